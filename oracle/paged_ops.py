@@ -1,0 +1,334 @@
+"""Torch (CPU) restatement of the reference's CPU semantics for the five ops on the
+paged-attention path.  TEST INFRASTRUCTURE: see ``oracle/__init__.py``.
+
+Every function names the reference lines it follows.  Shapes use
+B = users, Hq / Hkv = query / KV heads, D = head size, bs = block size,
+NB = physical blocks, W = page-table width.
+
+What pins each function (see tests/test_oracle_*.py):
+  paged_update_cache     brute-force per-(user, head) loop, negative index and
+                         padded-head cases, the reference's own parameter grid
+                         (tests/torch/ops/test_custom_ops.py:139-168)
+  paged_fill_cache       brute-force per-token loop over the reference's grid
+                         (test_custom_ops.py:171-203), tail block kept intact
+  paged_sdpa_decode      fp32 textbook attention over the first cur_pos+1 gathered
+                         tokens; GQA form against the chunked op with a 1-token chunk
+  chunked_sdpa           the reference's independent oracle and cases restated
+                         (tests/torch/ops/test_chunked_sdpa_op_cpu.py:27-147)
+  sdpa                   library routine (F.scaled_dot_product_attention)
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+
+
+# --------------------------------------------------------------------------- #
+# cache writes
+# --------------------------------------------------------------------------- #
+def paged_update_cache(
+    cache: torch.Tensor,
+    fill_value: torch.Tensor,
+    update_indices: torch.Tensor,
+    page_table: torch.Tensor,
+    share_cache: bool = False,
+) -> torch.Tensor:
+    """One-token-per-user scatter into a paged cache; functional (returns a copy).
+
+    Follows python_package/tt_torch/custom_ops.py:981-1000.
+    cache [NB, Hkv, bs, D]; fill_value [1, B, >=Hkv, D]; update_indices [B] (any int
+    dtype); page_table [B, W].  Index arithmetic is torch's floor division /
+    modulo, so position -1 means (column -1, offset bs-1), and column -1 is the
+    last page-table column (ordinary negative indexing).
+    """
+    out = cache.clone()
+    bs = out.shape[-2]
+    hkv = out.shape[-3]
+    users = update_indices.shape[0]
+    col = update_indices // bs
+    off = update_indices % bs
+    phys = page_table[torch.arange(users), col]
+    # two index tensors separated by a slice: the indexed dims move to the front,
+    # so the target view is [B, Hkv, D].
+    out[phys, :, off, :] = fill_value[0, :, :hkv, :]
+    return out
+
+
+def paged_fill_cache(
+    cache: torch.Tensor,
+    fill_value: torch.Tensor,
+    page_table: torch.Tensor,
+    batch_idx: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Block-wise prefill write for ONE user; functional.
+
+    Follows custom_ops.py:1037-1092.  cache [NB, Hkv, bs, D]; fill_value
+    [1, Hkv, S, D]; page_table [B, Wf]; batch_idx [1].  Writing always starts at
+    page-table column 0; the S // bs full blocks are replaced whole and the
+    S % bs remaining tokens go to the head of the next block, whose other rows keep
+    their old contents.
+    """
+    if batch_idx is None:
+        batch_idx = torch.tensor([0], dtype=torch.int32)
+    out = cache.clone()
+    bs = out.shape[-2]
+    s = fill_value.shape[-2]
+    h = fill_value.shape[-3]
+    d = fill_value.shape[-1]
+    row = page_table[batch_idx.item()]
+    n_full, rem = divmod(s, bs)
+    if n_full > 0:
+        body = fill_value[:, :, : n_full * bs, :]
+        # [1, H, n*bs, D] -> [n, H, bs, D]
+        body = body.reshape(1, h, n_full, bs, d).transpose(0, 2).reshape(n_full, h, bs, d)
+        out[row[:n_full]] = body
+    if rem > 0:
+        out[row[n_full : n_full + 1], :, :rem, :] = fill_value[:, :, s - rem :, :]
+    return out
+
+
+def paged_fill_cache_batched(
+    cache: torch.Tensor,
+    fill_value: torch.Tensor,
+    page_table: torch.Tensor,
+    batch_idx: torch.Tensor,
+) -> torch.Tensor:
+    """Batched prefill write: row i of fill_value [B, Hkv, S, D] goes through
+    page_table[batch_idx[i]].
+
+    The reference's CPU branch cannot run this form (``batch_idx.item()`` raises for
+    more than one element, custom_ops.py:1044); the plugin nevertheless calls the
+    device op this way (vllm_tt/attention_impls/attention.py:486-511).  The meaning
+    is fixed BY DEFINITION as the single-user op applied row by row, which is what
+    the MLA impl spells out (attention_impls/attention_mla.py:350-358).
+    """
+    out = cache
+    for i in range(fill_value.shape[0]):
+        out = paged_fill_cache(out, fill_value[i : i + 1], page_table, batch_idx[i : i + 1])
+    if fill_value.shape[0] == 0:
+        out = cache.clone()
+    return out
+
+
+def gather_paged_to_dense(cache: torch.Tensor, page_table: torch.Tensor) -> torch.Tensor:
+    """[NB, Hkv, bs, D] + [B, W] -> [B, Hkv, W*bs, D]; position p of user u is
+    block page_table[u, p // bs], row p % bs.
+
+    Follows attention.py:600-632 (without the final trim) and custom_ops.py:1387-1403.
+    """
+    users, w = page_table.shape
+    _, hkv, bs, d = cache.shape
+    g = torch.index_select(cache, 0, page_table.reshape(-1).long())
+    g = g.view(users, w, hkv, bs, d).permute(0, 2, 1, 3, 4).contiguous()
+    return g.reshape(users, hkv, w * bs, d)
+
+
+# --------------------------------------------------------------------------- #
+# decode attention
+# --------------------------------------------------------------------------- #
+def paged_sdpa_decode_mha(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    page_table: torch.Tensor,
+    cur_pos_tensor: torch.Tensor,
+    scale: Optional[float] = None,
+) -> torch.Tensor:
+    """The reference's causal decode branch, op by op, for Hq == Hkv.
+
+    Follows custom_ops.py:1256-1312: dense zero-initialised K/V of W*bs positions
+    per user, additive mask with -inf right of cur_pos, then
+    ``(q @ K^T) * scale + mask -> softmax -> @ V`` with every intermediate in the
+    query dtype.  query [1, B, H, D] -> [1, B, H, D].
+    """
+    bs = key.shape[-2]
+    h = key.shape[-3]
+    d = key.shape[-1]
+    users = cur_pos_tensor.shape[0]
+    w = page_table.shape[1]
+    span = w * bs
+    dt = query.dtype
+    mask = torch.zeros(users, span, dtype=dt)
+    dense_k = torch.zeros(users, h, span, d, dtype=dt)
+    dense_v = torch.zeros(users, h, span, d, dtype=dt)
+    for u in range(users):
+        blocks = page_table[u].long()
+        dense_k[u] = key[blocks].transpose(0, 1).reshape(h, span, d)
+        dense_v[u] = value[blocks].transpose(0, 1).reshape(h, span, d)
+        mask[u, int(cur_pos_tensor[u]) + 1 :] = float("-inf")
+    q = query.reshape(users, h, 1, d)
+    if scale is None:
+        scale = 1 / d**0.5
+    w_ = q @ dense_k.transpose(-2, -1) * scale
+    w_ += mask.reshape(users, 1, 1, span)
+    w_ = torch.softmax(w_, dim=-1)
+    out = w_ @ dense_v
+    return out.reshape(1, users, h, d)
+
+
+def paged_sdpa_decode_gqa(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    page_table: torch.Tensor,
+    cur_pos_tensor: torch.Tensor,
+    scale: Optional[float] = None,
+) -> torch.Tensor:
+    """Causal paged decode for Hq = G * Hkv (query head h reads KV head h // G).
+
+    The reference's own decode branch cannot run with Hq != Hkv (its
+    ``query.reshape(B, Hkv, 1, D)`` raises, custom_ops.py:1297).  This follows the
+    reference-held equivalent that does run grouped heads: the paged MLA decode CPU
+    branch with an explicit value cache, custom_ops.py:551-610 (gather, additive
+    -inf mask right of cur_pos, ``F.scaled_dot_product_attention(enable_gqa=True)``).
+    """
+    bs = key.shape[-2]
+    hkv = key.shape[-3]
+    d = key.shape[-1]
+    users = query.shape[1]
+    hq = query.shape[2]
+    span = page_table.shape[1] * bs
+    idx = page_table.long()
+    gk = key[idx].permute(0, 2, 1, 3, 4).reshape(users, hkv, span, d)
+    gv = value[idx].permute(0, 2, 1, 3, 4).reshape(users, hkv, span, value.shape[-1])
+    q = query.reshape(users, hq, 1, d)
+    mask = torch.zeros(users, 1, 1, span, dtype=query.dtype)
+    for u in range(users):
+        mask[u, :, :, int(cur_pos_tensor[u]) + 1 :] = float("-inf")
+    if scale is None:
+        scale = 1.0 / d**0.5
+    out = F.scaled_dot_product_attention(
+        q, gk, gv, mask, is_causal=False, scale=scale, enable_gqa=True
+    )
+    return out.reshape(1, users, hq, value.shape[-1])
+
+
+def paged_sdpa_decode(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    page_table: torch.Tensor,
+    is_causal: bool = False,
+    attn_mask: Optional[torch.Tensor] = None,
+    cur_pos_tensor: Optional[torch.Tensor] = None,
+    attention_sink: Optional[torch.Tensor] = None,
+    scale: Optional[float] = None,
+    sliding_window_size: Optional[int] = None,
+) -> torch.Tensor:
+    """Operator-level entry with the reference's argument list
+    (custom_ops.py:1203-1223).  ``attention_sink`` and ``sliding_window_size`` are
+    accepted and ignored, as on the reference's CPU branch.  Only the causal form
+    (the one the plugin issues, attention.py:646-664) is restated.
+    """
+    if is_causal:
+        assert attn_mask is None, "attention_mask must be None when is_causal is True."
+        assert cur_pos_tensor is not None, "cur_pos_tensor must be provided when is_causal is True."
+    else:
+        raise NotImplementedError("oracle restates the causal decode form only")
+    if query.shape[2] == key.shape[1]:
+        return paged_sdpa_decode_mha(query, key, value, page_table, cur_pos_tensor, scale)
+    return paged_sdpa_decode_gqa(query, key, value, page_table, cur_pos_tensor, scale)
+
+
+# --------------------------------------------------------------------------- #
+# prefill attention
+# --------------------------------------------------------------------------- #
+def chunked_sdpa(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    page_table: torch.Tensor,
+    chunk_start_idx_tensor: torch.Tensor,
+    scale: Optional[float] = None,
+) -> torch.Tensor:
+    """Chunked-prefill attention over the paged cache.
+
+    Follows custom_ops.py:1376-1429.  query [U, Hq, Lc, D]; row i of the chunk sits
+    at absolute position chunk_start + i and may see key position j iff
+    j <= chunk_start + i.  KV heads are repeated G times along the head dim; mask
+    and softmax run in the dtype of the score tensor.
+    """
+    users, hq, lc, d = query.shape
+    hkv = key.shape[1]
+    start = int(chunk_start_idx_tensor.reshape(-1)[0].item())
+    gk = gather_paged_to_dense(key, page_table)
+    gv = gather_paged_to_dense(value, page_table)
+    span = gk.shape[2]
+    if hkv != hq:
+        gk = gk.repeat_interleave(hq // hkv, dim=1)
+        gv = gv.repeat_interleave(hq // hkv, dim=1)
+    if scale is None:
+        scale = 1.0 / d**0.5
+    att = torch.matmul(query, gk.transpose(-2, -1)) * scale
+    qpos = start + torch.arange(lc).view(lc, 1)
+    kpos = torch.arange(span).view(1, span)
+    neg = torch.full((), float("-inf"), dtype=att.dtype)
+    zero = torch.zeros((), dtype=att.dtype)
+    att = att + torch.where(kpos <= qpos, zero, neg).view(1, 1, lc, span)
+    att = torch.softmax(att, dim=-1)
+    return torch.matmul(att, gv)
+
+
+def sdpa(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    attn_mask: Optional[torch.Tensor] = None,
+    is_causal: bool = True,
+    scale: Optional[float] = None,
+    sliding_window_size: Optional[int] = None,
+) -> torch.Tensor:
+    """Dense prefill attention with grouped heads.
+
+    Follows custom_ops.py:648-692 (argument checks) and :717-727 (the CPU branch is
+    the library routine with ``enable_gqa=True``; ``sliding_window_size`` ignored).
+    """
+    assert query.dim() == 4 and key.dim() == 4 and value.dim() == 4
+    assert key.shape == value.shape, "key and value must have the same shape."
+    assert key.shape[-1] == query.shape[-1], "key and query must have the same head size."
+    assert query.shape[1] % key.shape[1] == 0, "num_heads must be divisible by num_kv_heads."
+    assert query.shape[2] % 32 == 0, (
+        f"query sequence length must be divisible by 32 but got {query.shape[2]}."
+    )
+    assert query.shape[0] == key.shape[0], "query and key must have the same batch size."
+    if attn_mask is not None:
+        assert is_causal is False, "is_causal attribute can't be True if attn_mask is available."
+        assert query.shape[0] == attn_mask.shape[0]
+    return F.scaled_dot_product_attention(
+        query, key, value, attn_mask, is_causal=is_causal, scale=scale, enable_gqa=True
+    )
+
+
+# --------------------------------------------------------------------------- #
+# independent fp32 forms used by tests to pin the restatements above
+# --------------------------------------------------------------------------- #
+def textbook_decode_fp32(query, key, value, page_table, cur_pos, scale=None):
+    """softmax(q K^T * scale) V in fp32 over exactly the first cur_pos+1 tokens of
+    each user, one (user, head) at a time.  No masks, no padding: a plain loop.
+    Returns fp32 [1, B, Hq, D]; rows with cur_pos < 0 are NaN.
+    """
+    _, users, hq, d = query.shape
+    hkv, bs = key.shape[1], key.shape[2]
+    g = hq // hkv
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    out = torch.full((1, users, hq, value.shape[-1]), float("nan"), dtype=torch.float32)
+    for u in range(users):
+        n = int(cur_pos[u]) + 1
+        if n <= 0:
+            continue
+        n = min(n, page_table.shape[1] * bs)
+        pos = torch.arange(n)
+        blk = page_table[u, pos // bs].long()
+        off = pos % bs
+        for h in range(hq):
+            k = key[blk, h // g, off, :].float()  # [n, D]
+            v = value[blk, h // g, off, :].float()
+            s = (k @ query[0, u, h].float()) * scale
+            p = torch.softmax(s, dim=0)
+            out[0, u, h] = p @ v
+    return out
