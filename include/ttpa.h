@@ -1,0 +1,166 @@
+/*
+ * ttpa — paged KV-cache write and paged attention for MI355X (gfx950).
+ *
+ * C ABI of libttpa.so.  These entry points are what the device branch of the
+ * reference's five custom ops binds to; each comment names the reference
+ * interface the function replaces (paths relative to the tt-xla tree).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *   - activations and bf16 caches are bfloat16, indices int32 unless an
+ *     `_is_i64` flag says otherwise; strides are in ELEMENTS, the innermost
+ *     (head_size) dimension is always contiguous;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - calls only enqueue work: they never synchronise, never allocate and never
+ *     touch the caller's buffers from the host;
+ *   - return value: TTPA_OK, or a negative TTPA_ERR_*; ttpa_last_error() returns
+ *     a thread-local, human-readable reason for the last failure.
+ *
+ * Cache layout (reference: TTAttentionBackend.get_kv_cache_shape,
+ * integrations/vllm_plugin/vllm_tt/attention_impls/attention.py:104-112):
+ *   TTPA_KV_BF16  bfloat16 [num_blocks, kv_heads, block_size, head_size]
+ *   TTPA_KV_BFP8  uint8    [num_blocks, kv_heads, block_size + block_size/16, head_size]
+ *                 rows 0..block_size-1: one byte (sign<<7 | 7-bit magnitude) per element;
+ *                 the remaining bytes, read as [block_size][head_size/16], hold one
+ *                 shared exponent byte per 16 consecutive head_size elements;
+ *                 value = (-1)^s * m * 2^(e - 133).
+ * K and V are two separate tensors of that layout.
+ */
+#ifndef TTPA_H_
+#define TTPA_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TTPA_ABI_VERSION 1
+
+#define TTPA_OK 0
+#define TTPA_ERR_INVALID_ARGUMENT (-1) /* shape / stride / alignment the kernels cannot take */
+#define TTPA_ERR_UNSUPPORTED (-2)      /* valid request, no kernel instantiated for it */
+#define TTPA_ERR_WORKSPACE (-3)        /* workspace missing or too small */
+#define TTPA_ERR_LAUNCH (-4)           /* HIP reported an error at launch */
+
+#define TTPA_KV_BF16 0
+#define TTPA_KV_BFP8 1
+
+int ttpa_abi_version(void);
+const char *ttpa_last_error(void);
+
+/* Number of compute units of the current device (used to size persistent grids). */
+int ttpa_device_compute_units(void);
+
+/*
+ * One-token-per-user scatter, IN PLACE on `cache`.
+ * Replaces the device branch of tt::paged_update_cache
+ * (python_package/tt_torch/custom_ops.py:962-1002; CPU semantics :981-1000):
+ *   col = floor(idx[u] / block_size), off = idx[u] mod block_size (floor semantics,
+ *   col < 0 wraps once by table_width like a negative Python index);
+ *   cache[page_table[u, col], h, off, :] = fill[u, h, :]  for h < kv_heads.
+ * fill is the [1, users, >=kv_heads, head_size] operand addressed through
+ * fill_user_stride / fill_head_stride.  Users whose column or physical block falls
+ * outside the table / the cache are skipped (the reference raises IndexError).
+ * With TTPA_KV_BFP8 the bf16 row is encoded on the way in.
+ * The functional form of the op (fresh result tensor) is clone + this call.
+ */
+int ttpa_paged_update_cache(void *cache, const void *fill, int64_t fill_user_stride,
+                            int64_t fill_head_stride, const void *update_indices,
+                            int indices_is_i64, const int32_t *page_table,
+                            int64_t page_table_row_stride, int32_t users, int32_t kv_heads,
+                            int32_t block_size, int32_t head_size, int32_t table_width,
+                            int32_t num_blocks, int32_t kv_format, void *stream);
+
+/*
+ * Block-wise prefill write, IN PLACE on `cache`.
+ * Replaces the device branch of tt::paged_fill_cache (custom_ops.py:1016-1094; CPU
+ * semantics for one user :1037-1092; batched call site
+ * vllm_tt/attention_impls/attention.py:486-511):
+ *   for i < fill_users, t < seq_len:
+ *     cache[page_table[batch_idx[i], t / block_size], h, t % block_size, :] = fill[i, h, t, :]
+ * Writing always starts at table column 0; rows of the last block past seq_len keep
+ * their contents.  batch_idx may be NULL (= user 0, fill_users must then be 1).
+ * seq_len > table_width * block_size is rejected.  batch_idx values outside
+ * [0, table_rows) and physical blocks outside the cache are skipped.
+ */
+int ttpa_paged_fill_cache(void *cache, const void *fill, int64_t fill_user_stride,
+                          int64_t fill_head_stride, int64_t fill_token_stride,
+                          const int32_t *page_table, int64_t page_table_row_stride,
+                          const void *batch_idx, int batch_idx_is_i64, int32_t fill_users,
+                          int32_t table_rows, int32_t kv_heads, int32_t seq_len,
+                          int32_t block_size, int32_t head_size, int32_t table_width,
+                          int32_t num_blocks, int32_t kv_format, void *stream);
+
+/*
+ * Causal paged decode attention, one query token per user.
+ * Replaces the device branch of tt::paged_scaled_dot_product_attention_decode
+ * (custom_ops.py:1198-1315; CPU semantics :1256-1312, grouped heads as in :551-610):
+ *   out[u, hq, :] = softmax_j( scale * q[u, hq, :] . K[u, hq / G, j, :] ) . V[u, hq / G, j, :]
+ *   over cache positions j = 0 .. min(cur_pos[u], table_width * block_size - 1),
+ *   position j living in block page_table[u, j / block_size], row j % block_size.
+ * cur_pos[u] < 0 (padded batch row) gives a NaN output row, as on the reference.
+ * Physical block ids outside [0, num_blocks) are read as block 0.
+ * `workspace` holds split-K partial results: at least
+ * ttpa_paged_decode_workspace_bytes(...) bytes, 256-byte aligned, private to this
+ * call until the stream reaches its end.
+ */
+size_t ttpa_paged_decode_workspace_bytes(int32_t users, int32_t q_heads, int32_t kv_heads,
+                                         int32_t head_size);
+
+int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_t out_head_stride,
+                           const void *q, int64_t q_user_stride, int64_t q_head_stride,
+                           const void *k_cache, const void *v_cache,
+                           const int32_t *page_table, int64_t page_table_row_stride,
+                           const void *cur_pos, int cur_pos_is_i64, int32_t users,
+                           int32_t q_heads, int32_t kv_heads, int32_t head_size,
+                           int32_t block_size, int32_t table_width, int32_t num_blocks,
+                           float scale, int32_t kv_format, void *workspace,
+                           size_t workspace_bytes, void *stream);
+
+/*
+ * Prefill attention (bf16 MFMA), dense or paged K/V, grouped heads.
+ * Replaces the device branches of
+ *   tt::scaled_dot_product_attention        (custom_ops.py:635-729; CPU :717-727) and
+ *   tt::chunked_scaled_dot_product_attention (custom_ops.py:1334-1431; CPU :1376-1429).
+ *   out[b, hq, i, :] = softmax_j( scale * q[b,hq,i,:] . K[b, hq/G, j, :] + mask ) . V[b, hq/G, j, :]
+ * Dense form: page_table == NULL, k / v are [batch, kv_heads, kv_len, head_size]
+ *   addressed by the kv_* strides.
+ * Paged form: page_table != NULL, k / v are caches (bf16 layout above), kv_len is
+ *   ignored and the keys of user b are positions 0 .. table_width*block_size-1.
+ * Masking: causal != 0 allows key j for query row i iff j <= offset + i, where offset
+ *   is *chunk_start (device int32, may be NULL = 0) in the paged form and 0 in the
+ *   dense form (the library routine's top-left aligned causal mask).  `mask` (may be
+ *   NULL, requires causal == 0) is an additive bf16 mask [batch, 1, q_len, kv_len]
+ *   addressed by mask_batch_stride / mask_row_stride.
+ */
+int ttpa_sdpa_prefill(void *out, int64_t out_batch_stride, int64_t out_head_stride,
+                      int64_t out_token_stride, const void *q, int64_t q_batch_stride,
+                      int64_t q_head_stride, int64_t q_token_stride, const void *k,
+                      const void *v, int64_t kv_batch_stride, int64_t kv_head_stride,
+                      int64_t kv_token_stride, const int32_t *page_table,
+                      int64_t page_table_row_stride, const int32_t *chunk_start,
+                      const void *mask, int64_t mask_batch_stride, int64_t mask_row_stride,
+                      int32_t batch, int32_t q_heads, int32_t kv_heads, int32_t q_len,
+                      int32_t kv_len, int32_t head_size, int32_t block_size,
+                      int32_t table_width, int32_t num_blocks, int32_t causal, float scale,
+                      void *stream);
+
+/*
+ * Block-float-8 codec on flat arrays (n_elems % 16 == 0), for tests and cache
+ * conversion.  No reference counterpart: the reference forwards
+ * experimental_kv_cache_dtype="bfp_bf8" to an un-vendored compiler
+ * (vllm_tt/platform.py:165; pjrt_implementation/src/api/module_builder/module_builder.cc:1050-1063).
+ *   quantize:   bf16[n] -> elem uint8[n], exps uint8[n/16]
+ *   dequantize: -> bf16[n] (exact: 7-bit magnitudes fit bfloat16)
+ */
+int ttpa_bfp8_quantize(const void *src_bf16, void *elem_u8, void *exps_u8, int64_t n_elems,
+                       void *stream);
+int ttpa_bfp8_dequantize(const void *elem_u8, const void *exps_u8, void *dst_bf16,
+                         int64_t n_elems, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TTPA_H_ */

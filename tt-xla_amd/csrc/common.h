@@ -1,0 +1,95 @@
+// Shared host/device helpers for libttpa (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ttpa.h"
+
+namespace ttpa {
+
+// ---- host side -------------------------------------------------------------
+// Records a printf-style message for ttpa_last_error() and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int check_launch(const char *what);
+int device_cus();
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+#define TTPA_REQUIRE(cond, ...)                                            \
+  do {                                                                     \
+    if (!(cond)) return ::ttpa::fail(TTPA_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
+  } while (0)
+
+// ---- device side -----------------------------------------------------------
+constexpr int kWave = 64;
+
+// DPP controls valid on gfx9: each moves data inside a row of 16 lanes.
+constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane ^ 7
+constexpr int kDppMirror = 0x140;     // lane ^ 15
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) {
+  return __builtin_bit_cast(float, w & 0xffff0000u);
+}
+
+// float -> bfloat16 bits, round to nearest even (NaN stays NaN).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+__device__ __forceinline__ int64_t load_index(const void *p, int is_i64, int64_t i) {
+  return is_i64 ? static_cast<const int64_t *>(p)[i]
+                : static_cast<int64_t>(static_cast<const int32_t *>(p)[i]);
+}
+
+// ---- block-float-8 ---------------------------------------------------------
+// Encodes 16 bfloat16 values held as 8 packed dwords (element 2j in the low half of
+// w[j]).  Returns the shared exponent; out[0..3] receive the 16 element bytes.
+__device__ __forceinline__ uint32_t bfp8_encode16(const uint32_t (&w)[8], uint32_t (&out)[4]) {
+  uint32_t emax = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    uint32_t e0 = (w[j] >> 7) & 0xffu, e1 = (w[j] >> 23) & 0xffu;
+    emax = max(emax, max(e0, e1));
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) out[j] = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    uint32_t h = (i & 1) ? (w[i >> 1] >> 16) : (w[i >> 1] & 0xffffu);
+    uint32_t ex = (h >> 7) & 0xffu;
+    uint32_t sig = ex ? (0x80u | (h & 0x7fu)) : 0u;
+    uint32_t sh = min(emax - ex + 1u, 16u);
+    uint32_t q = sig >> sh;
+    uint32_t rem = sig & ((1u << sh) - 1u);
+    uint32_t half = 1u << (sh - 1u);
+    q += (rem > half || (rem == half && (q & 1u))) ? 1u : 0u;
+    q = min(q, 127u);
+    uint32_t byte = ((h >> 8) & 0x80u) | q;
+    out[i >> 2] |= byte << (8 * (i & 3));
+  }
+  return emax;
+}
+
+// Decodes one element byte with shared exponent e to float: (-1)^s * m * 2^(e-133).
+__device__ __forceinline__ float bfp8_decode(uint32_t byte, float group_scale) {
+  float m = static_cast<float>(byte & 0x7fu) * group_scale;
+  return (byte & 0x80u) ? -m : m;
+}
+__device__ __forceinline__ float bfp8_group_scale(uint32_t e) {
+  return __builtin_ldexpf(1.0f, static_cast<int>(e) - 133);
+}
+
+}  // namespace ttpa

@@ -1,0 +1,549 @@
+// Paged decode attention: split-K over a flattened list of 64-token tiles.
+//
+// Work decomposition
+//   A tile is 64 consecutive cache positions of one (user, kv_head) segment.  All
+//   tiles of all segments form one flat list ordered (user, kv_head, tile); the
+//   list is cut into n_waves equal ranges and every wavefront streams exactly one
+//   range, so ragged context lengths cost no imbalance.  A wavefront emits one
+//   partial result (un-normalised output, running max, running sum) per segment
+//   its range touches; a second kernel merges the partials of each segment.
+//
+// Inside a wavefront (lane = 16 * r + c)
+//   A K or V tile is read with 16 wide loads; load i gives lane (r, c) the
+//   head_size/16 elements c of token 4 i + r, so every load instruction covers 4
+//   whole token rows contiguously.  q.k is a per-lane partial dot product
+//   (v_dot2_f32_bf16) that must be summed over the 16 lanes c of a row; the 16
+//   loads of a tile are summed with a DPP reduce-scatter, after which lane (r, c)
+//   holds the score of ONE token for each of the G query heads of the group.
+//   The 16 lanes with equal r therefore own every fourth token: each such row of
+//   lanes runs its own online softmax and its own accumulators (4 streams per
+//   wavefront, merged once per segment).  Probabilities go through a wave-private
+//   LDS buffer so that lane (r, c) can read the weight of token 4 i + r when it
+//   multiplies its V elements.
+//   The G query heads of a group share every K/V load: each element is read once
+//   per KV head.
+#include "common.h"
+
+namespace ttpa {
+namespace {
+
+constexpr int kMaxUsers = 4096;
+constexpr int kTile = 64;
+constexpr int kWavesPerBlock = 4;
+
+struct DecodeArgs {
+  uint16_t *out;
+  int64_t out_us, out_hs;
+  const uint16_t *q;
+  int64_t q_us, q_hs;
+  const uint8_t *k, *v;
+  const int32_t *pt;
+  int64_t pt_rs;
+  const void *cur;
+  int cur_i64;
+  int users, hq, hkv, bs, w, nb;
+  float scale_log2e;
+  int *ws_pref;  // [users + 1] exclusive prefix of tile counts
+  float *ws_slots;
+  int n_waves;
+  int slot_floats;
+};
+
+__device__ __forceinline__ int tiles_of_user(const DecodeArgs &a, int u, int &len) {
+  int64_t cp = load_index(a.cur, a.cur_i64, u);
+  int64_t cap = (int64_t)a.w * a.bs;
+  int64_t l = cp < 0 ? 0 : (cp + 1 < cap ? cp + 1 : cap);
+  len = (int)l;
+  return (int)((l + kTile - 1) / kTile);
+}
+
+// Exclusive prefix sum of per-user tile counts into pref[0..users]; all 256 threads.
+__device__ void build_prefix(const DecodeArgs &a, int *pref, int *wave_sums) {
+  const int tid = threadIdx.x;
+  const int per = (a.users + 255) / 256;
+  const int beg = tid * per;
+  const int end = min(beg + per, a.users);
+  int local = 0, len;
+  for (int u = beg; u < end; ++u) local += tiles_of_user(a, u, len);
+  int incl = local;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    int o = __shfl_up(incl, d);
+    if ((tid & 63) >= d) incl += o;
+  }
+  if ((tid & 63) == 63) wave_sums[tid >> 6] = incl;
+  __syncthreads();
+  int base = 0;
+  for (int wv = 0; wv < (tid >> 6); ++wv) base += wave_sums[wv];
+  int run = base + incl - local;
+  if (tid == 0) pref[0] = 0;
+  for (int u = beg; u < end; ++u) {
+    run += tiles_of_user(a, u, len);
+    pref[u + 1] = run;
+  }
+  __syncthreads();
+}
+
+template <int DW>
+__device__ __forceinline__ void load_dwords(const uint16_t *p, uint32_t (&d)[DW]) {
+  if constexpr (DW == 4) {
+    uint4 t = *reinterpret_cast<const uint4 *>(p);
+    d[0] = t.x, d[1] = t.y, d[2] = t.z, d[3] = t.w;
+  } else {
+    uint2 t = *reinterpret_cast<const uint2 *>(p);
+    d[0] = t.x, d[1] = t.y;
+  }
+}
+
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf2;
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, a), __builtin_bit_cast(bf2, b), c,
+                                         false);
+}
+
+// Level L of the reduce-scatter exchanges along one lane bit inside a row of 16.
+// The exchange pattern of a level may flip lane bits that LATER levels partition on,
+// never earlier ones: mirror (^15) splits on bit 3, half-mirror (^7) on bit 2, then
+// ^2 on bit 1 and ^1 on bit 0.  After four levels lane c holds load bitrev4(c).
+template <int LEVEL>
+__device__ __forceinline__ float rs_exchange(float v) {
+  if constexpr (LEVEL == 1) return dpp_move<kDppMirror>(v);
+  if constexpr (LEVEL == 2) return dpp_move<kDppHalfMirror>(v);
+  if constexpr (LEVEL == 3) return dpp_move<kDppXor2>(v);
+  return dpp_move<kDppXor1>(v);
+}
+
+template <int LEVEL, int BASE, int G, int NH, int DW>
+__device__ __forceinline__ void qk_reduce_scatter(const uint32_t (&k)[NH][16][DW],
+                                                  const uint32_t (&q)[G][NH][DW], int c,
+                                                  float (&s)[G]) {
+  if constexpr (LEVEL == 0) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float acc = 0.f;
+#pragma unroll
+      for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+        for (int j = 0; j < DW; ++j) acc = dot2(k[hf][BASE][j], q[g][hf][j], acc);
+      s[g] = acc;
+    }
+  } else {
+    float lo[G], hi[G];
+    qk_reduce_scatter<LEVEL - 1, BASE, G, NH, DW>(k, q, c, lo);
+    qk_reduce_scatter<LEVEL - 1, BASE + (1 << (LEVEL - 1)), G, NH, DW>(k, q, c, hi);
+    const bool upper = (c >> (4 - LEVEL)) & 1;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float keep = upper ? hi[g] : lo[g];
+      float send = upper ? lo[g] : hi[g];
+      s[g] = keep + rs_exchange<LEVEL>(send);
+    }
+  }
+}
+
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_move<kDppXor1>(v));
+  v = fmaxf(v, dpp_move<kDppXor2>(v));
+  v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+  v = fmaxf(v, dpp_move<kDppMirror>(v));
+  return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_move<kDppXor1>(v);
+  v += dpp_move<kDppXor2>(v);
+  v += dpp_move<kDppHalfMirror>(v);
+  v += dpp_move<kDppMirror>(v);
+  return v;
+}
+
+__device__ __forceinline__ int bitrev4(int c) {
+  return ((c & 1) << 3) | ((c & 2) << 1) | ((c & 4) >> 1) | ((c & 8) >> 3);
+}
+
+template <int D, int G>
+struct Shape {
+  static constexpr int HD = D > 128 ? 128 : D;  // elements covered by one load pass
+  static constexpr int NH = D / HD;
+  static constexpr int EPL = HD / 16;  // elements per lane per pass
+  static constexpr int DW = EPL / 2;
+  static constexpr int GP = G <= 2 ? G : ((G + 3) / 4) * 4;  // padded heads in LDS
+};
+
+template <int D, int G>
+__global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeArgs a) {
+  using S = Shape<D, G>;
+  constexpr int NH = S::NH, EPL = S::EPL, DW = S::DW, GP = S::GP;
+
+  __shared__ int s_pref[kMaxUsers + 1];
+  __shared__ int s_wsum[kWavesPerBlock];
+  __shared__ float s_p[kWavesPerBlock][kTile * GP];
+
+  build_prefix(a, s_pref, s_wsum);
+  if (blockIdx.x == 0) {
+    for (int i = threadIdx.x; i <= a.users; i += 256) a.ws_pref[i] = s_pref[i];
+  }
+
+  const int lane = threadIdx.x & 63;
+  const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane >> 4, c = lane & 15;
+  const int wave = blockIdx.x * kWavesPerBlock + wib;
+  const int64_t total = (int64_t)__builtin_amdgcn_readfirstlane(s_pref[a.users]) * a.hkv;
+  int64_t x = (int64_t)wave * total / a.n_waves;
+  const int64_t x_hi = (int64_t)(wave + 1) * total / a.n_waves;
+  float *plds = s_p[wib];
+  const int my_step = bitrev4(c);
+  const int64_t row_elems = D;  // elements per token row in the cache
+
+  while (x < x_hi) {
+    // ---- locate the segment that owns unit x (uniform) -------------------------
+    int lo_u = 0, hi_u = a.users - 1;
+    while (lo_u < hi_u) {
+      int mid = (lo_u + hi_u + 1) >> 1;
+      if ((int64_t)__builtin_amdgcn_readfirstlane(s_pref[mid]) * a.hkv <= x) lo_u = mid; else hi_u = mid - 1;
+    }
+    const int u = lo_u;
+    const int pref_u = __builtin_amdgcn_readfirstlane(s_pref[u]);
+    const int nt = __builtin_amdgcn_readfirstlane(s_pref[u + 1]) - pref_u;
+    const int rem = (int)(x - (int64_t)pref_u * a.hkv);  // < nt * hkv
+    const int h = rem / nt;
+    int t = rem - h * nt;
+    const int64_t seg_end = x + (nt - t);
+    const int64_t x_end = seg_end < x_hi ? seg_end : x_hi;
+    int len;
+    tiles_of_user(a, u, len);
+    len = __builtin_amdgcn_readfirstlane(len);
+
+    // ---- query registers: q[g][pass][DW] ---------------------------------------
+    uint32_t q[G][NH][DW];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int hf = 0; hf < NH; ++hf)
+        load_dwords<DW>(a.q + u * a.q_us + (int64_t)(h * G + g) * a.q_hs + hf * S::HD + c * EPL,
+                        q[g][hf]);
+
+    float m[G], l[G], acc[G][NH][EPL];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      m[g] = -INFINITY;
+      l[g] = 0.f;
+#pragma unroll
+      for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) acc[g][hf][e] = 0.f;
+    }
+
+    const int32_t *pt_row = a.pt + (int64_t)u * a.pt_rs;
+    const bool big_block = (a.bs % kTile) == 0;
+
+    for (; x < x_end; ++x, ++t) {
+      const int tok0 = t * kTile;
+      const int nvalid = len - tok0;  // >= 1
+      const bool full = nvalid >= kTile;
+
+      // element offset of the first token row of each load, relative to the cache base
+      int64_t off[16];
+      if (big_block) {
+        int phys = __builtin_amdgcn_readfirstlane(pt_row[tok0 / a.bs]);
+        if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+        int64_t base = (((int64_t)phys * a.hkv + h) * a.bs + (tok0 % a.bs)) * row_elems;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) off[i] = base + (int64_t)i * 4 * row_elems;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          int tk = tok0 + 4 * i;
+          int col = tk / a.bs;
+          int phys = (col < a.w) ? __builtin_amdgcn_readfirstlane(pt_row[col]) : 0;
+          if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+          off[i] = (((int64_t)phys * a.hkv + h) * a.bs + (tk % a.bs)) * row_elems;
+        }
+      }
+      const int64_t lane_off = (int64_t)r * row_elems + c * EPL;
+
+      uint32_t kreg[NH][16][DW], vreg[NH][16][DW];
+      const uint16_t *kb = reinterpret_cast<const uint16_t *>(a.k);
+      const uint16_t *vb = reinterpret_cast<const uint16_t *>(a.v);
+#pragma unroll
+      for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          if (full || 4 * i + r < nvalid) {
+            load_dwords<DW>(kb + off[i] + lane_off + hf * S::HD, kreg[hf][i]);
+          } else {
+#pragma unroll
+            for (int j = 0; j < DW; ++j) kreg[hf][i][j] = 0;
+          }
+        }
+      if constexpr (NH == 1) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          if (full || 4 * i + r < nvalid) {
+            load_dwords<DW>(vb + off[i] + lane_off, vreg[0][i]);
+          } else {
+#pragma unroll
+            for (int j = 0; j < DW; ++j) vreg[0][i][j] = 0;
+          }
+        }
+      }
+
+      // ---- scores: lane (r, c) ends with token tok0 + 4 * bitrev4(c) + r --------
+      float s[G];
+      qk_reduce_scatter<4, 0, G, NH, DW>(kreg, q, c, s);
+      const bool valid = full || (4 * my_step + r < nvalid);
+      float p[G];
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float sv = valid ? s[g] * a.scale_log2e : -INFINITY;
+        float mx = fmaxf(m[g], row16_max(sv));
+        float msafe = (mx == -INFINITY) ? 0.f : mx;
+        float alpha = __builtin_amdgcn_exp2f(m[g] - msafe);
+        p[g] = __builtin_amdgcn_exp2f(sv - msafe);
+        l[g] = l[g] * alpha + p[g];
+        m[g] = mx;
+#pragma unroll
+        for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) acc[g][hf][e] *= alpha;
+      }
+      // publish the weights: plds[(r * 16 + step) * GP + g]
+      {
+        float *dst = plds + (r * 16 + my_step) * GP;
+#pragma unroll
+        for (int g = 0; g < G; ++g) dst[g] = p[g];
+      }
+
+      if constexpr (NH == 2) {
+        // head_size 256: V is fetched only now, one 128-element half at a time
+#pragma unroll
+        for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            if (full || 4 * i + r < nvalid) {
+              load_dwords<DW>(vb + off[i] + lane_off + hf * S::HD, vreg[hf][i]);
+            } else {
+#pragma unroll
+              for (int j = 0; j < DW; ++j) vreg[hf][i][j] = 0;
+            }
+          }
+      }
+
+      // ---- output accumulation ---------------------------------------------------
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float w[GP];
+        const float *src = plds + (r * 16 + i) * GP;
+        if constexpr (GP % 4 == 0) {
+#pragma unroll
+          for (int g4 = 0; g4 < GP / 4; ++g4) {
+            float4 t4 = *reinterpret_cast<const float4 *>(src + 4 * g4);
+            w[4 * g4] = t4.x, w[4 * g4 + 1] = t4.y, w[4 * g4 + 2] = t4.z, w[4 * g4 + 3] = t4.w;
+          }
+        } else {
+#pragma unroll
+          for (int g = 0; g < GP; ++g) w[g] = src[g];
+        }
+#pragma unroll
+        for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+          for (int j = 0; j < DW; ++j) {
+            float v0 = bf16_lo(vreg[hf][i][j]), v1 = bf16_hi(vreg[hf][i][j]);
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+              acc[g][hf][2 * j] = fmaf(w[g], v0, acc[g][hf][2 * j]);
+              acc[g][hf][2 * j + 1] = fmaf(w[g], v1, acc[g][hf][2 * j + 1]);
+            }
+          }
+      }
+    }
+
+    // ---- merge the 4 lane rows and write the partial of this (wave, segment) -----
+    float *slot = a.ws_slots + ((int64_t)wave + (int64_t)u * a.hkv + h) * a.slot_floats;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float lr = row16_sum(l[g]);
+      float mr = m[g];
+      float mall = fmaxf(mr, __shfl_xor(mr, 16));
+      mall = fmaxf(mall, __shfl_xor(mall, 32));
+      float wgt = (mr == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mr - mall);
+      lr *= wgt;
+      lr += __shfl_xor(lr, 16);
+      lr += __shfl_xor(lr, 32);
+#pragma unroll
+      for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+          float v = acc[g][hf][e] * wgt;
+          v += __shfl_xor(v, 16);
+          v += __shfl_xor(v, 32);
+          acc[g][hf][e] = v;
+        }
+      if (r == 0) {
+#pragma unroll
+        for (int hf = 0; hf < NH; ++hf) {
+          float *dst = slot + g * D + hf * S::HD + c * EPL;
+#pragma unroll
+          for (int e4 = 0; e4 < EPL / 4; ++e4)
+            *reinterpret_cast<float4 *>(dst + 4 * e4) =
+                make_float4(acc[g][hf][4 * e4], acc[g][hf][4 * e4 + 1], acc[g][hf][4 * e4 + 2],
+                            acc[g][hf][4 * e4 + 3]);
+        }
+        if (c == 0) {
+          slot[G * D + g] = mall;
+          slot[G * D + G + g] = lr;
+        }
+      }
+    }
+  }
+}
+
+// Merges the partials of one (user, kv_head) segment and writes bfloat16 output.
+template <int D, int G>
+__global__ __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a) {
+  const int seg = blockIdx.x;
+  const int u = seg / a.hkv, h = seg % a.hkv;
+  const int nt = a.ws_pref[u + 1] - a.ws_pref[u];
+  const int64_t total = (int64_t)a.ws_pref[a.users] * a.hkv;
+  uint16_t *out = a.out + u * a.out_us;
+  if (nt == 0) {  // padded row: no attended position -> NaN like softmax of all -inf
+    for (int i = threadIdx.x; i < G * D; i += 256)
+      out[(int64_t)(h * G + i / D) * a.out_hs + (i % D)] = 0x7fc0;
+    return;
+  }
+  const int64_t x0 = (int64_t)a.ws_pref[u] * a.hkv + (int64_t)h * nt;
+  const int64_t x1 = x0 + nt - 1;
+  // wave owning unit x: largest w with floor(w * total / n) <= x
+  const int w0 = (int)(((x0 + 1) * a.n_waves + total - 1) / total) - 1;
+  const int w1 = (int)(((x1 + 1) * a.n_waves + total - 1) / total) - 1;
+  const float *slots = a.ws_slots;
+  for (int i = threadIdx.x; i < G * D; i += 256) {
+    const int g = i / D;
+    float mall = -INFINITY;
+    for (int w = w0; w <= w1; ++w) {
+      if ((int64_t)w * total / a.n_waves == (int64_t)(w + 1) * total / a.n_waves) continue;
+      mall = fmaxf(mall, slots[((int64_t)w + seg) * a.slot_floats + G * D + g]);
+    }
+    float num = 0.f, den = 0.f;
+    for (int w = w0; w <= w1; ++w) {
+      if ((int64_t)w * total / a.n_waves == (int64_t)(w + 1) * total / a.n_waves) continue;
+      const float *sl = slots + ((int64_t)w + seg) * a.slot_floats;
+      float wgt = __builtin_amdgcn_exp2f(sl[G * D + g] - mall);
+      num = fmaf(wgt, sl[i], num);
+      den = fmaf(wgt, sl[G * D + G + g], den);
+    }
+    out[(int64_t)(h * G + g) * a.out_hs + (i % D)] = (uint16_t)f32_to_bf16_bits(num / den);
+  }
+}
+
+int slot_floats_for(int g, int d) { return ((g * d + 2 * g + 3) / 4) * 4; }
+size_t header_bytes(int users) { return (((size_t)(users + 1) * 4 + 255) / 256) * 256; }
+
+int waves_for_device() {
+  static int override_waves = -1;
+  if (override_waves < 0) {
+    const char *e = getenv("TTPA_DECODE_WAVES_PER_CU");
+    override_waves = e ? atoi(e) : 0;
+  }
+  int per_cu = override_waves > 0 ? override_waves : 8;
+  int cus = device_cus();
+  if (cus <= 0) cus = 256;
+  int waves = cus * per_cu;
+  return (waves + kWavesPerBlock - 1) / kWavesPerBlock * kWavesPerBlock;
+}
+
+template <int D, int G>
+void launch(const DecodeArgs &a, hipStream_t st) {
+  paged_decode_kernel<D, G><<<dim3(a.n_waves / kWavesPerBlock), dim3(256), 0, st>>>(a);
+  decode_combine_kernel<D, G><<<dim3(a.users * a.hkv), dim3(256), 0, st>>>(a);
+}
+
+template <int D>
+int launch_g(const DecodeArgs &a, int g, hipStream_t st) {
+  switch (g) {
+    case 1: launch<D, 1>(a, st); break;
+    case 2: launch<D, 2>(a, st); break;
+    case 3: launch<D, 3>(a, st); break;
+    case 4: launch<D, 4>(a, st); break;
+    case 5: launch<D, 5>(a, st); break;
+    case 6: launch<D, 6>(a, st); break;
+    case 7: launch<D, 7>(a, st); break;
+    case 8: launch<D, 8>(a, st); break;
+    default:
+      return fail(TTPA_ERR_UNSUPPORTED, "query heads per KV head = %d; supported 1..8", g);
+  }
+  return TTPA_OK;
+}
+
+}  // namespace
+}  // namespace ttpa
+
+using namespace ttpa;
+
+extern "C" size_t ttpa_paged_decode_workspace_bytes(int32_t users, int32_t q_heads,
+                                                    int32_t kv_heads, int32_t head_size) {
+  if (users <= 0 || q_heads <= 0 || kv_heads <= 0 || head_size <= 0 || q_heads % kv_heads) return 0;
+  int g = q_heads / kv_heads;
+  size_t slots = (size_t)waves_for_device() + (size_t)users * kv_heads;
+  return header_bytes(users) + slots * (size_t)slot_floats_for(g, head_size) * sizeof(float);
+}
+
+extern "C" int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_t out_head_stride,
+                                      const void *q, int64_t q_user_stride, int64_t q_head_stride,
+                                      const void *k_cache, const void *v_cache,
+                                      const int32_t *page_table, int64_t page_table_row_stride,
+                                      const void *cur_pos, int cur_pos_is_i64, int32_t users,
+                                      int32_t q_heads, int32_t kv_heads, int32_t head_size,
+                                      int32_t block_size, int32_t table_width, int32_t num_blocks,
+                                      float scale, int32_t kv_format, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
+  TTPA_REQUIRE(out && q && k_cache && v_cache && page_table && cur_pos, "null pointer argument");
+  TTPA_REQUIRE(users > 0 && q_heads > 0 && kv_heads > 0 && head_size > 0 && block_size > 0 &&
+                   table_width > 0 && num_blocks > 0,
+               "non-positive dimension");
+  TTPA_REQUIRE(q_heads % kv_heads == 0, "q_heads %d not divisible by kv_heads %d", q_heads,
+               kv_heads);
+  if (kv_format != TTPA_KV_BF16)
+    return fail(TTPA_ERR_UNSUPPORTED, "decode: kv_format %d not built", kv_format);
+  if (users > kMaxUsers)
+    return fail(TTPA_ERR_UNSUPPORTED, "decode: %d users exceeds the limit of %d", users, kMaxUsers);
+  if (head_size != 64 && head_size != 128 && head_size != 256)
+    return fail(TTPA_ERR_UNSUPPORTED, "decode: head_size %d; supported 64, 128, 256", head_size);
+  if (block_size % 4 != 0)
+    return fail(TTPA_ERR_UNSUPPORTED, "decode: block_size %d must be a multiple of 4", block_size);
+  TTPA_REQUIRE(aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && aligned16(out),
+               "decode: q / caches / out must be 16-byte aligned");
+  TTPA_REQUIRE(q_user_stride % 8 == 0 && q_head_stride % 8 == 0,
+               "decode: q strides must be multiples of 8 elements");
+  const size_t need = ttpa_paged_decode_workspace_bytes(users, q_heads, kv_heads, head_size);
+  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    return fail(TTPA_ERR_WORKSPACE, "decode: workspace of %zu bytes (256-byte aligned) required, got %zu",
+                need, workspace_bytes);
+
+  const int g = q_heads / kv_heads;
+  DecodeArgs a;
+  a.out = static_cast<uint16_t *>(out);
+  a.out_us = out_user_stride, a.out_hs = out_head_stride;
+  a.q = static_cast<const uint16_t *>(q);
+  a.q_us = q_user_stride, a.q_hs = q_head_stride;
+  a.k = static_cast<const uint8_t *>(k_cache);
+  a.v = static_cast<const uint8_t *>(v_cache);
+  a.pt = page_table, a.pt_rs = page_table_row_stride;
+  a.cur = cur_pos, a.cur_i64 = cur_pos_is_i64;
+  a.users = users, a.hq = q_heads, a.hkv = kv_heads, a.bs = block_size, a.w = table_width;
+  a.nb = num_blocks;
+  a.scale_log2e = scale * 1.4426950408889634f;
+  a.ws_pref = static_cast<int *>(workspace);
+  a.ws_slots = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + header_bytes(users));
+  a.n_waves = waves_for_device();
+  a.slot_floats = slot_floats_for(g, head_size);
+
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  int rc = TTPA_OK;
+  switch (head_size) {
+    case 64: rc = launch_g<64>(a, g, st); break;
+    case 128: rc = launch_g<128>(a, g, st); break;
+    default: rc = launch_g<256>(a, g, st); break;
+  }
+  if (rc) return rc;
+  return check_launch("paged_sdpa_decode");
+}

@@ -1,0 +1,14 @@
+"""MI355X-native paged KV-cache write and paged attention behind tt-xla's operator
+and attention-backend interface.
+
+Importing the package registers the ``torch.ops.tt.*`` operators for HIP devices
+(``custom_ops``); ``attention`` holds the vLLM-facing backend classes.  Every operator
+runs a hand-written gfx950 kernel from ``lib/libttpa.so``; there is no other
+implementation to fall back to, and a missing library is an error.
+"""
+
+from . import _native  # noqa: F401
+from . import custom_ops  # noqa: F401
+from .attention import TTAttentionBackend, TTAttentionBackendImpl, TTMetadata  # noqa: F401
+
+__all__ = ["TTAttentionBackend", "TTAttentionBackendImpl", "TTMetadata", "custom_ops"]

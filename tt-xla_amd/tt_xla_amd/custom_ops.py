@@ -1,0 +1,426 @@
+"""``torch.ops.tt.*`` operators of the paged-attention path for HIP devices.
+
+Names, argument order and defaults are those of tt-xla's
+``python_package/tt_torch/custom_ops.py`` (:635-646, :962-971, :1016-1024,
+:1198-1214, :1334-1346); the implementation of each is a launch of a gfx950 kernel
+through the C ABI in ``include/ttpa.h``.  As in the reference the five operators are
+functional (``mutates_args=[]``): the cache writers return a fresh tensor.  Because a
+functional write copies the whole cache, in-place twins ``tt::paged_update_cache_`` and
+``tt::paged_fill_cache_`` are provided for callers that own the cache (the attention
+backend uses them); their effect on the cache equals ``cache.copy_(functional_op(...))``.
+
+The operators are registered for the ``cuda`` (HIP) device type only.  There is no CPU
+implementation here: calling them with CPU tensors raises.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from . import _native as N
+
+# --------------------------------------------------------------------------- #
+# helpers
+# --------------------------------------------------------------------------- #
+_BFP8_GROUP = 16
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def _rows_contiguous(t: torch.Tensor) -> torch.Tensor:
+    """Last dim contiguous, every other stride a multiple of 8 elements, 16-byte base."""
+    if t.stride(-1) != 1 or t.data_ptr() % 16 or any(s % 8 for s in t.stride()[:-1]):
+        return t.contiguous()
+    return t
+
+
+def _index_tensor(t: torch.Tensor) -> torch.Tensor:
+    if t.dtype not in (torch.int32, torch.int64):
+        t = t.to(torch.int64)
+    return t.contiguous()
+
+
+def _table(t: torch.Tensor) -> torch.Tensor:
+    if t.dtype != torch.int32:
+        t = t.to(torch.int32)
+    if t.stride(-1) != 1:
+        t = t.contiguous()
+    return t
+
+
+def _kv_format(cache: torch.Tensor) -> int:
+    if cache.dtype == torch.uint8:
+        return N.KV_BFP8
+    if cache.dtype in (torch.bfloat16, torch.float16):
+        return N.KV_BF16  # 2-byte elements; the cache writers are pure copies
+    raise ValueError(f"unsupported cache dtype {cache.dtype}")
+
+
+def _cache_geometry(cache: torch.Tensor):
+    """(num_blocks, kv_heads, block_size, head_size, format) of a cache tensor."""
+    if cache.dim() != 4 or not cache.is_contiguous():
+        raise ValueError("cache must be a contiguous [num_blocks, kv_heads, block_size, head_size] tensor")
+    fmt = _kv_format(cache)
+    nb, hkv, rows, d = cache.shape
+    if fmt == N.KV_BFP8:
+        if rows % (_BFP8_GROUP + 1):
+            raise ValueError("block-float-8 cache must have block_size + block_size/16 rows")
+        bs = rows // (_BFP8_GROUP + 1) * _BFP8_GROUP
+    else:
+        bs = rows
+    return nb, hkv, bs, d, fmt
+
+
+def bfp8_cache_shape(num_blocks: int, num_kv_heads: int, block_size: int, head_size: int):
+    """Shape of the uint8 tensor that stores a block-float-8 cache."""
+    assert block_size % _BFP8_GROUP == 0 and head_size % _BFP8_GROUP == 0
+    return (num_blocks, num_kv_heads, block_size + block_size // _BFP8_GROUP, head_size)
+
+
+# --------------------------------------------------------------------------- #
+# cache writes
+# --------------------------------------------------------------------------- #
+def _update_inplace(cache, fill_value, update_indices, page_table):
+    nb, hkv, bs, d, fmt = _cache_geometry(cache)
+    if fill_value.dim() != 4 or fill_value.shape[0] != 1:
+        raise ValueError("fill_value must be [1, users, heads, head_size]")
+    users = update_indices.shape[0]
+    if fill_value.shape[1] != users or fill_value.shape[2] < hkv or fill_value.shape[3] != d:
+        raise ValueError(
+            f"fill_value {tuple(fill_value.shape)} does not match users={users}, "
+            f"kv_heads={hkv}, head_size={d}"
+        )
+    if page_table.dim() != 2 or page_table.shape[0] < users:
+        raise ValueError("page_table must be [users, blocks_per_user]")
+    if fill_value.dtype not in (torch.bfloat16, torch.float16) or (
+        fmt == N.KV_BF16 and fill_value.dtype != cache.dtype
+    ):
+        raise ValueError("fill_value dtype must match the cache (bfloat16 for block-float-8)")
+    fill_value = _rows_contiguous(fill_value)
+    idx = _index_tensor(update_indices)
+    pt = _table(page_table)
+    N.call(
+        "ttpa_paged_update_cache",
+        cache.data_ptr(), fill_value.data_ptr(), fill_value.stride(1), fill_value.stride(2),
+        idx.data_ptr(), int(idx.dtype == torch.int64), pt.data_ptr(), pt.stride(0),
+        users, hkv, bs, d, pt.shape[1], nb, fmt, _stream(),
+    )
+
+
+@torch.library.custom_op("tt::paged_update_cache", mutates_args=[], device_types=["cuda"])
+def paged_update_cache(
+    cache: torch.Tensor,
+    fill_value: torch.Tensor,
+    update_indices: torch.Tensor,
+    page_table: torch.Tensor,
+    share_cache: bool = False,
+) -> torch.Tensor:
+    out = cache.clone()
+    _update_inplace(out, fill_value, update_indices, page_table)
+    return out
+
+
+@paged_update_cache.register_fake
+def _(cache, fill_value, update_indices, page_table, share_cache=False):
+    return torch.empty_like(cache)
+
+
+@torch.library.custom_op("tt::paged_update_cache_", mutates_args=["cache"], device_types=["cuda"])
+def paged_update_cache_(
+    cache: torch.Tensor,
+    fill_value: torch.Tensor,
+    update_indices: torch.Tensor,
+    page_table: torch.Tensor,
+    share_cache: bool = False,
+) -> None:
+    _update_inplace(cache, fill_value, update_indices, page_table)
+
+
+@paged_update_cache_.register_fake
+def _(cache, fill_value, update_indices, page_table, share_cache=False):
+    return None
+
+
+def _fill_inplace(cache, fill_value, page_table, batch_idx):
+    nb, hkv, bs, d, fmt = _cache_geometry(cache)
+    if fill_value.dim() != 4:
+        raise ValueError("fill_value must be [users, heads, seq_len, head_size]")
+    fu, fh, s, fd = fill_value.shape
+    if fh != hkv or fd != d:
+        raise ValueError(
+            f"fill_value {tuple(fill_value.shape)} does not match kv_heads={hkv}, head_size={d}"
+        )
+    if page_table.dim() != 2:
+        raise ValueError("page_table must be [users, blocks_per_user]")
+    if batch_idx is None:
+        if fu != 1:
+            raise ValueError("batch_idx is required when fill_value holds more than one user")
+    else:
+        if batch_idx.numel() != fu:
+            raise ValueError("batch_idx must have one entry per fill_value row")
+        batch_idx = _index_tensor(batch_idx.reshape(-1))
+    if s > page_table.shape[1] * bs:
+        raise ValueError(
+            f"{s} tokens do not fit {page_table.shape[1]} page-table columns of {bs} tokens"
+        )
+    if fill_value.dtype not in (torch.bfloat16, torch.float16) or (
+        fmt == N.KV_BF16 and fill_value.dtype != cache.dtype
+    ):
+        raise ValueError("fill_value dtype must match the cache (bfloat16 for block-float-8)")
+    fill_value = _rows_contiguous(fill_value)
+    pt = _table(page_table)
+    N.call(
+        "ttpa_paged_fill_cache",
+        cache.data_ptr(), fill_value.data_ptr(), fill_value.stride(0), fill_value.stride(1),
+        fill_value.stride(2), pt.data_ptr(), pt.stride(0), _ptr(batch_idx),
+        int(batch_idx is not None and batch_idx.dtype == torch.int64),
+        fu, pt.shape[0], hkv, s, bs, d, pt.shape[1], nb, fmt, _stream(),
+    )
+
+
+@torch.library.custom_op("tt::paged_fill_cache", mutates_args=[], device_types=["cuda"])
+def paged_fill_cache(
+    cache: torch.Tensor,
+    fill_value: torch.Tensor,
+    page_table: torch.Tensor,
+    batch_idx: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    out = cache.clone()
+    _fill_inplace(out, fill_value, page_table, batch_idx)
+    return out
+
+
+@paged_fill_cache.register_fake
+def _(cache, fill_value, page_table, batch_idx=None):
+    return torch.empty_like(cache)
+
+
+@torch.library.custom_op("tt::paged_fill_cache_", mutates_args=["cache"], device_types=["cuda"])
+def paged_fill_cache_(
+    cache: torch.Tensor,
+    fill_value: torch.Tensor,
+    page_table: torch.Tensor,
+    batch_idx: Optional[torch.Tensor] = None,
+) -> None:
+    _fill_inplace(cache, fill_value, page_table, batch_idx)
+
+
+@paged_fill_cache_.register_fake
+def _(cache, fill_value, page_table, batch_idx=None):
+    return None
+
+
+# --------------------------------------------------------------------------- #
+# decode attention
+# --------------------------------------------------------------------------- #
+@torch.library.custom_op(
+    "tt::paged_scaled_dot_product_attention_decode", mutates_args=[], device_types=["cuda"]
+)
+def paged_scaled_dot_product_attention_decode(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    page_table: torch.Tensor,
+    is_causal: bool = False,
+    attn_mask: Optional[torch.Tensor] = None,
+    cur_pos_tensor: Optional[torch.Tensor] = None,
+    attention_sink: Optional[torch.Tensor] = None,
+    scale: Optional[float] = None,
+    sliding_window_size: Optional[int] = None,
+) -> torch.Tensor:
+    if is_causal:
+        assert attn_mask is None, "attention_mask must be None when is_causal is True."
+        assert cur_pos_tensor is not None, "cur_pos_tensor must be provided when is_causal is True."
+    if attn_mask is not None:
+        assert not is_causal, "attention_mask must be None when is_causal is True."
+    if not is_causal:
+        raise NotImplementedError(
+            "paged decode with an explicit attn_mask is not built; the serving path always "
+            "issues the causal form"
+        )
+    if attention_sink is not None or sliding_window_size is not None:
+        raise NotImplementedError("attention_sink / sliding_window_size are not built")
+    if query.dim() != 4 or query.shape[0] != 1:
+        raise ValueError("query must be [1, users, heads, head_size]")
+    nb, hkv, bs, d, fmt = _cache_geometry(key)
+    if _cache_geometry(value) != (nb, hkv, bs, d, fmt):
+        raise ValueError("key and value caches must have the same shape and dtype")
+    _, users, hq, qd = query.shape
+    if qd != d or hq % hkv:
+        raise ValueError(f"query {tuple(query.shape)} does not match the cache geometry")
+    if query.dtype != torch.bfloat16:
+        raise ValueError("query must be bfloat16")
+    if page_table.dim() != 2 or page_table.shape[0] != users or cur_pos_tensor.shape[0] != users:
+        raise ValueError("page_table / cur_pos_tensor must have one row per user")
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    q = _rows_contiguous(query)
+    pt = _table(page_table)
+    cur = _index_tensor(cur_pos_tensor)
+    out = torch.empty((1, users, hq, d), dtype=query.dtype, device=query.device)
+    ws_bytes = N.lib().ttpa_paged_decode_workspace_bytes(users, hq, hkv, d)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=query.device)
+    N.call(
+        "ttpa_paged_sdpa_decode",
+        out.data_ptr(), out.stride(1), out.stride(2), q.data_ptr(), q.stride(1), q.stride(2),
+        key.data_ptr(), value.data_ptr(), pt.data_ptr(), pt.stride(0), cur.data_ptr(),
+        int(cur.dtype == torch.int64), users, hq, hkv, d, bs, pt.shape[1], nb, float(scale), fmt,
+        ws.data_ptr(), ws_bytes, _stream(),
+    )
+    return out
+
+
+@paged_scaled_dot_product_attention_decode.register_fake
+def _(query, key, value, page_table, is_causal=False, attn_mask=None, cur_pos_tensor=None,
+      attention_sink=None, scale=None, sliding_window_size=None):
+    return torch.empty_like(query)
+
+
+# --------------------------------------------------------------------------- #
+# prefill attention
+# --------------------------------------------------------------------------- #
+def _prefill(query, key, value, page_table, chunk_start, attn_mask, is_causal, scale):
+    b, hq, s, d = query.shape
+    if query.dtype != torch.bfloat16:
+        raise ValueError("query must be bfloat16")
+    q = _rows_contiguous(query)
+    out = torch.empty_like(q)  # keeps q's (possibly token-major) strides
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    if page_table is None:
+        hkv, skv = key.shape[1], key.shape[2]
+        k = _rows_contiguous(key)
+        v = _rows_contiguous(value)
+        if k.stride() != v.stride():
+            k, v = k.contiguous(), v.contiguous()
+        kv_strides = (k.stride(0), k.stride(1), k.stride(2))
+        bs = w = nb = 0
+        pt_ptr, pt_rs = 0, 0
+    else:
+        nb, hkv, bs, kd, fmt = _cache_geometry(key)
+        if fmt != N.KV_BF16 or _cache_geometry(value) != (nb, hkv, bs, kd, fmt) or kd != d:
+            raise ValueError("chunked attention needs matching bfloat16 K/V caches")
+        k, v = key, value
+        pt = _table(page_table)
+        w = pt.shape[1]
+        skv = w * bs
+        kv_strides = (0, 0, 0)
+        pt_ptr, pt_rs = pt.data_ptr(), pt.stride(0)
+    mask_ptr, mask_bs, mask_rs = 0, 0, 0
+    if attn_mask is not None:
+        m = attn_mask
+        if m.dtype != torch.bfloat16:
+            m = m.to(torch.bfloat16)
+        if m.dim() != 4 or m.shape[1] != 1 or m.shape[2] != s or m.shape[3] != skv:
+            raise ValueError("attn_mask must be [batch, 1, q_len, kv_len]")
+        if m.stride(-1) != 1:
+            m = m.contiguous()
+        mask_ptr, mask_bs, mask_rs = m.data_ptr(), m.stride(0), m.stride(2)
+    N.call(
+        "ttpa_sdpa_prefill",
+        out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
+        q.data_ptr(), q.stride(0), q.stride(1), q.stride(2),
+        k.data_ptr(), v.data_ptr(), *kv_strides, pt_ptr, pt_rs, _ptr(chunk_start),
+        mask_ptr, mask_bs, mask_rs, b, hq, hkv, s, skv, d, bs, w, nb, int(is_causal),
+        float(scale), _stream(),
+    )
+    return out
+
+
+@torch.library.custom_op("tt::scaled_dot_product_attention", mutates_args=[], device_types=["cuda"])
+def scaled_dot_product_attention(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    attn_mask: Optional[torch.Tensor] = None,
+    is_causal: bool = True,
+    scale: Optional[float] = None,
+    sliding_window_size: Optional[int] = None,
+) -> torch.Tensor:
+    assert len(query.shape) == 4, "query must be a 4D tensor: [B, num_heads, query_seq_len, head_size]."
+    assert len(key.shape) == 4, "key must be a 4D tensor: [B, num_kv_heads, kv_seq_len, head_size]."
+    assert len(value.shape) == 4, "value must be a 4D tensor: [B, num_kv_heads, kv_seq_len, head_size]."
+    assert key.shape == value.shape, "key and value must have the same shape."
+    assert key.shape[-1] == query.shape[-1], "key and query must have the same head size."
+    assert query.shape[1] % key.shape[1] == 0, "num_heads must be divisible by num_kv_heads."
+    assert (
+        query.shape[2] % 32 == 0
+    ), f"query sequence length must be divisible by 32 but got {query.shape[2]}."
+    assert query.shape[0] == key.shape[0], "query and key must have the same batch size."
+    assert query.device == key.device == value.device, "query, key, and value must be on the same device."
+    if attn_mask is not None:
+        assert attn_mask.device == query.device, "attn_mask must be on the same device as query, key, and value."
+        assert is_causal == False, "is_causal attribute can't be True if attn_mask is available."  # noqa: E712
+        assert query.shape[0] == attn_mask.shape[0], "Attention mask batch size must match query batch size."
+    if sliding_window_size is not None:
+        raise NotImplementedError("sliding_window_size is not built")
+    return _prefill(query, key, value, None, None, attn_mask, is_causal, scale)
+
+
+@scaled_dot_product_attention.register_fake
+def _(query, key, value, attn_mask=None, is_causal=True, scale=None, sliding_window_size=None):
+    return torch.empty_like(query)
+
+
+@torch.library.custom_op(
+    "tt::chunked_scaled_dot_product_attention", mutates_args=[], device_types=["cuda"]
+)
+def chunked_scaled_dot_product_attention(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    page_table: torch.Tensor,
+    chunk_start_idx_tensor: torch.Tensor,
+    scale: Optional[float] = None,
+) -> torch.Tensor:
+    if query.dim() != 4:
+        raise ValueError("query must be [users, heads, chunk_len, head_size]")
+    if page_table.dim() != 2 or page_table.shape[0] != query.shape[0]:
+        raise ValueError("page_table must have one row per user")
+    start = chunk_start_idx_tensor.reshape(-1)
+    if start.dtype != torch.int32:
+        start = start.to(torch.int32)
+    return _prefill(query, key, value, page_table, start, None, True, scale)
+
+
+@chunked_scaled_dot_product_attention.register_fake
+def _(query, key, value, page_table, chunk_start_idx_tensor, scale=None):
+    return torch.empty_like(query)
+
+
+# --------------------------------------------------------------------------- #
+# block-float-8 helpers (cache conversion; no reference operator)
+# --------------------------------------------------------------------------- #
+def bfp8_pack_cache(cache: torch.Tensor) -> torch.Tensor:
+    """bf16 [NB, Hkv, bs, D] -> uint8 [NB, Hkv, bs + bs/16, D] on the device."""
+    nb, hkv, bs, d = cache.shape
+    cache = cache.contiguous()
+    out = torch.empty(bfp8_cache_shape(nb, hkv, bs, d), dtype=torch.uint8, device=cache.device)
+    elem = torch.empty((nb, hkv, bs, d), dtype=torch.uint8, device=cache.device)
+    exps = torch.empty((nb, hkv, bs * d // _BFP8_GROUP), dtype=torch.uint8, device=cache.device)
+    N.call("ttpa_bfp8_quantize", cache.data_ptr(), elem.data_ptr(), exps.data_ptr(),
+           cache.numel(), _stream())
+    out[:, :, :bs, :] = elem
+    out[:, :, bs:, :] = exps.view(nb, hkv, bs // _BFP8_GROUP, d)
+    return out
+
+
+def bfp8_unpack_cache(packed: torch.Tensor) -> torch.Tensor:
+    """uint8 [NB, Hkv, bs + bs/16, D] -> bf16 [NB, Hkv, bs, D] (exact decode)."""
+    nb, hkv, bs, d, fmt = _cache_geometry(packed)
+    assert fmt == N.KV_BFP8
+    elem = packed[:, :, :bs, :].contiguous()
+    exps = packed[:, :, bs:, :].contiguous()
+    out = torch.empty((nb, hkv, bs, d), dtype=torch.bfloat16, device=packed.device)
+    N.call("ttpa_bfp8_dequantize", elem.data_ptr(), exps.data_ptr(), out.data_ptr(),
+           out.numel(), _stream())
+    return out

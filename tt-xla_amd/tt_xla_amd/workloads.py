@@ -1,0 +1,153 @@
+"""Seeded synthetic workloads of the paged-attention path (the shapes the benchmark and
+the parity tests run).  Everything is generated on the CPU from one ``torch.Generator``
+and moved to the requested device by the caller, so the CPU checker and the GPU kernels
+see identical bits.
+
+The generators reproduce the invariants of the reference's host metadata
+(vllm_tt/model_runner.py:1727-1741, 1945-1985): ``cache_position`` is the position of the
+token written this step, page-table rows list a user's blocks in logical order and are
+zero beyond them, block 0 is the null block.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+
+
+@dataclass
+class DecodeWorkload:
+    name: str
+    q: torch.Tensor  # [1, B, Hq, D] bf16
+    k_new: torch.Tensor  # [1, B, Hkv, D] bf16 (token written this step)
+    v_new: torch.Tensor
+    k_cache: torch.Tensor  # [NB, Hkv, bs, D] bf16
+    v_cache: torch.Tensor
+    page_table: torch.Tensor  # [B, W] int32
+    cache_position: torch.Tensor  # [B] int32 = context length before this step
+    scale: float
+
+    @property
+    def shape(self):
+        nb, hkv, bs, d = self.k_cache.shape
+        return dict(users=self.q.shape[1], q_heads=self.q.shape[2], kv_heads=hkv, head_size=d,
+                    block_size=bs, num_blocks=nb, table_width=self.page_table.shape[1])
+
+    def to(self, device):
+        return DecodeWorkload(self.name, *[
+            t.to(device) for t in (self.q, self.k_new, self.v_new, self.k_cache, self.v_cache,
+                                   self.page_table, self.cache_position)
+        ], self.scale)
+
+    def decode_bytes(self, kv_bytes_per_elem: float = 2.0) -> int:
+        """Algorithmic HBM bytes of one decode-attention launch: every attended K and V
+        element once per KV head, q read, output written, page-table entries and
+        positions read."""
+        s = self.shape
+        attended = (self.cache_position.to(torch.int64) + 1).clamp(min=0)
+        kv = int(attended.sum()) * s["kv_heads"] * s["head_size"] * 2 * kv_bytes_per_elem
+        qo = 2 * s["users"] * s["q_heads"] * s["head_size"] * 2
+        tables = int(((attended + s["block_size"] - 1) // s["block_size"]).sum()) * 4 + s["users"] * 4
+        return int(kv + qo + tables)
+
+    def update_bytes(self) -> int:
+        """One-token K and V writes: row read + row written, two tensors."""
+        s = self.shape
+        return 2 * 2 * s["users"] * s["kv_heads"] * s["head_size"] * 2
+
+
+def _randn_bf16(gen, *shape):
+    return torch.randn(*shape, generator=gen).to(torch.bfloat16)
+
+
+def decode_config1(seed: int = 1) -> DecodeWorkload:
+    """Batch 1, 8/8 heads, head 64, block 32, context 128: the reference's CPU-runnable
+    case.  The cache is pre-filled for 128 tokens through a random permutation of the 16
+    physical blocks; the new token goes to position 128."""
+    g = torch.Generator().manual_seed(seed)
+    b, hq, hkv, d, bs, nb, ctx = 1, 8, 8, 64, 32, 16, 128
+    table = torch.randperm(nb, generator=g).view(1, nb).to(torch.int32)
+    k_cache = torch.zeros(nb, hkv, bs, d, dtype=torch.bfloat16)
+    v_cache = torch.zeros(nb, hkv, bs, d, dtype=torch.bfloat16)
+    k_ctx = _randn_bf16(g, hkv, ctx, d)
+    v_ctx = _randn_bf16(g, hkv, ctx, d)
+    for t in range(ctx):
+        k_cache[table[0, t // bs], :, t % bs] = k_ctx[:, t]
+        v_cache[table[0, t // bs], :, t % bs] = v_ctx[:, t]
+    return DecodeWorkload(
+        "config1-b1-h8x8-d64-bs32-ctx128",
+        _randn_bf16(g, 1, b, hq, d), _randn_bf16(g, 1, b, hkv, d), _randn_bf16(g, 1, b, hkv, d),
+        k_cache, v_cache, table, torch.tensor([ctx], dtype=torch.int32), 1.0 / math.sqrt(d),
+    )
+
+
+def decode_ragged(
+    name: str,
+    seed: int,
+    users: int,
+    q_heads: int,
+    kv_heads: int,
+    head_size: int,
+    block_size: int,
+    num_blocks: int,
+    context: List[int],
+    table_width: Optional[int] = None,
+    cache_fill: str = "randn",
+) -> DecodeWorkload:
+    """Ragged decode batch: user u has ``context[u]`` tokens cached and writes position
+    ``context[u]``; its blocks are a disjoint slice of a random permutation of the pool
+    (block 0 is kept out as the null block), zero-padded to ``table_width``."""
+    g = torch.Generator().manual_seed(seed)
+    need = [(c + 1 + block_size - 1) // block_size for c in context]
+    assert sum(need) <= num_blocks - 1, "pool too small"
+    width = table_width or (max(need) + 7) // 8 * 8
+    perm = torch.randperm(num_blocks - 1, generator=g) + 1
+    table = torch.zeros(users, width, dtype=torch.int32)
+    at = 0
+    for u, n in enumerate(need):
+        table[u, :n] = perm[at : at + n].to(torch.int32)
+        at += n
+    shape = (num_blocks, kv_heads, block_size, head_size)
+    if cache_fill == "randn":
+        # generated in slices so peak host memory stays near one cache
+        k_cache = torch.empty(shape, dtype=torch.bfloat16)
+        v_cache = torch.empty(shape, dtype=torch.bfloat16)
+        step = max(1, (1 << 24) // (kv_heads * block_size * head_size))
+        for s in range(0, num_blocks, step):
+            e = min(num_blocks, s + step)
+            k_cache[s:e] = torch.randn(e - s, *shape[1:], generator=g).to(torch.bfloat16)
+            v_cache[s:e] = torch.randn(e - s, *shape[1:], generator=g).to(torch.bfloat16)
+    else:
+        k_cache = torch.zeros(shape, dtype=torch.bfloat16)
+        v_cache = torch.zeros(shape, dtype=torch.bfloat16)
+    return DecodeWorkload(
+        name,
+        _randn_bf16(g, 1, users, q_heads, head_size),
+        _randn_bf16(g, 1, users, kv_heads, head_size),
+        _randn_bf16(g, 1, users, kv_heads, head_size),
+        k_cache, v_cache, table, torch.tensor(context, dtype=torch.int32),
+        1.0 / math.sqrt(head_size),
+    )
+
+
+def decode_config2(seed: int = 2, users: int = 32, num_blocks: int = 4096) -> DecodeWorkload:
+    """Llama-3-8B shape: 32/8 heads, head 128, block 64, batch 32, context uniform in
+    [512, 4096], blocks drawn without reuse from a pool of 4096."""
+    g = torch.Generator().manual_seed(seed)
+    ctx = torch.randint(512, 4097, (users,), generator=g).tolist()
+    return decode_ragged("config2-llama3-8b-b32-h32x8-d128-bs64-ctx512..4096", seed + 1000, users,
+                         32, 8, 128, 64, num_blocks, ctx, table_width=72)
+
+
+def decode_config4(seed: int = 4, users: int = 128, num_blocks: int = 16384) -> DecodeWorkload:
+    """Llama-3-70B shape on one GPU: 64/8 heads, head 128, block 64, batch 128, context
+    log-uniform in [256, 32768]."""
+    g = torch.Generator().manual_seed(seed)
+    u = torch.rand(users, generator=g)
+    ctx = torch.exp(math.log(256) + u * (math.log(32768) - math.log(256))).round().long()
+    ctx = ctx.clamp(256, 32767).tolist()
+    return decode_ragged("config4-llama3-70b-b128-h64x8-d128-bs64-ctx256..32768", seed + 1000,
+                         users, 64, 8, 128, 64, num_blocks, ctx, table_width=520)
