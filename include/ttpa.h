@@ -120,6 +120,15 @@ int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_t out_head_
                            size_t workspace_bytes, void *stream);
 
 /*
+ * Measurement hook, no reference counterpart: the NEXT attention call made by this host
+ * thread (decode or prefill) records `before` and `after` (hipEvent_t, as void*) on its
+ * stream immediately around its dominant kernel (the split-K main kernel for decode, the
+ * MFMA kernel for prefill), then forgets them.  Pass NULLs to clear.  Used by bench.py to
+ * time that kernel alone, the way a profiler's kernel trace does.
+ */
+int ttpa_profile_next_attention(void *before, void *after);
+
+/*
  * Prefill attention (bf16 MFMA), dense or paged K/V, grouped heads.
  * Replaces the device branches of
  *   tt::scaled_dot_product_attention        (custom_ops.py:635-729; CPU :717-727) and

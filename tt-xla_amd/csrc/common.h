@@ -14,6 +14,10 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int check_launch(const char *what);
 int device_cus();
 
+// Events armed by ttpa_profile_next_attention(); take_profile_events() hands them to the
+// launcher that brackets its dominant kernel and disarms them.
+void take_profile_events(hipEvent_t &before, hipEvent_t &after);
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 #define TTPA_REQUIRE(cond, ...)                                            \

@@ -22,6 +22,8 @@ int check_launch(const char *what) {
   return TTPA_OK;
 }
 
+void arm_profile_events(void *before, void *after);
+
 int device_cus() {
   static thread_local int cached_dev = -1, cached_cus = 0;
   int dev = 0;
@@ -35,7 +37,27 @@ int device_cus() {
   return cached_cus;
 }
 
+static thread_local hipEvent_t g_ev_before = nullptr, g_ev_after = nullptr;
+
+void take_profile_events(hipEvent_t &before, hipEvent_t &after) {
+  before = g_ev_before;
+  after = g_ev_after;
+  g_ev_before = g_ev_after = nullptr;
+}
+
+void arm_profile_events(void *before, void *after) {
+  g_ev_before = static_cast<hipEvent_t>(before);
+  g_ev_after = static_cast<hipEvent_t>(after);
+}
+
 }  // namespace ttpa
+
+extern "C" int ttpa_profile_next_attention(void *before, void *after) {
+  if ((before == nullptr) != (after == nullptr))
+    return ttpa::fail(TTPA_ERR_INVALID_ARGUMENT, "pass both events or neither");
+  ttpa::arm_profile_events(before, after);
+  return TTPA_OK;
+}
 
 extern "C" int ttpa_abi_version(void) { return TTPA_ABI_VERSION; }
 extern "C" const char *ttpa_last_error(void) { return ttpa::g_err; }

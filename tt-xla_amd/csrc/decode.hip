@@ -84,6 +84,28 @@ __device__ void build_prefix(const DecodeArgs &a, int *pref, int *wave_sums) {
   __syncthreads();
 }
 
+// LDS probabilities are written as 16-bit values and read back as 32-bit pairs
+typedef uint16_t __attribute__((may_alias)) lds_u16;
+typedef uint32_t __attribute__((may_alias)) lds_u32;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Streaming (non-temporal) load of DW dwords: K/V are read once per launch, so they
+// should not displace anything in L2 / MALL.
+// `ubase` is wavefront-uniform and `lane_bytes` a 32-bit per-lane offset, which lets the
+// load use the scalar-base addressing form: no per-load 64-bit address registers.
+template <int DW>
+__device__ __forceinline__ void load_stream(const uint16_t *ubase, uint32_t lane_bytes,
+                                            uint32_t (&d)[DW]) {
+  const char *p = reinterpret_cast<const char *>(ubase) + static_cast<uint64_t>(lane_bytes);
+  if constexpr (DW == 4) {
+    u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+    d[0] = t.x, d[1] = t.y, d[2] = t.z, d[3] = t.w;
+  } else {
+    u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(p));
+    d[0] = t.x, d[1] = t.y;
+  }
+}
 template <int DW>
 __device__ __forceinline__ void load_dwords(const uint16_t *p, uint32_t (&d)[DW]) {
   if constexpr (DW == 4) {
@@ -166,17 +188,26 @@ struct Shape {
   static constexpr int NH = D / HD;
   static constexpr int EPL = HD / 16;  // elements per lane per pass
   static constexpr int DW = EPL / 2;
-  static constexpr int GP = G <= 2 ? G : ((G + 3) / 4) * 4;  // padded heads in LDS
 };
 
-template <int D, int G>
+// Position of a wavefront in the flat tile list.
+struct Cursor {
+  int u, h, t;      // user, kv head, tile index inside the segment
+  int len;          // attended positions of user u
+  int tiles_left;   // tiles of this segment from t on (including t)
+};
+
+// BIG = block_size is a multiple of 64: a tile lies inside one physical block.
+template <int D, int G, bool BIG>
 __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeArgs a) {
   using S = Shape<D, G>;
-  constexpr int NH = S::NH, EPL = S::EPL, DW = S::DW, GP = S::GP;
+  constexpr int NH = S::NH, EPL = S::EPL, DW = S::DW;
+  constexpr int NOFF = BIG ? 1 : 16;  // distinct row-group bases per tile
 
   __shared__ int s_pref[kMaxUsers + 1];
   __shared__ int s_wsum[kWavesPerBlock];
-  __shared__ float s_p[kWavesPerBlock][kTile * GP];
+  // probabilities of one tile as bfloat16: [wave][lane row r][head g][16 loads]
+  __shared__ __attribute__((aligned(16))) uint16_t s_p[kWavesPerBlock][4 * G * 16];
 
   build_prefix(a, s_pref, s_wsum);
   if (blockIdx.x == 0) {
@@ -187,213 +218,231 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeArgs a) {
   const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane >> 4, c = lane & 15;
   const int wave = blockIdx.x * kWavesPerBlock + wib;
-  const int64_t total = (int64_t)__builtin_amdgcn_readfirstlane(s_pref[a.users]) * a.hkv;
-  int64_t x = (int64_t)wave * total / a.n_waves;
-  const int64_t x_hi = (int64_t)(wave + 1) * total / a.n_waves;
-  float *plds = s_p[wib];
+  const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
+  const int64_t total = (int64_t)total_tiles * a.hkv;
+  const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);  // waves that get work
+  if (wave >= n_eff) return;
+  int64_t x = (int64_t)wave * total / n_eff;
+  const int64_t x_hi = (int64_t)(wave + 1) * total / n_eff;
+  lds_u16 *plds = s_p[wib];
   const int my_step = bitrev4(c);
-  const int64_t row_elems = D;  // elements per token row in the cache
+  const uint16_t *kb = reinterpret_cast<const uint16_t *>(a.k);
+  const uint16_t *vb = reinterpret_cast<const uint16_t *>(a.v);
+  const uint32_t lane_bytes = (uint32_t)(r * D + c * EPL) * 2u;
 
-  while (x < x_hi) {
-    // ---- locate the segment that owns unit x (uniform) -------------------------
+  // ---- helpers (all uniform across the wavefront) ---------------------------------
+  auto locate = [&](int64_t xx) {
     int lo_u = 0, hi_u = a.users - 1;
     while (lo_u < hi_u) {
       int mid = (lo_u + hi_u + 1) >> 1;
-      if ((int64_t)__builtin_amdgcn_readfirstlane(s_pref[mid]) * a.hkv <= x) lo_u = mid; else hi_u = mid - 1;
+      if ((int64_t)__builtin_amdgcn_readfirstlane(s_pref[mid]) * a.hkv <= xx) lo_u = mid;
+      else hi_u = mid - 1;
     }
-    const int u = lo_u;
-    const int pref_u = __builtin_amdgcn_readfirstlane(s_pref[u]);
-    const int nt = __builtin_amdgcn_readfirstlane(s_pref[u + 1]) - pref_u;
-    const int rem = (int)(x - (int64_t)pref_u * a.hkv);  // < nt * hkv
-    const int h = rem / nt;
-    int t = rem - h * nt;
-    const int64_t seg_end = x + (nt - t);
-    const int64_t x_end = seg_end < x_hi ? seg_end : x_hi;
+    Cursor cu;
+    cu.u = lo_u;
+    const int pref_u = __builtin_amdgcn_readfirstlane(s_pref[lo_u]);
+    const int nt = __builtin_amdgcn_readfirstlane(s_pref[lo_u + 1]) - pref_u;
+    const int rem = (int)(xx - (int64_t)pref_u * a.hkv);
+    cu.h = rem / nt;
+    cu.t = rem - cu.h * nt;
+    cu.tiles_left = nt - cu.t;
     int len;
-    tiles_of_user(a, u, len);
-    len = __builtin_amdgcn_readfirstlane(len);
-
-    // ---- query registers: q[g][pass][DW] ---------------------------------------
-    uint32_t q[G][NH][DW];
+    tiles_of_user(a, lo_u, len);
+    cu.len = __builtin_amdgcn_readfirstlane(len);
+    return cu;
+  };
+  // element offset (relative to the cache base) of the first row of each 4-row load
+  auto tile_offsets = [&](const Cursor &cu, int64_t (&off)[NOFF]) {
+    const int32_t *pt_row = a.pt + (int64_t)cu.u * a.pt_rs;
+    const int tok0 = cu.t * kTile;
+    if constexpr (BIG) {
+      int phys = __builtin_amdgcn_readfirstlane(pt_row[tok0 / a.bs]);
+      if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+      off[0] = (((int64_t)phys * a.hkv + cu.h) * a.bs + (tok0 % a.bs)) * D;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        int tk = tok0 + 4 * i;
+        int col = tk / a.bs;
+        int phys = (col < a.w) ? __builtin_amdgcn_readfirstlane(pt_row[col]) : 0;
+        if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+        off[i] = (((int64_t)phys * a.hkv + cu.h) * a.bs + (tk % a.bs)) * D;
+      }
+    }
+  };
+  // Loads are unconditional: every row of a tile is readable memory (rows past the
+  // attended length sit in the same physical block, columns past the table map to block 0).
+  auto load_tile = [&](const uint16_t *base, const int64_t (&off)[NOFF],
+                       uint32_t (&dst)[NH][16][DW]) {
+#pragma unroll
+    for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const uint16_t *row = BIG ? base + off[0] + i * 4 * D : base + off[BIG ? 0 : i];
+        load_stream<DW>(row + hf * S::HD, lane_bytes, dst[hf][i]);
+      }
+  };
+  // Rows that are not attended get weight 0; their V bits are cleared so that stale
+  // Inf / NaN in unwritten cache rows cannot turn 0 * x into NaN.
+  auto clear_unattended = [&](int nvalid, uint32_t (&dst)[NH][16][DW]) {
+#pragma unroll
+    for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int j = 0; j < DW; ++j) dst[hf][i][j] = (4 * i + r < nvalid) ? dst[hf][i][j] : 0u;
+  };
+  auto load_q = [&](const Cursor &cu, uint32_t (&q)[G][NH][DW]) {
 #pragma unroll
     for (int g = 0; g < G; ++g)
 #pragma unroll
       for (int hf = 0; hf < NH; ++hf)
-        load_dwords<DW>(a.q + u * a.q_us + (int64_t)(h * G + g) * a.q_hs + hf * S::HD + c * EPL,
+        load_dwords<DW>(a.q + cu.u * a.q_us + (int64_t)(cu.h * G + g) * a.q_hs + hf * S::HD + c * EPL,
                         q[g][hf]);
+  };
 
-    float m[G], l[G], acc[G][NH][EPL];
+  Cursor cur = locate(x);
+  int64_t off[NOFF];
+  uint32_t kreg[NH][16][DW], q[G][NH][DW];
+  tile_offsets(cur, off);
+  load_tile(kb, off, kreg);
+  load_q(cur, q);
+
+  float m[G], l[G], acc[G][NH][EPL];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    m[g] = -INFINITY;
+    l[g] = 0.f;
+#pragma unroll
+    for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) acc[g][hf][e] = 0.f;
+  }
+
+  while (true) {
+    const int nvalid = cur.len - cur.t * kTile;  // >= 1
+    // V of this tile goes in flight behind K (which was requested one iteration ago)
+    uint32_t vreg[NH][16][DW];
+    if constexpr (NH == 1) load_tile(vb, off, vreg);
+
+    // ---- scores: lane (r, c) ends with token 4 * bitrev4(c) + r of the tile -----------
+    float s[G];
+    qk_reduce_scatter<4, 0, G, NH, DW>(kreg, q, c, s);
+
+    // ---- advance the cursor; K of the next tile goes in flight now --------------------
+    const bool has_next = x + 1 < x_hi;
+    const bool same_seg = has_next && cur.tiles_left > 1;
+    Cursor nxt = cur;
+    int64_t noff[NOFF];
+#pragma unroll
+    for (int i = 0; i < NOFF; ++i) noff[i] = off[i];
+    if (has_next) {
+      if (same_seg) {
+        nxt.t = cur.t + 1;
+        nxt.tiles_left = cur.tiles_left - 1;
+      } else {
+        nxt = locate(x + 1);
+      }
+      tile_offsets(nxt, noff);
+      load_tile(kb, noff, kreg);
+    }
+    if constexpr (NH == 2) load_tile(vb, off, vreg);  // head_size 256: V fetched late
+
+    // ---- online softmax, one stream per lane row ---------------------------------------
+    const bool valid = 4 * my_step + r < nvalid;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      m[g] = -INFINITY;
-      l[g] = 0.f;
+      float sv = valid ? s[g] * a.scale_log2e : -INFINITY;
+      float mx = fmaxf(m[g], row16_max(sv));
+      float msafe = (mx == -INFINITY) ? 0.f : mx;
+      float alpha = __builtin_amdgcn_exp2f(m[g] - msafe);
+      float p = __builtin_amdgcn_exp2f(sv - msafe);
+      // the weight that multiplies V is rounded to bfloat16; the normaliser sums the
+      // same rounded values
+      uint32_t pb = f32_to_bf16_bits(p);
+      l[g] = l[g] * alpha + __builtin_bit_cast(float, pb << 16);
+      m[g] = mx;
+      plds[(r * G + g) * 16 + my_step] = (uint16_t)pb;
 #pragma unroll
       for (int hf = 0; hf < NH; ++hf)
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) acc[g][hf][e] = 0.f;
+        for (int e = 0; e < EPL; ++e) acc[g][hf][e] *= alpha;
     }
 
-    const int32_t *pt_row = a.pt + (int64_t)u * a.pt_rs;
-    const bool big_block = (a.bs % kTile) == 0;
-
-    for (; x < x_end; ++x, ++t) {
-      const int tok0 = t * kTile;
-      const int nvalid = len - tok0;  // >= 1
-      const bool full = nvalid >= kTile;
-
-      // element offset of the first token row of each load, relative to the cache base
-      int64_t off[16];
-      if (big_block) {
-        int phys = __builtin_amdgcn_readfirstlane(pt_row[tok0 / a.bs]);
-        if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
-        int64_t base = (((int64_t)phys * a.hkv + h) * a.bs + (tok0 % a.bs)) * row_elems;
+    // ---- output accumulation: two tokens per dot2 ----------------------------------------
+    if (nvalid < kTile) clear_unattended(nvalid, vreg);
+    const lds_u32 *pw = reinterpret_cast<const lds_u32 *>(plds) + r * G * 8;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) off[i] = base + (int64_t)i * 4 * row_elems;
-      } else {
+    for (int k2 = 0; k2 < 8; ++k2) {
+      uint32_t pk[G];  // weights of loads (2 k2, 2 k2 + 1) as a bf16 pair, per head
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          int tk = tok0 + 4 * i;
-          int col = tk / a.bs;
-          int phys = (col < a.w) ? __builtin_amdgcn_readfirstlane(pt_row[col]) : 0;
-          if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
-          off[i] = (((int64_t)phys * a.hkv + h) * a.bs + (tk % a.bs)) * row_elems;
-        }
-      }
-      const int64_t lane_off = (int64_t)r * row_elems + c * EPL;
-
-      uint32_t kreg[NH][16][DW], vreg[NH][16][DW];
-      const uint16_t *kb = reinterpret_cast<const uint16_t *>(a.k);
-      const uint16_t *vb = reinterpret_cast<const uint16_t *>(a.v);
+      for (int g = 0; g < G; ++g) pk[g] = pw[g * 8 + k2];
 #pragma unroll
       for (int hf = 0; hf < NH; ++hf)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          if (full || 4 * i + r < nvalid) {
-            load_dwords<DW>(kb + off[i] + lane_off + hf * S::HD, kreg[hf][i]);
-          } else {
+        for (int j = 0; j < DW; ++j) {
+          const uint32_t va = vreg[hf][2 * k2][j], vb2 = vreg[hf][2 * k2 + 1][j];
+          const uint32_t even = __builtin_amdgcn_perm(vb2, va, 0x05040100u);  // element 2j
+          const uint32_t odd = __builtin_amdgcn_perm(vb2, va, 0x07060302u);   // element 2j+1
 #pragma unroll
-            for (int j = 0; j < DW; ++j) kreg[hf][i][j] = 0;
+          for (int g = 0; g < G; ++g) {
+            acc[g][hf][2 * j] = dot2(even, pk[g], acc[g][hf][2 * j]);
+            acc[g][hf][2 * j + 1] = dot2(odd, pk[g], acc[g][hf][2 * j + 1]);
           }
         }
-      if constexpr (NH == 1) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          if (full || 4 * i + r < nvalid) {
-            load_dwords<DW>(vb + off[i] + lane_off, vreg[0][i]);
-          } else {
-#pragma unroll
-            for (int j = 0; j < DW; ++j) vreg[0][i][j] = 0;
-          }
-        }
-      }
+    }
 
-      // ---- scores: lane (r, c) ends with token tok0 + 4 * bitrev4(c) + r --------
-      float s[G];
-      qk_reduce_scatter<4, 0, G, NH, DW>(kreg, q, c, s);
-      const bool valid = full || (4 * my_step + r < nvalid);
-      float p[G];
+    // ---- close the segment if it ends here ----------------------------------------------
+    if (!same_seg) {
+      float *slot = a.ws_slots + ((int64_t)wave + (int64_t)cur.u * a.hkv + cur.h) * a.slot_floats;
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        float sv = valid ? s[g] * a.scale_log2e : -INFINITY;
-        float mx = fmaxf(m[g], row16_max(sv));
-        float msafe = (mx == -INFINITY) ? 0.f : mx;
-        float alpha = __builtin_amdgcn_exp2f(m[g] - msafe);
-        p[g] = __builtin_amdgcn_exp2f(sv - msafe);
-        l[g] = l[g] * alpha + p[g];
-        m[g] = mx;
+        float lr = row16_sum(l[g]);
+        float mr = m[g];
+        float mall = fmaxf(mr, __shfl_xor(mr, 16));
+        mall = fmaxf(mall, __shfl_xor(mall, 32));
+        float wgt = (mr == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mr - mall);
+        lr *= wgt;
+        lr += __shfl_xor(lr, 16);
+        lr += __shfl_xor(lr, 32);
 #pragma unroll
         for (int hf = 0; hf < NH; ++hf)
 #pragma unroll
-          for (int e = 0; e < EPL; ++e) acc[g][hf][e] *= alpha;
-      }
-      // publish the weights: plds[(r * 16 + step) * GP + g]
-      {
-        float *dst = plds + (r * 16 + my_step) * GP;
-#pragma unroll
-        for (int g = 0; g < G; ++g) dst[g] = p[g];
-      }
-
-      if constexpr (NH == 2) {
-        // head_size 256: V is fetched only now, one 128-element half at a time
-#pragma unroll
-        for (int hf = 0; hf < NH; ++hf)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            if (full || 4 * i + r < nvalid) {
-              load_dwords<DW>(vb + off[i] + lane_off + hf * S::HD, vreg[hf][i]);
-            } else {
-#pragma unroll
-              for (int j = 0; j < DW; ++j) vreg[hf][i][j] = 0;
-            }
+          for (int e = 0; e < EPL; ++e) {
+            float v = acc[g][hf][e] * wgt;
+            v += __shfl_xor(v, 16);
+            v += __shfl_xor(v, 32);
+            acc[g][hf][e] = v;
           }
-      }
-
-      // ---- output accumulation ---------------------------------------------------
+        if (r == 0) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float w[GP];
-        const float *src = plds + (r * 16 + i) * GP;
-        if constexpr (GP % 4 == 0) {
+          for (int hf = 0; hf < NH; ++hf) {
+            float *dst = slot + g * D + hf * S::HD + c * EPL;
 #pragma unroll
-          for (int g4 = 0; g4 < GP / 4; ++g4) {
-            float4 t4 = *reinterpret_cast<const float4 *>(src + 4 * g4);
-            w[4 * g4] = t4.x, w[4 * g4 + 1] = t4.y, w[4 * g4 + 2] = t4.z, w[4 * g4 + 3] = t4.w;
+            for (int e4 = 0; e4 < EPL / 4; ++e4)
+              *reinterpret_cast<float4 *>(dst + 4 * e4) =
+                  make_float4(acc[g][hf][4 * e4], acc[g][hf][4 * e4 + 1], acc[g][hf][4 * e4 + 2],
+                              acc[g][hf][4 * e4 + 3]);
           }
-        } else {
-#pragma unroll
-          for (int g = 0; g < GP; ++g) w[g] = src[g];
+          if (c == 0) {
+            slot[G * D + g] = mall;
+            slot[G * D + G + g] = lr;
+          }
         }
+        m[g] = -INFINITY;
+        l[g] = 0.f;
 #pragma unroll
         for (int hf = 0; hf < NH; ++hf)
 #pragma unroll
-          for (int j = 0; j < DW; ++j) {
-            float v0 = bf16_lo(vreg[hf][i][j]), v1 = bf16_hi(vreg[hf][i][j]);
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-              acc[g][hf][2 * j] = fmaf(w[g], v0, acc[g][hf][2 * j]);
-              acc[g][hf][2 * j + 1] = fmaf(w[g], v1, acc[g][hf][2 * j + 1]);
-            }
-          }
+          for (int e = 0; e < EPL; ++e) acc[g][hf][e] = 0.f;
       }
+      if (has_next) load_q(nxt, q);
     }
-
-    // ---- merge the 4 lane rows and write the partial of this (wave, segment) -----
-    float *slot = a.ws_slots + ((int64_t)wave + (int64_t)u * a.hkv + h) * a.slot_floats;
+    if (!has_next) break;
+    cur = nxt;
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float lr = row16_sum(l[g]);
-      float mr = m[g];
-      float mall = fmaxf(mr, __shfl_xor(mr, 16));
-      mall = fmaxf(mall, __shfl_xor(mall, 32));
-      float wgt = (mr == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mr - mall);
-      lr *= wgt;
-      lr += __shfl_xor(lr, 16);
-      lr += __shfl_xor(lr, 32);
-#pragma unroll
-      for (int hf = 0; hf < NH; ++hf)
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-          float v = acc[g][hf][e] * wgt;
-          v += __shfl_xor(v, 16);
-          v += __shfl_xor(v, 32);
-          acc[g][hf][e] = v;
-        }
-      if (r == 0) {
-#pragma unroll
-        for (int hf = 0; hf < NH; ++hf) {
-          float *dst = slot + g * D + hf * S::HD + c * EPL;
-#pragma unroll
-          for (int e4 = 0; e4 < EPL / 4; ++e4)
-            *reinterpret_cast<float4 *>(dst + 4 * e4) =
-                make_float4(acc[g][hf][4 * e4], acc[g][hf][4 * e4 + 1], acc[g][hf][4 * e4 + 2],
-                            acc[g][hf][4 * e4 + 3]);
-        }
-        if (c == 0) {
-          slot[G * D + g] = mall;
-          slot[G * D + G + g] = lr;
-        }
-      }
-    }
+    for (int i = 0; i < NOFF; ++i) off[i] = noff[i];
+    ++x;
   }
 }
 
@@ -403,30 +452,29 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a) {
   const int seg = blockIdx.x;
   const int u = seg / a.hkv, h = seg % a.hkv;
   const int nt = a.ws_pref[u + 1] - a.ws_pref[u];
-  const int64_t total = (int64_t)a.ws_pref[a.users] * a.hkv;
   uint16_t *out = a.out + u * a.out_us;
-  if (nt == 0) {  // padded row: no attended position -> NaN like softmax of all -inf
+  if (nt == 0) {  // padded row: no attended position -> NaN like softmax over nothing
     for (int i = threadIdx.x; i < G * D; i += 256)
       out[(int64_t)(h * G + i / D) * a.out_hs + (i % D)] = 0x7fc0;
     return;
   }
+  const int64_t total = (int64_t)a.ws_pref[a.users] * a.hkv;
+  const int64_t n_eff = total < a.n_waves ? total : a.n_waves;
   const int64_t x0 = (int64_t)a.ws_pref[u] * a.hkv + (int64_t)h * nt;
   const int64_t x1 = x0 + nt - 1;
-  // wave owning unit x: largest w with floor(w * total / n) <= x
-  const int w0 = (int)(((x0 + 1) * a.n_waves + total - 1) / total) - 1;
-  const int w1 = (int)(((x1 + 1) * a.n_waves + total - 1) / total) - 1;
-  const float *slots = a.ws_slots;
+  // wave owning unit x: largest w with floor(w * total / n_eff) <= x; with n_eff <= total
+  // every wave in [w0, w1] owns at least one unit of this segment
+  const int w0 = (int)(((x0 + 1) * n_eff + total - 1) / total) - 1;
+  const int w1 = (int)(((x1 + 1) * n_eff + total - 1) / total) - 1;
+  const float *base = a.ws_slots + ((int64_t)w0 + seg) * a.slot_floats;
+  const int nw = w1 - w0 + 1;
   for (int i = threadIdx.x; i < G * D; i += 256) {
     const int g = i / D;
     float mall = -INFINITY;
-    for (int w = w0; w <= w1; ++w) {
-      if ((int64_t)w * total / a.n_waves == (int64_t)(w + 1) * total / a.n_waves) continue;
-      mall = fmaxf(mall, slots[((int64_t)w + seg) * a.slot_floats + G * D + g]);
-    }
+    for (int w = 0; w < nw; ++w) mall = fmaxf(mall, base[(int64_t)w * a.slot_floats + G * D + g]);
     float num = 0.f, den = 0.f;
-    for (int w = w0; w <= w1; ++w) {
-      if ((int64_t)w * total / a.n_waves == (int64_t)(w + 1) * total / a.n_waves) continue;
-      const float *sl = slots + ((int64_t)w + seg) * a.slot_floats;
+    for (int w = 0; w < nw; ++w) {
+      const float *sl = base + (int64_t)w * a.slot_floats;
       float wgt = __builtin_amdgcn_exp2f(sl[G * D + g] - mall);
       num = fmaf(wgt, sl[i], num);
       den = fmaf(wgt, sl[G * D + G + g], den);
@@ -453,7 +501,14 @@ int waves_for_device() {
 
 template <int D, int G>
 void launch(const DecodeArgs &a, hipStream_t st) {
-  paged_decode_kernel<D, G><<<dim3(a.n_waves / kWavesPerBlock), dim3(256), 0, st>>>(a);
+  hipEvent_t ev0, ev1;
+  take_profile_events(ev0, ev1);
+  if (ev0) (void)hipEventRecord(ev0, st);
+  if (a.bs % kTile == 0)
+    paged_decode_kernel<D, G, true><<<dim3(a.n_waves / kWavesPerBlock), dim3(256), 0, st>>>(a);
+  else
+    paged_decode_kernel<D, G, false><<<dim3(a.n_waves / kWavesPerBlock), dim3(256), 0, st>>>(a);
+  if (ev1) (void)hipEventRecord(ev1, st);
   decode_combine_kernel<D, G><<<dim3(a.users * a.hkv), dim3(256), 0, st>>>(a);
 }
 

@@ -26,6 +26,7 @@ SIGNATURES = {
     "ttpa_abi_version": (_int, []),
     "ttpa_last_error": (C.c_char_p, []),
     "ttpa_device_compute_units": (_int, []),
+    "ttpa_profile_next_attention": (_int, [_p, _p]),
     "ttpa_paged_update_cache": (
         _int,
         [_p, _p, _i64, _i64, _p, _int, _p, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _p],

@@ -96,10 +96,13 @@ def decode_ragged(
     context: List[int],
     table_width: Optional[int] = None,
     cache_fill: str = "randn",
+    cache_device: Optional[str] = None,
 ) -> DecodeWorkload:
     """Ragged decode batch: user u has ``context[u]`` tokens cached and writes position
     ``context[u]``; its blocks are a disjoint slice of a random permutation of the pool
-    (block 0 is kept out as the null block), zero-padded to ``table_width``."""
+    (block 0 is kept out as the null block), zero-padded to ``table_width``.
+    ``cache_device`` draws the cache contents on that device instead of the CPU (for
+    benchmarks of full-size pools, where the values only need to be N(0, 1))."""
     g = torch.Generator().manual_seed(seed)
     need = [(c + 1 + block_size - 1) // block_size for c in context]
     assert sum(need) <= num_blocks - 1, "pool too small"
@@ -111,7 +114,11 @@ def decode_ragged(
         table[u, :n] = perm[at : at + n].to(torch.int32)
         at += n
     shape = (num_blocks, kv_heads, block_size, head_size)
-    if cache_fill == "randn":
+    if cache_fill == "randn" and cache_device is not None:
+        dg = torch.Generator(device=cache_device).manual_seed(seed)
+        k_cache = torch.randn(shape, generator=dg, device=cache_device, dtype=torch.bfloat16)
+        v_cache = torch.randn(shape, generator=dg, device=cache_device, dtype=torch.bfloat16)
+    elif cache_fill == "randn":
         # generated in slices so peak host memory stays near one cache
         k_cache = torch.empty(shape, dtype=torch.bfloat16)
         v_cache = torch.empty(shape, dtype=torch.bfloat16)
@@ -133,16 +140,19 @@ def decode_ragged(
     )
 
 
-def decode_config2(seed: int = 2, users: int = 32, num_blocks: int = 4096) -> DecodeWorkload:
+def decode_config2(seed: int = 2, users: int = 32, num_blocks: int = 4096,
+                   cache_device: Optional[str] = None) -> DecodeWorkload:
     """Llama-3-8B shape: 32/8 heads, head 128, block 64, batch 32, context uniform in
     [512, 4096], blocks drawn without reuse from a pool of 4096."""
     g = torch.Generator().manual_seed(seed)
     ctx = torch.randint(512, 4097, (users,), generator=g).tolist()
     return decode_ragged("config2-llama3-8b-b32-h32x8-d128-bs64-ctx512..4096", seed + 1000, users,
-                         32, 8, 128, 64, num_blocks, ctx, table_width=72)
+                         32, 8, 128, 64, num_blocks, ctx, table_width=72,
+                         cache_device=cache_device)
 
 
-def decode_config4(seed: int = 4, users: int = 128, num_blocks: int = 16384) -> DecodeWorkload:
+def decode_config4(seed: int = 4, users: int = 128, num_blocks: int = 16384,
+                   cache_device: Optional[str] = None) -> DecodeWorkload:
     """Llama-3-70B shape on one GPU: 64/8 heads, head 128, block 64, batch 128, context
     log-uniform in [256, 32768]."""
     g = torch.Generator().manual_seed(seed)
@@ -150,4 +160,5 @@ def decode_config4(seed: int = 4, users: int = 128, num_blocks: int = 16384) -> 
     ctx = torch.exp(math.log(256) + u * (math.log(32768) - math.log(256))).round().long()
     ctx = ctx.clamp(256, 32767).tolist()
     return decode_ragged("config4-llama3-70b-b128-h64x8-d128-bs64-ctx256..32768", seed + 1000,
-                         users, 64, 8, 128, 64, num_blocks, ctx, table_width=520)
+                         users, 64, 8, 128, 64, num_blocks, ctx, table_width=520,
+                         cache_device=cache_device)
