@@ -24,6 +24,8 @@
 //   per KV head.
 #include "common.h"
 
+#include <type_traits>
+
 namespace ttpa {
 namespace {
 
@@ -49,8 +51,9 @@ struct DecodeArgs {
   int slot_floats;
 };
 
-__device__ __forceinline__ int tiles_of_user(const DecodeArgs &a, int u, int &len) {
-  int64_t cp = load_index(a.cur, a.cur_i64, u);
+__device__ __forceinline__ int tiles_of_user(const DecodeArgs &a, const void *__restrict__ cur,
+                                             int u, int &len) {
+  int64_t cp = load_index(cur, a.cur_i64, u);
   int64_t cap = (int64_t)a.w * a.bs;
   int64_t l = cp < 0 ? 0 : (cp + 1 < cap ? cp + 1 : cap);
   len = (int)l;
@@ -58,13 +61,14 @@ __device__ __forceinline__ int tiles_of_user(const DecodeArgs &a, int u, int &le
 }
 
 // Exclusive prefix sum of per-user tile counts into pref[0..users]; all 256 threads.
-__device__ void build_prefix(const DecodeArgs &a, int *pref, int *wave_sums) {
+__device__ void build_prefix(const DecodeArgs &a, const void *__restrict__ cur, int *pref,
+                             int *wave_sums) {
   const int tid = threadIdx.x;
   const int per = (a.users + 255) / 256;
   const int beg = tid * per;
   const int end = min(beg + per, a.users);
   int local = 0, len;
-  for (int u = beg; u < end; ++u) local += tiles_of_user(a, u, len);
+  for (int u = beg; u < end; ++u) local += tiles_of_user(a, cur, u, len);
   int incl = local;
 #pragma unroll
   for (int d = 1; d < kWave; d <<= 1) {
@@ -78,7 +82,7 @@ __device__ void build_prefix(const DecodeArgs &a, int *pref, int *wave_sums) {
   int run = base + incl - local;
   if (tid == 0) pref[0] = 0;
   for (int u = beg; u < end; ++u) {
-    run += tiles_of_user(a, u, len);
+    run += tiles_of_user(a, cur, u, len);
     pref[u + 1] = run;
   }
   __syncthreads();
@@ -199,7 +203,11 @@ struct Cursor {
 
 // BIG = block_size is a multiple of 64: a tile lies inside one physical block.
 template <int D, int G, bool BIG>
-__global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeArgs a) {
+__global__ __launch_bounds__(256, 2) void paged_decode_kernel(
+    DecodeArgs a, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
+  // page_table / cur_pos are separate restrict parameters so that their wavefront-uniform
+  // reads become scalar loads: a vector load + readfirstlane would have to wait for every
+  // K/V tile load in flight (one shared counter) and stall the stream between tiles.
   using S = Shape<D, G>;
   constexpr int NH = S::NH, EPL = S::EPL, DW = S::DW;
   constexpr int NOFF = BIG ? 1 : 16;  // distinct row-group bases per tile
@@ -209,7 +217,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeArgs a) {
   // probabilities of one tile as bfloat16: [wave][lane row r][head g][16 loads]
   __shared__ __attribute__((aligned(16))) uint16_t s_p[kWavesPerBlock][4 * G * 16];
 
-  build_prefix(a, s_pref, s_wsum);
+  build_prefix(a, cur_pos, s_pref, s_wsum);
   if (blockIdx.x == 0) {
     for (int i = threadIdx.x; i <= a.users; i += 256) a.ws_pref[i] = s_pref[i];
   }
@@ -247,13 +255,13 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeArgs a) {
     cu.t = rem - cu.h * nt;
     cu.tiles_left = nt - cu.t;
     int len;
-    tiles_of_user(a, lo_u, len);
+    tiles_of_user(a, cur_pos, lo_u, len);
     cu.len = __builtin_amdgcn_readfirstlane(len);
     return cu;
   };
   // element offset (relative to the cache base) of the first row of each 4-row load
   auto tile_offsets = [&](const Cursor &cu, int64_t (&off)[NOFF]) {
-    const int32_t *pt_row = a.pt + (int64_t)cu.u * a.pt_rs;
+    const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
     const int tok0 = cu.t * kTile;
     if constexpr (BIG) {
       int phys = __builtin_amdgcn_readfirstlane(pt_row[tok0 / a.bs]);
@@ -319,24 +327,33 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeArgs a) {
       for (int e = 0; e < EPL; ++e) acc[g][hf][e] = 0.f;
   }
 
-  while (true) {
+  // One tile.  HAS_NEXT is a compile-time property of the call site: the steady-state
+  // loop always prefetches the next K tile unconditionally (a conditional prefetch makes
+  // the wait-count bookkeeping pessimistic and PV would wait for the prefetch), the last
+  // tile of the wavefront's range is peeled off below.
+  auto process_tile = [&](auto has_next_tag) {
+    constexpr bool has_next = decltype(has_next_tag)::value;
     const int nvalid = cur.len - cur.t * kTile;  // >= 1
     // V of this tile goes in flight behind K (which was requested one iteration ago)
     uint32_t vreg[NH][16][DW];
     if constexpr (NH == 1) load_tile(vb, off, vreg);
+    // scheduling fences pin the order "V(t) loads, QK(t), K(t+1) loads, softmax, PV(t)":
+    // left alone the scheduler sinks the V loads below the K(t+1) loads, and PV(t) then
+    // has to wait for K(t+1) (loads complete in issue order)
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- scores: lane (r, c) ends with token 4 * bitrev4(c) + r of the tile -----------
     float s[G];
     qk_reduce_scatter<4, 0, G, NH, DW>(kreg, q, c, s);
 
+    __builtin_amdgcn_sched_barrier(0);
     // ---- advance the cursor; K of the next tile goes in flight now --------------------
-    const bool has_next = x + 1 < x_hi;
     const bool same_seg = has_next && cur.tiles_left > 1;
     Cursor nxt = cur;
     int64_t noff[NOFF];
 #pragma unroll
     for (int i = 0; i < NOFF; ++i) noff[i] = off[i];
-    if (has_next) {
+    if constexpr (has_next) {
       if (same_seg) {
         nxt.t = cur.t + 1;
         nxt.tiles_left = cur.tiles_left - 1;
@@ -347,6 +364,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeArgs a) {
       load_tile(kb, noff, kreg);
     }
     if constexpr (NH == 2) load_tile(vb, off, vreg);  // head_size 256: V fetched late
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- online softmax, one stream per lane row ---------------------------------------
     const bool valid = 4 * my_step + r < nvalid;
@@ -436,14 +454,15 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeArgs a) {
 #pragma unroll
           for (int e = 0; e < EPL; ++e) acc[g][hf][e] = 0.f;
       }
-      if (has_next) load_q(nxt, q);
+      if constexpr (has_next) load_q(nxt, q);
     }
-    if (!has_next) break;
     cur = nxt;
 #pragma unroll
     for (int i = 0; i < NOFF; ++i) off[i] = noff[i];
     ++x;
-  }
+  };
+  while (x + 1 < x_hi) process_tile(std::true_type{});
+  process_tile(std::false_type{});
 }
 
 // Merges the partials of one (user, kv_head) segment and writes bfloat16 output.
@@ -505,9 +524,9 @@ void launch(const DecodeArgs &a, hipStream_t st) {
   take_profile_events(ev0, ev1);
   if (ev0) (void)hipEventRecord(ev0, st);
   if (a.bs % kTile == 0)
-    paged_decode_kernel<D, G, true><<<dim3(a.n_waves / kWavesPerBlock), dim3(256), 0, st>>>(a);
+    paged_decode_kernel<D, G, true><<<dim3(a.n_waves / kWavesPerBlock), dim3(256), 0, st>>>(a, a.pt, a.cur);
   else
-    paged_decode_kernel<D, G, false><<<dim3(a.n_waves / kWavesPerBlock), dim3(256), 0, st>>>(a);
+    paged_decode_kernel<D, G, false><<<dim3(a.n_waves / kWavesPerBlock), dim3(256), 0, st>>>(a, a.pt, a.cur);
   if (ev1) (void)hipEventRecord(ev1, st);
   decode_combine_kernel<D, G><<<dim3(a.users * a.hkv), dim3(256), 0, st>>>(a);
 }
