@@ -29,7 +29,7 @@
 namespace ttpa {
 namespace {
 
-constexpr int kMaxUsers = 4096;
+constexpr int kMaxUsers = 2048;
 constexpr int kTile = 64;
 constexpr int kWavesPerBlock = 4;
 
@@ -45,7 +45,7 @@ struct DecodeArgs {
   int cur_i64;
   int users, hq, hkv, bs, w, nb;
   float scale_log2e;
-  int *ws_pref;  // [users + 1] exclusive prefix of tile counts
+  int *ws_seg;   // [users * hkv][2]: first partial slot and number of partials per segment
   float *ws_slots;
   int n_waves;
   int slot_floats;
@@ -60,15 +60,22 @@ __device__ __forceinline__ int tiles_of_user(const DecodeArgs &a, const void *__
   return (int)((l + kTile - 1) / kTile);
 }
 
-// Exclusive prefix sum of per-user tile counts into pref[0..users]; all 256 threads.
+// Exclusive prefix sum of per-user tile counts into pref[0..users] and attended lengths into
+// lens[0..users); all 256 threads.  Each position is read from global memory once.
 __device__ void build_prefix(const DecodeArgs &a, const void *__restrict__ cur, int *pref,
-                             int *wave_sums) {
+                             int *lens, int *wave_sums) {
   const int tid = threadIdx.x;
   const int per = (a.users + 255) / 256;
   const int beg = tid * per;
   const int end = min(beg + per, a.users);
-  int local = 0, len;
-  for (int u = beg; u < end; ++u) local += tiles_of_user(a, cur, u, len);
+  int local = 0;
+  for (int u = beg; u < end; ++u) {
+    int len;
+    int nt = tiles_of_user(a, cur, u, len);
+    lens[u] = len;
+    pref[u + 1] = nt;  // replaced by the running sum below
+    local += nt;
+  }
   int incl = local;
 #pragma unroll
   for (int d = 1; d < kWave; d <<= 1) {
@@ -77,12 +84,11 @@ __device__ void build_prefix(const DecodeArgs &a, const void *__restrict__ cur, 
   }
   if ((tid & 63) == 63) wave_sums[tid >> 6] = incl;
   __syncthreads();
-  int base = 0;
-  for (int wv = 0; wv < (tid >> 6); ++wv) base += wave_sums[wv];
-  int run = base + incl - local;
+  int run = incl - local;
+  for (int wv = 0; wv < (tid >> 6); ++wv) run += wave_sums[wv];
   if (tid == 0) pref[0] = 0;
   for (int u = beg; u < end; ++u) {
-    run += tiles_of_user(a, cur, u, len);
+    run += pref[u + 1];
     pref[u + 1] = run;
   }
   __syncthreads();
@@ -213,15 +219,12 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   constexpr int NOFF = BIG ? 1 : 16;  // distinct row-group bases per tile
 
   __shared__ int s_pref[kMaxUsers + 1];
+  __shared__ int s_len[kMaxUsers];
   __shared__ int s_wsum[kWavesPerBlock];
   // probabilities of one tile as bfloat16: [wave][lane row r][head g][16 loads]
   __shared__ __attribute__((aligned(16))) uint16_t s_p[kWavesPerBlock][4 * G * 16];
 
-  build_prefix(a, cur_pos, s_pref, s_wsum);
-  if (blockIdx.x == 0) {
-    for (int i = threadIdx.x; i <= a.users; i += 256) a.ws_pref[i] = s_pref[i];
-  }
-
+  build_prefix(a, cur_pos, s_pref, s_len, s_wsum);
   const int lane = threadIdx.x & 63;
   const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane >> 4, c = lane & 15;
@@ -229,7 +232,31 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
   const int64_t total = (int64_t)total_tiles * a.hkv;
   const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);  // waves that get work
-  if (wave >= n_eff) return;
+  // The first blocks publish, for every segment, which partial slots the merge kernel has
+  // to read (one segment per thread; idle wavefronts do their share before leaving).
+  auto publish_segment_row = [&]() {
+    const int seg = blockIdx.x * 256 + threadIdx.x;
+    if (seg >= a.users * a.hkv) return;
+    const int su = seg / a.hkv, sh = seg - su * a.hkv;
+    const int snt = s_pref[su + 1] - s_pref[su];
+    int first = 0, count = 0;
+    if (snt > 0) {
+      const int64_t x0 = (int64_t)s_pref[su] * a.hkv + (int64_t)sh * snt;
+      const int64_t x1 = x0 + snt - 1;
+      // wave owning unit x: largest w with floor(w * total / n_eff) <= x; every wave in
+      // [w0, w1] owns at least one unit of the segment because n_eff <= total
+      const int w0 = (int)(((x0 + 1) * n_eff + total - 1) / total) - 1;
+      const int w1 = (int)(((x1 + 1) * n_eff + total - 1) / total) - 1;
+      first = w0 + seg;
+      count = w1 - w0 + 1;
+    }
+    a.ws_seg[2 * seg] = first;
+    a.ws_seg[2 * seg + 1] = count;
+  };
+  if (total == 0 || wave >= n_eff) {
+    publish_segment_row();
+    return;
+  }
   int64_t x = (int64_t)wave * total / n_eff;
   const int64_t x_hi = (int64_t)(wave + 1) * total / n_eff;
   lds_u16 *plds = s_p[wib];
@@ -254,9 +281,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
     cu.h = rem / nt;
     cu.t = rem - cu.h * nt;
     cu.tiles_left = nt - cu.t;
-    int len;
-    tiles_of_user(a, cur_pos, lo_u, len);
-    cu.len = __builtin_amdgcn_readfirstlane(len);
+    cu.len = __builtin_amdgcn_readfirstlane(s_len[lo_u]);
     return cu;
   };
   // element offset (relative to the cache base) of the first row of each 4-row load
@@ -315,6 +340,8 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   tile_offsets(cur, off);
   load_tile(kb, off, kreg);
   load_q(cur, q);
+
+  publish_segment_row();  // hidden behind the latency of the first tile
 
   float m[G], l[G], acc[G][NH][EPL];
 #pragma unroll
@@ -466,44 +493,49 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
 }
 
 // Merges the partials of one (user, kv_head) segment and writes bfloat16 output.
+// Partials are read four at a time so that their loads overlap.
 template <int D, int G>
 __global__ __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a) {
   const int seg = blockIdx.x;
   const int u = seg / a.hkv, h = seg % a.hkv;
-  const int nt = a.ws_pref[u + 1] - a.ws_pref[u];
+  const int first = a.ws_seg[2 * seg], nw = a.ws_seg[2 * seg + 1];
   uint16_t *out = a.out + u * a.out_us;
-  if (nt == 0) {  // padded row: no attended position -> NaN like softmax over nothing
+  if (nw == 0) {  // padded row: no attended position -> NaN like softmax over nothing
     for (int i = threadIdx.x; i < G * D; i += 256)
       out[(int64_t)(h * G + i / D) * a.out_hs + (i % D)] = 0x7fc0;
     return;
   }
-  const int64_t total = (int64_t)a.ws_pref[a.users] * a.hkv;
-  const int64_t n_eff = total < a.n_waves ? total : a.n_waves;
-  const int64_t x0 = (int64_t)a.ws_pref[u] * a.hkv + (int64_t)h * nt;
-  const int64_t x1 = x0 + nt - 1;
-  // wave owning unit x: largest w with floor(w * total / n_eff) <= x; with n_eff <= total
-  // every wave in [w0, w1] owns at least one unit of this segment
-  const int w0 = (int)(((x0 + 1) * n_eff + total - 1) / total) - 1;
-  const int w1 = (int)(((x1 + 1) * n_eff + total - 1) / total) - 1;
-  const float *base = a.ws_slots + ((int64_t)w0 + seg) * a.slot_floats;
-  const int nw = w1 - w0 + 1;
+  const float *base = a.ws_slots + (int64_t)first * a.slot_floats;
   for (int i = threadIdx.x; i < G * D; i += 256) {
     const int g = i / D;
-    float mall = -INFINITY;
-    for (int w = 0; w < nw; ++w) mall = fmaxf(mall, base[(int64_t)w * a.slot_floats + G * D + g]);
-    float num = 0.f, den = 0.f;
-    for (int w = 0; w < nw; ++w) {
-      const float *sl = base + (int64_t)w * a.slot_floats;
-      float wgt = __builtin_amdgcn_exp2f(sl[G * D + g] - mall);
-      num = fmaf(wgt, sl[i], num);
-      den = fmaf(wgt, sl[G * D + G + g], den);
+    float mall = -INFINITY, num = 0.f, den = 0.f;
+    for (int w = 0; w < nw; w += 4) {
+      float mv[4], lv[4], av[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float *sl = base + (int64_t)min(w + j, nw - 1) * a.slot_floats;
+        mv[j] = (w + j < nw) ? sl[G * D + g] : -INFINITY;
+        lv[j] = sl[G * D + G + g];
+        av[j] = sl[i];
+      }
+      float mnew = fmaxf(fmaxf(fmaxf(mv[0], mv[1]), fmaxf(mv[2], mv[3])), mall);
+      float resc = __builtin_amdgcn_exp2f(mall - mnew);
+      num *= resc;
+      den *= resc;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float wgt = __builtin_amdgcn_exp2f(mv[j] - mnew);  // 0 for the padding entries
+        num = fmaf(wgt, av[j], num);
+        den = fmaf(wgt, lv[j], den);
+      }
+      mall = mnew;
     }
     out[(int64_t)(h * G + g) * a.out_hs + (i % D)] = (uint16_t)f32_to_bf16_bits(num / den);
   }
 }
 
 int slot_floats_for(int g, int d) { return ((g * d + 2 * g + 3) / 4) * 4; }
-size_t header_bytes(int users) { return (((size_t)(users + 1) * 4 + 255) / 256) * 256; }
+size_t header_bytes(int users, int hkv) { return (((size_t)users * hkv * 8 + 255) / 256) * 256; }
 
 int waves_for_device() {
   static int override_waves = -1;
@@ -511,7 +543,7 @@ int waves_for_device() {
     const char *e = getenv("TTPA_DECODE_WAVES_PER_CU");
     override_waves = e ? atoi(e) : 0;
   }
-  int per_cu = override_waves > 0 ? override_waves : 8;
+  int per_cu = override_waves > 0 ? override_waves : 4;
   int cus = device_cus();
   if (cus <= 0) cus = 256;
   int waves = cus * per_cu;
@@ -523,10 +555,14 @@ void launch(const DecodeArgs &a, hipStream_t st) {
   hipEvent_t ev0, ev1;
   take_profile_events(ev0, ev1);
   if (ev0) (void)hipEventRecord(ev0, st);
+  // With one workgroup per CU in the grid, a 64 KiB dynamic LDS request (unused) makes two
+  // workgroups too large to share a CU, so the dispatcher has to spread them over all CUs.
+  const int blocks = a.n_waves / kWavesPerBlock;
+  const size_t pad = blocks <= device_cus() ? 65536 : 0;
   if (a.bs % kTile == 0)
-    paged_decode_kernel<D, G, true><<<dim3(a.n_waves / kWavesPerBlock), dim3(256), 0, st>>>(a, a.pt, a.cur);
+    paged_decode_kernel<D, G, true><<<dim3(blocks), dim3(256), pad, st>>>(a, a.pt, a.cur);
   else
-    paged_decode_kernel<D, G, false><<<dim3(a.n_waves / kWavesPerBlock), dim3(256), 0, st>>>(a, a.pt, a.cur);
+    paged_decode_kernel<D, G, false><<<dim3(blocks), dim3(256), pad, st>>>(a, a.pt, a.cur);
   if (ev1) (void)hipEventRecord(ev1, st);
   decode_combine_kernel<D, G><<<dim3(a.users * a.hkv), dim3(256), 0, st>>>(a);
 }
@@ -558,7 +594,7 @@ extern "C" size_t ttpa_paged_decode_workspace_bytes(int32_t users, int32_t q_hea
   if (users <= 0 || q_heads <= 0 || kv_heads <= 0 || head_size <= 0 || q_heads % kv_heads) return 0;
   int g = q_heads / kv_heads;
   size_t slots = (size_t)waves_for_device() + (size_t)users * kv_heads;
-  return header_bytes(users) + slots * (size_t)slot_floats_for(g, head_size) * sizeof(float);
+  return header_bytes(users, kv_heads) + slots * (size_t)slot_floats_for(g, head_size) * sizeof(float);
 }
 
 extern "C" int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_t out_head_stride,
@@ -606,8 +642,8 @@ extern "C" int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_
   a.users = users, a.hq = q_heads, a.hkv = kv_heads, a.bs = block_size, a.w = table_width;
   a.nb = num_blocks;
   a.scale_log2e = scale * 1.4426950408889634f;
-  a.ws_pref = static_cast<int *>(workspace);
-  a.ws_slots = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + header_bytes(users));
+  a.ws_seg = static_cast<int *>(workspace);
+  a.ws_slots = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + header_bytes(users, kv_heads));
   a.n_waves = waves_for_device();
   a.slot_floats = slot_floats_for(g, head_size);
 
