@@ -168,30 +168,37 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
       }
     }
 
-    // ---- scale, mask, online softmax (one query row per lane) ---------------------------
+    // ---- mask, online softmax (one query row per lane) -----------------------------------
+    // The softmax scale is positive, so the running maximum is tracked on raw scores and
+    // the scale is folded into the exponent: p = exp2(s * c - m * c).
     const int qrow = row0 + n;
-    const int limit = a.causal ? offset + qrow : a.skv - 1;  // last visible key of this row
-    const bool need_mask = (key0 + kKeysPerTile - 1 > offset + row0 && a.causal) ||
-                           key0 + kKeysPerTile > a.skv;
-    float mloc = -INFINITY;
+    const bool need_mask = (a.causal && key0 + kKeysPerTile - 1 > offset + row0) ||
+                           key0 + kKeysPerTile > a.skv || a.mask != nullptr;
+    if (need_mask) {  // wavefront-uniform: only diagonal / ragged / explicitly masked tiles
+      const int limit = a.causal ? min(offset + qrow, a.skv - 1) : a.skv - 1;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float v = st[kb][r] * a.scale_log2e;
-        const int key = key0 + 32 * kb + 8 * (r >> 2) + 4 * h + (r & 3);
-        if (a.mask) {
-          const int kc = min(key, a.skv - 1), qc = min(qrow, a.sq - 1);
-          v += bf16_lo(a.mask[b * a.mask_bs + (int64_t)qc * a.mask_rs + kc]) * 1.4426950408889634f;
+        for (int r = 0; r < 16; ++r) {
+          const int key = key0 + 32 * kb + 8 * (r >> 2) + 4 * h + (r & 3);
+          float v = st[kb][r];
+          if (a.mask) {
+            const int kc = min(key, a.skv - 1), qc = min(qrow, a.sq - 1);
+            // additive mask is in natural-log units of the scaled score
+            v += bf16_lo(a.mask[b * a.mask_bs + (int64_t)qc * a.mask_rs + kc]) *
+                 (1.4426950408889634f / a.scale_log2e);
+          }
+          st[kb][r] = key > limit ? -INFINITY : v;
         }
-        if (need_mask && (key > limit || key >= a.skv)) v = -INFINITY;
-        st[kb][r] = v;
-        mloc = fmaxf(mloc, v);
-      }
+    }
+    float mloc = fmaxf(st[0][0], st[1][0]);
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(st[0][r], st[1][r]));
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
     const float m_new = fmaxf(m_run, mloc);
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * a.scale_log2e);
+    const float mc = m_safe * a.scale_log2e;
     m_run = m_new;
     float lsum = 0.f;
     bf16x8 pf[2][2];
@@ -202,10 +209,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           // B-operand element e of k-step s <-> accumulator register 8 s + e
-          float p = __builtin_amdgcn_exp2f(st[kb][8 * s + e] - m_safe);
-          __bf16 pb = (__bf16)p;
-          lsum += (float)pb;
-          pf[kb][s][e] = pb;
+          float p = __builtin_amdgcn_exp2f(fmaf(st[kb][8 * s + e], a.scale_log2e, -mc));
+          lsum += p;
+          pf[kb][s][e] = (__bf16)p;
         }
     l_run = l_run * alpha + lsum;
     // skip the accumulator rescale when no row of the wavefront moved its maximum
