@@ -22,190 +22,10 @@
 //   multiplies its V elements.
 //   The G query heads of a group share every K/V load: each element is read once
 //   per KV head.
-#include "common.h"
-
-#include <type_traits>
+#include "decode_common.h"
 
 namespace ttpa {
-namespace {
-
-constexpr int kMaxUsers = 2048;
-constexpr int kTile = 64;
-constexpr int kWavesPerBlock = 4;
-
-struct DecodeArgs {
-  uint16_t *out;
-  int64_t out_us, out_hs;
-  const uint16_t *q;
-  int64_t q_us, q_hs;
-  const uint8_t *k, *v;
-  const int32_t *pt;
-  int64_t pt_rs;
-  const void *cur;
-  int cur_i64;
-  int users, hq, hkv, bs, w, nb;
-  float scale_log2e;
-  int *ws_seg;   // [users * hkv][2]: first partial slot and number of partials per segment
-  float *ws_slots;
-  int n_waves;
-  int slot_floats;
-};
-
-__device__ __forceinline__ int tiles_of_user(const DecodeArgs &a, const void *__restrict__ cur,
-                                             int u, int &len) {
-  int64_t cp = load_index(cur, a.cur_i64, u);
-  int64_t cap = (int64_t)a.w * a.bs;
-  int64_t l = cp < 0 ? 0 : (cp + 1 < cap ? cp + 1 : cap);
-  len = (int)l;
-  return (int)((l + kTile - 1) / kTile);
-}
-
-// Exclusive prefix sum of per-user tile counts into pref[0..users] and attended lengths into
-// lens[0..users); all 256 threads.  Each position is read from global memory once.
-__device__ void build_prefix(const DecodeArgs &a, const void *__restrict__ cur, int *pref,
-                             int *lens, int *wave_sums) {
-  const int tid = threadIdx.x;
-  const int per = (a.users + 255) / 256;
-  const int beg = tid * per;
-  const int end = min(beg + per, a.users);
-  int local = 0;
-  for (int u = beg; u < end; ++u) {
-    int len;
-    int nt = tiles_of_user(a, cur, u, len);
-    lens[u] = len;
-    pref[u + 1] = nt;  // replaced by the running sum below
-    local += nt;
-  }
-  int incl = local;
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    int o = __shfl_up(incl, d);
-    if ((tid & 63) >= d) incl += o;
-  }
-  if ((tid & 63) == 63) wave_sums[tid >> 6] = incl;
-  __syncthreads();
-  int run = incl - local;
-  for (int wv = 0; wv < (tid >> 6); ++wv) run += wave_sums[wv];
-  if (tid == 0) pref[0] = 0;
-  for (int u = beg; u < end; ++u) {
-    run += pref[u + 1];
-    pref[u + 1] = run;
-  }
-  __syncthreads();
-}
-
-// LDS probabilities are written as 16-bit values and read back as 32-bit pairs
-typedef uint16_t __attribute__((may_alias)) lds_u16;
-typedef uint32_t __attribute__((may_alias)) lds_u32;
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-// Streaming (non-temporal) load of DW dwords: K/V are read once per launch, so they
-// should not displace anything in L2 / MALL.
-// `ubase` is wavefront-uniform and `lane_bytes` a 32-bit per-lane offset, which lets the
-// load use the scalar-base addressing form: no per-load 64-bit address registers.
-template <int DW>
-__device__ __forceinline__ void load_stream(const uint16_t *ubase, uint32_t lane_bytes,
-                                            uint32_t (&d)[DW]) {
-  const char *p = reinterpret_cast<const char *>(ubase) + static_cast<uint64_t>(lane_bytes);
-  if constexpr (DW == 4) {
-    u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
-    d[0] = t.x, d[1] = t.y, d[2] = t.z, d[3] = t.w;
-  } else {
-    u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(p));
-    d[0] = t.x, d[1] = t.y;
-  }
-}
-template <int DW>
-__device__ __forceinline__ void load_dwords(const uint16_t *p, uint32_t (&d)[DW]) {
-  if constexpr (DW == 4) {
-    uint4 t = *reinterpret_cast<const uint4 *>(p);
-    d[0] = t.x, d[1] = t.y, d[2] = t.z, d[3] = t.w;
-  } else {
-    uint2 t = *reinterpret_cast<const uint2 *>(p);
-    d[0] = t.x, d[1] = t.y;
-  }
-}
-
-__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
-  typedef __attribute__((ext_vector_type(2))) __bf16 bf2;
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, a), __builtin_bit_cast(bf2, b), c,
-                                         false);
-}
-
-// Level L of the reduce-scatter exchanges along one lane bit inside a row of 16.
-// The exchange pattern of a level may flip lane bits that LATER levels partition on,
-// never earlier ones: mirror (^15) splits on bit 3, half-mirror (^7) on bit 2, then
-// ^2 on bit 1 and ^1 on bit 0.  After four levels lane c holds load bitrev4(c).
-template <int LEVEL>
-__device__ __forceinline__ float rs_exchange(float v) {
-  if constexpr (LEVEL == 1) return dpp_move<kDppMirror>(v);
-  if constexpr (LEVEL == 2) return dpp_move<kDppHalfMirror>(v);
-  if constexpr (LEVEL == 3) return dpp_move<kDppXor2>(v);
-  return dpp_move<kDppXor1>(v);
-}
-
-template <int LEVEL, int BASE, int G, int NH, int DW>
-__device__ __forceinline__ void qk_reduce_scatter(const uint32_t (&k)[NH][16][DW],
-                                                  const uint32_t (&q)[G][NH][DW], int c,
-                                                  float (&s)[G]) {
-  if constexpr (LEVEL == 0) {
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float acc = 0.f;
-#pragma unroll
-      for (int hf = 0; hf < NH; ++hf)
-#pragma unroll
-        for (int j = 0; j < DW; ++j) acc = dot2(k[hf][BASE][j], q[g][hf][j], acc);
-      s[g] = acc;
-    }
-  } else {
-    float lo[G], hi[G];
-    qk_reduce_scatter<LEVEL - 1, BASE, G, NH, DW>(k, q, c, lo);
-    qk_reduce_scatter<LEVEL - 1, BASE + (1 << (LEVEL - 1)), G, NH, DW>(k, q, c, hi);
-    const bool upper = (c >> (4 - LEVEL)) & 1;
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float keep = upper ? hi[g] : lo[g];
-      float send = upper ? lo[g] : hi[g];
-      s[g] = keep + rs_exchange<LEVEL>(send);
-    }
-  }
-}
-
-__device__ __forceinline__ float row16_max(float v) {
-  v = fmaxf(v, dpp_move<kDppXor1>(v));
-  v = fmaxf(v, dpp_move<kDppXor2>(v));
-  v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
-  v = fmaxf(v, dpp_move<kDppMirror>(v));
-  return v;
-}
-__device__ __forceinline__ float row16_sum(float v) {
-  v += dpp_move<kDppXor1>(v);
-  v += dpp_move<kDppXor2>(v);
-  v += dpp_move<kDppHalfMirror>(v);
-  v += dpp_move<kDppMirror>(v);
-  return v;
-}
-
-__device__ __forceinline__ int bitrev4(int c) {
-  return ((c & 1) << 3) | ((c & 2) << 1) | ((c & 4) >> 1) | ((c & 8) >> 3);
-}
-
-template <int D, int G>
-struct Shape {
-  static constexpr int HD = D > 128 ? 128 : D;  // elements covered by one load pass
-  static constexpr int NH = D / HD;
-  static constexpr int EPL = HD / 16;  // elements per lane per pass
-  static constexpr int DW = EPL / 2;
-};
-
-// Position of a wavefront in the flat tile list.
-struct Cursor {
-  int u, h, t;      // user, kv head, tile index inside the segment
-  int len;          // attended positions of user u
-  int tiles_left;   // tiles of this segment from t on (including t)
-};
+namespace decode {
 
 // BIG = block_size is a multiple of 64: a tile lies inside one physical block.
 template <int D, int G, bool BIG>
@@ -232,29 +52,8 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
   const int64_t total = (int64_t)total_tiles * a.hkv;
   const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);  // waves that get work
-  // The first blocks publish, for every segment, which partial slots the merge kernel has
-  // to read (one segment per thread; idle wavefronts do their share before leaving).
-  auto publish_segment_row = [&]() {
-    const int seg = blockIdx.x * 256 + threadIdx.x;
-    if (seg >= a.users * a.hkv) return;
-    const int su = seg / a.hkv, sh = seg - su * a.hkv;
-    const int snt = s_pref[su + 1] - s_pref[su];
-    int first = 0, count = 0;
-    if (snt > 0) {
-      const int64_t x0 = (int64_t)s_pref[su] * a.hkv + (int64_t)sh * snt;
-      const int64_t x1 = x0 + snt - 1;
-      // wave owning unit x: largest w with floor(w * total / n_eff) <= x; every wave in
-      // [w0, w1] owns at least one unit of the segment because n_eff <= total
-      const int w0 = (int)(((x0 + 1) * n_eff + total - 1) / total) - 1;
-      const int w1 = (int)(((x1 + 1) * n_eff + total - 1) / total) - 1;
-      first = w0 + seg;
-      count = w1 - w0 + 1;
-    }
-    a.ws_seg[2 * seg] = first;
-    a.ws_seg[2 * seg + 1] = count;
-  };
-  if (total == 0 || wave >= n_eff) {
-    publish_segment_row();
+  if (total == 0 || wave >= n_eff) {  // idle wavefronts still do their share of the table
+    publish_segment_row(a, s_pref, total, n_eff);
     return;
   }
   int64_t x = (int64_t)wave * total / n_eff;
@@ -266,24 +65,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   const uint32_t lane_bytes = (uint32_t)(r * D + c * EPL) * 2u;
 
   // ---- helpers (all uniform across the wavefront) ---------------------------------
-  auto locate = [&](int64_t xx) {
-    int lo_u = 0, hi_u = a.users - 1;
-    while (lo_u < hi_u) {
-      int mid = (lo_u + hi_u + 1) >> 1;
-      if ((int64_t)__builtin_amdgcn_readfirstlane(s_pref[mid]) * a.hkv <= xx) lo_u = mid;
-      else hi_u = mid - 1;
-    }
-    Cursor cu;
-    cu.u = lo_u;
-    const int pref_u = __builtin_amdgcn_readfirstlane(s_pref[lo_u]);
-    const int nt = __builtin_amdgcn_readfirstlane(s_pref[lo_u + 1]) - pref_u;
-    const int rem = (int)(xx - (int64_t)pref_u * a.hkv);
-    cu.h = rem / nt;
-    cu.t = rem - cu.h * nt;
-    cu.tiles_left = nt - cu.t;
-    cu.len = __builtin_amdgcn_readfirstlane(s_len[lo_u]);
-    return cu;
-  };
+  auto locate = [&](int64_t xx) { return locate_unit(s_pref, s_len, a.users, a.hkv, xx); };
   // element offset (relative to the cache base) of the first row of each 4-row load
   auto tile_offsets = [&](const Cursor &cu, int64_t (&off)[NOFF]) {
     const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
@@ -341,7 +123,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   load_tile(kb, off, kreg);
   load_q(cur, q);
 
-  publish_segment_row();  // hidden behind the latency of the first tile
+  publish_segment_row(a, s_pref, total, n_eff);  // hidden behind the first tile's latency
 
   float m[G], l[G], acc[G][NH][EPL];
 #pragma unroll
@@ -492,51 +274,6 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   process_tile(std::false_type{});
 }
 
-// Merges the partials of one (user, kv_head) segment and writes bfloat16 output.
-// Partials are read four at a time so that their loads overlap.
-template <int D, int G>
-__global__ __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a) {
-  const int seg = blockIdx.x;
-  const int u = seg / a.hkv, h = seg % a.hkv;
-  const int first = a.ws_seg[2 * seg], nw = a.ws_seg[2 * seg + 1];
-  uint16_t *out = a.out + u * a.out_us;
-  if (nw == 0) {  // padded row: no attended position -> NaN like softmax over nothing
-    for (int i = threadIdx.x; i < G * D; i += 256)
-      out[(int64_t)(h * G + i / D) * a.out_hs + (i % D)] = 0x7fc0;
-    return;
-  }
-  const float *base = a.ws_slots + (int64_t)first * a.slot_floats;
-  for (int i = threadIdx.x; i < G * D; i += 256) {
-    const int g = i / D;
-    float mall = -INFINITY, num = 0.f, den = 0.f;
-    for (int w = 0; w < nw; w += 4) {
-      float mv[4], lv[4], av[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float *sl = base + (int64_t)min(w + j, nw - 1) * a.slot_floats;
-        mv[j] = (w + j < nw) ? sl[G * D + g] : -INFINITY;
-        lv[j] = sl[G * D + G + g];
-        av[j] = sl[i];
-      }
-      float mnew = fmaxf(fmaxf(fmaxf(mv[0], mv[1]), fmaxf(mv[2], mv[3])), mall);
-      float resc = __builtin_amdgcn_exp2f(mall - mnew);
-      num *= resc;
-      den *= resc;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float wgt = __builtin_amdgcn_exp2f(mv[j] - mnew);  // 0 for the padding entries
-        num = fmaf(wgt, av[j], num);
-        den = fmaf(wgt, lv[j], den);
-      }
-      mall = mnew;
-    }
-    out[(int64_t)(h * G + g) * a.out_hs + (i % D)] = (uint16_t)f32_to_bf16_bits(num / den);
-  }
-}
-
-int slot_floats_for(int g, int d) { return ((g * d + 2 * g + 3) / 4) * 4; }
-size_t header_bytes(int users, int hkv) { return (((size_t)users * hkv * 8 + 255) / 256) * 256; }
-
 int waves_for_device() {
   static int override_waves = -1;
   if (override_waves < 0) {
@@ -555,14 +292,18 @@ void launch(const DecodeArgs &a, hipStream_t st) {
   hipEvent_t ev0, ev1;
   take_profile_events(ev0, ev1);
   if (ev0) (void)hipEventRecord(ev0, st);
-  // With one workgroup per CU in the grid, a 64 KiB dynamic LDS request (unused) makes two
-  // workgroups too large to share a CU, so the dispatcher has to spread them over all CUs.
-  const int blocks = a.n_waves / kWavesPerBlock;
-  const size_t pad = blocks <= device_cus() ? 65536 : 0;
-  if (a.bs % kTile == 0)
-    paged_decode_kernel<D, G, true><<<dim3(blocks), dim3(256), pad, st>>>(a, a.pt, a.cur);
-  else
-    paged_decode_kernel<D, G, false><<<dim3(blocks), dim3(256), pad, st>>>(a, a.pt, a.cur);
+  if (a.kv_format == TTPA_KV_BFP8) {
+    launch_bfp8_main(a, D, G, st);
+  } else {
+    // With one workgroup per CU in the grid, a 64 KiB dynamic LDS request (unused) makes two
+    // workgroups too large to share a CU, so the dispatcher has to spread them over all CUs.
+    const int blocks = a.n_waves / kWavesPerBlock;
+    const size_t pad = blocks <= device_cus() ? 65536 : 0;
+    if (a.bs % kTile == 0)
+      paged_decode_kernel<D, G, true><<<dim3(blocks), dim3(256), pad, st>>>(a, a.pt, a.cur);
+    else
+      paged_decode_kernel<D, G, false><<<dim3(blocks), dim3(256), pad, st>>>(a, a.pt, a.cur);
+  }
   if (ev1) (void)hipEventRecord(ev1, st);
   decode_combine_kernel<D, G><<<dim3(a.users * a.hkv), dim3(256), 0, st>>>(a);
 }
@@ -584,10 +325,11 @@ int launch_g(const DecodeArgs &a, int g, hipStream_t st) {
   return TTPA_OK;
 }
 
-}  // namespace
+}  // namespace decode
 }  // namespace ttpa
 
 using namespace ttpa;
+using namespace ttpa::decode;
 
 extern "C" size_t ttpa_paged_decode_workspace_bytes(int32_t users, int32_t q_heads,
                                                     int32_t kv_heads, int32_t head_size) {
@@ -612,8 +354,11 @@ extern "C" int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_
                "non-positive dimension");
   TTPA_REQUIRE(q_heads % kv_heads == 0, "q_heads %d not divisible by kv_heads %d", q_heads,
                kv_heads);
-  if (kv_format != TTPA_KV_BF16)
-    return fail(TTPA_ERR_UNSUPPORTED, "decode: kv_format %d not built", kv_format);
+  if (kv_format != TTPA_KV_BF16 && kv_format != TTPA_KV_BFP8)
+    return fail(TTPA_ERR_INVALID_ARGUMENT, "decode: unknown kv_format %d", kv_format);
+  if (kv_format == TTPA_KV_BFP8 && ((head_size != 64 && head_size != 128) || block_size % 16))
+    return fail(TTPA_ERR_UNSUPPORTED,
+                "decode: block-float-8 is built for head_size 64 / 128 and block_size %% 16 == 0");
   if (users > kMaxUsers)
     return fail(TTPA_ERR_UNSUPPORTED, "decode: %d users exceeds the limit of %d", users, kMaxUsers);
   if (head_size != 64 && head_size != 128 && head_size != 256)
@@ -646,6 +391,7 @@ extern "C" int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_
   a.ws_slots = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + header_bytes(users, kv_heads));
   a.n_waves = waves_for_device();
   a.slot_floats = slot_floats_for(g, head_size);
+  a.kv_format = kv_format;
 
   hipStream_t st = static_cast<hipStream_t>(stream);
   int rc = TTPA_OK;

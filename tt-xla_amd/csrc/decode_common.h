@@ -1,0 +1,328 @@
+// Pieces shared by the bf16 and block-float-8 paged decode kernels: launch arguments,
+// tile-list prefix, wave-level reductions, the partial-merge kernel and workspace sizing.
+#pragma once
+
+#include "common.h"
+
+#include <type_traits>
+
+namespace ttpa {
+namespace decode {
+
+
+constexpr int kMaxUsers = 2048;
+constexpr int kTile = 64;
+constexpr int kWavesPerBlock = 4;
+
+struct DecodeArgs {
+  uint16_t *out;
+  int64_t out_us, out_hs;
+  const uint16_t *q;
+  int64_t q_us, q_hs;
+  const uint8_t *k, *v;
+  const int32_t *pt;
+  int64_t pt_rs;
+  const void *cur;
+  int cur_i64;
+  int users, hq, hkv, bs, w, nb;
+  float scale_log2e;
+  int *ws_seg;   // [users * hkv][2]: first partial slot and number of partials per segment
+  float *ws_slots;
+  int n_waves;
+  int slot_floats;
+  int kv_format;
+};
+
+__device__ __forceinline__ int tiles_of_user(const DecodeArgs &a, const void *__restrict__ cur,
+                                             int u, int &len) {
+  int64_t cp = load_index(cur, a.cur_i64, u);
+  int64_t cap = (int64_t)a.w * a.bs;
+  int64_t l = cp < 0 ? 0 : (cp + 1 < cap ? cp + 1 : cap);
+  len = (int)l;
+  return (int)((l + kTile - 1) / kTile);
+}
+
+// Exclusive prefix sum of per-user tile counts into pref[0..users] and attended lengths into
+// lens[0..users); all 256 threads.  Each position is read from global memory once.
+__device__ inline void build_prefix(const DecodeArgs &a, const void *__restrict__ cur, int *pref,
+                             int *lens, int *wave_sums) {
+  const int tid = threadIdx.x;
+  const int per = (a.users + 255) / 256;
+  const int beg = tid * per;
+  const int end = min(beg + per, a.users);
+  int local = 0;
+  for (int u = beg; u < end; ++u) {
+    int len;
+    int nt = tiles_of_user(a, cur, u, len);
+    lens[u] = len;
+    pref[u + 1] = nt;  // replaced by the running sum below
+    local += nt;
+  }
+  int incl = local;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    int o = __shfl_up(incl, d);
+    if ((tid & 63) >= d) incl += o;
+  }
+  if ((tid & 63) == 63) wave_sums[tid >> 6] = incl;
+  __syncthreads();
+  int run = incl - local;
+  for (int wv = 0; wv < (tid >> 6); ++wv) run += wave_sums[wv];
+  if (tid == 0) pref[0] = 0;
+  for (int u = beg; u < end; ++u) {
+    run += pref[u + 1];
+    pref[u + 1] = run;
+  }
+  __syncthreads();
+}
+
+// LDS probabilities are written as 16-bit values and read back as 32-bit pairs
+typedef uint16_t __attribute__((may_alias)) lds_u16;
+typedef uint32_t __attribute__((may_alias)) lds_u32;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Streaming (non-temporal) load of DW dwords: K/V are read once per launch, so they
+// should not displace anything in L2 / MALL.
+// `ubase` is wavefront-uniform and `lane_bytes` a 32-bit per-lane offset, which lets the
+// load use the scalar-base addressing form: no per-load 64-bit address registers.
+template <int DW>
+__device__ __forceinline__ void load_stream(const uint16_t *ubase, uint32_t lane_bytes,
+                                            uint32_t (&d)[DW]) {
+  const char *p = reinterpret_cast<const char *>(ubase) + static_cast<uint64_t>(lane_bytes);
+  if constexpr (DW == 4) {
+    u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+    d[0] = t.x, d[1] = t.y, d[2] = t.z, d[3] = t.w;
+  } else {
+    u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(p));
+    d[0] = t.x, d[1] = t.y;
+  }
+}
+template <int DW>
+__device__ __forceinline__ void load_dwords(const uint16_t *p, uint32_t (&d)[DW]) {
+  if constexpr (DW == 4) {
+    uint4 t = *reinterpret_cast<const uint4 *>(p);
+    d[0] = t.x, d[1] = t.y, d[2] = t.z, d[3] = t.w;
+  } else {
+    uint2 t = *reinterpret_cast<const uint2 *>(p);
+    d[0] = t.x, d[1] = t.y;
+  }
+}
+
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf2;
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, a), __builtin_bit_cast(bf2, b), c,
+                                         false);
+}
+
+// Level L of the reduce-scatter exchanges along one lane bit inside a row of 16.
+// The exchange pattern of a level may flip lane bits that LATER levels partition on,
+// never earlier ones: mirror (^15) splits on bit 3, half-mirror (^7) on bit 2, then
+// ^2 on bit 1 and ^1 on bit 0.  After four levels lane c holds load bitrev4(c).
+template <int LEVEL>
+__device__ __forceinline__ float rs_exchange(float v) {
+  if constexpr (LEVEL == 1) return dpp_move<kDppMirror>(v);
+  if constexpr (LEVEL == 2) return dpp_move<kDppHalfMirror>(v);
+  if constexpr (LEVEL == 3) return dpp_move<kDppXor2>(v);
+  return dpp_move<kDppXor1>(v);
+}
+
+template <int LEVEL, int BASE, int G, int NH, int DW>
+__device__ __forceinline__ void qk_reduce_scatter(const uint32_t (&k)[NH][16][DW],
+                                                  const uint32_t (&q)[G][NH][DW], int c,
+                                                  float (&s)[G]) {
+  if constexpr (LEVEL == 0) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float acc = 0.f;
+#pragma unroll
+      for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+        for (int j = 0; j < DW; ++j) acc = dot2(k[hf][BASE][j], q[g][hf][j], acc);
+      s[g] = acc;
+    }
+  } else {
+    float lo[G], hi[G];
+    qk_reduce_scatter<LEVEL - 1, BASE, G, NH, DW>(k, q, c, lo);
+    qk_reduce_scatter<LEVEL - 1, BASE + (1 << (LEVEL - 1)), G, NH, DW>(k, q, c, hi);
+    const bool upper = (c >> (4 - LEVEL)) & 1;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float keep = upper ? hi[g] : lo[g];
+      float send = upper ? lo[g] : hi[g];
+      s[g] = keep + rs_exchange<LEVEL>(send);
+    }
+  }
+}
+
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_move<kDppXor1>(v));
+  v = fmaxf(v, dpp_move<kDppXor2>(v));
+  v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+  v = fmaxf(v, dpp_move<kDppMirror>(v));
+  return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_move<kDppXor1>(v);
+  v += dpp_move<kDppXor2>(v);
+  v += dpp_move<kDppHalfMirror>(v);
+  v += dpp_move<kDppMirror>(v);
+  return v;
+}
+
+__device__ __forceinline__ int bitrev4(int c) {
+  return ((c & 1) << 3) | ((c & 2) << 1) | ((c & 4) >> 1) | ((c & 8) >> 3);
+}
+
+template <int D, int G>
+struct Shape {
+  static constexpr int HD = D > 128 ? 128 : D;  // elements covered by one load pass
+  static constexpr int NH = D / HD;
+  static constexpr int EPL = HD / 16;  // elements per lane per pass
+  static constexpr int DW = EPL / 2;
+};
+
+// Position of a wavefront in the flat tile list.
+struct Cursor {
+  int u, h, t;      // user, kv head, tile index inside the segment
+  int len;          // attended positions of user u
+  int tiles_left;   // tiles of this segment from t on (including t)
+};
+
+// Finds the segment that owns unit `x` of the flat tile list (binary search over the
+// per-user prefix in LDS).  Everything is wavefront-uniform.
+__device__ __forceinline__ Cursor locate_unit(const int *s_pref, const int *s_len, int users,
+                                              int hkv, int64_t x) {
+  int lo_u = 0, hi_u = users - 1;
+  while (lo_u < hi_u) {
+    int mid = (lo_u + hi_u + 1) >> 1;
+    if ((int64_t)__builtin_amdgcn_readfirstlane(s_pref[mid]) * hkv <= x) lo_u = mid;
+    else hi_u = mid - 1;
+  }
+  Cursor cu;
+  cu.u = lo_u;
+  const int pref_u = __builtin_amdgcn_readfirstlane(s_pref[lo_u]);
+  const int nt = __builtin_amdgcn_readfirstlane(s_pref[lo_u + 1]) - pref_u;
+  const int rem = (int)(x - (int64_t)pref_u * hkv);
+  cu.h = rem / nt;
+  cu.t = rem - cu.h * nt;
+  cu.tiles_left = nt - cu.t;
+  cu.len = __builtin_amdgcn_readfirstlane(s_len[lo_u]);
+  return cu;
+}
+
+// One thread per segment (the first blocks of the grid): publishes which partial slots the
+// merge kernel has to read for that segment.
+__device__ __forceinline__ void publish_segment_row(const DecodeArgs &a, const int *s_pref,
+                                                    int64_t total, int n_eff) {
+  const int seg = blockIdx.x * 256 + threadIdx.x;
+  if (seg >= a.users * a.hkv) return;
+  const int su = seg / a.hkv, sh = seg - su * a.hkv;
+  const int snt = s_pref[su + 1] - s_pref[su];
+  int first = 0, count = 0;
+  if (snt > 0) {
+    const int64_t x0 = (int64_t)s_pref[su] * a.hkv + (int64_t)sh * snt;
+    const int64_t x1 = x0 + snt - 1;
+    // wave owning unit x: largest w with floor(w * total / n_eff) <= x; every wave in
+    // [w0, w1] owns at least one unit of the segment because n_eff <= total
+    const int w0 = (int)(((x0 + 1) * n_eff + total - 1) / total) - 1;
+    const int w1 = (int)(((x1 + 1) * n_eff + total - 1) / total) - 1;
+    first = w0 + seg;
+    count = w1 - w0 + 1;
+  }
+  a.ws_seg[2 * seg] = first;
+  a.ws_seg[2 * seg + 1] = count;
+}
+
+// Merges the row streams of a wavefront (4 rows of 16 lanes) for one head and writes the
+// partial (un-normalised output, running max, running sum) of (wave, segment).
+template <int D, int NH, int EPL>
+__device__ __forceinline__ void write_partial(float *slot, int g, int G, int r, int c, float m,
+                                              float l, float (&acc)[NH][EPL]) {
+  float lr = row16_sum(l);
+  float mall = fmaxf(m, __shfl_xor(m, 16));
+  mall = fmaxf(mall, __shfl_xor(mall, 32));
+  float wgt = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - mall);
+  lr *= wgt;
+  lr += __shfl_xor(lr, 16);
+  lr += __shfl_xor(lr, 32);
+#pragma unroll
+  for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      float v = acc[hf][e] * wgt;
+      v += __shfl_xor(v, 16);
+      v += __shfl_xor(v, 32);
+      acc[hf][e] = v;
+    }
+  if (r == 0) {
+    constexpr int HD = D > 128 ? 128 : D;
+#pragma unroll
+    for (int hf = 0; hf < NH; ++hf) {
+      float *dst = slot + g * D + hf * HD + c * EPL;
+#pragma unroll
+      for (int e4 = 0; e4 < EPL / 4; ++e4)
+        *reinterpret_cast<float4 *>(dst + 4 * e4) = make_float4(
+            acc[hf][4 * e4], acc[hf][4 * e4 + 1], acc[hf][4 * e4 + 2], acc[hf][4 * e4 + 3]);
+    }
+    if (c == 0) {
+      slot[G * D + g] = mall;
+      slot[G * D + G + g] = lr;
+    }
+  }
+}
+
+// Merges the partials of one (user, kv_head) segment and writes bfloat16 output.
+// Partials are read four at a time so that their loads overlap.
+template <int D, int G>
+__global__ __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a) {
+  const int seg = blockIdx.x;
+  const int u = seg / a.hkv, h = seg % a.hkv;
+  const int first = a.ws_seg[2 * seg], nw = a.ws_seg[2 * seg + 1];
+  uint16_t *out = a.out + u * a.out_us;
+  if (nw == 0) {  // padded row: no attended position -> NaN like softmax over nothing
+    for (int i = threadIdx.x; i < G * D; i += 256)
+      out[(int64_t)(h * G + i / D) * a.out_hs + (i % D)] = 0x7fc0;
+    return;
+  }
+  const float *base = a.ws_slots + (int64_t)first * a.slot_floats;
+  for (int i = threadIdx.x; i < G * D; i += 256) {
+    const int g = i / D;
+    float mall = -INFINITY, num = 0.f, den = 0.f;
+    for (int w = 0; w < nw; w += 4) {
+      float mv[4], lv[4], av[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float *sl = base + (int64_t)min(w + j, nw - 1) * a.slot_floats;
+        mv[j] = (w + j < nw) ? sl[G * D + g] : -INFINITY;
+        lv[j] = sl[G * D + G + g];
+        av[j] = sl[i];
+      }
+      float mnew = fmaxf(fmaxf(fmaxf(mv[0], mv[1]), fmaxf(mv[2], mv[3])), mall);
+      float resc = __builtin_amdgcn_exp2f(mall - mnew);
+      num *= resc;
+      den *= resc;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float wgt = __builtin_amdgcn_exp2f(mv[j] - mnew);  // 0 for the padding entries
+        num = fmaf(wgt, av[j], num);
+        den = fmaf(wgt, lv[j], den);
+      }
+      mall = mnew;
+    }
+    out[(int64_t)(h * G + g) * a.out_hs + (i % D)] = (uint16_t)f32_to_bf16_bits(num / den);
+  }
+}
+
+inline int slot_floats_for(int g, int d) { return ((g * d + 2 * g + 3) / 4) * 4; }
+inline size_t header_bytes(int users, int hkv) { return (((size_t)users * hkv * 8 + 255) / 256) * 256; }
+
+
+int waves_for_device();
+constexpr int kWavesPerBlockHost = kWavesPerBlock;
+
+// Launches the block-float-8 main kernel (decode_bfp8.hip); false = shape not built.
+bool launch_bfp8_main(const DecodeArgs &a, int head_size, int g, hipStream_t st);
+
+}  // namespace decode
+}  // namespace ttpa

@@ -162,3 +162,29 @@ def decode_config4(seed: int = 4, users: int = 128, num_blocks: int = 16384,
     return decode_ragged("config4-llama3-70b-b128-h64x8-d128-bs64-ctx256..32768", seed + 1000,
                          users, 64, 8, 128, 64, num_blocks, ctx, table_width=520,
                          cache_device=cache_device)
+
+
+def add_outlier_channels(wl: DecodeWorkload, seed: int, fraction: float = 0.01, gain: float = 20.0):
+    """Scales a random `fraction` of the (kv_head, head_dim) channels of K and V (cache and new
+    token) by `gain`: the outlier-channel distribution of the block-float-8 configuration."""
+    g = torch.Generator().manual_seed(seed)
+    _, hkv, _, d = wl.k_cache.shape
+    n = max(1, int(round(fraction * hkv * d)))
+    for cache, new in ((wl.k_cache, wl.k_new), (wl.v_cache, wl.v_new)):
+        ch = torch.randperm(hkv * d, generator=g)[:n]
+        hh, dd = (ch // d).to(cache.device), (ch % d).to(cache.device)
+        cache[:, hh, :, dd] = (cache[:, hh, :, dd].float() * gain).to(cache.dtype)
+        new[:, :, hh.cpu(), dd.cpu()] = (new[:, :, hh.cpu(), dd.cpu()].float() * gain).to(new.dtype)
+    return wl
+
+
+def decode_config5(seed: int = 5, users: int = 32, num_blocks: int = 4096,
+                   cache_device: Optional[str] = None) -> DecodeWorkload:
+    """The Llama-3-8B decode shape with N(0, 1) K/V where 1% of the channels are scaled x20.
+    The caches are returned in bfloat16; the caller packs them to block-float-8."""
+    g = torch.Generator().manual_seed(seed)
+    ctx = torch.randint(512, 4097, (users,), generator=g).tolist()
+    wl = decode_ragged("config5-llama3-8b-bfp8-b32-h32x8-d128-bs64-ctx512..4096", seed + 1000,
+                       users, 32, 8, 128, 64, num_blocks, ctx, table_width=72,
+                       cache_device=cache_device)
+    return add_outlier_channels(wl, seed + 2000)
