@@ -1,15 +1,23 @@
 #!/usr/bin/env python3
-"""Headline benchmark: Llama-3-8B-shaped paged decode on one MI355X.
+"""Benchmark of the paged KV-cache write + paged attention path on one MI355X.
 
-A step is what one attention layer does for one generated token of every sequence:
-K cache update + V cache update + paged decode attention, on synthetic data of the
-workload's shape already resident in HBM.  The timed region replays a HIP graph of that
-step (captured through the torch.ops.tt operators) on `--rotate` independent copies of
-the workload, so consecutive steps never touch the same cache lines.
+Default (the headline): Llama-3-8B-shaped paged decode (`--workload config2`).  A step is
+what one attention layer does for one generated token of every sequence: K cache update +
+V cache update + paged decode attention, on synthetic data of the workload's shape already
+resident in HBM.  The timed region replays a HIP graph of that step (captured through the
+torch.ops.tt operators) over `--rotate` independent copies of the workload, so consecutive
+steps never touch the same cache lines.
 
-Prints ONE JSON line: value = algorithmic HBM bytes of a step / time of a step (GB/s),
-with tokens/s alongside, the roofline of the dominant kernel (the split-K decode kernel,
-timed alone with HIP events) and the CPU oracle timed on this box's host cores.
+Other workloads (same JSON contract):
+  config4  Llama-3-70B-shaped decode, batch 128, context 256..32768, fragmented pool
+           (its 4 x 512-token chunked-prefill pass is timed separately, see "chunk_pass")
+  config5  config2 with a block-float-8 KV cache (dequantised inside the decode kernel)
+  config3  causal prefill, 4 x 2048 tokens: K fill + V fill + MFMA attention; value is
+           useful TFLOP/s
+
+Prints ONE JSON line.  `roofline` is the dominant kernel alone, bracketed by HIP events
+inside the library; `cpu_baseline` is the CPU oracle timed on this box's host cores on a
+bounded sample of the same workload.
 """
 
 import argparse
@@ -25,7 +33,9 @@ for _p in (ROOT, os.path.join(ROOT, "tt-xla_amd")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
-HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
+CPU_THREADS_CAP = 16        # host cores a one-GPU box grants, whatever os.cpu_count() says
 
 
 def parse():
@@ -35,9 +45,12 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--rotate", type=int, default=3, help="independent workload copies cycled through")
     ap.add_argument("--launch", choices=["graph", "eager"], default="graph")
-    ap.add_argument("--workload", choices=["config2", "config4"], default="config2")
+    ap.add_argument("--workload", choices=["config2", "config3", "config4", "config5"], default="config2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-users", type=int, default=0, help="users in the CPU sample (0 = auto)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain 256 MiB device copies, so that a counter run of this "
+                         "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     return ap.parse_args()
 
 
@@ -48,7 +61,6 @@ class HipEvents:
         self.hip = ctypes.CDLL("libamdhip64.so")
         self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
         self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
-        self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
 
     def create(self):
         ev = ctypes.c_void_p()
@@ -63,15 +75,16 @@ class HipEvents:
         return ms.value
 
 
-def make_workload(name, seed, device):
+# --------------------------------------------------------------------------- workloads
+def make_decode(name, seed, device):
     from tt_xla_amd import workloads
 
-    if name == "config2":
-        return workloads.decode_config2(seed=seed, cache_device=device)
-    return workloads.decode_config4(seed=seed, cache_device=device)
+    fn = {"config2": workloads.decode_config2, "config4": workloads.decode_config4,
+          "config5": workloads.decode_config5}[name]
+    return fn(seed=seed, cache_device=device)
 
 
-def step(g):
+def decode_step(g):
     import torch
 
     torch.ops.tt.paged_update_cache_(g.k_cache, g.k_new, g.cache_position, g.page_table)
@@ -82,51 +95,283 @@ def step(g):
     )
 
 
-def cpu_baseline(args):
-    """The CPU oracle (restated reference CPU ops, functional cache clones included) on a
-    bounded sample of the same workload: the first `n` users, full-size pool."""
+def make_prefill_impl(w):
+    from tt_xla_amd import TTAttentionBackendImpl
+
+    return TTAttentionBackendImpl(w.q_heads, w.head_size, w.head_size**-0.5, w.kv_heads, None, None, "auto")
+
+
+def prefill_step(impl, w, out):
+    """The backend's prefill pass: K fill + V fill + causal attention (dense on the fresh K/V
+    for a first chunk, paged with the cached prefix for a continuation chunk)."""
+    from tt_xla_amd import TTMetadata
+
+    md = TTMetadata(cache_position=None, page_table=w.page_table, num_users=w.users,
+                    batch_idx=w.batch_idx, fill_page_table=w.fill_page_table,
+                    chunk_start_idx=w.chunk_start)
+    impl.forward(None, w.q, w.k, w.v, [w.k_cache, w.v_cache], md, output=out)
+    return out
+
+
+# --------------------------------------------------------------------------- timing helpers
+def build_launchers(fns, use_graph):
     import torch
 
+    if not use_graph:
+        return fns, None
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for f in fns:  # warm allocator and kernels outside capture
+            f()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graphs, keep = [], []
+    for f in fns:
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            keep.append(f())
+        graphs.append(gr)
+    return [gr.replay for gr in graphs], keep
+
+
+def time_steps(launchers, steps, warmup):
+    import torch
+
+    n = len(launchers)
+    for i in range(warmup):
+        launchers[i % n]()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        launchers[i % n]()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def time_dominant_kernel(fns, iters):
+    """Eager launches with HIP events armed around the dominant kernel of each call."""
+    import torch
+
+    from tt_xla_amd import _native
+
+    ev = HipEvents()
+    pairs, n = [], len(fns)
+    for i in range(iters + 5):
+        a, b = ev.create(), ev.create()
+        _native.call("ttpa_profile_next_attention", a, b)
+        fns[i % n]()
+        if i >= 5:
+            pairs.append((a, b, i % n))
+    torch.cuda.synchronize()
+    return [(ev.elapsed_ms(a, b), which) for a, b, which in pairs]
+
+
+# --------------------------------------------------------------------------- CPU baselines
+def cpu_decode_baseline(args):
+    """The CPU oracle (restated reference CPU ops, functional cache clones included) on the
+    first `n` users of the workload, full-size pool.  For the block-float-8 workload the CPU
+    leg is the codec round trip followed by the same attention."""
+    import torch
+
+    from oracle import bfp8_codec
     from oracle import paged_ops as O
     from tt_xla_amd import workloads
 
-    cores = os.cpu_count() or 1
-    # the box grants 16 cores per GPU whatever os.cpu_count() says
-    threads = min(cores, 16)
+    threads = min(os.cpu_count() or 1, CPU_THREADS_CAP)
     torch.set_num_threads(threads)
-    wl = make_workload(args.workload, 2, None)
+    if args.workload == "config4":
+        wl = workloads.decode_config4(seed=2, num_blocks=16384)
+    else:
+        wl = make_decode(args.workload, 2, None)
     total_users = wl.q.shape[1]
+    k_cache, v_cache = wl.k_cache, wl.v_cache
+    note = ""
+    if args.workload == "config5":
+        t0 = time.perf_counter()
+        k_cache = bfp8_codec.roundtrip(k_cache).to(torch.bfloat16)
+        v_cache = bfp8_codec.roundtrip(v_cache).to(torch.bfloat16)
+        note = f"; codec round trip of both caches (not in the step time) took {time.perf_counter() - t0:.1f} s"
 
     def run(n):
         q, kn, vn = wl.q[:, :n], wl.k_new[:, :n], wl.v_new[:, :n]
         pt, pos = wl.page_table[:n], wl.cache_position[:n]
         t0 = time.perf_counter()
-        k = O.paged_update_cache(wl.k_cache, kn, pos, pt)
-        v = O.paged_update_cache(wl.v_cache, vn, pos, pt)
+        k = O.paged_update_cache(k_cache, kn, pos, pt)
+        v = O.paged_update_cache(v_cache, vn, pos, pt)
         O.paged_sdpa_decode(q, k, v, pt, True, None, pos, None, wl.scale)
         return time.perf_counter() - t0
 
-    n = args.cpu_users or min(4, total_users)
-    first = run(n)  # warm-up, also sizes the sample
+    n = args.cpu_users or min(2, total_users)
+    first = run(n)
     if not args.cpu_users:
-        per_user = max(first / n, 1e-3)
-        n = max(1, min(total_users, int(6.0 / per_user)))
+        n = max(1, min(total_users, 16 if args.workload == "config4" else total_users,
+                       int(6.0 / max(first / n, 1e-3))))
     times = [run(n) for _ in range(3)]
     t = statistics.median(times)
     sub = workloads.DecodeWorkload(wl.name, wl.q[:, :n], wl.k_new[:, :n], wl.v_new[:, :n],
                                    wl.k_cache, wl.v_cache, wl.page_table[:n],
                                    wl.cache_position[:n], wl.scale)
-    nbytes = sub.decode_bytes() + sub.update_bytes()
+    e_kv = 17.0 / 16.0 if args.workload == "config5" else 2.0
+    nbytes = sub.decode_bytes(e_kv) + sub.update_bytes()
     return {
-        "value": nbytes / t / 1e9,
-        "unit": "GB/s",
-        "cores": threads,
-        "kind": "port",
-        "sample": f"first {n} of {total_users} users of {wl.name}, full-size cache pool, "
-                  f"median of 3 steps after 1 warm-up ({t * 1e3:.0f} ms/step, "
-                  f"{n / t:.1f} tokens/s), torch {torch.__version__}",
-        "tokens_per_s": n / t,
+        "value": nbytes / t / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"first {n} of {total_users} users of {wl.name}, full-size cache pool, median of 3 "
+                  f"steps after 1 warm-up ({t * 1e3:.0f} ms/step, {n / t:.1f} tokens/s), "
+                  f"torch {torch.__version__}{note}",
+        "tokens_per_s": n / t, "ms_per_step": t * 1e3,
+    }
+
+
+def cpu_prefill_baseline(args):
+    import torch
+
+    from oracle import paged_ops as O
+    from tt_xla_amd import workloads
+
+    threads = min(os.cpu_count() or 1, CPU_THREADS_CAP)
+    torch.set_num_threads(threads)
+    w = workloads.prefill_config3()
+    n, s = 1, w.seq
+    q = w.q[: n * s].view(n, s, w.q_heads, w.head_size).transpose(1, 2)
+    k = w.k[: n * s].view(n, s, w.kv_heads, w.head_size).transpose(1, 2)
+    v = w.v[: n * s].view(n, s, w.kv_heads, w.head_size).transpose(1, 2)
+    bidx = w.batch_idx[:n]
+
+    def run():
+        t0 = time.perf_counter()
+        kc = O.paged_fill_cache_batched(w.k_cache, k, w.fill_page_table, bidx)
+        vc = O.paged_fill_cache_batched(w.v_cache, v, w.fill_page_table, bidx)
+        O.sdpa(q, k, v, None, True, w.head_size**-0.5)
+        del kc, vc
+        return time.perf_counter() - t0
+
+    run()
+    t = statistics.median([run() for _ in range(3)])
+    flops = w.useful_flops() * n / w.users
+    return {
+        "value": flops / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": f"first {n} of {w.users} prompts of {w.name} (fill K, fill V with functional cache "
+                  f"clones, causal attention), median of 3 after 1 warm-up ({t * 1e3:.0f} ms), "
+                  f"torch {torch.__version__}",
         "ms_per_step": t * 1e3,
+    }
+
+
+# --------------------------------------------------------------------------- runs
+def run_decode(args):
+    import torch
+
+    from tt_xla_amd import custom_ops as ops
+
+    dev = "cuda:0"
+    copies = [make_decode(args.workload, 2 + i, dev).to(dev) for i in range(max(1, args.rotate))]
+    e_kv, dtype = 2.0, "bf16"
+    if args.workload == "config5":
+        for c in copies:  # caches become block-float-8 (uint8) tensors
+            c.k_cache = ops.bfp8_pack_cache(c.k_cache)
+            c.v_cache = ops.bfp8_pack_cache(c.v_cache)
+        e_kv, dtype = 17.0 / 16.0, "bfp8 cache, bf16 activations, f32 accumulate"
+        torch.cuda.empty_cache()
+    wl = copies[0]
+    nb, hkv, _, d = wl.k_cache.shape
+    shape = dict(users=wl.q.shape[1], q_heads=wl.q.shape[2], kv_heads=hkv, head_size=d,
+                 block_size=64, num_blocks=nb, table_width=wl.page_table.shape[1])
+    dec_bytes = [c.decode_bytes(e_kv) for c in copies]
+    step_bytes = [b + c.update_bytes() for b, c in zip(dec_bytes, copies)]
+    fns = [(lambda c=c: decode_step(c)) for c in copies]
+    launchers, _keep = build_launchers(fns, args.launch == "graph")
+    ms = time_steps(launchers, args.steps, args.warmup)
+    n = len(copies)
+    avg_step_bytes = sum(step_bytes[i % n] for i in range(args.steps)) / args.steps
+    durs = time_dominant_kernel(fns, min(args.steps, 100))
+    kern_ms = sum(d for d, _ in durs) / len(durs)
+    kern_bytes = sum(dec_bytes[w] for _, w in durs) / len(durs)
+    achieved = kern_bytes / (kern_ms * 1e-3) / 1e9
+    out = {
+        "metric": "paged_decode_attention_hbm_throughput",
+        "value": avg_step_bytes / (ms * 1e-3) / 1e9,
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic",
+        "config": {
+            "workload": wl.name,
+            "step": "K update + V update + paged decode attention, one layer, one token per sequence",
+            "launch": args.launch, "rotating_copies": n, **shape,
+            "mean_context": float(wl.cache_position.float().mean()),
+        },
+        "tokens_per_s": shape["users"] / (ms * 1e-3),
+        "pct_of_hbm_peak": 100.0 * avg_step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "roofline": {
+            "kernel": "paged_decode_bfp8_kernel" if args.workload == "config5" else "paged_decode_kernel",
+            "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+            "kernel_us": kern_ms * 1e3, "kernel_us_min": min(d for d, _ in durs) * 1e3,
+            "bytes_per_launch": kern_bytes, "timed_launches": len(durs),
+        },
+    }
+    if args.workload == "config4":
+        from tt_xla_amd import workloads
+
+        w = workloads.prefill_config4_chunks(device=dev).to(dev)
+        impl = make_prefill_impl(w)
+        outbuf = torch.empty_like(w.q)
+        chunk = [lambda: prefill_step(impl, w, outbuf)]
+        cl, _k2 = build_launchers(chunk, args.launch == "graph")
+        cms = time_steps(cl, min(args.steps, 50), 5)
+        cd = time_dominant_kernel(chunk, 20)
+        ck = sum(x for x, _ in cd) / len(cd)
+        out["chunk_pass"] = {
+            "workload": w.name, "ms_per_pass": cms, "attention_kernel_us": ck * 1e3,
+            "useful_tflops": w.useful_flops() / (ck * 1e-3) / 1e12,
+            "frac_of_bf16_mfma_peak": w.useful_flops() / (ck * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+        }
+    return out
+
+
+def run_prefill(args):
+    import torch
+
+    from tt_xla_amd import workloads
+
+    dev = "cuda:0"
+    copies = [workloads.prefill_config3(seed=3 + i, device=dev).to(dev) for i in range(max(1, args.rotate))]
+    impls = [make_prefill_impl(w) for w in copies]
+    outs = [torch.empty_like(w.q) for w in copies]
+    fns = [(lambda i=i: prefill_step(impls[i], copies[i], outs[i])) for i in range(len(copies))]
+    launchers, _keep = build_launchers(fns, args.launch == "graph")
+    steps = min(args.steps, 100)
+    ms = time_steps(launchers, steps, min(args.warmup, 10))
+    w = copies[0]
+    flops = w.useful_flops()
+    durs = time_dominant_kernel(fns, min(steps, 50))
+    kern_ms = sum(d for d, _ in durs) / len(durs)
+    achieved = flops / (kern_ms * 1e-3) / 1e12
+    return {
+        "metric": "paged_prefill_attention_useful_tflops",
+        "value": flops / (ms * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": steps, "warmup": min(args.warmup, 10), "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "workload": w.name,
+            "step": "K fill + V fill through the fill page table + causal attention on the fresh K/V",
+            "launch": args.launch, "rotating_copies": len(copies), "users": w.users,
+            "tokens_per_user": w.seq, "q_heads": w.q_heads, "kv_heads": w.kv_heads,
+            "head_size": w.head_size, "block_size": 64,
+        },
+        "tokens_per_s": w.users * w.seq / (ms * 1e-3),
+        "fill_bytes_per_step": w.fill_bytes(),
+        "roofline": {
+            "kernel": "prefill_kernel", "bound": "mfma", "achieved": achieved,
+            "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+            "kernel_us": kern_ms * 1e3, "kernel_us_min": min(d for d, _ in durs) * 1e3,
+            "flops_per_launch": flops, "timed_launches": len(durs),
+            "note": "useful (causal) FLOPs only; the dense 4*B*Hq*S^2*D figure is twice this",
+        },
     }
 
 
@@ -144,105 +389,24 @@ def main():
 
     entry.ensure_built()
     import tt_xla_amd  # noqa: F401
-    from tt_xla_amd import _native
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
-    dev = "cuda:0"
     torch.cuda.set_device(0)
-    copies = [make_workload(args.workload, 2 + i, dev).to(dev) for i in range(max(1, args.rotate))]
-    wl = copies[0]
-    shape = wl.shape
-    step_bytes = [c.decode_bytes() + c.update_bytes() for c in copies]
-    decode_bytes = [c.decode_bytes() for c in copies]
-
-    # ---- build the launchers -------------------------------------------------------
-    if args.launch == "graph":
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for c in copies:  # warm allocator and kernels outside capture
-                step(c)
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        graphs, keep = [], []
-        for c in copies:
-            gr = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(gr):
-                keep.append(step(c))
-            graphs.append(gr)
-        launchers = [gr.replay for gr in graphs]
+    if args.workload == "config3":
+        out = run_prefill(args)
+        if not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_prefill_baseline(args)
     else:
-        launchers = [(lambda c=c: step(c)) for c in copies]
-
-    n = len(launchers)
-    for i in range(args.warmup):
-        launchers[i % n]()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        launchers[i % n]()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    avg_step_bytes = sum(step_bytes[i % n] for i in range(args.steps)) / args.steps
-    users = shape["users"]
-
-    # ---- dominant kernel alone: HIP events armed around the split-K decode kernel -------
-    ev = HipEvents()
-    pairs = []
-    k_iters = min(args.steps, 100)
-    for i in range(k_iters + 5):
-        c = copies[i % n]
-        a, b = ev.create(), ev.create()
-        _native.call("ttpa_profile_next_attention", a, b)
-        step(c)
-        if i >= 5:
-            pairs.append((a, b, decode_bytes[i % n]))
-    torch.cuda.synchronize()
-    durs = [ev.elapsed_ms(a, b) for a, b, _ in pairs]
-    kern_ms = sum(durs) / len(durs)
-    kern_bytes = sum(nb for _, _, nb in pairs) / len(pairs)
-    achieved = kern_bytes / (kern_ms * 1e-3) / 1e9
-
-    out = {
-        "metric": "paged_decode_attention_hbm_throughput",
-        "value": avg_step_bytes / (ms_per_step * 1e-3) / 1e9,
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
-        "config": {
-            "workload": wl.name,
-            "step": "K update + V update + paged decode attention, one layer, one token per sequence",
-            "launch": args.launch,
-            "rotating_copies": n,
-            **shape,
-            "mean_context": float(wl.cache_position.float().mean()),
-        },
-        "tokens_per_s": users / (ms_per_step * 1e-3),
-        "pct_of_hbm_peak": 100.0 * avg_step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-        "roofline": {
-            "kernel": "paged_decode_kernel",
-            "bound": "hbm",
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None,
-            "kernel_us": kern_ms * 1e3,
-            "kernel_us_min": min(durs) * 1e3,
-            "bytes_per_launch": kern_bytes,
-            "timed_launches": len(durs),
-        },
-    }
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(args)
+        out = run_decode(args)
+        if not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_decode_baseline(args)
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        out["calibration"] = {"kernel": "torch device copy", "bytes_read": 256 << 20, "bytes_written": 256 << 20}
     print(json.dumps(out), flush=True)
 
 

@@ -151,17 +151,141 @@ def decode_config2(seed: int = 2, users: int = 32, num_blocks: int = 4096,
                          cache_device=cache_device)
 
 
+def fragmented_block_order(gen: torch.Generator, num_blocks: int, rounds: int = 4) -> List[int]:
+    """Order in which a block pool hands out blocks after a seeded history of interleaved
+    allocations and frees (free list = queue, freed blocks return to its tail, as in vLLM's
+    block pool).  Block 0 stays reserved as the null block."""
+    free = list(range(1, num_blocks))
+    live: List[List[int]] = []
+    for _ in range(rounds):
+        # allocate variable-length requests until ~85% of the pool is in use
+        while len(free) > 0.15 * num_blocks:
+            n = int(torch.randint(1, 96, (1,), generator=gen))
+            n = min(n, len(free))
+            live.append(free[:n])
+            del free[:n]
+        # free a random half of the live requests, in random order
+        order = torch.randperm(len(live), generator=gen).tolist()
+        keep = []
+        for j, idx in enumerate(order):
+            if j % 2 == 0:
+                free.extend(live[idx])
+            else:
+                keep.append(live[idx])
+        live = keep
+    order = torch.randperm(len(live), generator=gen).tolist()
+    for idx in order:
+        free.extend(live[idx])
+    return free
+
+
 def decode_config4(seed: int = 4, users: int = 128, num_blocks: int = 16384,
                    cache_device: Optional[str] = None) -> DecodeWorkload:
     """Llama-3-70B shape on one GPU: 64/8 heads, head 128, block 64, batch 128, context
-    log-uniform in [256, 32768]."""
+    log-uniform in [256, 32768]; block tables come out of a pool fragmented by interleaved
+    allocations and frees, so they are non-contiguous and interleaved between users."""
     g = torch.Generator().manual_seed(seed)
     u = torch.rand(users, generator=g)
     ctx = torch.exp(math.log(256) + u * (math.log(32768) - math.log(256))).round().long()
     ctx = ctx.clamp(256, 32767).tolist()
-    return decode_ragged("config4-llama3-70b-b128-h64x8-d128-bs64-ctx256..32768", seed + 1000,
-                         users, 64, 8, 128, 64, num_blocks, ctx, table_width=520,
-                         cache_device=cache_device)
+    wl = decode_ragged("config4-llama3-70b-b128-h64x8-d128-bs64-ctx256..32768", seed + 1000,
+                       users, 64, 8, 128, 64, num_blocks, ctx, table_width=520,
+                       cache_device=cache_device)
+    order = fragmented_block_order(g, num_blocks)
+    need = [(c + 1 + 63) // 64 for c in ctx]
+    assert sum(need) <= len(order), "pool too small"
+    # users grow in round-robin bursts, like requests decoding side by side
+    table = torch.zeros_like(wl.page_table)
+    have = [0] * users
+    at = 0
+    while any(h < n for h, n in zip(have, need)):
+        for uu in range(users):
+            burst = min(4, need[uu] - have[uu])
+            for _ in range(burst):
+                table[uu, have[uu]] = order[at]
+                have[uu] += 1
+                at += 1
+    wl.page_table = table
+    return wl
+
+
+@dataclass
+class PrefillWorkload:
+    name: str
+    q: torch.Tensor  # [users * S, Hq * D] token-major, as the attention layer hands it over
+    k: torch.Tensor  # [users * S, Hkv * D]
+    v: torch.Tensor
+    k_cache: torch.Tensor
+    v_cache: torch.Tensor
+    page_table: torch.Tensor  # [users, W]
+    fill_page_table: torch.Tensor
+    batch_idx: torch.Tensor
+    chunk_start: Optional[torch.Tensor]  # [1] int32 or None (first chunk)
+    users: int
+    seq: int
+    q_heads: int
+    kv_heads: int
+    head_size: int
+
+    def to(self, device):
+        mv = lambda t: None if t is None else t.to(device)  # noqa: E731
+        return PrefillWorkload(self.name, mv(self.q), mv(self.k), mv(self.v), mv(self.k_cache),
+                               mv(self.v_cache), mv(self.page_table), mv(self.fill_page_table),
+                               mv(self.batch_idx), mv(self.chunk_start), self.users, self.seq,
+                               self.q_heads, self.kv_heads, self.head_size)
+
+    def useful_flops(self) -> float:
+        """4 * D * Hq * sum over users of (Lc * start + Lc (Lc + 1) / 2): the causal part only."""
+        start = 0 if self.chunk_start is None else int(self.chunk_start[0])
+        lc = self.seq
+        return 4.0 * self.head_size * self.q_heads * self.users * (lc * start + lc * (lc + 1) / 2)
+
+    def fill_bytes(self) -> int:
+        return 2 * 2 * self.users * self.seq * self.kv_heads * self.head_size * 2
+
+
+def prefill_workload(name: str, seed: int, users: int, seq: int, q_heads: int, kv_heads: int,
+                     head_size: int, block_size: int, start: int = 0,
+                     device: Optional[str] = None) -> PrefillWorkload:
+    """`users` prompts (or continuation chunks after `start` cached tokens, start a multiple of
+    the block size) of `seq` tokens; blocks from a random permutation of the pool."""
+    dev = device or "cpu"
+    g = torch.Generator(device=dev).manual_seed(seed)
+    cg = torch.Generator().manual_seed(seed)
+    assert start % block_size == 0
+    w = (start + seq + block_size - 1) // block_size
+    w = (w + 7) // 8 * 8
+    nb = users * w + 1
+    table = (torch.randperm(nb - 1, generator=cg) + 1).view(users, w).to(torch.int32)
+    mk = lambda *sh: torch.randn(*sh, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)  # noqa: E731
+    shape = (nb, kv_heads, block_size, head_size)
+    if start:
+        k_cache, v_cache = mk(*shape), mk(*shape)
+    else:
+        k_cache = torch.zeros(shape, dtype=torch.bfloat16, device=dev)
+        v_cache = torch.zeros(shape, dtype=torch.bfloat16, device=dev)
+    return PrefillWorkload(
+        name, mk(users * seq, q_heads * head_size), mk(users * seq, kv_heads * head_size),
+        mk(users * seq, kv_heads * head_size), k_cache, v_cache, table,
+        torch.roll(table, -(start // block_size), dims=1),
+        torch.arange(users, dtype=torch.int32),
+        torch.tensor([start], dtype=torch.int32) if start else None,
+        users, seq, q_heads, kv_heads, head_size,
+    )
+
+
+def prefill_config3(seed: int = 3, device: Optional[str] = None) -> PrefillWorkload:
+    """Causal prefill at the Llama-3-8B head shape: 4 prompts of 2048 tokens, 32/8 heads,
+    head 128, block 64."""
+    return prefill_workload("config3-llama3-8b-prefill-b4x2048-h32x8-d128-bs64", seed, 4, 2048,
+                            32, 8, 128, 64, 0, device)
+
+
+def prefill_config4_chunks(seed: int = 44, device: Optional[str] = None) -> PrefillWorkload:
+    """The chunked-prefill pass of the 70B configuration: 4 sequences, 512-token chunks on top
+    of 4096 cached tokens, 64/8 heads."""
+    return prefill_workload("config4-chunks-b4x512-start4096-h64x8-d128-bs64", seed, 4, 512, 64,
+                            8, 128, 64, 4096, device)
 
 
 def add_outlier_channels(wl: DecodeWorkload, seed: int, fraction: float = 0.01, gain: float = 20.0):
