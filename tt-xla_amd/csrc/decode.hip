@@ -24,6 +24,9 @@
 //   per KV head.
 #include "decode_common.h"
 
+#include <cstdlib>
+#include <cstring>
+
 namespace ttpa {
 namespace decode {
 
@@ -274,13 +277,13 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   process_tile(std::false_type{});
 }
 
-int waves_for_device() {
+int waves_for_device(int kv_format) {
   static int override_waves = -1;
   if (override_waves < 0) {
     const char *e = getenv("TTPA_DECODE_WAVES_PER_CU");
     override_waves = e ? atoi(e) : 0;
   }
-  int per_cu = override_waves > 0 ? override_waves : 4;
+  int per_cu = override_waves > 0 ? override_waves : (kv_format == TTPA_KV_BFP8 ? 8 : 4);
   int cus = device_cus();
   if (cus <= 0) cus = 256;
   int waves = cus * per_cu;
@@ -289,9 +292,6 @@ int waves_for_device() {
 
 template <int D, int G>
 void launch(const DecodeArgs &a, hipStream_t st) {
-  hipEvent_t ev0, ev1;
-  take_profile_events(ev0, ev1);
-  if (ev0) (void)hipEventRecord(ev0, st);
   if (a.kv_format == TTPA_KV_BFP8) {
     launch_bfp8_main(a, D, G, st);
   } else {
@@ -304,8 +304,6 @@ void launch(const DecodeArgs &a, hipStream_t st) {
     else
       paged_decode_kernel<D, G, false><<<dim3(blocks), dim3(256), pad, st>>>(a, a.pt, a.cur);
   }
-  if (ev1) (void)hipEventRecord(ev1, st);
-  decode_combine_kernel<D, G><<<dim3(a.users * a.hkv), dim3(256), 0, st>>>(a);
 }
 
 template <int D>
@@ -335,7 +333,7 @@ extern "C" size_t ttpa_paged_decode_workspace_bytes(int32_t users, int32_t q_hea
                                                     int32_t kv_heads, int32_t head_size) {
   if (users <= 0 || q_heads <= 0 || kv_heads <= 0 || head_size <= 0 || q_heads % kv_heads) return 0;
   int g = q_heads / kv_heads;
-  size_t slots = (size_t)waves_for_device() + (size_t)users * kv_heads;
+  size_t slots = (size_t)waves_for_device(TTPA_KV_BFP8) + (size_t)users * kv_heads;  // the larger grid
   return header_bytes(users, kv_heads) + slots * (size_t)slot_floats_for(g, head_size) * sizeof(float);
 }
 
@@ -389,17 +387,41 @@ extern "C" int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_
   a.scale_log2e = scale * 1.4426950408889634f;
   a.ws_seg = static_cast<int *>(workspace);
   a.ws_slots = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + header_bytes(users, kv_heads));
-  a.n_waves = waves_for_device();
+  a.n_waves = waves_for_device(kv_format);
   a.slot_floats = slot_floats_for(g, head_size);
   a.kv_format = kv_format;
 
   hipStream_t st = static_cast<hipStream_t>(stream);
-  int rc = TTPA_OK;
-  switch (head_size) {
-    case 64: rc = launch_g<64>(a, g, st); break;
-    case 128: rc = launch_g<128>(a, g, st); break;
-    default: rc = launch_g<256>(a, g, st); break;
+  // Kernel choice: the VALU kernel streams at the HBM ceiling up to 4 query heads per KV head;
+  // beyond that its per-head VALU work becomes the limiter and the matrix-core kernel takes
+  // over (its cost per tile does not depend on the group width).  The block-float-8 cache is
+  // bound by the byte -> bfloat16 expansion in either kernel.  TTPA_DECODE_KERNEL=valu|mfma
+  // overrides the choice.
+  static int forced = -1;
+  if (forced < 0) {
+    const char *e = getenv("TTPA_DECODE_KERNEL");
+    forced = !e ? 0 : (!strcmp(e, "valu") ? 1 : (!strcmp(e, "mfma") ? 2 : 0));
   }
+  const bool mfma_ok = mfma_decode_supported(a, head_size, g);
+  bool use_mfma = mfma_ok && g >= 5;
+  if (forced == 1) use_mfma = false;
+  if (forced == 2) use_mfma = mfma_ok;
+  hipEvent_t ev0, ev1;
+  take_profile_events(ev0, ev1);
+  if (ev0) (void)hipEventRecord(ev0, st);
+  int rc = TTPA_OK;
+  if (use_mfma) {
+    if (!launch_mfma_main(a, head_size, st))
+      rc = fail(TTPA_ERR_LAUNCH, "decode: cannot configure the matrix-core kernel");
+  } else {
+    switch (head_size) {
+      case 64: rc = launch_g<64>(a, g, st); break;
+      case 128: rc = launch_g<128>(a, g, st); break;
+      default: rc = launch_g<256>(a, g, st); break;
+    }
+  }
+  if (ev1) (void)hipEventRecord(ev1, st);
   if (rc) return rc;
+  decode_combine_kernel<<<dim3(users * kv_heads), dim3(256), 0, st>>>(a, g, head_size);
   return check_launch("paged_sdpa_decode");
 }

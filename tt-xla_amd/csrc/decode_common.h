@@ -273,9 +273,9 @@ __device__ __forceinline__ void write_partial(float *slot, int g, int G, int r, 
 }
 
 // Merges the partials of one (user, kv_head) segment and writes bfloat16 output.
-// Partials are read four at a time so that their loads overlap.
-template <int D, int G>
-__global__ __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a) {
+// Partials are read four at a time so that their loads overlap.  G and D are run-time values:
+// the matrix-core kernel serves any group width up to 32.
+__global__ inline __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a, int G, int D) {
   const int seg = blockIdx.x;
   const int u = seg / a.hkv, h = seg % a.hkv;
   const int first = a.ws_seg[2 * seg], nw = a.ws_seg[2 * seg + 1];
@@ -318,11 +318,14 @@ inline int slot_floats_for(int g, int d) { return ((g * d + 2 * g + 3) / 4) * 4;
 inline size_t header_bytes(int users, int hkv) { return (((size_t)users * hkv * 8 + 255) / 256) * 256; }
 
 
-int waves_for_device();
+int waves_for_device(int kv_format);
 constexpr int kWavesPerBlockHost = kWavesPerBlock;
 
-// Launches the block-float-8 main kernel (decode_bfp8.hip); false = shape not built.
+// Launches the block-float-8 VALU main kernel (decode_bfp8.hip); false = shape not built.
 bool launch_bfp8_main(const DecodeArgs &a, int head_size, int g, hipStream_t st);
+// Matrix-core main kernel (decode_mfma.hip) for wide head groups and block-float-8.
+bool mfma_decode_supported(const DecodeArgs &a, int head_size, int g);
+bool launch_mfma_main(const DecodeArgs &a, int head_size, hipStream_t st);
 
 }  // namespace decode
 }  // namespace ttpa

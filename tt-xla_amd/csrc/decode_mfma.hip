@@ -1,0 +1,372 @@
+// Paged decode attention, matrix-core formulation for wide head groups and for the
+// block-float-8 cache.
+//
+// The work decomposition is the one of decode.hip (flat list of 64-token tiles cut into
+// equal wavefront ranges, one partial per (wavefront, segment), merge kernel afterwards).
+// What differs is the arithmetic inside a wavefront.  The VALU kernel spends per-head work
+// on every tile (dot products, cross-lane reduction, softmax), which stops hiding behind
+// the HBM stream at 8 query heads per KV head, and the block-float-8 cache adds a byte ->
+// bfloat16 expansion on top.  Here a tile goes global -> registers -> wave-private LDS
+// (expanded to bfloat16 on the way for block-float-8), and the two products run on
+// v_mfma_f32_32x32x16_bf16 with the G query heads of the group as the 32-wide N dimension:
+//   S^T[key, head] = K[key, :] . Q[head, :]        A = K rows from LDS, B = Q in registers
+//   O^T[d, head]  += V^T[d, key] . P^T[key, head]  A = V through the transposing LDS load
+// Each lane owns one head column, so softmax statistics are per-lane scalars and the
+// probabilities are already the B operand of the second product.  Cost per tile is
+// independent of G (up to 32 heads per KV head).
+//
+// LDS: 37 KiB per wavefront (K rows padded to 68 dwords, V rows to 80), four wavefronts
+// per workgroup, one workgroup per CU.
+#include "decode_common.h"
+
+namespace ttpa {
+namespace decode {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kMaxUsersMfma = 1024;
+
+// 4 element bytes with shared scale -> two packed bfloat16 pairs (exact).
+__device__ __forceinline__ void expand4_scaled(uint32_t w, float scale, uint32_t &p01,
+                                               uint32_t &p23) {
+  const uint32_t mag = w & 0x7f7f7f7fu;
+  const float f0 = (float)(mag & 0xffu) * scale, f1 = (float)((mag >> 8) & 0xffu) * scale;
+  const float f2 = (float)((mag >> 16) & 0xffu) * scale, f3 = (float)(mag >> 24) * scale;
+  p01 = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f1), __builtin_bit_cast(uint32_t, f0),
+                              0x07060302u);
+  p23 = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f3), __builtin_bit_cast(uint32_t, f2),
+                              0x07060302u);
+  p01 ^= __builtin_amdgcn_perm(w, w, 0x010c000cu) & 0x80008000u;
+  p23 ^= __builtin_amdgcn_perm(w, w, 0x030c020cu) & 0x80008000u;
+}
+__device__ __forceinline__ float group_scale(uint32_t e) {
+  return e >= 7u ? __builtin_bit_cast(float, (e - 6u) << 23) : 0.f;
+}
+
+template <int D, bool BFP8, bool BIG>
+__global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
+    DecodeArgs a, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
+  static_assert(D == 64 || D == 128, "matrix-core decode is built for head sizes 64 and 128");
+  constexpr int KS = D + 8, VS = D + 32;    // LDS row strides in elements
+  constexpr int KSTEPS = D / 16, DBLK = D / 32;
+  // staging geometry: a load instruction covers RPL whole token rows
+  constexpr int BPE = BFP8 ? 1 : 2;         // bytes per cache element
+  constexpr int LPR = D * BPE / 16;         // lanes per token row (16 bytes per lane)
+  constexpr int RPL = 64 / LPR;             // rows per load
+  constexpr int NL = kTile / RPL;           // loads per tile and tensor
+  constexpr int GPR = D / 16;               // exponent bytes per row (block-float-8)
+  constexpr int NOFF = BIG ? 1 : NL;
+
+  __shared__ int s_pref[kMaxUsersMfma + 1];
+  __shared__ int s_len[kMaxUsersMfma];
+  __shared__ int s_wsum[kWavesPerBlock];
+  extern __shared__ __attribute__((aligned(16))) uint16_t tiles[];
+
+  build_prefix(a, cur_pos, s_pref, s_len, s_wsum);
+
+  const int lane = threadIdx.x & 63;
+  const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int wave = blockIdx.x * kWavesPerBlock + wib;
+  const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
+  const int64_t total = (int64_t)total_tiles * a.hkv;
+  const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);
+  if (total == 0 || wave >= n_eff) {
+    publish_segment_row(a, s_pref, total, n_eff);
+    return;
+  }
+  int64_t x = (int64_t)wave * total / n_eff;
+  const int64_t x_hi = (int64_t)(wave + 1) * total / n_eff;
+  uint16_t *ks = tiles + wib * (kTile * (KS + VS));
+  uint16_t *vs = ks + kTile * KS;
+  const int G = a.hq / a.hkv;
+
+  // staging lane mapping
+  const int sr = lane / LPR, sc = lane % LPR;
+  const uint32_t lane_bytes = (uint32_t)(sr * D * BPE + sc * 16);
+  const uint32_t lane_exp = (uint32_t)(sr * GPR + sc);  // block-float-8: one group per lane
+  const int64_t slab = BFP8 ? (int64_t)(a.bs + a.bs / 16) * D : (int64_t)a.bs * D * 2;  // bytes
+
+  auto locate = [&](int64_t xx) { return locate_unit(s_pref, s_len, a.users, a.hkv, xx); };
+  auto tile_offsets = [&](const Cursor &cu, int64_t (&eo)[NOFF], int64_t (&xo)[NOFF]) {
+    const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
+    const int tok0 = cu.t * kTile;
+#pragma unroll
+    for (int i = 0; i < NOFF; ++i) {
+      const int tk = tok0 + RPL * i;
+      const int col = tk / a.bs;
+      int phys = (col < a.w) ? __builtin_amdgcn_readfirstlane(pt_row[col]) : 0;
+      if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+      const int64_t base = ((int64_t)phys * a.hkv + cu.h) * slab;
+      const int row = tk - col * a.bs;
+      eo[i] = base + (int64_t)row * D * BPE;
+      xo[i] = base + (int64_t)a.bs * D + (int64_t)row * GPR;
+    }
+  };
+  auto fetch = [&](const uint8_t *base, const int64_t (&eo)[NOFF], const int64_t (&xo)[NOFF],
+                   u32x4 (&raw)[NL], uint32_t (&ex)[NL]) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const uint8_t *erow = BIG ? base + eo[0] + i * (RPL * D * BPE) : base + eo[BIG ? 0 : i];
+      raw[i] = __builtin_nontemporal_load(
+          reinterpret_cast<const u32x4 *>(erow + static_cast<uint64_t>(lane_bytes)));
+      if constexpr (BFP8) {
+        const uint8_t *xrow = BIG ? base + xo[0] + i * (RPL * GPR) : base + xo[BIG ? 0 : i];
+        ex[i] = __builtin_nontemporal_load(xrow + static_cast<uint64_t>(lane_exp));
+      }
+    }
+  };
+  // registers -> LDS tile (rows past `nvalid` are cleared when `clear` is set)
+  auto stage = [&](uint16_t *dst, int stride, const u32x4 (&raw)[NL], const uint32_t (&ex)[NL],
+                   int nvalid, bool clear) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int row = RPL * i + sr;
+      const bool keep = !clear || row < nvalid;
+      if constexpr (BFP8) {
+        const float gs = keep ? group_scale(ex[i]) : 0.f;
+        uint32_t o[8];
+        expand4_scaled(raw[i].x, gs, o[0], o[1]);
+        expand4_scaled(raw[i].y, gs, o[2], o[3]);
+        expand4_scaled(raw[i].z, gs, o[4], o[5]);
+        expand4_scaled(raw[i].w, gs, o[6], o[7]);
+        if (!keep) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) o[j] = 0;  // -0 from a cleared scale is harmless, but be exact
+        }
+        uint4 *p = reinterpret_cast<uint4 *>(dst + row * stride + sc * 16);
+        p[0] = make_uint4(o[0], o[1], o[2], o[3]);
+        p[1] = make_uint4(o[4], o[5], o[6], o[7]);
+      } else {
+        uint4 v = keep ? make_uint4(raw[i].x, raw[i].y, raw[i].z, raw[i].w) : make_uint4(0, 0, 0, 0);
+        *reinterpret_cast<uint4 *>(dst + row * stride + sc * 8) = v;
+      }
+    }
+  };
+  // Q fragments: B operand, lane n = head of the group (zero beyond G)
+  auto load_q = [&](const Cursor &cu, bf16x8 (&qf)[KSTEPS]) {
+    const uint16_t *qp = a.q + cu.u * a.q_us + (int64_t)(cu.h * G + min(n, G - 1)) * a.q_hs + 8 * h;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      uint4 t = *reinterpret_cast<const uint4 *>(qp + 16 * s);
+      if (n >= G) t = make_uint4(0, 0, 0, 0);
+      qf[s] = __builtin_bit_cast(bf16x8, t);
+    }
+  };
+
+  Cursor cur = locate(x);
+  int64_t eo[NOFF], xo[NOFF];
+  u32x4 kraw[NL], vraw[NL];
+  uint32_t kex[NL], vex[NL];
+  bf16x8 qf[KSTEPS];
+  tile_offsets(cur, eo, xo);
+  fetch(a.k, eo, xo, kraw, kex);
+  fetch(a.v, eo, xo, vraw, vex);
+  load_q(cur, qf);
+  publish_segment_row(a, s_pref, total, n_eff);
+
+  floatx16 acc[DBLK];
+#pragma unroll
+  for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  auto process_tile = [&](auto has_next_tag) {
+    constexpr bool has_next = decltype(has_next_tag)::value;
+    const int nvalid = cur.len - cur.t * kTile;
+    const bool partial = nvalid < kTile;
+    // ---- this tile: registers -> LDS; next tile: global -> registers ----------------------
+    const bool same_seg = has_next && cur.tiles_left > 1;
+    Cursor nxt = cur;
+    auto prefetch_next = [&]() {
+      if constexpr (has_next) {
+        if (same_seg) {
+          nxt.t = cur.t + 1;
+          nxt.tiles_left = cur.tiles_left - 1;
+        } else {
+          nxt = locate(x + 1);
+        }
+        tile_offsets(nxt, eo, xo);
+        fetch(a.k, eo, xo, kraw, kex);
+        fetch(a.v, eo, xo, vraw, vex);
+      }
+    };
+    if constexpr (BFP8) {
+      // expansion is long: move the raw tile to a second register set so that the loads of
+      // the next tile are in flight while this one is expanded and staged
+      u32x4 kcur[NL], vcur[NL];
+      uint32_t kexc[NL], vexc[NL];
+#pragma unroll
+      for (int i = 0; i < NL; ++i) kcur[i] = kraw[i], vcur[i] = vraw[i], kexc[i] = kex[i], vexc[i] = vex[i];
+      prefetch_next();
+      __builtin_amdgcn_sched_barrier(0);
+      stage(ks, KS, kcur, kexc, nvalid, false);
+      stage(vs, VS, vcur, vexc, nvalid, partial);
+    } else {
+      stage(ks, KS, kraw, kex, nvalid, false);
+      stage(vs, VS, vraw, vex, nvalid, partial);  // unattended V rows must not carry Inf / NaN
+      prefetch_next();
+    }
+
+    // ---- S^T = K . Q^T ----------------------------------------------------------------------
+    floatx16 st[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[kb][r] = 0.f;
+      const uint16_t *krow = ks + (32 * kb + n) * KS + 8 * h;
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {
+        bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(krow + 16 * s));
+        st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], st[kb], 0, 0, 0);
+      }
+    }
+    // ---- online softmax, one head per lane --------------------------------------------------
+    if (partial) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = 32 * kb + 8 * (r >> 2) + 4 * h + (r & 3);
+          if (key >= nvalid) st[kb][r] = -INFINITY;
+        }
+    }
+    float mloc = fmaxf(st[0][0], st[1][0]);
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(st[0][r], st[1][r]));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+    const float scale = a.scale_log2e;  // > 0 or < 0: the maximum is tracked on scaled scores
+    mloc *= scale;
+    // a negative scale would turn the max into a min; scores are scaled before comparing then
+    if (scale < 0.f) {
+      mloc = -INFINITY;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, st[kb][r] * scale);
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+    }
+    const float m_new = fmaxf(m_run, mloc);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
+    m_run = m_new;
+    float lsum = 0.f;
+    bf16x8 pf[2][2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float p = __builtin_amdgcn_exp2f(fmaf(st[kb][8 * s + e], scale, -m_safe));
+          __bf16 pb = (__bf16)p;
+          lsum += (float)pb;  // the normaliser sums the weights that multiply V
+          pf[kb][s][e] = pb;
+        }
+    l_run = l_run * alpha + lsum;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+      for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] *= alpha;
+    }
+    // ---- O^T += V^T . P^T (V^T fragments through the transposing LDS load) -------------------
+    const int grp = lane >> 4, a16 = lane & 15;
+    const uint16_t *vbase = vs + (4 * (grp >> 1) + (a16 >> 2)) * VS + 16 * (grp & 1) + 4 * (a16 & 3);
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const uint16_t *vk = vbase + (32 * kb + 16 * s) * VS;
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db) {
+          typedef __attribute__((address_space(3))) shortx4 *lds_v4;
+          shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk + 32 * db));
+          shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk + 8 * VS + 32 * db));
+          bf16x8 vf;
+          bf16x4 l4 = __builtin_bit_cast(bf16x4, lo), h4 = __builtin_bit_cast(bf16x4, hi);
+          vf[0] = l4[0], vf[1] = l4[1], vf[2] = l4[2], vf[3] = l4[3];
+          vf[4] = h4[0], vf[5] = h4[1], vf[6] = h4[2], vf[7] = h4[3];
+          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kb][s], acc[db], 0, 0, 0);
+        }
+      }
+
+    // ---- close the segment --------------------------------------------------------------------
+    if (!same_seg) {
+      float *slot = a.ws_slots + ((int64_t)wave + (int64_t)cur.u * a.hkv + cur.h) * a.slot_floats;
+      const float l_tot = l_run + __shfl_xor(l_run, 32);
+      if (n < G) {
+        float *dst = slot + n * D + 4 * h;
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            *reinterpret_cast<float4 *>(dst + 32 * db + 8 * j) = make_float4(
+                acc[db][4 * j], acc[db][4 * j + 1], acc[db][4 * j + 2], acc[db][4 * j + 3]);
+        if (h == 0) {
+          slot[G * D + n] = m_run;
+          slot[G * D + G + n] = l_tot;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+      m_run = -INFINITY;
+      l_run = 0.f;
+      if constexpr (has_next) load_q(nxt, qf);
+    }
+    cur = nxt;
+    ++x;
+  };
+  while (x + 1 < x_hi) process_tile(std::true_type{});
+  process_tile(std::false_type{});
+}
+
+template <int D, bool BFP8>
+bool launch(const DecodeArgs &a, hipStream_t st) {
+  const int blocks = a.n_waves / kWavesPerBlock;
+  const size_t lds = (size_t)kWavesPerBlock * kTile * ((D + 8) + (D + 32)) * 2;
+  if (a.bs % kTile == 0) {
+    static bool once = false;
+    if (!once) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(&paged_decode_mfma_kernel<D, BFP8, true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return false;
+      once = true;
+    }
+    paged_decode_mfma_kernel<D, BFP8, true><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
+  } else {
+    static bool once = false;
+    if (!once) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(&paged_decode_mfma_kernel<D, BFP8, false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return false;
+      once = true;
+    }
+    paged_decode_mfma_kernel<D, BFP8, false><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
+  }
+  return true;
+}
+
+}  // namespace
+
+bool mfma_decode_supported(const DecodeArgs &a, int head_size, int g) {
+  return (head_size == 64 || head_size == 128) && g <= 32 && a.users <= kMaxUsersMfma &&
+         a.bs % 8 == 0;
+}
+
+bool launch_mfma_main(const DecodeArgs &a, int head_size, hipStream_t st) {
+  const bool bfp8 = a.kv_format == TTPA_KV_BFP8;
+  if (head_size == 64) return bfp8 ? launch<64, true>(a, st) : launch<64, false>(a, st);
+  if (head_size == 128) return bfp8 ? launch<128, true>(a, st) : launch<128, false>(a, st);
+  return false;
+}
+
+}  // namespace decode
+}  // namespace ttpa
