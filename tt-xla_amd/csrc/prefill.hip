@@ -19,6 +19,8 @@
 // element (row 8 (r / 4) + 4 h + r % 4, column n).
 #include "common.h"
 
+#include <cstdlib>
+
 namespace ttpa {
 namespace {
 
@@ -26,6 +28,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kKeysPerTile = 64;
 constexpr int kRowsPerWave = 32;
@@ -67,22 +70,29 @@ __device__ __forceinline__ const uint16_t *kv_chunk(const PrefillArgs &a, const 
   return base + b * a.kv_bs + hk * a.kv_hs + (int64_t)key * a.kv_ts + c * 8;
 }
 
-template <int D, int HPW>
-__global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(PrefillArgs a) {
-  constexpr int RPW = 4 / HPW;            // row blocks per workgroup
+// MODE 0: dense K/V; 1: paged, block_size a multiple of 64 (a tile lies in one block);
+// 2: paged, any block size (per-chunk table lookups).
+// R = blocks of 32 query rows per wavefront.  R = 2 reuses every K / V fragment read from
+// LDS for two matrix instructions (LDS operand traffic per FLOP halves) and gives the
+// scheduler two independent row blocks to overlap: the score product of block 1 runs on the
+// matrix pipe while block 0's softmax runs on the VALU.  It needs the 512-register budget
+// (one workgroup per CU); R = 1 keeps two workgroups per CU and serves short queries.
+template <int D, int HPW, int MODE, int R>
+__global__ __launch_bounds__(256, (D <= 128 && R == 1 ? 2 : 1)) void prefill_kernel(PrefillArgs a) {
+  constexpr int RPW = 4 / HPW;            // wavefront row slots per workgroup
+  constexpr int ROWS = kRowsPerWave * R;  // query rows per wavefront
   constexpr int KSTEPS = D / 16;          // MFMA k-steps over the head dimension
   constexpr int DBLK = D / 32;            // 32-wide output blocks over the head dimension
   constexpr int CPT = D / 32;             // 16-byte chunks per thread per tile and tensor
   using L = Lds<D>;
+  constexpr int STAGE = kKeysPerTile * (L::KS + L::VS);  // elements per LDS stage
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-  uint16_t *ks = smem;
-  uint16_t *vs = smem + kKeysPerTile * L::KS;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int n = lane & 31, h = lane >> 5;
-  const int nqt = (a.sq + kRowsPerWave * RPW - 1) / (kRowsPerWave * RPW);
+  const int nqt = (a.sq + ROWS * RPW - 1) / (ROWS * RPW);
   const int qt = nqt - 1 - (int)blockIdx.x;  // heavy (late) tiles are scheduled first
   const int groups = a.hq / HPW;
   const int b = blockIdx.y / groups;
@@ -90,192 +100,257 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
   const int g = a.hq / a.hkv;
   const int hk = hq0 / g;
   const int hq = hq0 + wave % HPW;
-  const int row0 = (qt * RPW + wave / HPW) * kRowsPerWave;  // first query row of the wave
+  const int row0 = (qt * RPW + wave / HPW) * ROWS;  // first query row of the wavefront
   const int offset = a.causal ? (a.chunk_start ? a.chunk_start[0] : 0) : 0;
 
   // keys this workgroup / this wavefront can see
-  const int wg_last_row = min(a.sq, (qt + 1) * kRowsPerWave * RPW) - 1;
+  const int wg_last_row = min(a.sq, (qt + 1) * ROWS * RPW) - 1;
   const int kv_end_wg = a.causal ? min(a.skv, offset + wg_last_row + 1) : a.skv;
   const int ntiles = (kv_end_wg + kKeysPerTile - 1) / kKeysPerTile;
-  const int wave_last_key = a.causal ? offset + min(a.sq - 1, row0 + kRowsPerWave - 1) : a.skv - 1;
+  const int wave_last_key = a.causal ? offset + min(a.sq - 1, row0 + ROWS - 1) : a.skv - 1;
   const bool wave_active = row0 < a.sq;
 
   // ---- Q fragments (B operand: lane n = query row, 8 head-dim elements per k-step) -----
-  bf16x8 qf[KSTEPS];
-  {
-    const int qrow = min(row0 + n, a.sq - 1);
+  bf16x8 qf[R][KSTEPS];
+#pragma unroll
+  for (int rb = 0; rb < R; ++rb) {
+    const int qrow = min(row0 + 32 * rb + n, a.sq - 1);
     const uint16_t *qp = a.q + b * a.q_bs + hq * a.q_hs + (int64_t)qrow * a.q_ts + 8 * h;
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s)
-      qf[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 16 * s));
+      qf[rb][s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 16 * s));
   }
 
-  floatx16 acc[DBLK];
+  floatx16 acc[R][DBLK];
+  float m_run[R], l_run[R];
 #pragma unroll
-  for (int i = 0; i < DBLK; ++i)
+  for (int rb = 0; rb < R; ++rb) {
+    m_run[rb] = -INFINITY;
+    l_run[rb] = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+    for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[rb][i][r] = 0.f;
+  }
 
   // ---- global -> register staging of one K/V tile -------------------------------------
-  uint4 kst[CPT], vst[CPT];
+  // A thread's chunks sit at fixed (key, column) positions of every tile: their offsets are
+  // computed once, and per tile only a wavefront-uniform base moves (modes 0 and 1).
+  u32x4 kst[CPT], vst[CPT];  // native vectors: struct-typed uint4 arrays end up in scratch memory
+  uint32_t chunk_off[CPT];  // element offset of chunk i inside a tile
+  int chunk_key[CPT], chunk_col[CPT];
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int id = tid + 256 * i;
+    const int key = id / (D / 8), c = id - key * (D / 8);
+    chunk_key[i] = key;
+    chunk_col[i] = c;
+    chunk_off[i] = (uint32_t)(key * (MODE == 0 ? (int)a.kv_ts : D) + c * 8);
+  }
+  // Loads are unconditional (a predicated load would make the compiler wait for the prefetch
+  // right after issuing it): keys past the end of a dense K/V are clamped to the last row,
+  // whose scores are masked and whose V rows therefore carry weight 0.
   auto fetch_tile = [&](int kt) {
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int id = tid + 256 * i;
-      const int key = id / (D / 8), c = id - key * (D / 8);
-      const int kabs = kt * kKeysPerTile + key;
-      if (kabs < a.skv) {
-        kst[i] = *reinterpret_cast<const uint4 *>(kv_chunk(a, a.k, b, hk, kabs, c, D));
-        vst[i] = *reinterpret_cast<const uint4 *>(kv_chunk(a, a.v, b, hk, kabs, c, D));
-      } else {
-        kst[i] = make_uint4(0, 0, 0, 0);
-        vst[i] = make_uint4(0, 0, 0, 0);
-      }
-    }
-  };
-  auto stage_tile = [&]() {
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int id = tid + 256 * i;
-      const int key = id / (D / 8), c = id - key * (D / 8);
-      *reinterpret_cast<uint4 *>(ks + key * L::KS + c * 8) = kst[i];
-      *reinterpret_cast<uint4 *>(vs + key * L::VS + c * 8) = vst[i];
-    }
-  };
-
-  if (ntiles > 0) fetch_tile(0);
-  for (int kt = 0; kt < ntiles; ++kt) {
-    __syncthreads();  // every wavefront is done reading the previous tile
-    stage_tile();
-    __syncthreads();
-    if (kt + 1 < ntiles) fetch_tile(kt + 1);  // in flight while this tile is consumed
-
     const int key0 = kt * kKeysPerTile;
-    if (!wave_active || key0 > wave_last_key) continue;  // nothing visible to this wavefront
-
-    // ---- S^T = K . Q^T for the two 32-key blocks of the tile ----------------------------
-    floatx16 st[2];
+    int64_t base;  // uniform element offset of the tile
+    if constexpr (MODE == 0) {
+      base = b * a.kv_bs + hk * a.kv_hs + (int64_t)key0 * a.kv_ts;
+    } else if constexpr (MODE == 1) {
+      int phys = __builtin_amdgcn_readfirstlane(a.pt[(int64_t)b * a.pt_rs + key0 / a.bs]);
+      if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+      base = (((int64_t)phys * a.hkv + hk) * a.bs + (key0 % a.bs)) * D;
+    } else {
+      base = 0;
+    }
+    const int last = a.skv - 1 - key0;  // last valid key of this tile, relative (>= 0)
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) st[kb][r] = 0.f;
-      const uint16_t *krow = ks + (32 * kb + n) * L::KS + 8 * h;
-#pragma unroll
-      for (int s = 0; s < KSTEPS; ++s) {
-        bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(krow + 16 * s));
-        st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], st[kb], 0, 0, 0);
+    for (int i = 0; i < CPT; ++i) {
+      if constexpr (MODE == 2) {
+        const int key = key0 + min(chunk_key[i], last);
+        kst[i] = *reinterpret_cast<const u32x4 *>(kv_chunk(a, a.k, b, hk, key, chunk_col[i], D));
+        vst[i] = *reinterpret_cast<const u32x4 *>(kv_chunk(a, a.v, b, hk, key, chunk_col[i], D));
+      } else if constexpr (MODE == 1) {  // table_width * block_size is a multiple of the tile
+        kst[i] = *reinterpret_cast<const u32x4 *>(a.k + base + chunk_off[i]);
+        vst[i] = *reinterpret_cast<const u32x4 *>(a.v + base + chunk_off[i]);
+      } else {
+        const uint32_t off = (uint32_t)(min(chunk_key[i], last) * (int)a.kv_ts + chunk_col[i] * 8);
+        kst[i] = *reinterpret_cast<const u32x4 *>(a.k + base + off);
+        vst[i] = *reinterpret_cast<const u32x4 *>(a.v + base + off);
       }
     }
+  };
+  auto stage_tile = [&](int buf) {
+    uint16_t *ks = smem + buf * STAGE;
+    uint16_t *vs = ks + kKeysPerTile * L::KS;
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      *reinterpret_cast<u32x4 *>(ks + chunk_key[i] * L::KS + chunk_col[i] * 8) = kst[i];
+      *reinterpret_cast<u32x4 *>(vs + chunk_key[i] * L::VS + chunk_col[i] * 8) = vst[i];
+    }
+  };
 
-    // ---- mask, online softmax (one query row per lane) -----------------------------------
-    // The softmax scale is positive, so the running maximum is tracked on raw scores and
-    // the scale is folded into the exponent: p = exp2(s * c - m * c).
-    const int qrow = row0 + n;
-    const bool need_mask = (a.causal && key0 + kKeysPerTile - 1 > offset + row0) ||
-                           key0 + kKeysPerTile > a.skv || a.mask != nullptr;
-    if (need_mask) {  // wavefront-uniform: only diagonal / ragged / explicitly masked tiles
-      const int limit = a.causal ? min(offset + qrow, a.skv - 1) : a.skv - 1;
+  // Pipeline: LDS holds two stages.  While tile kt is consumed from stage kt & 1, tile kt + 1
+  // (fetched one iteration ago) is written to the other stage and tile kt + 2 is in flight
+  // from global memory.  One barrier per tile.  Staging and prefetch are unconditional (past
+  // the last tile they repeat it into a stage nobody reads): straight-line code keeps the
+  // staged tile in registers and the wait counters exact.  ntiles >= 1 always (row 0 sees
+  // key 0).
+  const int last_tile = ntiles - 1;
+  fetch_tile(0);
+  stage_tile(0);
+  fetch_tile(min(1, last_tile));
+  __syncthreads();
+  for (int kt = 0; kt < ntiles; ++kt) {
+    stage_tile((kt + 1) & 1);
+    fetch_tile(min(kt + 2, last_tile));
+    const uint16_t *ks = smem + (kt & 1) * STAGE;
+    const uint16_t *vs = ks + kKeysPerTile * L::KS;
+    const int key0 = kt * kKeysPerTile;
+
+    if (wave_active && key0 <= wave_last_key) {
+      // ---- K fragments: read once, used for every row block ------------------------------
+      bf16x8 kf[2][KSTEPS];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+      for (int kb = 0; kb < 2; ++kb) {
+        const uint16_t *krow = ks + (32 * kb + n) * L::KS + 8 * h;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = key0 + 32 * kb + 8 * (r >> 2) + 4 * h + (r & 3);
-          float v = st[kb][r];
-          if (a.mask) {
-            const int kc = min(key, a.skv - 1), qc = min(qrow, a.sq - 1);
-            // additive mask is in natural-log units of the scaled score
-            v += bf16_lo(a.mask[b * a.mask_bs + (int64_t)qc * a.mask_rs + kc]) *
-                 (1.4426950408889634f / a.scale_log2e);
+        for (int s = 0; s < KSTEPS; ++s)
+          kf[kb][s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(krow + 16 * s));
+      }
+      // ---- S^T = K . Q^T, row block after row block ------------------------------------------
+      floatx16 st[R][2];
+#pragma unroll
+      for (int rb = 0; rb < R; ++rb)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) st[rb][kb][r] = 0.f;
+#pragma unroll
+          for (int s = 0; s < KSTEPS; ++s)
+            st[rb][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb][s], qf[rb][s], st[rb][kb], 0, 0, 0);
+        }
+      bf16x8 pf[R][2][2];
+#pragma unroll
+      for (int rb = 0; rb < R; ++rb) {
+        // ---- mask, online softmax (one query row per lane) -----------------------------------
+        // The softmax scale is positive, so the running maximum is tracked on raw scores and
+        // the scale is folded into the exponent: p = exp2(s * c - m * c).
+        const int rrow0 = row0 + 32 * rb;
+        const int qrow = rrow0 + n;
+        const bool need_mask = (a.causal && key0 + kKeysPerTile - 1 > offset + rrow0) ||
+                               key0 + kKeysPerTile > a.skv || a.mask != nullptr;
+        if (need_mask) {  // wavefront-uniform: only diagonal / ragged / explicitly masked tiles
+          const int limit = a.causal ? min(offset + qrow, a.skv - 1) : a.skv - 1;
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int key = key0 + 32 * kb + 8 * (r >> 2) + 4 * h + (r & 3);
+              float v = st[rb][kb][r];
+              if (a.mask) {
+                const int kc = min(key, a.skv - 1), qc = min(qrow, a.sq - 1);
+                // additive mask is in natural-log units of the scaled score
+                v += bf16_lo(a.mask[b * a.mask_bs + (int64_t)qc * a.mask_rs + kc]) *
+                     (1.4426950408889634f / a.scale_log2e);
+              }
+              st[rb][kb][r] = key > limit ? -INFINITY : v;
+            }
+        }
+        float mloc = fmaxf(st[rb][0][0], st[rb][1][0]);
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(st[rb][0][r], st[rb][1][r]));
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+        const float m_new = fmaxf(m_run[rb], mloc);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f((m_run[rb] - m_safe) * a.scale_log2e);
+        const float mc = m_safe * a.scale_log2e;
+        m_run[rb] = m_new;
+        float lsum = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              // B-operand element e of k-step s <-> accumulator register 8 s + e
+              float p = __builtin_amdgcn_exp2f(fmaf(st[rb][kb][8 * s + e], a.scale_log2e, -mc));
+              lsum += p;
+              pf[rb][kb][s][e] = (__bf16)p;
+            }
+        l_run[rb] = l_run[rb] * alpha + lsum;
+        // skip the accumulator rescale when no row of the wavefront moved its maximum
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+          for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[rb][i][r] *= alpha;
+        }
+      }
+      // ---- O^T += V^T . P^T: V^T fragments come through the transposing LDS load (per group
+      //      of 16 lanes, lane i receives element i % 4 of the 8-byte chunks addressed by lanes
+      //      4 j + i / 4); each fragment feeds every row block -------------------------------
+      {
+        const int grp = lane >> 4, a16 = lane & 15;
+        const uint16_t *vbase =
+            vs + (4 * (grp >> 1) + (a16 >> 2)) * L::VS + 16 * (grp & 1) + 4 * (a16 & 3);
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) {
+          bf16x8 vf[DBLK];
+#pragma unroll
+          for (int db = 0; db < DBLK; ++db) {
+            typedef __attribute__((address_space(3))) shortx4 *lds_v4;
+            const uint16_t *vk = vbase + 16 * k4 * L::VS + 32 * db;
+            shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk));
+            shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk + 8 * L::VS));
+            bf16x4 l4 = __builtin_bit_cast(bf16x4, lo), h4 = __builtin_bit_cast(bf16x4, hi);
+            bf16x8 t;
+            t[0] = l4[0], t[1] = l4[1], t[2] = l4[2], t[3] = l4[3];
+            t[4] = h4[0], t[5] = h4[1], t[6] = h4[2], t[7] = h4[3];
+            vf[db] = t;
           }
-          st[kb][r] = key > limit ? -INFINITY : v;
-        }
-    }
-    float mloc = fmaxf(st[0][0], st[1][0]);
 #pragma unroll
-    for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(st[0][r], st[1][r]));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-    const float m_new = fmaxf(m_run, mloc);
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * a.scale_log2e);
-    const float mc = m_safe * a.scale_log2e;
-    m_run = m_new;
-    float lsum = 0.f;
-    bf16x8 pf[2][2];
+          for (int rb = 0; rb < R; ++rb)
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int s = 0; s < 2; ++s)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          // B-operand element e of k-step s <-> accumulator register 8 s + e
-          float p = __builtin_amdgcn_exp2f(fmaf(st[kb][8 * s + e], a.scale_log2e, -mc));
-          lsum += p;
-          pf[kb][s][e] = (__bf16)p;
-        }
-    l_run = l_run * alpha + lsum;
-    // skip the accumulator rescale when no row of the wavefront moved its maximum
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-      for (int i = 0; i < DBLK; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][r] *= alpha;
-    }
-
-    // ---- O^T += V^T . P^T ------------------------------------------------------------------
-    // transposing LDS load, per group of 16 lanes: lane i receives element (i % 4) of the
-    // 8-byte chunks addressed by lanes 4 j + i / 4 (j = 0..3).  Lane a of a group therefore
-    // points at key (a / 4) of the wanted four and at head-dim chunk 4 (a % 4) of the 16
-    // columns the group covers.
-    const int grp = lane >> 4, a16 = lane & 15;
-    const uint16_t *vbase =
-        vs + (4 * (grp >> 1) + (a16 >> 2)) * L::VS + 16 * (grp & 1) + 4 * (a16 & 3);
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        const uint16_t *vk = vbase + (32 * kb + 16 * s) * L::VS;
-#pragma unroll
-        for (int db = 0; db < DBLK; ++db) {
-          typedef __attribute__((address_space(3))) shortx4 *lds_v4;
-          shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk + 32 * db));
-          shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk + 8 * L::VS + 32 * db));
-          bf16x8 vf;
-          bf16x4 l4 = __builtin_bit_cast(bf16x4, lo), h4 = __builtin_bit_cast(bf16x4, hi);
-          vf[0] = l4[0], vf[1] = l4[1], vf[2] = l4[2], vf[3] = l4[3];
-          vf[4] = h4[0], vf[5] = h4[1], vf[6] = h4[2], vf[7] = h4[3];
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kb][s], acc[db], 0, 0, 0);
+            for (int db = 0; db < DBLK; ++db)
+              acc[rb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db], pf[rb][k4 >> 1][k4 & 1],
+                                                                    acc[rb][db], 0, 0, 0);
         }
       }
+    }
+    __syncthreads();  // tile kt + 1 is staged; everyone is done with stage kt & 1
   }
 
   // ---- normalise and store: lane (n, h) holds head-dim elements 32 db + 8 j + 4 h + i ----
   if (!wave_active) return;
-  const float l_tot = l_run + __shfl_xor(l_run, 32);
-  const float inv = 1.0f / l_tot;
-  const int qrow = row0 + n;
-  if (qrow >= a.sq) return;
-  uint16_t *op = a.out + b * a.out_bs + hq * a.out_hs + (int64_t)qrow * a.out_ts + 4 * h;
 #pragma unroll
-  for (int db = 0; db < DBLK; ++db)
+  for (int rb = 0; rb < R; ++rb) {
+    const float l_tot = l_run[rb] + __shfl_xor(l_run[rb], 32);
+    const float inv = 1.0f / l_tot;
+    const int qrow = row0 + 32 * rb + n;
+    if (qrow >= a.sq) continue;
+    uint16_t *op = a.out + b * a.out_bs + hq * a.out_hs + (int64_t)qrow * a.out_ts + 4 * h;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      uint32_t lo = f32_to_bf16_bits(acc[db][4 * j] * inv) |
-                    (f32_to_bf16_bits(acc[db][4 * j + 1] * inv) << 16);
-      uint32_t hi = f32_to_bf16_bits(acc[db][4 * j + 2] * inv) |
-                    (f32_to_bf16_bits(acc[db][4 * j + 3] * inv) << 16);
-      *reinterpret_cast<uint2 *>(op + 32 * db + 8 * j) = make_uint2(lo, hi);
-    }
+    for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t lo = f32_to_bf16_bits(acc[rb][db][4 * j] * inv) |
+                      (f32_to_bf16_bits(acc[rb][db][4 * j + 1] * inv) << 16);
+        uint32_t hi = f32_to_bf16_bits(acc[rb][db][4 * j + 2] * inv) |
+                      (f32_to_bf16_bits(acc[rb][db][4 * j + 3] * inv) << 16);
+        *reinterpret_cast<uint2 *>(op + 32 * db + 8 * j) = make_uint2(lo, hi);
+      }
+  }
 }
 
-template <int D, int HPW>
-int launch(const PrefillArgs &a, hipStream_t st) {
+template <int D, int HPW, int MODE, int R>
+int launch_mode(const PrefillArgs &a, hipStream_t st) {
   constexpr int RPW = 4 / HPW;
-  const int nqt = (a.sq + kRowsPerWave * RPW - 1) / (kRowsPerWave * RPW);
-  const size_t lds = Lds<D>::BYTES;
+  constexpr int ROWS = kRowsPerWave * R;
+  const int nqt = (a.sq + ROWS * RPW - 1) / (ROWS * RPW);
+  const size_t lds = 2 * Lds<D>::BYTES;  // two stages
   static bool attr_set = false;
-  if (!attr_set && lds > 48 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&prefill_kernel<D, HPW>),
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&prefill_kernel<D, HPW, MODE, R>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return fail(TTPA_ERR_LAUNCH, "prefill: cannot reserve %zu bytes of LDS", lds);
     attr_set = true;
@@ -283,9 +358,32 @@ int launch(const PrefillArgs &a, hipStream_t st) {
   hipEvent_t ev0, ev1;
   take_profile_events(ev0, ev1);
   if (ev0) (void)hipEventRecord(ev0, st);
-  prefill_kernel<D, HPW><<<dim3(nqt, a.batch * (a.hq / HPW)), dim3(256), lds, st>>>(a);
+  prefill_kernel<D, HPW, MODE, R><<<dim3(nqt, a.batch * (a.hq / HPW)), dim3(256), lds, st>>>(a);
   if (ev1) (void)hipEventRecord(ev1, st);
   return check_launch("sdpa_prefill");
+}
+
+template <int D, int HPW, int MODE>
+int launch_rows(const PrefillArgs &a, hipStream_t st) {
+  // 64 rows per wavefront once the query is long enough to fill them; head size 256 keeps
+  // 32 (its accumulators alone take 128 registers per row block)
+  if constexpr (D <= 128) {
+    static int forced = -1;
+    if (forced < 0) {
+      const char *e = getenv("TTPA_PREFILL_ROWS");
+      forced = e ? atoi(e) : 0;
+    }
+    const bool two = forced == 64;  // 64 rows per wavefront is experimental (TTPA_PREFILL_ROWS=64)
+    if (two) return launch_mode<D, HPW, MODE, 2>(a, st);
+  }
+  return launch_mode<D, HPW, MODE, 1>(a, st);
+}
+
+template <int D, int HPW>
+int launch(const PrefillArgs &a, hipStream_t st) {
+  if (!a.pt) return launch_rows<D, HPW, 0>(a, st);
+  if (a.bs % kKeysPerTile == 0) return launch_rows<D, HPW, 1>(a, st);
+  return launch_rows<D, HPW, 2>(a, st);
 }
 
 template <int D>
