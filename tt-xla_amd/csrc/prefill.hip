@@ -260,9 +260,15 @@ __global__ __launch_bounds__(256, (D <= 128 && R == 1 ? 2 : 1)) void prefill_ker
 #pragma unroll
         for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(st[rb][0][r], st[rb][1][r]));
         mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-        const float m_new = fmaxf(m_run[rb], mloc);
+        // Lazy rescaling: the running maximum only moves when a row's new maximum exceeds it
+        // by more than 2^8 in the exponent domain.  Until then probabilities are taken
+        // relative to the stale maximum (they may reach 2^8, harmless in bf16 / fp32), the
+        // accumulators need no rescale, and the final division by the row sum is unchanged.
+        const float kLazy = 8.0f;
+        const bool move = !((mloc - m_run[rb]) * a.scale_log2e <= kLazy);  // also true from -inf
+        const float m_new = move ? mloc : m_run[rb];
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f((m_run[rb] - m_safe) * a.scale_log2e);
+        const float alpha = move ? __builtin_amdgcn_exp2f((m_run[rb] - m_safe) * a.scale_log2e) : 1.0f;
         const float mc = m_safe * a.scale_log2e;
         m_run[rb] = m_new;
         float lsum = 0.f;
