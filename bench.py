@@ -87,8 +87,9 @@ def make_decode(name, seed, device):
 def decode_step(g):
     import torch
 
-    torch.ops.tt.paged_update_cache_(g.k_cache, g.k_new, g.cache_position, g.page_table)
-    torch.ops.tt.paged_update_cache_(g.v_cache, g.v_new, g.cache_position, g.page_table)
+    # what the attention backend issues for a decode step: both cache scatters in one launch
+    torch.ops.tt.paged_update_kv_cache_(g.k_cache, g.v_cache, g.k_new, g.v_new, g.cache_position,
+                                        g.page_table)
     return torch.ops.tt.paged_scaled_dot_product_attention_decode(
         g.q, g.k_cache, g.v_cache, g.page_table, is_causal=True,
         cur_pos_tensor=g.cache_position, scale=g.scale,
@@ -162,6 +163,44 @@ def time_dominant_kernel(fns, iters):
         _native.call("ttpa_profile_next_attention", a, b)
         fns[i % n]()
         if i >= 5:
+            pairs.append((a, b, i % n))
+    torch.cuda.synchronize()
+    return [(ev.elapsed_ms(a, b), which) for a, b, which in pairs]
+
+
+def time_decode_kernel_direct(copies, iters):
+    """The decode kernel alone, driven through the C ABI with preallocated output and
+    workspace: the host enqueues far faster than the GPU executes, so the stream never runs
+    dry and the armed event pair brackets the kernel the way a kernel trace does.  Returns
+    [(milliseconds, copy index)]."""
+    import torch
+
+    from tt_xla_amd import _native
+    from tt_xla_amd import custom_ops as ops
+
+    lib = _native.lib()
+    ev = HipEvents()
+    stream = torch.cuda.current_stream().cuda_stream
+    prepared = []
+    for c in copies:
+        nb, hkv, bs, d, fmt = ops._cache_geometry(c.k_cache)
+        users, hq = c.q.shape[1], c.q.shape[2]
+        out = torch.empty_like(c.q)
+        nbytes = lib.ttpa_paged_decode_workspace_bytes(users, hq, hkv, d)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=c.q.device)
+        prepared.append((c, out, ws, nbytes, (users, hq, hkv, d, bs, c.page_table.shape[1], nb, fmt)))
+    pairs, n = [], len(prepared)
+    torch.cuda.synchronize()
+    for i in range(iters + 10):
+        c, out, ws, nbytes, (users, hq, hkv, d, bs, w, nb, fmt) = prepared[i % n]
+        a, b = ev.create(), ev.create()
+        _native.call("ttpa_profile_next_attention", a, b)
+        _native.call(
+            "ttpa_paged_sdpa_decode", out.data_ptr(), out.stride(1), out.stride(2),
+            c.q.data_ptr(), c.q.stride(1), c.q.stride(2), c.k_cache.data_ptr(), c.v_cache.data_ptr(),
+            c.page_table.data_ptr(), c.page_table.stride(0), c.cache_position.data_ptr(), 0,
+            users, hq, hkv, d, bs, w, nb, float(c.scale), fmt, ws.data_ptr(), nbytes, stream)
+        if i >= 10:
             pairs.append((a, b, i % n))
     torch.cuda.synchronize()
     return [(ev.elapsed_ms(a, b), which) for a, b, which in pairs]
@@ -284,7 +323,7 @@ def run_decode(args):
     ms = time_steps(launchers, args.steps, args.warmup)
     n = len(copies)
     avg_step_bytes = sum(step_bytes[i % n] for i in range(args.steps)) / args.steps
-    durs = time_dominant_kernel(fns, min(args.steps, 100))
+    durs = time_decode_kernel_direct(copies, min(args.steps, 100))
     kern_ms = sum(d for d, _ in durs) / len(durs)
     kern_bytes = sum(dec_bytes[w] for _, w in durs) / len(durs)
     achieved = kern_bytes / (kern_ms * 1e-3) / 1e9
@@ -297,7 +336,7 @@ def run_decode(args):
         "dtype": dtype, "data": "synthetic",
         "config": {
             "workload": wl.name,
-            "step": "K update + V update + paged decode attention, one layer, one token per sequence",
+            "step": "K + V cache update (one launch) + paged decode attention, one layer, one token per sequence",
             "launch": args.launch, "rotating_copies": n, **shape,
             "mean_context": float(wl.cache_position.float().mean()),
         },

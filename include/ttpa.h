@@ -74,6 +74,20 @@ int ttpa_paged_update_cache(void *cache, const void *fill, int64_t fill_user_str
                             int32_t num_blocks, int32_t kv_format, void *stream);
 
 /*
+ * The decode step's two scatters in one launch: ttpa_paged_update_cache applied to the K cache
+ * with k_fill and to the V cache with v_fill (same indices, same page table, same geometry,
+ * same fill strides).  The reference issues the op twice
+ * (vllm_tt/attention_impls/attention.py:473-484); the result is identical.
+ */
+int ttpa_paged_update_cache_kv(void *k_cache, void *v_cache, const void *k_fill, const void *v_fill,
+                               int64_t fill_user_stride, int64_t fill_head_stride,
+                               const void *update_indices, int indices_is_i64,
+                               const int32_t *page_table, int64_t page_table_row_stride,
+                               int32_t users, int32_t kv_heads, int32_t block_size,
+                               int32_t head_size, int32_t table_width, int32_t num_blocks,
+                               int32_t kv_format, void *stream);
+
+/*
  * Block-wise prefill write, IN PLACE on `cache`.
  * Replaces the device branch of tt::paged_fill_cache (custom_ops.py:1016-1094; CPU
  * semantics for one user :1037-1092; batched call site

@@ -72,6 +72,32 @@ def test_update_backend_view_padded_heads_and_padded_rows():
     assert torch.equal(row, key[4, 0, :hkv]) or torch.equal(row, key[5, 0, :hkv])
 
 
+@pytest.mark.parametrize("fmt", ["bf16", "bfp8"])
+def test_update_kv_single_launch_equals_two_updates(fmt):
+    """tt::paged_update_kv_cache_ (one launch for K and V) against the oracle applied twice."""
+    from oracle import bfp8_codec as C
+
+    g = torch.Generator().manual_seed(21)
+    users, hkv, bs, d, w = 7, 8, 32, 128, 3
+    nb = users * w
+    kc = torch.randn(nb, hkv, bs, d, generator=g).to(torch.bfloat16)
+    vc = torch.randn(nb, hkv, bs, d, generator=g).to(torch.bfloat16)
+    key = torch.randn(users, 1, hkv, d, generator=g).to(torch.bfloat16)
+    val = torch.randn(users, 1, hkv, d, generator=g).to(torch.bfloat16)
+    table = _table(g, users, w)
+    idx = torch.randint(0, w * bs, (users,), generator=g, dtype=torch.int32)
+    k_want = O.paged_update_cache(kc, key.transpose(0, 1), idx, table)
+    v_want = O.paged_update_cache(vc, val.transpose(0, 1), idx, table)
+    if fmt == "bfp8":
+        k_dev, v_dev = C.pack_cache(kc).cuda(), C.pack_cache(vc).cuda()
+        k_want, v_want = C.pack_cache(k_want), C.pack_cache(v_want)
+    else:
+        k_dev, v_dev = kc.cuda(), vc.cuda()
+    torch.ops.tt.paged_update_kv_cache_(k_dev, v_dev, key.cuda().transpose(0, 1),
+                                        val.cuda().transpose(0, 1), idx.cuda(), table.cuda())
+    assert torch.equal(k_dev.cpu(), k_want) and torch.equal(v_dev.cpu(), v_want)
+
+
 def test_update_out_of_table_positions_are_skipped():
     cache = torch.zeros(4, 1, 32, 64, dtype=torch.bfloat16)
     fill = torch.ones(1, 2, 1, 64, dtype=torch.bfloat16)

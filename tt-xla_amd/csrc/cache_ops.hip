@@ -13,6 +13,8 @@ namespace {
 struct UpdateArgs {
   void *cache;
   const uint16_t *fill;
+  void *cache2;           // second (V) cache and fill when both are written in one launch
+  const uint16_t *fill2;
   int64_t fill_us, fill_hs;
   const void *idx;
   int idx_i64;
@@ -55,6 +57,30 @@ __global__ __launch_bounds__(256) void update_bf16_kernel(UpdateArgs a) {
   } else {
     *dst = *src;
   }
+  if (a.cache2) {
+    const int64_t so = src - a.fill, dof = dst - static_cast<uint16_t *>(a.cache);
+    if constexpr (VEC == 8) {
+      *reinterpret_cast<uint4 *>(static_cast<uint16_t *>(a.cache2) + dof) =
+          *reinterpret_cast<const uint4 *>(a.fill2 + so);
+    } else {
+      static_cast<uint16_t *>(a.cache2)[dof] = a.fill2[so];
+    }
+  }
+}
+
+__device__ __forceinline__ void update_bfp8_row(void *cache, const uint16_t *fill, const UpdateArgs &a,
+                                                int u, int h, int grp, int phys, int off) {
+  const int gpr = a.d / 16;
+  const uint4 *src = reinterpret_cast<const uint4 *>(fill + u * a.fill_us + h * a.fill_hs + grp * 16);
+  uint4 lo = src[0], hi = src[1];
+  uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  uint32_t bytes[4];
+  uint32_t e = bfp8_encode16(w, bytes);
+  uint8_t *slab = static_cast<uint8_t *>(cache) +
+                  ((int64_t)phys * a.hkv + h) * (int64_t)(a.bs + a.bs / 16) * a.d;
+  *reinterpret_cast<uint4 *>(slab + (int64_t)off * a.d + grp * 16) =
+      make_uint4(bytes[0], bytes[1], bytes[2], bytes[3]);
+  slab[(int64_t)a.bs * a.d + (int64_t)off * gpr + grp] = (uint8_t)e;
 }
 
 __global__ __launch_bounds__(256) void update_bfp8_kernel(UpdateArgs a) {
@@ -66,17 +92,8 @@ __global__ __launch_bounds__(256) void update_bfp8_kernel(UpdateArgs a) {
   int u = (int)(row / a.hkv), h = (int)(row % a.hkv);
   int phys, off;
   if (!resolve_update(a, u, phys, off)) return;
-  const uint4 *src =
-      reinterpret_cast<const uint4 *>(a.fill + u * a.fill_us + h * a.fill_hs + grp * 16);
-  uint4 lo = src[0], hi = src[1];
-  uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-  uint32_t bytes[4];
-  uint32_t e = bfp8_encode16(w, bytes);
-  uint8_t *slab = static_cast<uint8_t *>(a.cache) +
-                  ((int64_t)phys * a.hkv + h) * (int64_t)(a.bs + a.bs / 16) * a.d;
-  *reinterpret_cast<uint4 *>(slab + (int64_t)off * a.d + grp * 16) =
-      make_uint4(bytes[0], bytes[1], bytes[2], bytes[3]);
-  slab[(int64_t)a.bs * a.d + (int64_t)off * gpr + grp] = (uint8_t)e;
+  update_bfp8_row(a.cache, a.fill, a, u, h, grp, phys, off);
+  if (a.cache2) update_bfp8_row(a.cache2, a.fill2, a, u, h, grp, phys, off);
 }
 
 struct FillArgs {
@@ -170,13 +187,12 @@ int common_checks(const void *cache, const void *fill, const int32_t *pt, int hk
 
 using namespace ttpa;
 
-extern "C" int ttpa_paged_update_cache(void *cache, const void *fill, int64_t fill_user_stride,
-                                       int64_t fill_head_stride, const void *update_indices,
-                                       int indices_is_i64, const int32_t *page_table,
-                                       int64_t page_table_row_stride, int32_t users,
-                                       int32_t kv_heads, int32_t block_size, int32_t head_size,
-                                       int32_t table_width, int32_t num_blocks, int32_t kv_format,
-                                       void *stream) {
+static int launch_update(void *cache, void *cache2, const void *fill, const void *fill2,
+                         int64_t fill_user_stride, int64_t fill_head_stride,
+                         const void *update_indices, int indices_is_i64, const int32_t *page_table,
+                         int64_t page_table_row_stride, int32_t users, int32_t kv_heads,
+                         int32_t block_size, int32_t head_size, int32_t table_width,
+                         int32_t num_blocks, int32_t kv_format, void *stream) {
   if (int rc = common_checks(cache, fill, page_table, kv_heads, block_size, head_size, table_width,
                              num_blocks, kv_format))
     return rc;
@@ -184,6 +200,7 @@ extern "C" int ttpa_paged_update_cache(void *cache, const void *fill, int64_t fi
   TTPA_REQUIRE(users >= 0, "negative user count");
   if (users == 0) return TTPA_OK;
   UpdateArgs a{cache,      static_cast<const uint16_t *>(fill),
+               cache2,     static_cast<const uint16_t *>(fill2),
                fill_user_stride, fill_head_stride,
                update_indices,   indices_is_i64,
                page_table, page_table_row_stride,
@@ -192,6 +209,7 @@ extern "C" int ttpa_paged_update_cache(void *cache, const void *fill, int64_t fi
                table_width, num_blocks};
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool vec_ok = head_size % 8 == 0 && aligned16(cache) && aligned16(fill) &&
+                      (!cache2 || (aligned16(cache2) && aligned16(fill2))) &&
                       fill_user_stride % 8 == 0 && fill_head_stride % 8 == 0;
   if (kv_format == TTPA_KV_BFP8) {
     TTPA_REQUIRE(vec_ok, "block-float-8 update needs 16-byte aligned fill rows");
@@ -205,6 +223,32 @@ extern "C" int ttpa_paged_update_cache(void *cache, const void *fill, int64_t fi
     update_bf16_kernel<1><<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st>>>(a);
   }
   return check_launch("paged_update_cache");
+}
+
+extern "C" int ttpa_paged_update_cache(void *cache, const void *fill, int64_t fill_user_stride,
+                                       int64_t fill_head_stride, const void *update_indices,
+                                       int indices_is_i64, const int32_t *page_table,
+                                       int64_t page_table_row_stride, int32_t users,
+                                       int32_t kv_heads, int32_t block_size, int32_t head_size,
+                                       int32_t table_width, int32_t num_blocks, int32_t kv_format,
+                                       void *stream) {
+  return launch_update(cache, nullptr, fill, nullptr, fill_user_stride, fill_head_stride,
+                       update_indices, indices_is_i64, page_table, page_table_row_stride, users,
+                       kv_heads, block_size, head_size, table_width, num_blocks, kv_format, stream);
+}
+
+extern "C" int ttpa_paged_update_cache_kv(void *k_cache, void *v_cache, const void *k_fill,
+                                          const void *v_fill, int64_t fill_user_stride,
+                                          int64_t fill_head_stride, const void *update_indices,
+                                          int indices_is_i64, const int32_t *page_table,
+                                          int64_t page_table_row_stride, int32_t users,
+                                          int32_t kv_heads, int32_t block_size, int32_t head_size,
+                                          int32_t table_width, int32_t num_blocks,
+                                          int32_t kv_format, void *stream) {
+  TTPA_REQUIRE(v_cache && v_fill, "null V cache / fill pointer");
+  return launch_update(k_cache, v_cache, k_fill, v_fill, fill_user_stride, fill_head_stride,
+                       update_indices, indices_is_i64, page_table, page_table_row_stride, users,
+                       kv_heads, block_size, head_size, table_width, num_blocks, kv_format, stream);
 }
 
 extern "C" int ttpa_paged_fill_cache(void *cache, const void *fill, int64_t fill_user_stride,

@@ -31,6 +31,10 @@ SIGNATURES = {
         _int,
         [_p, _p, _i64, _i64, _p, _int, _p, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _p],
     ),
+    "ttpa_paged_update_cache_kv": (
+        _int,
+        [_p, _p, _p, _p, _i64, _i64, _p, _int, _p, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _p],
+    ),
     "ttpa_paged_fill_cache": (
         _int,
         [_p, _p, _i64, _i64, _i64, _p, _i64, _p, _int, _i32, _i32, _i32, _i32, _i32, _i32, _i32,

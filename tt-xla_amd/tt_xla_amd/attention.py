@@ -326,9 +326,8 @@ class TTAttentionBackendImpl(_ImplBase):
             if self.functional_cache_ops:
                 kv_cache[0].copy_(ops.paged_update_cache(kv_cache[0], k_new, *args))
                 kv_cache[1].copy_(ops.paged_update_cache(kv_cache[1], v_new, *args))
-            else:
-                ops.paged_update_cache_(kv_cache[0], k_new, *args)
-                ops.paged_update_cache_(kv_cache[1], v_new, *args)
+            else:  # both scatters in one launch
+                ops.paged_update_kv_cache_(kv_cache[0], kv_cache[1], k_new, v_new, *args)
             return
         # prefill: [users, S, Hkv, D] -> [users, Hkv, S, D], all users in one call
         k_new = inputs.key.transpose(1, 2)

@@ -150,6 +150,48 @@ def _(cache, fill_value, update_indices, page_table, share_cache=False):
     return None
 
 
+@torch.library.custom_op("tt::paged_update_kv_cache_", mutates_args=["k_cache", "v_cache"],
+                         device_types=["cuda"])
+def paged_update_kv_cache_(
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    k_fill: torch.Tensor,
+    v_fill: torch.Tensor,
+    update_indices: torch.Tensor,
+    page_table: torch.Tensor,
+) -> None:
+    """``paged_update_cache_`` on the K cache and on the V cache in one launch (the decode
+    step always writes both with the same indices and table)."""
+    geo = _cache_geometry(k_cache)
+    if _cache_geometry(v_cache) != geo or k_fill.shape != v_fill.shape or k_fill.dtype != v_fill.dtype:
+        raise ValueError("K and V caches / fills must agree in shape and dtype")
+    k_fill, v_fill = _rows_contiguous(k_fill), _rows_contiguous(v_fill)
+    if k_fill.stride() != v_fill.stride():
+        paged_update_cache_(k_cache, k_fill, update_indices, page_table)
+        paged_update_cache_(v_cache, v_fill, update_indices, page_table)
+        return
+    nb, hkv, bs, d, fmt = geo
+    users = update_indices.shape[0]
+    if (k_fill.dim() != 4 or k_fill.shape[0] != 1 or k_fill.shape[1] != users
+            or k_fill.shape[2] < hkv or k_fill.shape[3] != d):
+        raise ValueError(f"fill {tuple(k_fill.shape)} does not match users={users}, kv_heads={hkv}, head_size={d}")
+    if page_table.dim() != 2 or page_table.shape[0] < users:
+        raise ValueError("page_table must be [users, blocks_per_user]")
+    idx = _index_tensor(update_indices)
+    pt = _table(page_table)
+    N.call(
+        "ttpa_paged_update_cache_kv",
+        k_cache.data_ptr(), v_cache.data_ptr(), k_fill.data_ptr(), v_fill.data_ptr(),
+        k_fill.stride(1), k_fill.stride(2), idx.data_ptr(), int(idx.dtype == torch.int64),
+        pt.data_ptr(), pt.stride(0), users, hkv, bs, d, pt.shape[1], nb, fmt, _stream(),
+    )
+
+
+@paged_update_kv_cache_.register_fake
+def _(k_cache, v_cache, k_fill, v_fill, update_indices, page_table):
+    return None
+
+
 def _fill_inplace(cache, fill_value, page_table, batch_idx):
     nb, hkv, bs, d, fmt = _cache_geometry(cache)
     if fill_value.dim() != 4:
