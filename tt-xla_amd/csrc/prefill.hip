@@ -70,17 +70,29 @@ __device__ __forceinline__ const uint16_t *kv_chunk(const PrefillArgs &a, const 
   return base + b * a.kv_bs + hk * a.kv_hs + (int64_t)key * a.kv_ts + c * 8;
 }
 
+// v_max3_f32 without the input canonicalisation the compiler adds around fmaxf (scores are
+// never signalling NaNs).  Callers order it after a compiler-visible read of the matrix
+// results, which is where the matrix-to-vector hazard wait states are inserted.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float d;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+  return d;
+}
+
 // MODE 0: dense K/V; 1: paged, block_size a multiple of 64 (a tile lies in one block);
 // 2: paged, any block size (per-chunk table lookups).
-// R = blocks of 32 query rows per wavefront.  R = 2 reuses every K / V fragment read from
-// LDS for two matrix instructions (LDS operand traffic per FLOP halves) and gives the
-// scheduler two independent row blocks to overlap: the score product of block 1 runs on the
-// matrix pipe while block 0's softmax runs on the VALU.  It needs the 512-register budget
-// (one workgroup per CU); R = 1 keeps two workgroups per CU and serves short queries.
-template <int D, int HPW, int MODE, int R>
-__global__ __launch_bounds__(256, (D <= 128 && R == 1 ? 2 : 1)) void prefill_kernel(PrefillArgs a) {
+//
+// Per-tile schedule of a workgroup (LDS holds two K stages and two V stages):
+//   write K(t+1) to LDS | fetch K(t+2) | S^T = K(t) Q^T | barrier |
+//   write V(t+1) to LDS | fetch V(t+2) | softmax | O^T += V(t)^T P^T
+// One barrier per tile: K(t+1) is complete for everyone at the barrier of tile t and is read
+// after it; V(t+1) is written after that barrier (so every wavefront has finished reading
+// V(t-1) from the same stage) and read after the barrier of tile t+1.  LDS operand reads run
+// a few fragments ahead of the matrix instructions that consume them.
+template <int D, int HPW, int MODE>
+__global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(PrefillArgs a) {
   constexpr int RPW = 4 / HPW;            // wavefront row slots per workgroup
-  constexpr int ROWS = kRowsPerWave * R;  // query rows per wavefront
+  constexpr int ROWS = kRowsPerWave;      // query rows per wavefront
   constexpr int KSTEPS = D / 16;          // MFMA k-steps over the head dimension
   constexpr int DBLK = D / 32;            // 32-wide output blocks over the head dimension
   constexpr int CPT = D / 32;             // 16-byte chunks per thread per tile and tensor
@@ -92,11 +104,19 @@ __global__ __launch_bounds__(256, (D <= 128 && R == 1 ? 2 : 1)) void prefill_ker
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int n = lane & 31, h = lane >> 5;
+  // Workgroups are dealt to the 8 XCDs round-robin by linear id, and each XCD has its own
+  // L2: all query tiles of one (batch, KV-head group) run on the same XCD, one after the
+  // other, so that K/V of a group is fetched from HBM by one L2 only and stays resident there
+  // while its query tiles stream through.
   const int nqt = (a.sq + ROWS * RPW - 1) / (ROWS * RPW);
-  const int qt = nqt - 1 - (int)blockIdx.x;  // heavy (late) tiles are scheduled first
   const int groups = a.hq / HPW;
-  const int b = blockIdx.y / groups;
-  const int hq0 = (blockIdx.y - b * groups) * HPW;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int yl = slot / nqt;
+  const int y = yl * 8 + xcd;
+  if (y >= a.batch * groups) return;  // grid is padded to a multiple of 8 groups
+  const int qt = nqt - 1 - (slot - yl * nqt);  // heavy (late) tiles are scheduled first
+  const int b = y / groups;
+  const int hq0 = (y - b * groups) * HPW;
   const int g = a.hq / a.hkv;
   const int hk = hq0 / g;
   const int hq = hq0 + wave % HPW;
@@ -111,33 +131,28 @@ __global__ __launch_bounds__(256, (D <= 128 && R == 1 ? 2 : 1)) void prefill_ker
   const bool wave_active = row0 < a.sq;
 
   // ---- Q fragments (B operand: lane n = query row, 8 head-dim elements per k-step) -----
-  bf16x8 qf[R][KSTEPS];
-#pragma unroll
-  for (int rb = 0; rb < R; ++rb) {
-    const int qrow = min(row0 + 32 * rb + n, a.sq - 1);
+  bf16x8 qf[KSTEPS];
+  {
+    const int qrow = min(row0 + n, a.sq - 1);
     const uint16_t *qp = a.q + b * a.q_bs + hq * a.q_hs + (int64_t)qrow * a.q_ts + 8 * h;
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s)
-      qf[rb][s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 16 * s));
+      qf[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 16 * s));
   }
 
-  floatx16 acc[R][DBLK];
-  float m_run[R], l_run[R];
+  floatx16 acc[DBLK];
+  float m_run = -INFINITY, l_run = 0.f;
 #pragma unroll
-  for (int rb = 0; rb < R; ++rb) {
-    m_run[rb] = -INFINITY;
-    l_run[rb] = 0.f;
+  for (int i = 0; i < DBLK; ++i)
 #pragma unroll
-    for (int i = 0; i < DBLK; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[rb][i][r] = 0.f;
-  }
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
 
   // ---- global -> register staging of one K/V tile -------------------------------------
   // A thread's chunks sit at fixed (key, column) positions of every tile: their offsets are
   // computed once, and per tile only a wavefront-uniform base moves (modes 0 and 1).
   u32x4 kst[CPT], vst[CPT];  // native vectors: struct-typed uint4 arrays end up in scratch memory
-  uint32_t chunk_off[CPT];  // element offset of chunk i inside a tile
+  uint32_t chunk_off[CPT];   // element offset of chunk i inside a tile
+  uint32_t lds_k[CPT], lds_v[CPT];  // element offset of chunk i inside an LDS stage
   int chunk_key[CPT], chunk_col[CPT];
 #pragma unroll
   for (int i = 0; i < CPT; ++i) {
@@ -146,217 +161,242 @@ __global__ __launch_bounds__(256, (D <= 128 && R == 1 ? 2 : 1)) void prefill_ker
     chunk_key[i] = key;
     chunk_col[i] = c;
     chunk_off[i] = (uint32_t)(key * (MODE == 0 ? (int)a.kv_ts : D) + c * 8);
+    lds_k[i] = (uint32_t)(key * L::KS + c * 8);
+    lds_v[i] = (uint32_t)(kKeysPerTile * L::KS + key * L::VS + c * 8);
   }
   // Loads are unconditional (a predicated load would make the compiler wait for the prefetch
   // right after issuing it): keys past the end of a dense K/V are clamped to the last row,
   // whose scores are masked and whose V rows therefore carry weight 0.
-  auto fetch_tile = [&](int kt) {
+  auto tile_base = [&](int kt) -> int64_t {  // uniform element offset of the tile
     const int key0 = kt * kKeysPerTile;
-    int64_t base;  // uniform element offset of the tile
     if constexpr (MODE == 0) {
-      base = b * a.kv_bs + hk * a.kv_hs + (int64_t)key0 * a.kv_ts;
+      return b * a.kv_bs + hk * a.kv_hs + (int64_t)key0 * a.kv_ts;
     } else if constexpr (MODE == 1) {
       int phys = __builtin_amdgcn_readfirstlane(a.pt[(int64_t)b * a.pt_rs + key0 / a.bs]);
       if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
-      base = (((int64_t)phys * a.hkv + hk) * a.bs + (key0 % a.bs)) * D;
+      return (((int64_t)phys * a.hkv + hk) * a.bs + (key0 % a.bs)) * D;
     } else {
-      base = 0;
+      return 0;
     }
+  };
+  auto fetch = [&](const uint16_t *src, u32x4 (&dst)[CPT], int kt) {
+    const int key0 = kt * kKeysPerTile;
+    const int64_t base = tile_base(kt);
     const int last = a.skv - 1 - key0;  // last valid key of this tile, relative (>= 0)
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
       if constexpr (MODE == 2) {
         const int key = key0 + min(chunk_key[i], last);
-        kst[i] = *reinterpret_cast<const u32x4 *>(kv_chunk(a, a.k, b, hk, key, chunk_col[i], D));
-        vst[i] = *reinterpret_cast<const u32x4 *>(kv_chunk(a, a.v, b, hk, key, chunk_col[i], D));
+        dst[i] = *reinterpret_cast<const u32x4 *>(kv_chunk(a, src, b, hk, key, chunk_col[i], D));
       } else if constexpr (MODE == 1) {  // table_width * block_size is a multiple of the tile
-        kst[i] = *reinterpret_cast<const u32x4 *>(a.k + base + chunk_off[i]);
-        vst[i] = *reinterpret_cast<const u32x4 *>(a.v + base + chunk_off[i]);
+        dst[i] = *reinterpret_cast<const u32x4 *>(src + base + chunk_off[i]);
       } else {
         const uint32_t off = (uint32_t)(min(chunk_key[i], last) * (int)a.kv_ts + chunk_col[i] * 8);
-        kst[i] = *reinterpret_cast<const u32x4 *>(a.k + base + off);
-        vst[i] = *reinterpret_cast<const u32x4 *>(a.v + base + off);
+        dst[i] = *reinterpret_cast<const u32x4 *>(src + base + off);
       }
     }
   };
-  auto stage_tile = [&](int buf) {
-    uint16_t *ks = smem + buf * STAGE;
-    uint16_t *vs = ks + kKeysPerTile * L::KS;
+  auto stage = [&](const u32x4 (&srcv)[CPT], const uint32_t (&off)[CPT], int buf) {
+    uint16_t *base = smem + buf * STAGE;
 #pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      *reinterpret_cast<u32x4 *>(ks + chunk_key[i] * L::KS + chunk_col[i] * 8) = kst[i];
-      *reinterpret_cast<u32x4 *>(vs + chunk_key[i] * L::VS + chunk_col[i] * 8) = vst[i];
-    }
+    for (int i = 0; i < CPT; ++i) *reinterpret_cast<u32x4 *>(base + off[i]) = srcv[i];
   };
 
-  // Pipeline: LDS holds two stages.  While tile kt is consumed from stage kt & 1, tile kt + 1
-  // (fetched one iteration ago) is written to the other stage and tile kt + 2 is in flight
-  // from global memory.  One barrier per tile.  Staging and prefetch are unconditional (past
-  // the last tile they repeat it into a stage nobody reads): straight-line code keeps the
-  // staged tile in registers and the wait counters exact.  ntiles >= 1 always (row 0 sees
-  // key 0).
+  // LDS operand addresses of this lane inside a stage
+  const uint32_t k_lane = (uint32_t)(n * L::KS + 8 * h);
+  const int grp = lane >> 4, a16 = lane & 15;
+  const uint32_t v_lane = (uint32_t)(kKeysPerTile * L::KS +
+                                     (4 * (grp >> 1) + (a16 >> 2)) * L::VS + 16 * (grp & 1) + 4 * (a16 & 3));
+  // K fragment i of a tile in issue order: k-step i / 2 of key block i % 2 (the two score
+  // blocks alternate so consecutive matrix instructions are independent).
+  auto read_k = [&](const uint16_t *st_base, int i) -> bf16x8 {
+    const int s = i >> 1, kb = i & 1;
+    return __builtin_bit_cast(
+        bf16x8, *reinterpret_cast<const uint4 *>(st_base + k_lane + 32 * kb * L::KS + 16 * s));
+  };
+  // V^T fragment j in issue order: key step j / DBLK, output block j % DBLK.  Through the
+  // transposing LDS load, per group of 16 lanes, lane i receives element i % 4 of the 8-byte
+  // chunks addressed by lanes 4 j + i / 4.
+  auto read_v = [&](const uint16_t *st_base, int j) -> bf16x8 {
+    typedef __attribute__((address_space(3))) shortx4 *lds_v4;
+    const int k4 = j / DBLK, db = j % DBLK;
+    const uint16_t *vk = st_base + v_lane + 16 * k4 * L::VS + 32 * db;
+    shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk));
+    shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk + 8 * L::VS));
+    bf16x4 l4 = __builtin_bit_cast(bf16x4, lo), h4 = __builtin_bit_cast(bf16x4, hi);
+    bf16x8 t;
+    t[0] = l4[0], t[1] = l4[1], t[2] = l4[2], t[3] = l4[3];
+    t[4] = h4[0], t[5] = h4[1], t[6] = h4[2], t[7] = h4[3];
+    return t;
+  };
+
+  constexpr int NK = 2 * KSTEPS;  // K fragments per tile
+  constexpr int NV = 4 * DBLK;    // V^T fragments per tile
+  constexpr int KPRE = 6;         // K fragments in flight
+  constexpr int VPRE = 4;         // V^T fragments in flight
+
+  // ntiles >= 1 always (row 0 sees key 0).  Past the last tile the prefetch repeats it into a
+  // stage nobody reads: straight-line code keeps staged tiles in registers and the wait
+  // counters exact.
   const int last_tile = ntiles - 1;
-  fetch_tile(0);
-  stage_tile(0);
-  fetch_tile(min(1, last_tile));
+  fetch(a.k, kst, 0);
+  fetch(a.v, vst, 0);
+  stage(kst, lds_k, 0);
+  stage(vst, lds_v, 0);
+  fetch(a.k, kst, min(1, last_tile));
+  fetch(a.v, vst, min(1, last_tile));
   __syncthreads();
   for (int kt = 0; kt < ntiles; ++kt) {
-    stage_tile((kt + 1) & 1);
-    fetch_tile(min(kt + 2, last_tile));
-    const uint16_t *ks = smem + (kt & 1) * STAGE;
-    const uint16_t *vs = ks + kKeysPerTile * L::KS;
+    const uint16_t *cur = smem + (kt & 1) * STAGE;
     const int key0 = kt * kKeysPerTile;
+    const bool compute = wave_active && key0 <= wave_last_key;  // wavefront-uniform
 
-    if (wave_active && key0 <= wave_last_key) {
-      // ---- K fragments: read once, used for every row block ------------------------------
-      bf16x8 kf[2][KSTEPS];
+    stage(kst, lds_k, (kt + 1) & 1);
+    fetch(a.k, kst, min(kt + 2, last_tile));
+
+    // ---- S^T = K . Q^T -------------------------------------------------------------------
+    floatx16 st[2];
+    if (compute) {
+      bf16x8 ring[KPRE];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        const uint16_t *krow = ks + (32 * kb + n) * L::KS + 8 * h;
+      for (int i = 0; i < KPRE; ++i) ring[i] = read_k(cur, i);
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s)
-          kf[kb][s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(krow + 16 * s));
+      for (int r = 0; r < 16; ++r) st[0][r] = 0.f, st[1][r] = 0.f;
+#pragma unroll
+      for (int i = 0; i < NK; ++i) {
+        st[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % KPRE], qf[i >> 1], st[i & 1], 0, 0, 0);
+        if (i + KPRE < NK) ring[i % KPRE] = read_k(cur, i + KPRE);
       }
-      // ---- S^T = K . Q^T, row block after row block ------------------------------------------
-      floatx16 st[R][2];
+      // pin the order: KPRE reads up front, then one read behind every matrix instruction
+      __builtin_amdgcn_sched_group_barrier(0x100, KPRE, 0);
 #pragma unroll
-      for (int rb = 0; rb < R; ++rb)
+      for (int i = 0; i < NK; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i + KPRE < NK) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+    }
+    __syncthreads();  // K(kt+1) staged by everyone; everyone is done with V(kt-1)
+    stage(vst, lds_v, (kt + 1) & 1);
+    fetch(a.v, vst, min(kt + 2, last_tile));
+
+    if (compute) {
+      bf16x8 vring[VPRE];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) st[rb][kb][r] = 0.f;
-#pragma unroll
-          for (int s = 0; s < KSTEPS; ++s)
-            st[rb][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb][s], qf[rb][s], st[rb][kb], 0, 0, 0);
-        }
-      bf16x8 pf[R][2][2];
-#pragma unroll
-      for (int rb = 0; rb < R; ++rb) {
-        // ---- mask, online softmax (one query row per lane) -----------------------------------
-        // The softmax scale is positive, so the running maximum is tracked on raw scores and
-        // the scale is folded into the exponent: p = exp2(s * c - m * c).
-        const int rrow0 = row0 + 32 * rb;
-        const int qrow = rrow0 + n;
-        const bool need_mask = (a.causal && key0 + kKeysPerTile - 1 > offset + rrow0) ||
-                               key0 + kKeysPerTile > a.skv || a.mask != nullptr;
-        if (need_mask) {  // wavefront-uniform: only diagonal / ragged / explicitly masked tiles
-          const int limit = a.causal ? min(offset + qrow, a.skv - 1) : a.skv - 1;
-#pragma unroll
-          for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int key = key0 + 32 * kb + 8 * (r >> 2) + 4 * h + (r & 3);
-              float v = st[rb][kb][r];
-              if (a.mask) {
-                const int kc = min(key, a.skv - 1), qc = min(qrow, a.sq - 1);
-                // additive mask is in natural-log units of the scaled score
-                v += bf16_lo(a.mask[b * a.mask_bs + (int64_t)qc * a.mask_rs + kc]) *
-                     (1.4426950408889634f / a.scale_log2e);
-              }
-              st[rb][kb][r] = key > limit ? -INFINITY : v;
-            }
-        }
-        float mloc = fmaxf(st[rb][0][0], st[rb][1][0]);
-#pragma unroll
-        for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(st[rb][0][r], st[rb][1][r]));
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-        // Lazy rescaling: the running maximum only moves when a row's new maximum exceeds it
-        // by more than 2^8 in the exponent domain.  Until then probabilities are taken
-        // relative to the stale maximum (they may reach 2^8, harmless in bf16 / fp32), the
-        // accumulators need no rescale, and the final division by the row sum is unchanged.
-        const float kLazy = 8.0f;
-        const bool move = !((mloc - m_run[rb]) * a.scale_log2e <= kLazy);  // also true from -inf
-        const float m_new = move ? mloc : m_run[rb];
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = move ? __builtin_amdgcn_exp2f((m_run[rb] - m_safe) * a.scale_log2e) : 1.0f;
-        const float mc = m_safe * a.scale_log2e;
-        m_run[rb] = m_new;
-        float lsum = 0.f;
+      for (int j = 0; j < VPRE; ++j) vring[j] = read_v(cur, j);
+
+      // ---- mask, online softmax (one query row per lane) -----------------------------------
+      // The softmax scale is positive, so the running maximum is tracked on raw scores and
+      // the scale is folded into the exponent: p = exp2(s * c - m * c).
+      const int qrow = row0 + n;
+      const bool need_mask = (a.causal && key0 + kKeysPerTile - 1 > offset + row0) ||
+                             key0 + kKeysPerTile > a.skv || a.mask != nullptr;
+      if (need_mask) {  // wavefront-uniform: only diagonal / ragged / explicitly masked tiles
+        const int limit = a.causal ? min(offset + qrow, a.skv - 1) : a.skv - 1;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-          for (int s = 0; s < 2; ++s)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-              // B-operand element e of k-step s <-> accumulator register 8 s + e
-              float p = __builtin_amdgcn_exp2f(fmaf(st[rb][kb][8 * s + e], a.scale_log2e, -mc));
-              lsum += p;
-              pf[rb][kb][s][e] = (__bf16)p;
+          for (int r = 0; r < 16; ++r) {
+            const int key = key0 + 32 * kb + 8 * (r >> 2) + 4 * h + (r & 3);
+            float v = st[kb][r];
+            if (a.mask) {
+              const int kc = min(key, a.skv - 1), qc = min(qrow, a.sq - 1);
+              // additive mask is in natural-log units of the scaled score
+              v += bf16_lo(a.mask[b * a.mask_bs + (int64_t)qc * a.mask_rs + kc]) *
+                   (1.4426950408889634f / a.scale_log2e);
             }
-        l_run[rb] = l_run[rb] * alpha + lsum;
-        // skip the accumulator rescale when no row of the wavefront moved its maximum
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-          for (int i = 0; i < DBLK; ++i)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[rb][i][r] *= alpha;
-        }
-      }
-      // ---- O^T += V^T . P^T: V^T fragments come through the transposing LDS load (per group
-      //      of 16 lanes, lane i receives element i % 4 of the 8-byte chunks addressed by lanes
-      //      4 j + i / 4); each fragment feeds every row block -------------------------------
-      {
-        const int grp = lane >> 4, a16 = lane & 15;
-        const uint16_t *vbase =
-            vs + (4 * (grp >> 1) + (a16 >> 2)) * L::VS + 16 * (grp & 1) + 4 * (a16 & 3);
-#pragma unroll
-        for (int k4 = 0; k4 < 4; ++k4) {
-          bf16x8 vf[DBLK];
-#pragma unroll
-          for (int db = 0; db < DBLK; ++db) {
-            typedef __attribute__((address_space(3))) shortx4 *lds_v4;
-            const uint16_t *vk = vbase + 16 * k4 * L::VS + 32 * db;
-            shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk));
-            shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk + 8 * L::VS));
-            bf16x4 l4 = __builtin_bit_cast(bf16x4, lo), h4 = __builtin_bit_cast(bf16x4, hi);
-            bf16x8 t;
-            t[0] = l4[0], t[1] = l4[1], t[2] = l4[2], t[3] = l4[3];
-            t[4] = h4[0], t[5] = h4[1], t[6] = h4[2], t[7] = h4[3];
-            vf[db] = t;
+            st[kb][r] = key > limit ? -INFINITY : v;
           }
+      }
+      // The first maximum is an ordinary compiler-visible read of both score blocks.
+      float mloc = fmaxf(st[0][0], st[1][0]);
 #pragma unroll
-          for (int rb = 0; rb < R; ++rb)
+      for (int r = 1; r < 16; r += 3) {
+        mloc = max3(mloc, st[0][r], st[1][r]);
+        mloc = max3(mloc, st[0][r + 1], st[1][r + 1]);
+        mloc = max3(mloc, st[0][r + 2], st[1][r + 2]);
+      }
+      {  // the other half of the key rows sits 32 lanes away: exchange through v_permlane32_swap
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        const uint32_t mb = __builtin_bit_cast(uint32_t, mloc);
+        const u32x2 sw = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
+        mloc = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+      }
+      // Lazy rescaling: the running maximum only moves when a row's new maximum exceeds it
+      // by more than 2^8 in the exponent domain.  Until then probabilities are taken
+      // relative to the stale maximum (they may reach 2^8, harmless in bf16 / fp32), the
+      // accumulators need no rescale, and the final division by the row sum is unchanged.
+      const float kLazy = 8.0f;
+      const bool move = !((mloc - m_run) * a.scale_log2e <= kLazy);  // also true from -inf
+      const float m_new = move ? mloc : m_run;
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = move ? __builtin_amdgcn_exp2f((m_run - m_safe) * a.scale_log2e) : 1.0f;
+      const float mc = m_safe * a.scale_log2e;
+      m_run = m_new;
+      // skip the accumulator rescale when no row of the wavefront moved its maximum
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-            for (int db = 0; db < DBLK; ++db)
-              acc[rb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db], pf[rb][k4 >> 1][k4 & 1],
-                                                                    acc[rb][db], 0, 0, 0);
+        for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][r] *= alpha;
+      }
+      // Probabilities as bf16 B-operand fragments: element e of key step k4 = 2 kb + s is
+      // accumulator register 8 s + e of score block kb.  The row sum is taken over the rounded
+      // values (two per v_dot2_f32_bf16), i.e. over exactly what the second product sees.
+      typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+      const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+      bf16x8 pf[4];
+      float lsum = 0.f;
+#pragma unroll
+      for (int k4 = 0; k4 < 4; ++k4)
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          const int r = 8 * (k4 & 1) + e;
+          const float p0 = __builtin_amdgcn_exp2f(fmaf(st[k4 >> 1][r], a.scale_log2e, -mc));
+          const float p1 = __builtin_amdgcn_exp2f(fmaf(st[k4 >> 1][r + 1], a.scale_log2e, -mc));
+          const bf16x2 pp = {(__bf16)p0, (__bf16)p1};
+          pf[k4][e] = pp[0], pf[k4][e + 1] = pp[1];
+          lsum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, lsum, false);
         }
+      l_run = l_run * alpha + lsum;
+
+      // ---- O^T += V^T . P^T -----------------------------------------------------------------
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        acc[j % DBLK] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vring[j % VPRE], pf[j / DBLK],
+                                                                acc[j % DBLK], 0, 0, 0);
+        if (j + VPRE < NV) vring[j % VPRE] = read_v(cur, j + VPRE);
       }
     }
-    __syncthreads();  // tile kt + 1 is staged; everyone is done with stage kt & 1
   }
 
   // ---- normalise and store: lane (n, h) holds head-dim elements 32 db + 8 j + 4 h + i ----
   if (!wave_active) return;
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float inv = 1.0f / l_tot;
+  const int qrow = row0 + n;
+  if (qrow >= a.sq) return;
+  uint16_t *op = a.out + b * a.out_bs + hq * a.out_hs + (int64_t)qrow * a.out_ts + 4 * h;
 #pragma unroll
-  for (int rb = 0; rb < R; ++rb) {
-    const float l_tot = l_run[rb] + __shfl_xor(l_run[rb], 32);
-    const float inv = 1.0f / l_tot;
-    const int qrow = row0 + 32 * rb + n;
-    if (qrow >= a.sq) continue;
-    uint16_t *op = a.out + b * a.out_bs + hq * a.out_hs + (int64_t)qrow * a.out_ts + 4 * h;
+  for (int db = 0; db < DBLK; ++db)
 #pragma unroll
-    for (int db = 0; db < DBLK; ++db)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        uint32_t lo = f32_to_bf16_bits(acc[rb][db][4 * j] * inv) |
-                      (f32_to_bf16_bits(acc[rb][db][4 * j + 1] * inv) << 16);
-        uint32_t hi = f32_to_bf16_bits(acc[rb][db][4 * j + 2] * inv) |
-                      (f32_to_bf16_bits(acc[rb][db][4 * j + 3] * inv) << 16);
-        *reinterpret_cast<uint2 *>(op + 32 * db + 8 * j) = make_uint2(lo, hi);
-      }
-  }
+    for (int j = 0; j < 4; ++j) {
+      uint32_t lo = f32_to_bf16_bits(acc[db][4 * j] * inv) |
+                    (f32_to_bf16_bits(acc[db][4 * j + 1] * inv) << 16);
+      uint32_t hi = f32_to_bf16_bits(acc[db][4 * j + 2] * inv) |
+                    (f32_to_bf16_bits(acc[db][4 * j + 3] * inv) << 16);
+      *reinterpret_cast<uint2 *>(op + 32 * db + 8 * j) = make_uint2(lo, hi);
+    }
 }
 
-template <int D, int HPW, int MODE, int R>
+template <int D, int HPW, int MODE>
 int launch_mode(const PrefillArgs &a, hipStream_t st) {
   constexpr int RPW = 4 / HPW;
-  constexpr int ROWS = kRowsPerWave * R;
+  constexpr int ROWS = kRowsPerWave;
   const int nqt = (a.sq + ROWS * RPW - 1) / (ROWS * RPW);
   const size_t lds = 2 * Lds<D>::BYTES;  // two stages
   static bool attr_set = false;
   if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&prefill_kernel<D, HPW, MODE, R>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&prefill_kernel<D, HPW, MODE>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return fail(TTPA_ERR_LAUNCH, "prefill: cannot reserve %zu bytes of LDS", lds);
     attr_set = true;
@@ -364,32 +404,17 @@ int launch_mode(const PrefillArgs &a, hipStream_t st) {
   hipEvent_t ev0, ev1;
   take_profile_events(ev0, ev1);
   if (ev0) (void)hipEventRecord(ev0, st);
-  prefill_kernel<D, HPW, MODE, R><<<dim3(nqt, a.batch * (a.hq / HPW)), dim3(256), lds, st>>>(a);
+  const int ny8 = (a.batch * (a.hq / HPW) + 7) / 8;
+  prefill_kernel<D, HPW, MODE><<<dim3(nqt * ny8 * 8), dim3(256), lds, st>>>(a);
   if (ev1) (void)hipEventRecord(ev1, st);
   return check_launch("sdpa_prefill");
 }
 
-template <int D, int HPW, int MODE>
-int launch_rows(const PrefillArgs &a, hipStream_t st) {
-  // 64 rows per wavefront once the query is long enough to fill them; head size 256 keeps
-  // 32 (its accumulators alone take 128 registers per row block)
-  if constexpr (D <= 128) {
-    static int forced = -1;
-    if (forced < 0) {
-      const char *e = getenv("TTPA_PREFILL_ROWS");
-      forced = e ? atoi(e) : 0;
-    }
-    const bool two = forced == 64;  // 64 rows per wavefront is experimental (TTPA_PREFILL_ROWS=64)
-    if (two) return launch_mode<D, HPW, MODE, 2>(a, st);
-  }
-  return launch_mode<D, HPW, MODE, 1>(a, st);
-}
-
 template <int D, int HPW>
 int launch(const PrefillArgs &a, hipStream_t st) {
-  if (!a.pt) return launch_rows<D, HPW, 0>(a, st);
-  if (a.bs % kKeysPerTile == 0) return launch_rows<D, HPW, 1>(a, st);
-  return launch_rows<D, HPW, 2>(a, st);
+  if (!a.pt) return launch_mode<D, HPW, 0>(a, st);
+  if (a.bs % kKeysPerTile == 0) return launch_mode<D, HPW, 1>(a, st);
+  return launch_mode<D, HPW, 2>(a, st);
 }
 
 template <int D>
@@ -439,7 +464,8 @@ extern "C" int ttpa_sdpa_prefill(void *out, int64_t out_batch_stride, int64_t ou
   TTPA_REQUIRE(q_batch_stride % 8 == 0 && q_head_stride % 8 == 0 && q_token_stride % 8 == 0 &&
                    out_batch_stride % 4 == 0 && out_head_stride % 4 == 0 && out_token_stride % 4 == 0,
                "prefill: q strides must be multiples of 8 elements, out strides of 4");
-  TTPA_REQUIRE((int64_t)batch * q_heads < 65536, "prefill: batch * heads too large for one launch");
+  TTPA_REQUIRE((int64_t)batch * q_heads * ((q_len + 31) / 32) < (1ll << 30),
+               "prefill: batch * heads * query tiles too large for one launch");
 
   PrefillArgs a;
   a.out = static_cast<uint16_t *>(out);
