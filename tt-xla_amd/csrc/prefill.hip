@@ -17,6 +17,12 @@
 //
 // Accumulator layout of a 32x32 tile (lane = 32 h + n): register r holds
 // element (row 8 (r / 4) + 4 h + r % 4, column n).
+//
+// K/V tiles travel global memory -> LDS directly (global_load_lds_dwordx4: 64 lanes x 16
+// bytes land in 1 KiB of consecutive LDS), with no staging registers.  Rows are therefore
+// unpadded in LDS; bank conflicts are avoided by an XOR swizzle of the 16-byte chunk
+// position inside a row, applied on the global side (which chunk a lane fetches) and again
+// when fragments are read.
 #include "common.h"
 
 #include <cstdlib>
@@ -26,9 +32,10 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef short shortx4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kKeysPerTile = 64;
 constexpr int kRowsPerWave = 32;
@@ -49,26 +56,23 @@ struct PrefillArgs {
   float scale_log2e;
 };
 
+// LDS geometry of one stage: the K tile (64 rows of D elements) followed by the V tile.
+// Chunk c (16 bytes) of row r is stored at chunk position c ^ swz(r).
+//   K fragments are read by 16 lanes of consecutive rows at one logical chunk: the 16
+//   positions must differ (rows of >= 256 bytes) or, for 128-byte rows, differ within each
+//   pair of rows that shares a 256-byte bank line.
+//   V fragments are read, per 32 lanes, as 4 consecutive rows x 4 consecutive chunks.
 template <int D>
-struct Lds {
-  // K rows: 16-byte fragments read by 32 lanes of consecutive rows -> row stride = 4 banks
-  // (mod 64); V rows: four consecutive rows read 64 bytes each -> row stride = 16 banks.
-  static constexpr int KS = D + 8;    // elements per K row   (D=128: 68 dwords)
-  static constexpr int VS = D + 32;   // elements per V row   (D=128: 80 dwords)
-  static constexpr int BYTES = kKeysPerTile * (KS + VS) * 2;
+struct Tile {
+  static constexpr int RB = 2 * D;                 // row bytes
+  static constexpr int CPR = D / 8;                // 16-byte chunks per row
+  static constexpr int RPI = 1024 / RB;            // rows covered by one wavefront load
+  static constexpr int NI = kKeysPerTile / RPI / 4;  // loads per wavefront per tile and tensor
+  static constexpr int TILE_BYTES = kKeysPerTile * RB;
+  static constexpr int STAGE_BYTES = 2 * TILE_BYTES;
+  __device__ static constexpr int swz_k(int r) { return RB >= 256 ? (r & 15) : ((r >> 1) & 7); }
+  __device__ static constexpr int swz_v(int r) { return RB >= 256 ? 4 * (r & 3) : 4 * ((r >> 1) & 1); }
 };
-
-// Address of the 8-element chunk `c` of key `key` (absolute position) for (batch b, kv head).
-__device__ __forceinline__ const uint16_t *kv_chunk(const PrefillArgs &a, const uint16_t *base,
-                                                    int b, int hk, int key, int c, int d) {
-  if (a.pt) {
-    int col = key / a.bs;
-    int phys = a.pt[(int64_t)b * a.pt_rs + col];
-    if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
-    return base + (((int64_t)phys * a.hkv + hk) * a.bs + (key - col * a.bs)) * d + c * 8;
-  }
-  return base + b * a.kv_bs + hk * a.kv_hs + (int64_t)key * a.kv_ts + c * 8;
-}
 
 // v_max3_f32 without the input canonicalisation the compiler adds around fmaxf (scores are
 // never signalling NaNs).  Callers order it after a compiler-visible read of the matrix
@@ -79,30 +83,45 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   return d;
 }
 
+// 64 lanes x 16 bytes, global memory -> 1 KiB of LDS starting at byte address `lds_addr`
+// (wavefront-uniform, passed in M0); lane l's 16 bytes land at lds_addr + 16 l.  Written as
+// assembly so that the compiler does not make every later LDS read wait for these loads: the
+// kernel waits for them itself (vmcnt(0)) before the barrier that publishes the tile.
+__device__ __forceinline__ void dma16(const void *uniform_base, uint32_t lane_bytes, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(lane_bytes), "s"(uniform_base), "s"(lds_addr)
+               : "memory");
+}
+__device__ __forceinline__ void dma16_lane(const void *lane_ptr, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(lane_ptr), "s"(lds_addr)
+               : "memory");
+}
+
 // MODE 0: dense K/V; 1: paged, block_size a multiple of 64 (a tile lies in one block);
-// 2: paged, any block size (per-chunk table lookups).
+// 2: paged, any block size (per-row table lookups).
 //
 // Per-tile schedule of a workgroup (LDS holds two K stages and two V stages):
-//   write K(t+1) to LDS | fetch K(t+2) | S^T = K(t) Q^T | barrier |
-//   write V(t+1) to LDS | fetch V(t+2) | softmax | O^T += V(t)^T P^T
-// One barrier per tile: K(t+1) is complete for everyone at the barrier of tile t and is read
-// after it; V(t+1) is written after that barrier (so every wavefront has finished reading
-// V(t-1) from the same stage) and read after the barrier of tile t+1.  LDS operand reads run
-// a few fragments ahead of the matrix instructions that consume them.
+//   S^T = K(t) Q^T | barrier | issue loads of K(t+2) and V(t+1) | softmax | O^T += V(t)^T P^T
+// Every load is issued right after a barrier and has to have landed by the next one, one
+// whole tile later.  K(t+2) overwrites the stage of K(t), which everybody has finished
+// reading at the barrier of tile t; V(t+1) overwrites the stage of V(t-1), read before that
+// barrier too.  LDS operand reads run a few fragments ahead of the matrix instructions that
+// consume them.
 template <int D, int HPW, int MODE>
 __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(PrefillArgs a) {
   constexpr int RPW = 4 / HPW;            // wavefront row slots per workgroup
   constexpr int ROWS = kRowsPerWave;      // query rows per wavefront
   constexpr int KSTEPS = D / 16;          // MFMA k-steps over the head dimension
   constexpr int DBLK = D / 32;            // 32-wide output blocks over the head dimension
-  constexpr int CPT = D / 32;             // 16-byte chunks per thread per tile and tensor
-  using L = Lds<D>;
-  constexpr int STAGE = kKeysPerTile * (L::KS + L::VS);  // elements per LDS stage
-  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  using T = Tile<D>;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
   // Workgroups are dealt to the 8 XCDs round-robin by linear id, and each XCD has its own
   // L2: all query tiles of one (batch, KV-head group) run on the same XCD, one after the
@@ -147,82 +166,95 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
 
-  // ---- global -> register staging of one K/V tile -------------------------------------
-  // A thread's chunks sit at fixed (key, column) positions of every tile: their offsets are
-  // computed once, and per tile only a wavefront-uniform base moves (modes 0 and 1).
-  u32x4 kst[CPT], vst[CPT];  // native vectors: struct-typed uint4 arrays end up in scratch memory
-  uint32_t chunk_off[CPT];   // element offset of chunk i inside a tile
-  uint32_t lds_k[CPT], lds_v[CPT];  // element offset of chunk i inside an LDS stage
-  int chunk_key[CPT], chunk_col[CPT];
+  // ---- global -> LDS tile loads ----------------------------------------------------------
+  // Load j of this wavefront fills LDS segment 4 j + wave of a tile: RPI whole rows.  Lane l
+  // writes chunk position l % CPR of row seg * RPI + l / CPR, so it fetches logical chunk
+  // (l % CPR) ^ swz(row).  The per-lane part of the source address is fixed for all tiles.
+  int ld_row[T::NI];       // row inside the tile
+  uint32_t ld_k[T::NI], ld_v[T::NI];  // byte offset of the lane's chunk inside a tile (modes 0 and 1)
 #pragma unroll
-  for (int i = 0; i < CPT; ++i) {
-    const int id = tid + 256 * i;
-    const int key = id / (D / 8), c = id - key * (D / 8);
-    chunk_key[i] = key;
-    chunk_col[i] = c;
-    chunk_off[i] = (uint32_t)(key * (MODE == 0 ? (int)a.kv_ts : D) + c * 8);
-    lds_k[i] = (uint32_t)(key * L::KS + c * 8);
-    lds_v[i] = (uint32_t)(kKeysPerTile * L::KS + key * L::VS + c * 8);
+  for (int j = 0; j < T::NI; ++j) {
+    const int r = (4 * j + wave) * T::RPI + lane / T::CPR;
+    const int cp = lane % T::CPR;
+    const uint32_t row_bytes = MODE == 0 ? 2u * (uint32_t)a.kv_ts : (uint32_t)T::RB;
+    ld_row[j] = r;
+    ld_k[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_k(r));
+    ld_v[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_v(r));
   }
-  // Loads are unconditional (a predicated load would make the compiler wait for the prefetch
-  // right after issuing it): keys past the end of a dense K/V are clamped to the last row,
-  // whose scores are masked and whose V rows therefore carry weight 0.
-  auto tile_base = [&](int kt) -> int64_t {  // uniform element offset of the tile
+  // Issues the loads of one tile of one tensor.  Keys past the end of K/V are clamped to the
+  // last row, whose scores are masked and whose V rows therefore carry weight 0.
+  auto issue = [&](const uint16_t *src, const uint32_t (&ld)[T::NI], bool is_v, int kt, int buf) {
     const int key0 = kt * kKeysPerTile;
+    const int last = a.skv - 1 - key0;  // last valid key of this tile, relative (>= 0)
+    const uint32_t lds_base = (uint32_t)(buf * T::STAGE_BYTES + (is_v ? T::TILE_BYTES : 0));
+    const char *base = nullptr;  // uniform address of the tile (modes 0 and 1)
     if constexpr (MODE == 0) {
-      return b * a.kv_bs + hk * a.kv_hs + (int64_t)key0 * a.kv_ts;
+      base = reinterpret_cast<const char *>(src + b * a.kv_bs + hk * a.kv_hs + (int64_t)key0 * a.kv_ts);
     } else if constexpr (MODE == 1) {
       int phys = __builtin_amdgcn_readfirstlane(a.pt[(int64_t)b * a.pt_rs + key0 / a.bs]);
       if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
-      return (((int64_t)phys * a.hkv + hk) * a.bs + (key0 % a.bs)) * D;
-    } else {
-      return 0;
+      base = reinterpret_cast<const char *>(src + (((int64_t)phys * a.hkv + hk) * a.bs + (key0 % a.bs)) * D);
     }
-  };
-  auto fetch = [&](const uint16_t *src, u32x4 (&dst)[CPT], int kt) {
-    const int key0 = kt * kKeysPerTile;
-    const int64_t base = tile_base(kt);
-    const int last = a.skv - 1 - key0;  // last valid key of this tile, relative (>= 0)
+    auto lds_dst = [&](int j) { return lds_base + (uint32_t)(4 * j + wave) * 1024u; };
+    if constexpr (MODE == 2) {
 #pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      if constexpr (MODE == 2) {
-        const int key = key0 + min(chunk_key[i], last);
-        dst[i] = *reinterpret_cast<const u32x4 *>(kv_chunk(a, src, b, hk, key, chunk_col[i], D));
-      } else if constexpr (MODE == 1) {  // table_width * block_size is a multiple of the tile
-        dst[i] = *reinterpret_cast<const u32x4 *>(src + base + chunk_off[i]);
-      } else {
-        const uint32_t off = (uint32_t)(min(chunk_key[i], last) * (int)a.kv_ts + chunk_col[i] * 8);
-        dst[i] = *reinterpret_cast<const u32x4 *>(src + base + off);
+      for (int j = 0; j < T::NI; ++j) {
+        const int key = key0 + min(ld_row[j], last);
+        const int col = key / a.bs;
+        int phys = a.pt[(int64_t)b * a.pt_rs + col];
+        if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+        const int c = (lane % T::CPR) ^ (is_v ? T::swz_v(ld_row[j]) : T::swz_k(ld_row[j]));
+        dma16_lane(src + (((int64_t)phys * a.hkv + hk) * a.bs + (key - col * a.bs)) * D + c * 8, lds_dst(j));
       }
+    } else if (MODE == 0 && last < kKeysPerTile - 1) {  // uniform: dense K/V ending inside the tile
+#pragma unroll
+      for (int j = 0; j < T::NI; ++j) {
+        const int c = (lane % T::CPR) ^ (is_v ? T::swz_v(ld_row[j]) : T::swz_k(ld_row[j]));
+        const uint32_t off = (uint32_t)min(ld_row[j], last) * 2u * (uint32_t)a.kv_ts + 16u * (uint32_t)c;
+        dma16(base, off, lds_dst(j));
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < T::NI; ++j) dma16(base, ld[j], lds_dst(j));
     }
   };
-  auto stage = [&](const u32x4 (&srcv)[CPT], const uint32_t (&off)[CPT], int buf) {
-    uint16_t *base = smem + buf * STAGE;
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) *reinterpret_cast<u32x4 *>(base + off[i]) = srcv[i];
+  auto wait_loads_and_sync = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's tile loads have landed
+    __syncthreads();
   };
 
-  // LDS operand addresses of this lane inside a stage
-  const uint32_t k_lane = (uint32_t)(n * L::KS + 8 * h);
+  // ---- LDS operand addresses of this lane inside a stage (bytes) ------------------------
+  uint32_t koff[KSTEPS];  // K fragment of k-step s, key block 0 (key block 1: + 32 rows)
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s)
+    koff[s] = (uint32_t)(n * T::RB + 16 * ((2 * s + h) ^ T::swz_k(n)));
+  // V^T fragment: through the transposing LDS load, per group of 16 lanes, lane i receives
+  // element i % 4 of the 8-byte chunks addressed by lanes 4 j + i / 4.  This lane addresses
+  // row 4 (grp / 2) + a16 / 4 (+ 16 per key step, + 8 for the second half), elements
+  // 32 db + 16 (grp % 2) + 4 (a16 % 4).
   const int grp = lane >> 4, a16 = lane & 15;
-  const uint32_t v_lane = (uint32_t)(kKeysPerTile * L::KS +
-                                     (4 * (grp >> 1) + (a16 >> 2)) * L::VS + 16 * (grp & 1) + 4 * (a16 & 3));
+  uint32_t voff[DBLK];
+  {
+    const int vr = 4 * (grp >> 1) + (a16 >> 2);
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db) {
+      const int c = 4 * db + 2 * (grp & 1) + ((a16 & 3) >> 1);
+      voff[db] = (uint32_t)(T::TILE_BYTES + vr * T::RB + 16 * (c ^ T::swz_v(vr)) + 8 * (a16 & 1));
+    }
+  }
   // K fragment i of a tile in issue order: k-step i / 2 of key block i % 2 (the two score
   // blocks alternate so consecutive matrix instructions are independent).
-  auto read_k = [&](const uint16_t *st_base, int i) -> bf16x8 {
+  auto read_k = [&](const unsigned char *st_base, int i) -> bf16x8 {
     const int s = i >> 1, kb = i & 1;
-    return __builtin_bit_cast(
-        bf16x8, *reinterpret_cast<const uint4 *>(st_base + k_lane + 32 * kb * L::KS + 16 * s));
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(st_base + koff[s] + 32 * kb * T::RB));
   };
-  // V^T fragment j in issue order: key step j / DBLK, output block j % DBLK.  Through the
-  // transposing LDS load, per group of 16 lanes, lane i receives element i % 4 of the 8-byte
-  // chunks addressed by lanes 4 j + i / 4.
-  auto read_v = [&](const uint16_t *st_base, int j) -> bf16x8 {
+  // V^T fragment j in issue order: key step j / DBLK, output block j % DBLK.
+  auto read_v = [&](const unsigned char *st_base, int j) -> bf16x8 {
     typedef __attribute__((address_space(3))) shortx4 *lds_v4;
     const int k4 = j / DBLK, db = j % DBLK;
-    const uint16_t *vk = st_base + v_lane + 16 * k4 * L::VS + 32 * db;
+    const unsigned char *vk = st_base + voff[db] + 16 * k4 * T::RB;
     shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk));
-    shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk + 8 * L::VS));
+    shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk + 8 * T::RB));
     bf16x4 l4 = __builtin_bit_cast(bf16x4, lo), h4 = __builtin_bit_cast(bf16x4, hi);
     bf16x8 t;
     t[0] = l4[0], t[1] = l4[1], t[2] = l4[2], t[3] = l4[3];
@@ -235,24 +267,16 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
   constexpr int KPRE = 6;         // K fragments in flight
   constexpr int VPRE = 4;         // V^T fragments in flight
 
-  // ntiles >= 1 always (row 0 sees key 0).  Past the last tile the prefetch repeats it into a
-  // stage nobody reads: straight-line code keeps staged tiles in registers and the wait
-  // counters exact.
+  // ntiles >= 1 always (row 0 sees key 0).
   const int last_tile = ntiles - 1;
-  fetch(a.k, kst, 0);
-  fetch(a.v, vst, 0);
-  stage(kst, lds_k, 0);
-  stage(vst, lds_v, 0);
-  fetch(a.k, kst, min(1, last_tile));
-  fetch(a.v, vst, min(1, last_tile));
-  __syncthreads();
+  issue(a.k, ld_k, false, 0, 0);
+  issue(a.v, ld_v, true, 0, 0);
+  if (last_tile >= 1) issue(a.k, ld_k, false, 1, 1);
+  wait_loads_and_sync();
   for (int kt = 0; kt < ntiles; ++kt) {
-    const uint16_t *cur = smem + (kt & 1) * STAGE;
+    const unsigned char *cur = smem + (kt & 1) * T::STAGE_BYTES;
     const int key0 = kt * kKeysPerTile;
     const bool compute = wave_active && key0 <= wave_last_key;  // wavefront-uniform
-
-    stage(kst, lds_k, (kt + 1) & 1);
-    fetch(a.k, kst, min(kt + 2, last_tile));
 
     // ---- S^T = K . Q^T -------------------------------------------------------------------
     floatx16 st[2];
@@ -275,9 +299,10 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
         if (i + KPRE < NK) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
     }
-    __syncthreads();  // K(kt+1) staged by everyone; everyone is done with V(kt-1)
-    stage(vst, lds_v, (kt + 1) & 1);
-    fetch(a.v, vst, min(kt + 2, last_tile));
+    // K(kt+1) and V(kt) have landed for everyone; everyone is done with K(kt) and V(kt-1)
+    wait_loads_and_sync();
+    if (kt + 2 <= last_tile) issue(a.k, ld_k, false, kt + 2, kt & 1);
+    if (kt + 1 <= last_tile) issue(a.v, ld_v, true, kt + 1, (kt + 1) & 1);
 
     if (compute) {
       bf16x8 vring[VPRE];
@@ -316,7 +341,6 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
         mloc = max3(mloc, st[0][r + 2], st[1][r + 2]);
       }
       {  // the other half of the key rows sits 32 lanes away: exchange through v_permlane32_swap
-        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
         const uint32_t mb = __builtin_bit_cast(uint32_t, mloc);
         const u32x2 sw = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
         mloc = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
@@ -342,7 +366,6 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
       // Probabilities as bf16 B-operand fragments: element e of key step k4 = 2 kb + s is
       // accumulator register 8 s + e of score block kb.  The row sum is taken over the rounded
       // values (two per v_dot2_f32_bf16), i.e. over exactly what the second product sees.
-      typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
       const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
       bf16x8 pf[4];
       float lsum = 0.f;
@@ -393,7 +416,7 @@ int launch_mode(const PrefillArgs &a, hipStream_t st) {
   constexpr int RPW = 4 / HPW;
   constexpr int ROWS = kRowsPerWave;
   const int nqt = (a.sq + ROWS * RPW - 1) / (ROWS * RPW);
-  const size_t lds = 2 * Lds<D>::BYTES;  // two stages
+  const size_t lds = 2 * Tile<D>::STAGE_BYTES;  // two stages
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(&prefill_kernel<D, HPW, MODE>),
