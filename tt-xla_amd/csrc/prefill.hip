@@ -273,6 +273,13 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
   issue(a.v, ld_v, true, 0, 0);
   if (last_tile >= 1) issue(a.k, ld_k, false, 1, 1);
   wait_loads_and_sync();
+  // The first K fragments of a tile are read one tile ahead (K(t+1) has landed at the barrier
+  // of tile t), so the score product starts without waiting for LDS.
+  bf16x8 ring[KPRE];
+  if (wave_active) {
+#pragma unroll
+    for (int i = 0; i < KPRE; ++i) ring[i] = read_k(smem, i);
+  }
   for (int kt = 0; kt < ntiles; ++kt) {
     const unsigned char *cur = smem + (kt & 1) * T::STAGE_BYTES;
     const int key0 = kt * kKeysPerTile;
@@ -281,9 +288,6 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
     // ---- S^T = K . Q^T -------------------------------------------------------------------
     floatx16 st[2];
     if (compute) {
-      bf16x8 ring[KPRE];
-#pragma unroll
-      for (int i = 0; i < KPRE; ++i) ring[i] = read_k(cur, i);
 #pragma unroll
       for (int r = 0; r < 16; ++r) st[0][r] = 0.f, st[1][r] = 0.f;
 #pragma unroll
@@ -291,8 +295,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
         st[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % KPRE], qf[i >> 1], st[i & 1], 0, 0, 0);
         if (i + KPRE < NK) ring[i % KPRE] = read_k(cur, i + KPRE);
       }
-      // pin the order: KPRE reads up front, then one read behind every matrix instruction
-      __builtin_amdgcn_sched_group_barrier(0x100, KPRE, 0);
+      // pin the order: one fragment read behind every matrix instruction
 #pragma unroll
       for (int i = 0; i < NK; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -388,6 +391,11 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
         acc[j % DBLK] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vring[j % VPRE], pf[j / DBLK],
                                                                 acc[j % DBLK], 0, 0, 0);
         if (j + VPRE < NV) vring[j % VPRE] = read_v(cur, j + VPRE);
+      }
+      if (kt + 1 < ntiles && key0 + kKeysPerTile <= wave_last_key) {  // this wavefront computes tile kt + 1
+        const unsigned char *nxt = smem + ((kt + 1) & 1) * T::STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < KPRE; ++i) ring[i] = read_k(nxt, i);
       }
     }
   }
