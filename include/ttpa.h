@@ -134,6 +134,31 @@ int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_t out_head_
                            size_t workspace_bytes, void *stream);
 
 /*
+ * The same decode attention with the two arguments of
+ * tt::paged_scaled_dot_product_attention_decode that the reference forwards to its device
+ * kernel and its CPU branch ignores (custom_ops.py:1207-1209, 1233-1247; the backend passes
+ * them at attention.py:646-656):
+ *   sliding_window > 0: only positions j > cur_pos[u] - sliding_window are attended
+ *                       (the newest `sliding_window` positions, the current one included);
+ *                       0 = no window.
+ *   attention_sink:     [q_heads] float32 logits on the device, or NULL.  Head hq's sink is
+ *                       one more entry of its softmax that contributes no value:
+ *                       denominator += exp(attention_sink[hq] - max).  It is in the units of
+ *                       the scaled scores (it is not multiplied by `scale`).
+ * With sliding_window = 0 and attention_sink = NULL this is ttpa_paged_sdpa_decode.
+ */
+int ttpa_paged_sdpa_decode_windowed(void *out, int64_t out_user_stride, int64_t out_head_stride,
+                                    const void *q, int64_t q_user_stride, int64_t q_head_stride,
+                                    const void *k_cache, const void *v_cache,
+                                    const int32_t *page_table, int64_t page_table_row_stride,
+                                    const void *cur_pos, int cur_pos_is_i64, int32_t users,
+                                    int32_t q_heads, int32_t kv_heads, int32_t head_size,
+                                    int32_t block_size, int32_t table_width, int32_t num_blocks,
+                                    float scale, int32_t kv_format, int32_t sliding_window,
+                                    const float *attention_sink, void *workspace,
+                                    size_t workspace_bytes, void *stream);
+
+/*
  * Measurement hook, no reference counterpart: the NEXT attention call made by this host
  * thread (decode or prefill) records `before` and `after` (hipEvent_t, as void*) on its
  * stream immediately around its dominant kernel (the split-K main kernel for decode, the
@@ -169,6 +194,26 @@ int ttpa_sdpa_prefill(void *out, int64_t out_batch_stride, int64_t out_head_stri
                       int32_t kv_len, int32_t head_size, int32_t block_size,
                       int32_t table_width, int32_t num_blocks, int32_t causal, float scale,
                       void *stream);
+
+/*
+ * The same prefill attention with the `sliding_window_size` argument of
+ * tt::scaled_dot_product_attention, which the reference forwards to its device kernel and
+ * its CPU branch ignores (custom_ops.py:645, 704-706; passed by the backend at
+ * attention.py:586-587).  sliding_window > 0 needs causal = 1: query row i then attends
+ * keys  chunk_start + i - sliding_window < j <= chunk_start + i  (the newest
+ * `sliding_window` keys, its own position included).  0 = no window = ttpa_sdpa_prefill.
+ */
+int ttpa_sdpa_prefill_windowed(void *out, int64_t out_batch_stride, int64_t out_head_stride,
+                               int64_t out_token_stride, const void *q, int64_t q_batch_stride,
+                               int64_t q_head_stride, int64_t q_token_stride, const void *k,
+                               const void *v, int64_t kv_batch_stride, int64_t kv_head_stride,
+                               int64_t kv_token_stride, const int32_t *page_table,
+                               int64_t page_table_row_stride, const int32_t *chunk_start,
+                               const void *mask, int64_t mask_batch_stride, int64_t mask_row_stride,
+                               int32_t batch, int32_t q_heads, int32_t kv_heads, int32_t q_len,
+                               int32_t kv_len, int32_t head_size, int32_t block_size,
+                               int32_t table_width, int32_t num_blocks, int32_t causal, float scale,
+                               int32_t sliding_window, void *stream);
 
 /*
  * Block-float-8 codec on flat arrays (n_elems % 16 == 0), for tests and cache

@@ -9,7 +9,9 @@ Modules
 -------
 paged_ops   torch restatement of the reference's CPU branches
             (python_package/tt_torch/custom_ops.py:635-742, 962-1104, 1198-1443,
-            GQA decode form :551-610).
+            GQA decode form :551-610), plus the sliding-window / attention-sink forms
+            that the reference's CPU branches ignore: semantics specified here,
+            PARITY UNPINNED against the reference.
 bfp8_codec  numpy block-float-8 quantise / dequantise.  The reference holds no
             CPU codec for this format (it lives in un-vendored tt-metal), so the
             codec is specified here and pinned by invariants: PARITY UNPINNED

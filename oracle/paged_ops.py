@@ -16,6 +16,16 @@ What pins each function (see tests/test_oracle_*.py):
   chunked_sdpa           the reference's independent oracle and cases restated
                          (tests/torch/ops/test_chunked_sdpa_op_cpu.py:27-147)
   sdpa                   library routine (F.scaled_dot_product_attention)
+  paged_sdpa_decode_windowed / sdpa_windowed
+                         PARITY UNPINNED against the reference: its CPU branches ignore
+                         `sliding_window_size` and `attention_sink`
+                         (custom_ops.py:1256-1312, 717-727) and the device kernels that
+                         honour them are not in the tree.  The semantics are specified
+                         here (window = newest W positions, current one included; sink =
+                         one value-less softmax entry per head) and pinned by mathematics:
+                         a window at least as long as the context changes nothing, a
+                         brute-force loop over the attended range, and the closed form
+                         out_sink = out * sigmoid(logsumexp(scores) - sink).
 """
 
 from __future__ import annotations
@@ -332,3 +342,64 @@ def textbook_decode_fp32(query, key, value, page_table, cur_pos, scale=None):
             p = torch.softmax(s, dim=0)
             out[0, u, h] = p @ v
     return out
+
+
+# --------------------------------------------------------------------------- #
+# sliding window and attention sink (semantics specified here, see module docstring)
+# --------------------------------------------------------------------------- #
+def paged_sdpa_decode_windowed(query, key, value, page_table, cur_pos, scale=None,
+                               sliding_window=None, attention_sink=None):
+    """Decode attention in fp32 over positions max(0, cur_pos - W + 1) .. cur_pos of each
+    user, with an optional per-head sink logit in the softmax denominator.
+
+    Argument meaning follows tt::paged_scaled_dot_product_attention_decode
+    (custom_ops.py:1198-1214): query [1, B, Hq, D], caches [NB, Hkv, bs, D], page_table
+    [B, W], cur_pos [B]; attention_sink [Hq] in the units of the scaled scores.
+    Returns fp32 [1, B, Hq, D]; rows with cur_pos < 0 are NaN.
+    """
+    _, users, hq, d = query.shape
+    hkv, bs = key.shape[1], key.shape[2]
+    g = hq // hkv
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    out = torch.full((1, users, hq, value.shape[-1]), float("nan"), dtype=torch.float32)
+    for u in range(users):
+        n = int(cur_pos[u]) + 1
+        if n <= 0:
+            continue
+        n = min(n, page_table.shape[1] * bs)
+        lo = max(0, n - int(sliding_window)) if sliding_window else 0
+        pos = torch.arange(lo, n)
+        blk = page_table[u, pos // bs].long()
+        off = pos % bs
+        for h in range(hq):
+            k = key[blk, h // g, off, :].float()
+            v = value[blk, h // g, off, :].float()
+            s = (k @ query[0, u, h].float()) * scale
+            if attention_sink is not None:
+                s = torch.cat([s, attention_sink[h].float().reshape(1)])
+                p = torch.softmax(s, dim=0)[:-1]
+            else:
+                p = torch.softmax(s, dim=0)
+            out[0, u, h] = p @ v
+    return out
+
+
+def sdpa_windowed(query, key, value, scale=None, sliding_window=None):
+    """Causal prefill attention in fp32 where query row i attends keys
+    max(0, i - W + 1) .. i.  Argument meaning follows tt::scaled_dot_product_attention
+    (custom_ops.py:635-646): query [B, Hq, S, D], key / value [B, Hkv, S, D]."""
+    b, hq, sq, d = query.shape
+    hkv, skv = key.shape[1], key.shape[2]
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    kk = key.float().repeat_interleave(hq // hkv, dim=1)
+    vv = value.float().repeat_interleave(hq // hkv, dim=1)
+    scores = query.float() @ kk.transpose(-1, -2) * scale
+    i = torch.arange(sq).view(sq, 1)
+    j = torch.arange(skv).view(1, skv)
+    banned = j > i
+    if sliding_window:
+        banned = banned | (j < i - int(sliding_window) + 1)
+    scores = scores.masked_fill(banned, float("-inf"))
+    return torch.softmax(scores, dim=-1) @ vv

@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   const uint32_t lane_bytes = (uint32_t)(r * D + c * EPL) * 2u;
 
   // ---- helpers (all uniform across the wavefront) ---------------------------------
-  auto locate = [&](int64_t xx) { return locate_unit(s_pref, s_len, a.users, a.hkv, xx); };
+  auto locate = [&](int64_t xx) { return locate_unit(a, s_pref, s_len, xx); };
   // element offset (relative to the cache base) of the first row of each 4-row load
   auto tile_offsets = [&](const Cursor &cu, int64_t (&off)[NOFF]) {
     const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
@@ -179,7 +179,9 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- online softmax, one stream per lane row ---------------------------------------
-    const bool valid = 4 * my_step + r < nvalid;
+    // positions below the sliding window's lower edge can only occur in a segment's first tile
+    const int nbelow = cur.lo - cur.t * kTile;
+    const bool valid = 4 * my_step + r < nvalid && 4 * my_step + r >= nbelow;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       float sv = valid ? s[g] * a.scale_log2e : -INFINITY;
@@ -337,15 +339,15 @@ extern "C" size_t ttpa_paged_decode_workspace_bytes(int32_t users, int32_t q_hea
   return header_bytes(users, kv_heads) + slots * (size_t)slot_floats_for(g, head_size) * sizeof(float);
 }
 
-extern "C" int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_t out_head_stride,
-                                      const void *q, int64_t q_user_stride, int64_t q_head_stride,
-                                      const void *k_cache, const void *v_cache,
-                                      const int32_t *page_table, int64_t page_table_row_stride,
-                                      const void *cur_pos, int cur_pos_is_i64, int32_t users,
-                                      int32_t q_heads, int32_t kv_heads, int32_t head_size,
-                                      int32_t block_size, int32_t table_width, int32_t num_blocks,
-                                      float scale, int32_t kv_format, void *workspace,
-                                      size_t workspace_bytes, void *stream) {
+static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stride, const void *q,
+                       int64_t q_user_stride, int64_t q_head_stride, const void *k_cache,
+                       const void *v_cache, const int32_t *page_table,
+                       int64_t page_table_row_stride, const void *cur_pos, int cur_pos_is_i64,
+                       int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
+                       int32_t block_size, int32_t table_width, int32_t num_blocks, float scale,
+                       int32_t kv_format, int32_t sliding_window, const float *attention_sink,
+                       void *workspace, size_t workspace_bytes, void *stream) {
+  TTPA_REQUIRE(sliding_window >= 0, "decode: sliding_window %d is negative", sliding_window);
   TTPA_REQUIRE(out && q && k_cache && v_cache && page_table && cur_pos, "null pointer argument");
   TTPA_REQUIRE(users > 0 && q_heads > 0 && kv_heads > 0 && head_size > 0 && block_size > 0 &&
                    table_width > 0 && num_blocks > 0,
@@ -390,6 +392,8 @@ extern "C" int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_
   a.n_waves = waves_for_device(kv_format);
   a.slot_floats = slot_floats_for(g, head_size);
   a.kv_format = kv_format;
+  a.window = sliding_window;
+  a.sink = attention_sink;
 
   hipStream_t st = static_cast<hipStream_t>(stream);
   // Kernel choice: the VALU kernel streams at the HBM ceiling up to 4 query heads per KV head;
@@ -424,4 +428,33 @@ extern "C" int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_
   if (rc) return rc;
   decode_combine_kernel<<<dim3(users * kv_heads), dim3(256), 0, st>>>(a, g, head_size);
   return check_launch("paged_sdpa_decode");
+}
+
+extern "C" int ttpa_paged_sdpa_decode(void *out, int64_t out_user_stride, int64_t out_head_stride,
+                                      const void *q, int64_t q_user_stride, int64_t q_head_stride,
+                                      const void *k_cache, const void *v_cache,
+                                      const int32_t *page_table, int64_t page_table_row_stride,
+                                      const void *cur_pos, int cur_pos_is_i64, int32_t users,
+                                      int32_t q_heads, int32_t kv_heads, int32_t head_size,
+                                      int32_t block_size, int32_t table_width, int32_t num_blocks,
+                                      float scale, int32_t kv_format, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
+  return decode_impl(out, out_user_stride, out_head_stride, q, q_user_stride, q_head_stride, k_cache,
+                     v_cache, page_table, page_table_row_stride, cur_pos, cur_pos_is_i64, users,
+                     q_heads, kv_heads, head_size, block_size, table_width, num_blocks, scale,
+                     kv_format, 0, nullptr, workspace, workspace_bytes, stream);
+}
+
+extern "C" int ttpa_paged_sdpa_decode_windowed(
+    void *out, int64_t out_user_stride, int64_t out_head_stride, const void *q,
+    int64_t q_user_stride, int64_t q_head_stride, const void *k_cache, const void *v_cache,
+    const int32_t *page_table, int64_t page_table_row_stride, const void *cur_pos,
+    int cur_pos_is_i64, int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
+    int32_t block_size, int32_t table_width, int32_t num_blocks, float scale, int32_t kv_format,
+    int32_t sliding_window, const float *attention_sink, void *workspace, size_t workspace_bytes,
+    void *stream) {
+  return decode_impl(out, out_user_stride, out_head_stride, q, q_user_stride, q_head_stride, k_cache,
+                     v_cache, page_table, page_table_row_stride, cur_pos, cur_pos_is_i64, users,
+                     q_heads, kv_heads, head_size, block_size, table_width, num_blocks, scale,
+                     kv_format, sliding_window, attention_sink, workspace, workspace_bytes, stream);
 }

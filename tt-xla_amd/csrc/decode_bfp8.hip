@@ -74,7 +74,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_kernel(
   const uint32_t lane_exp = (uint32_t)(r * GPR + grp);
   const int64_t slab_bytes = (int64_t)(a.bs + a.bs / 16) * D;  // one (block, head) slab
 
-  auto locate = [&](int64_t xx) { return locate_unit(s_pref, s_len, a.users, a.hkv, xx); };
+  auto locate = [&](int64_t xx) { return locate_unit(a, s_pref, s_len, xx); };
   // byte offsets of the element rows / exponent rows of each 4-row load of a tile
   auto tile_offsets = [&](const Cursor &cu, int64_t (&eo)[NOFF], int64_t (&xo)[NOFF]) {
     const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
@@ -200,7 +200,8 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_kernel(
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- online softmax, one stream per lane row ------------------------------------------
-    const bool valid = 4 * my_step + r < nvalid;
+    const int nbelow = cur.lo - cur.t * kTile;  // sliding window: only in a segment's first tile
+    const bool valid = 4 * my_step + r < nvalid && 4 * my_step + r >= nbelow;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       float sv = valid ? s[g] * a.scale_log2e : -INFINITY;

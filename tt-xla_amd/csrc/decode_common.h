@@ -31,15 +31,24 @@ struct DecodeArgs {
   int n_waves;
   int slot_floats;
   int kv_format;
+  int window;         // > 0: only the last `window` positions up to cur_pos are attended
+  const float *sink;  // [q_heads] extra logit per head in the softmax denominator, or null
 };
 
+// First attended position of a user whose attended range ends at `len` (exclusive).
+__device__ __forceinline__ int window_lo(const DecodeArgs &a, int len) {
+  return (a.window > 0 && len > a.window) ? len - a.window : 0;
+}
+
+// Attended positions of user u are [window_lo(len), len); returns the number of 64-token tiles
+// they touch.
 __device__ __forceinline__ int tiles_of_user(const DecodeArgs &a, const void *__restrict__ cur,
                                              int u, int &len) {
   int64_t cp = load_index(cur, a.cur_i64, u);
   int64_t cap = (int64_t)a.w * a.bs;
   int64_t l = cp < 0 ? 0 : (cp + 1 < cap ? cp + 1 : cap);
   len = (int)l;
-  return (int)((l + kTile - 1) / kTile);
+  return (int)((l + kTile - 1) / kTile) - window_lo(a, len) / kTile;
 }
 
 // Exclusive prefix sum of per-user tile counts into pref[0..users] and attended lengths into
@@ -184,15 +193,16 @@ struct Shape {
 
 // Position of a wavefront in the flat tile list.
 struct Cursor {
-  int u, h, t;      // user, kv head, tile index inside the segment
-  int len;          // attended positions of user u
+  int u, h, t;      // user, kv head, absolute tile index (tile t covers positions 64 t ..)
+  int len, lo;      // user u attends positions [lo, len)
   int tiles_left;   // tiles of this segment from t on (including t)
 };
 
 // Finds the segment that owns unit `x` of the flat tile list (binary search over the
 // per-user prefix in LDS).  Everything is wavefront-uniform.
-__device__ __forceinline__ Cursor locate_unit(const int *s_pref, const int *s_len, int users,
-                                              int hkv, int64_t x) {
+__device__ __forceinline__ Cursor locate_unit(const DecodeArgs &a, const int *s_pref,
+                                              const int *s_len, int64_t x) {
+  const int users = a.users, hkv = a.hkv;
   int lo_u = 0, hi_u = users - 1;
   while (lo_u < hi_u) {
     int mid = (lo_u + hi_u + 1) >> 1;
@@ -205,9 +215,11 @@ __device__ __forceinline__ Cursor locate_unit(const int *s_pref, const int *s_le
   const int nt = __builtin_amdgcn_readfirstlane(s_pref[lo_u + 1]) - pref_u;
   const int rem = (int)(x - (int64_t)pref_u * hkv);
   cu.h = rem / nt;
-  cu.t = rem - cu.h * nt;
-  cu.tiles_left = nt - cu.t;
+  const int rel = rem - cu.h * nt;
+  cu.tiles_left = nt - rel;
   cu.len = __builtin_amdgcn_readfirstlane(s_len[lo_u]);
+  cu.lo = window_lo(a, cu.len);
+  cu.t = cu.lo / kTile + rel;
   return cu;
 }
 
@@ -309,6 +321,13 @@ __global__ inline __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a
         den = fmaf(wgt, lv[j], den);
       }
       mall = mnew;
+    }
+    if (a.sink) {  // the sink logit (natural-log units, not scaled) only enlarges the normaliser
+      const float sk = a.sink[h * G + g] * 1.4426950408889634f;
+      const float mnew = fmaxf(mall, sk);
+      const float resc = __builtin_amdgcn_exp2f(mall - mnew);
+      num *= resc;
+      den = den * resc + __builtin_amdgcn_exp2f(sk - mnew);
     }
     out[(int64_t)(h * G + g) * a.out_hs + (i % D)] = (uint16_t)f32_to_bf16_bits(num / den);
   }

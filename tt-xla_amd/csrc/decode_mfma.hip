@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
   const uint32_t lane_exp = (uint32_t)(sr * GPR + sc);  // block-float-8: one group per lane
   const int64_t slab = BFP8 ? (int64_t)(a.bs + a.bs / 16) * D : (int64_t)a.bs * D * 2;  // bytes
 
-  auto locate = [&](int64_t xx) { return locate_unit(s_pref, s_len, a.users, a.hkv, xx); };
+  auto locate = [&](int64_t xx) { return locate_unit(a, s_pref, s_len, xx); };
   auto tile_offsets = [&](const Cursor &cu, int64_t (&eo)[NOFF], int64_t (&xo)[NOFF]) {
     const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
     const int tok0 = cu.t * kTile;
@@ -180,6 +180,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
     constexpr bool has_next = decltype(has_next_tag)::value;
     const int nvalid = cur.len - cur.t * kTile;
     const bool partial = nvalid < kTile;
+    const int nbelow = cur.lo - cur.t * kTile;  // sliding window: > 0 only in a segment's first tile
     // ---- this tile: registers -> LDS; next tile: global -> registers ----------------------
     const bool same_seg = has_next && cur.tiles_left > 1;
     Cursor nxt = cur;
@@ -227,13 +228,13 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
       }
     }
     // ---- online softmax, one head per lane --------------------------------------------------
-    if (partial) {
+    if (partial || nbelow > 0) {
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = 32 * kb + 8 * (r >> 2) + 4 * h + (r & 3);
-          if (key >= nvalid) st[kb][r] = -INFINITY;
+          if (key >= nvalid || key < nbelow) st[kb][r] = -INFINITY;
         }
     }
     float mloc = fmaxf(st[0][0], st[1][0]);

@@ -53,6 +53,7 @@ struct PrefillArgs {
   const uint16_t *mask;
   int64_t mask_bs, mask_rs;
   int batch, hq, hkv, sq, skv, bs, w, nb, causal;
+  int window;  // > 0 (causal only): row i attends keys offset + i - window < j <= offset + i
   float scale_log2e;
 };
 
@@ -148,6 +149,10 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
   const int ntiles = (kv_end_wg + kKeysPerTile - 1) / kKeysPerTile;
   const int wave_last_key = a.causal ? offset + min(a.sq - 1, row0 + ROWS - 1) : a.skv - 1;
   const bool wave_active = row0 < a.sq;
+  // sliding window: first key any row of the workgroup / of this wavefront can see
+  const int wg_first_key = a.window > 0 ? max(0, offset + qt * ROWS * RPW - a.window + 1) : 0;
+  const int wave_first_key = a.window > 0 ? max(0, offset + row0 - a.window + 1) : 0;
+  const int first_tile = wg_first_key / kKeysPerTile;
 
   // ---- Q fragments (B operand: lane n = query row, 8 head-dim elements per k-step) -----
   bf16x8 qf[KSTEPS];
@@ -269,21 +274,22 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
 
   // ntiles >= 1 always (row 0 sees key 0).
   const int last_tile = ntiles - 1;
-  issue(a.k, ld_k, false, 0, 0);
-  issue(a.v, ld_v, true, 0, 0);
-  if (last_tile >= 1) issue(a.k, ld_k, false, 1, 1);
+  issue(a.k, ld_k, false, first_tile, first_tile & 1);
+  issue(a.v, ld_v, true, first_tile, first_tile & 1);
+  if (last_tile >= first_tile + 1) issue(a.k, ld_k, false, first_tile + 1, (first_tile + 1) & 1);
   wait_loads_and_sync();
   // The first K fragments of a tile are read one tile ahead (K(t+1) has landed at the barrier
   // of tile t), so the score product starts without waiting for LDS.
   bf16x8 ring[KPRE];
   if (wave_active) {
 #pragma unroll
-    for (int i = 0; i < KPRE; ++i) ring[i] = read_k(smem, i);
+    for (int i = 0; i < KPRE; ++i) ring[i] = read_k(smem + (first_tile & 1) * T::STAGE_BYTES, i);
   }
-  for (int kt = 0; kt < ntiles; ++kt) {
+  for (int kt = first_tile; kt < ntiles; ++kt) {
     const unsigned char *cur = smem + (kt & 1) * T::STAGE_BYTES;
     const int key0 = kt * kKeysPerTile;
-    const bool compute = wave_active && key0 <= wave_last_key;  // wavefront-uniform
+    // wavefront-uniform; with a window, tiles wholly below this wavefront's rows are skipped
+    const bool compute = wave_active && key0 <= wave_last_key && key0 + kKeysPerTile > wave_first_key;
 
     // ---- S^T = K . Q^T -------------------------------------------------------------------
     floatx16 st[2];
@@ -317,9 +323,11 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
       // the scale is folded into the exponent: p = exp2(s * c - m * c).
       const int qrow = row0 + n;
       const bool need_mask = (a.causal && key0 + kKeysPerTile - 1 > offset + row0) ||
-                             key0 + kKeysPerTile > a.skv || a.mask != nullptr;
-      if (need_mask) {  // wavefront-uniform: only diagonal / ragged / explicitly masked tiles
+                             key0 + kKeysPerTile > a.skv || a.mask != nullptr ||
+                             (a.window > 0 && key0 <= offset + row0 + ROWS - 1 - a.window);
+      if (need_mask) {  // wavefront-uniform: only diagonal / ragged / window-edge / explicitly masked tiles
         const int limit = a.causal ? min(offset + qrow, a.skv - 1) : a.skv - 1;
+        const int lowest = a.window > 0 ? offset + qrow - a.window + 1 : 0;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -332,7 +340,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
               v += bf16_lo(a.mask[b * a.mask_bs + (int64_t)qc * a.mask_rs + kc]) *
                    (1.4426950408889634f / a.scale_log2e);
             }
-            st[kb][r] = key > limit ? -INFINITY : v;
+            st[kb][r] = (key > limit || key < lowest) ? -INFINITY : v;
           }
       }
       // The first maximum is an ordinary compiler-visible read of both score blocks.
@@ -343,10 +351,13 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
         mloc = max3(mloc, st[0][r + 1], st[1][r + 1]);
         mloc = max3(mloc, st[0][r + 2], st[1][r + 2]);
       }
-      {  // the other half of the key rows sits 32 lanes away: exchange through v_permlane32_swap
-        const uint32_t mb = __builtin_bit_cast(uint32_t, mloc);
-        const u32x2 sw = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
-        mloc = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+      {  // The other half of the key rows sits 32 lanes away.  v_permlane32_swap exchanges the
+         // upper 32 lanes of its first operand with the lower 32 of its second; with two copies
+         // of the value each lane ends up holding its own and its partner's.  Written as
+         // assembly: through the builtin the compiler folds the two results into one.
+        float ma = mloc, mb = mloc;
+        asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(ma), "+v"(mb));
+        mloc = max3(ma, mb, mb);
       }
       // Lazy rescaling: the running maximum only moves when a row's new maximum exceeds it
       // by more than 2^8 in the exponent domain.  Until then probabilities are taken
@@ -392,11 +403,12 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
                                                                 acc[j % DBLK], 0, 0, 0);
         if (j + VPRE < NV) vring[j % VPRE] = read_v(cur, j + VPRE);
       }
-      if (kt + 1 < ntiles && key0 + kKeysPerTile <= wave_last_key) {  // this wavefront computes tile kt + 1
-        const unsigned char *nxt = smem + ((kt + 1) & 1) * T::STAGE_BYTES;
+    }
+    if (wave_active && kt + 1 < ntiles && key0 + kKeysPerTile <= wave_last_key &&
+        key0 + 2 * kKeysPerTile > wave_first_key) {  // this wavefront computes tile kt + 1
+      const unsigned char *nxt = smem + ((kt + 1) & 1) * T::STAGE_BYTES;
 #pragma unroll
-        for (int i = 0; i < KPRE; ++i) ring[i] = read_k(nxt, i);
-      }
+      for (int i = 0; i < KPRE; ++i) ring[i] = read_k(nxt, i);
     }
   }
 
@@ -461,7 +473,7 @@ int launch_d(const PrefillArgs &a, hipStream_t st) {
 
 using namespace ttpa;
 
-extern "C" int ttpa_sdpa_prefill(void *out, int64_t out_batch_stride, int64_t out_head_stride,
+static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_stride,
                                  int64_t out_token_stride, const void *q, int64_t q_batch_stride,
                                  int64_t q_head_stride, int64_t q_token_stride, const void *k,
                                  const void *v, int64_t kv_batch_stride, int64_t kv_head_stride,
@@ -471,8 +483,10 @@ extern "C" int ttpa_sdpa_prefill(void *out, int64_t out_batch_stride, int64_t ou
                                  int64_t mask_row_stride, int32_t batch, int32_t q_heads,
                                  int32_t kv_heads, int32_t q_len, int32_t kv_len, int32_t head_size,
                                  int32_t block_size, int32_t table_width, int32_t num_blocks,
-                                 int32_t causal, float scale, void *stream) {
+                                 int32_t causal, float scale, int32_t sliding_window, void *stream) {
   TTPA_REQUIRE(out && q && k && v, "null pointer argument");
+  TTPA_REQUIRE(sliding_window >= 0, "prefill: sliding_window %d is negative", sliding_window);
+  TTPA_REQUIRE(sliding_window == 0 || causal, "prefill: a sliding window needs causal masking");
   TTPA_REQUIRE(batch > 0 && q_heads > 0 && kv_heads > 0 && q_len > 0 && head_size > 0,
                "non-positive dimension");
   TTPA_REQUIRE(q_heads % kv_heads == 0, "q_heads %d not divisible by kv_heads %d", q_heads,
@@ -512,6 +526,7 @@ extern "C" int ttpa_sdpa_prefill(void *out, int64_t out_batch_stride, int64_t ou
   a.mask_bs = mask_batch_stride, a.mask_rs = mask_row_stride;
   a.batch = batch, a.hq = q_heads, a.hkv = kv_heads, a.sq = q_len, a.skv = kv_len;
   a.bs = block_size, a.w = table_width, a.nb = num_blocks, a.causal = causal ? 1 : 0;
+  a.window = sliding_window;
   a.scale_log2e = scale * 1.4426950408889634f;
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (head_size) {
@@ -519,4 +534,28 @@ extern "C" int ttpa_sdpa_prefill(void *out, int64_t out_batch_stride, int64_t ou
     case 128: return launch_d<128>(a, st);
     default: return launch_d<256>(a, st);
   }
+}
+
+#define TTPA_PREFILL_PARAMS                                                                        \
+  void *out, int64_t out_batch_stride, int64_t out_head_stride, int64_t out_token_stride,          \
+      const void *q, int64_t q_batch_stride, int64_t q_head_stride, int64_t q_token_stride,        \
+      const void *k, const void *v, int64_t kv_batch_stride, int64_t kv_head_stride,               \
+      int64_t kv_token_stride, const int32_t *page_table, int64_t page_table_row_stride,           \
+      const int32_t *chunk_start, const void *mask, int64_t mask_batch_stride,                     \
+      int64_t mask_row_stride, int32_t batch, int32_t q_heads, int32_t kv_heads, int32_t q_len,    \
+      int32_t kv_len, int32_t head_size, int32_t block_size, int32_t table_width,                  \
+      int32_t num_blocks, int32_t causal, float scale
+#define TTPA_PREFILL_ARGS                                                                          \
+  out, out_batch_stride, out_head_stride, out_token_stride, q, q_batch_stride, q_head_stride,      \
+      q_token_stride, k, v, kv_batch_stride, kv_head_stride, kv_token_stride, page_table,          \
+      page_table_row_stride, chunk_start, mask, mask_batch_stride, mask_row_stride, batch,         \
+      q_heads, kv_heads, q_len, kv_len, head_size, block_size, table_width, num_blocks, causal,    \
+      scale
+
+extern "C" int ttpa_sdpa_prefill(TTPA_PREFILL_PARAMS, void *stream) {
+  return prefill_impl(TTPA_PREFILL_ARGS, 0, stream);
+}
+
+extern "C" int ttpa_sdpa_prefill_windowed(TTPA_PREFILL_PARAMS, int32_t sliding_window, void *stream) {
+  return prefill_impl(TTPA_PREFILL_ARGS, sliding_window, stream);
 }

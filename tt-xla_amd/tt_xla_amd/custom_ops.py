@@ -289,8 +289,8 @@ def paged_scaled_dot_product_attention_decode(
             "paged decode with an explicit attn_mask is not built; the serving path always "
             "issues the causal form"
         )
-    if attention_sink is not None or sliding_window_size is not None:
-        raise NotImplementedError("attention_sink / sliding_window_size are not built")
+    if sliding_window_size is not None and sliding_window_size <= 0:
+        raise ValueError("sliding_window_size must be positive")
     if query.dim() != 4 or query.shape[0] != 1:
         raise ValueError("query must be [1, users, heads, head_size]")
     nb, hkv, bs, d, fmt = _cache_geometry(key)
@@ -311,11 +311,17 @@ def paged_scaled_dot_product_attention_decode(
     out = torch.empty((1, users, hq, d), dtype=query.dtype, device=query.device)
     ws_bytes = N.lib().ttpa_paged_decode_workspace_bytes(users, hq, hkv, d)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=query.device)
+    sink = None
+    if attention_sink is not None:
+        if attention_sink.numel() != hq:
+            raise ValueError(f"attention_sink must hold one logit per query head ({hq})")
+        sink = attention_sink.reshape(hq).to(device=query.device, dtype=torch.float32).contiguous()
     N.call(
-        "ttpa_paged_sdpa_decode",
+        "ttpa_paged_sdpa_decode_windowed",
         out.data_ptr(), out.stride(1), out.stride(2), q.data_ptr(), q.stride(1), q.stride(2),
         key.data_ptr(), value.data_ptr(), pt.data_ptr(), pt.stride(0), cur.data_ptr(),
         int(cur.dtype == torch.int64), users, hq, hkv, d, bs, pt.shape[1], nb, float(scale), fmt,
+        int(sliding_window_size or 0), sink.data_ptr() if sink is not None else None,
         ws.data_ptr(), ws_bytes, _stream(),
     )
     return out
@@ -330,7 +336,7 @@ def _(query, key, value, page_table, is_causal=False, attn_mask=None, cur_pos_te
 # --------------------------------------------------------------------------- #
 # prefill attention
 # --------------------------------------------------------------------------- #
-def _prefill(query, key, value, page_table, chunk_start, attn_mask, is_causal, scale):
+def _prefill(query, key, value, page_table, chunk_start, attn_mask, is_causal, scale, window=0):
     b, hq, s, d = query.shape
     if query.dtype != torch.bfloat16:
         raise ValueError("query must be bfloat16")
@@ -368,12 +374,12 @@ def _prefill(query, key, value, page_table, chunk_start, attn_mask, is_causal, s
             m = m.contiguous()
         mask_ptr, mask_bs, mask_rs = m.data_ptr(), m.stride(0), m.stride(2)
     N.call(
-        "ttpa_sdpa_prefill",
+        "ttpa_sdpa_prefill_windowed",
         out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
         q.data_ptr(), q.stride(0), q.stride(1), q.stride(2),
         k.data_ptr(), v.data_ptr(), *kv_strides, pt_ptr, pt_rs, _ptr(chunk_start),
         mask_ptr, mask_bs, mask_rs, b, hq, hkv, s, skv, d, bs, w, nb, int(is_causal),
-        float(scale), _stream(),
+        float(scale), int(window), _stream(),
     )
     return out
 
@@ -404,8 +410,12 @@ def scaled_dot_product_attention(
         assert is_causal == False, "is_causal attribute can't be True if attn_mask is available."  # noqa: E712
         assert query.shape[0] == attn_mask.shape[0], "Attention mask batch size must match query batch size."
     if sliding_window_size is not None:
-        raise NotImplementedError("sliding_window_size is not built")
-    return _prefill(query, key, value, None, None, attn_mask, is_causal, scale)
+        if sliding_window_size <= 0:
+            raise ValueError("sliding_window_size must be positive")
+        if not is_causal:
+            raise NotImplementedError("sliding_window_size is built for the causal form only")
+    return _prefill(query, key, value, None, None, attn_mask, is_causal, scale,
+                    window=sliding_window_size or 0)
 
 
 @scaled_dot_product_attention.register_fake
