@@ -16,6 +16,11 @@ What pins each function (see tests/test_oracle_*.py):
   chunked_sdpa           the reference's independent oracle and cases restated
                          (tests/torch/ops/test_chunked_sdpa_op_cpu.py:27-147)
   sdpa                   library routine (F.scaled_dot_product_attention)
+  update_cache / fill_cache / sdpa_decode_static
+                         the non-paged forms (custom_ops.py:745-950): plain slice
+                         assignments, checked element by element, and the library SDPA
+                         with the reference's own additive mask, checked against the fp32
+                         loop and against the paged oracle on an identity page table
   paged_sdpa_decode_windowed / sdpa_windowed
                          PARITY UNPINNED against the reference: its CPU branches ignore
                          `sliding_window_size` and `attention_sink`
@@ -403,3 +408,37 @@ def sdpa_windowed(query, key, value, scale=None, sliding_window=None):
         banned = banned | (j < i - int(sliding_window) + 1)
     scores = scores.masked_fill(banned, float("-inf"))
     return torch.softmax(scores, dim=-1) @ vv
+
+
+# --------------------------------------------------------------------------- #
+# non-paged (static) caches [B, H, max_seq_len, D]
+# --------------------------------------------------------------------------- #
+def update_cache(cache, fill_value, cache_position, batch_offset=None):
+    """custom_ops.py:857-891: one token, one position shared by the whole batch."""
+    assert fill_value.shape[-2] == 1 and cache_position.shape == (1,)
+    assert not batch_offset
+    out = cache.clone()
+    out[:, :, cache_position, :] = fill_value
+    return out
+
+
+def fill_cache(cache, fill_value, batch_offset=None):
+    """custom_ops.py:903-940: the first seq_len positions of every (batch, head)."""
+    assert fill_value.shape[-2] <= cache.shape[-2]
+    assert not batch_offset
+    out = cache.clone()
+    out[:, :, : fill_value.shape[-2], :] = fill_value
+    return out
+
+
+def sdpa_decode_static(query, key, value, cur_pos_tensor, scale=None):
+    """custom_ops.py:817-842 with attn_mask=None: additive mask of -inf to the right of each
+    user's position, then the library SDPA with grouped heads, in the query's dtype."""
+    batch, heads, d = query.shape[1], query.shape[2], query.shape[3]
+    max_seq = key.shape[-2]
+    q = query.reshape(batch, heads, 1, d)
+    mask = torch.zeros(batch, heads, 1, max_seq, dtype=q.dtype)
+    for b in range(batch):
+        mask[b, ..., int(cur_pos_tensor[b]) + 1 :] = float("-inf")
+    out = F.scaled_dot_product_attention(q, key, value, mask, is_causal=False, scale=scale, enable_gqa=True)
+    return out.reshape(1, batch, heads, d)

@@ -2,7 +2,7 @@
 
 Names, argument order and defaults are those of tt-xla's
 ``python_package/tt_torch/custom_ops.py`` (:635-646, :962-971, :1016-1024,
-:1198-1214, :1334-1346); the implementation of each is a launch of a gfx950 kernel
+:1198-1214, :1334-1346, and the static-cache forms :745-759, :857-867, :903-906); the implementation of each is a launch of a gfx950 kernel
 through the C ABI in ``include/ttpa.h``.  As in the reference the five operators are
 functional (``mutates_args=[]``): the cache writers return a fresh tensor.  Because a
 functional write copies the whole cache, in-place twins ``tt::paged_update_cache_`` and
@@ -446,6 +446,156 @@ def chunked_scaled_dot_product_attention(
 
 @chunked_scaled_dot_product_attention.register_fake
 def _(query, key, value, page_table, chunk_start_idx_tensor, scale=None):
+    return torch.empty_like(query)
+
+
+# --------------------------------------------------------------------------- #
+# non-paged (static) cache: [batch, kv_heads, max_seq_len, head_size]
+# --------------------------------------------------------------------------- #
+# A static cache is a paged cache whose block u is the whole sequence of user u: the same
+# kernels run with block_size = max_seq_len and the one-column page table [[0], [1], ...].
+def _identity_table(batch: int, device) -> torch.Tensor:
+    return torch.arange(batch, dtype=torch.int32, device=device).view(batch, 1)
+
+
+def _static_geometry(cache: torch.Tensor):
+    if cache.dim() != 4:
+        raise ValueError("cache must be a 4D tensor: [B, num_heads, max_seq_len, head_size].")
+    if cache.dtype not in (torch.bfloat16, torch.float16) or not cache.is_contiguous():
+        raise ValueError("static caches must be contiguous 16-bit floating point tensors")
+    return cache.shape
+
+
+def _static_update_inplace(cache, fill_value, cache_position, batch_offset):
+    assert len(cache.shape) == 4, "cache must be a 4D tensor: [B, num_heads, max_seq_len, head_size]."
+    assert len(fill_value.shape) == 4, "fill_value must be a 4D tensor: [B, num_heads, 1, head_size]."
+    assert fill_value.shape[-2] == 1, (
+        "fill_value must have dim -2 equal to 1 as the cache cannot be updated with more than one "
+        "token at a time."
+    )
+    assert batch_offset is not None or cache.shape[0] == 1, "batch_offset must be provided if the batch size is not 1."
+    assert cache_position.shape == (1,), "cache_position must be a 1D tensor."
+    assert not batch_offset, "Only batch_offset == 0 is supported for currently."
+    b = _static_geometry(cache)[0]
+    if fill_value.shape[0] != b:
+        raise ValueError("fill_value and cache must have the same batch size")
+    _update_inplace(cache, fill_value.permute(2, 0, 1, 3), cache_position.expand(b), _identity_table(b, cache.device))
+
+
+@torch.library.custom_op("tt::update_cache", mutates_args=[], device_types=["cuda"])
+def update_cache(
+    cache: torch.Tensor,
+    fill_value: torch.Tensor,
+    cache_position: torch.Tensor,
+    batch_offset: Optional[int] = None,
+) -> torch.Tensor:
+    """cache[:, :, cache_position, :] = fill_value on a copy (reference custom_ops.py:857-900);
+    one position shared by the whole batch.  Positions outside [0, max_seq_len) write nothing."""
+    out = cache.clone()
+    _static_update_inplace(out, fill_value, cache_position, batch_offset)
+    return out
+
+
+@update_cache.register_fake
+def _(cache, fill_value, cache_position, batch_offset=None):
+    return torch.empty_like(cache)
+
+
+@torch.library.custom_op("tt::update_cache_", mutates_args=["cache"], device_types=["cuda"])
+def update_cache_(
+    cache: torch.Tensor,
+    fill_value: torch.Tensor,
+    cache_position: torch.Tensor,
+    batch_offset: Optional[int] = None,
+) -> None:
+    _static_update_inplace(cache, fill_value, cache_position, batch_offset)
+
+
+@update_cache_.register_fake
+def _(cache, fill_value, cache_position, batch_offset=None):
+    return None
+
+
+def _static_fill_inplace(cache, fill_value, batch_offset):
+    assert len(cache.shape) == 4, "cache must be a 4D tensor: [B, num_heads, max_seq_len, head_size]."
+    assert len(fill_value.shape) == 4, "fill_value must be a 4D tensor: [B, num_heads, seq_len, head_size]."
+    assert fill_value.shape[-2] <= cache.shape[-2], (
+        "fill_value must have dim -2 less than or equal to cache.shape[-2] as the cache cannot be "
+        f"filled with more tokens than the cache can hold. Recieved fill_value.shape = {fill_value.shape}, "
+        f"cache.shape = {cache.shape}."
+    )
+    assert batch_offset is not None or cache.shape[0] == 1, "batch_offset must be provided if the batch size is not 1."
+    assert not batch_offset, "Only batch_offset == 0 is supported for currently."
+    b = _static_geometry(cache)[0]
+    if fill_value.shape[0] != b:
+        raise ValueError("fill_value and cache must have the same batch size")
+    _fill_inplace(cache, fill_value, _identity_table(b, cache.device),
+                  torch.arange(b, dtype=torch.int32, device=cache.device))
+
+
+@torch.library.custom_op("tt::fill_cache", mutates_args=[], device_types=["cuda"])
+def fill_cache(cache: torch.Tensor, fill_value: torch.Tensor, batch_offset: Optional[int] = None) -> torch.Tensor:
+    """cache[:, :, :seq_len, :] = fill_value on a copy (reference custom_ops.py:903-950)."""
+    out = cache.clone()
+    _static_fill_inplace(out, fill_value, batch_offset)
+    return out
+
+
+@fill_cache.register_fake
+def _(cache, fill_value, batch_offset=None):
+    return torch.empty_like(cache)
+
+
+@torch.library.custom_op("tt::fill_cache_", mutates_args=["cache"], device_types=["cuda"])
+def fill_cache_(cache: torch.Tensor, fill_value: torch.Tensor, batch_offset: Optional[int] = None) -> None:
+    _static_fill_inplace(cache, fill_value, batch_offset)
+
+
+@fill_cache_.register_fake
+def _(cache, fill_value, batch_offset=None):
+    return None
+
+
+@torch.library.custom_op("tt::scaled_dot_product_attention_decode", mutates_args=[], device_types=["cuda"])
+def scaled_dot_product_attention_decode(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    cur_pos_tensor: torch.Tensor,
+    attn_mask: Optional[torch.Tensor] = None,
+    attention_sink: Optional[torch.Tensor] = None,
+    is_causal: bool = True,
+    scale: Optional[float] = None,
+) -> torch.Tensor:
+    """Decode attention over static caches (reference custom_ops.py:745-842): user b attends
+    positions 0 .. cur_pos_tensor[b] of key[b] / value[b]; grouped heads; optional sink."""
+    assert len(query.shape) == 4, "query must be a 4D tensor: [1, B, num_heads, head_size]."
+    assert len(key.shape) == 4, "key must be a 4D tensor: [B, num_kv_heads, seq_len, head_size]."
+    assert len(value.shape) == 4, "value must be a 4D tensor: [B, num_kv_heads, seq_len, head_size]."
+    assert len(cur_pos_tensor.shape) == 1, "cur_pos_tensor must be a 1D tensor: [B]."
+    assert key.shape == value.shape, "key and value must have the same shape."
+    assert key.shape[-1] == query.shape[-1], "key and query must have the same head size."
+    assert query.shape[2] % key.shape[1] == 0, (
+        f"num_heads must be divisible by num_kv_heads. Query shape: {query.shape}, key shape: {key.shape}."
+    )
+    assert query.shape[0] == 1, "query must have dim 0 equal to 1."
+    assert query.shape[1] == key.shape[0], "query and key must have the same batch size."
+    if is_causal:
+        assert attn_mask is None, "attn_mask must be None when is_causal is True."
+    if attn_mask is not None:
+        raise NotImplementedError("static-cache decode with an explicit attn_mask is not built")
+    _static_geometry(key), _static_geometry(value)
+    if key.shape[2] % 4:
+        raise NotImplementedError("static-cache decode needs max_seq_len to be a multiple of 4")
+    # the cache tensor already has the paged layout [blocks = B, kv_heads, block_size = S, D]
+    return paged_scaled_dot_product_attention_decode(
+        query, key, value, _identity_table(key.shape[0], key.device), is_causal=True,
+        cur_pos_tensor=cur_pos_tensor, attention_sink=attention_sink, scale=scale,
+    )
+
+
+@scaled_dot_product_attention_decode.register_fake
+def _(query, key, value, cur_pos_tensor, attn_mask=None, attention_sink=None, is_causal=True, scale=None):
     return torch.empty_like(query)
 
 
