@@ -159,6 +159,34 @@ int ttpa_paged_sdpa_decode_windowed(void *out, int64_t out_user_stride, int64_t 
                                     size_t workspace_bytes, void *stream);
 
 /*
+ * Paged decode attention for latent-style (multi-head latent attention) caches.
+ * Replaces the device branch of tt::paged_flash_mla_decode
+ * (python_package/tt_torch/custom_ops.py:381-632; CPU semantics :551-610), causal form:
+ *   out[u, hq, :head_dim_v] = softmax_j( scale * q[u, hq, :] . K[u, hq / G, j, :] ) . V[u, hq / G, j, :]
+ *   over cache positions j = 0 .. min(cur_pos[u], table_width * block_size - 1).
+ * k_cache is [num_blocks, kv_heads, block_size, head_size] bf16.  v_cache is either a cache
+ * [num_blocks, kv_heads, block_size, head_dim_v] or NULL: then V is the first head_dim_v
+ * features of K (the latent path, custom_ops.py:573-575).  q is [users, q_heads, head_size]
+ * by strides, out is [users, q_heads, head_dim_v] by strides.  Built shapes: head_size 64,
+ * 128, 192, 576 with head_dim_v a multiple of 64 up to 512 (256 with a separate v_cache);
+ * q_heads / kv_heads up to 32 or a multiple of 32.  attention_sink as in
+ * ttpa_paged_sdpa_decode_windowed, or NULL.  cur_pos[u] < 0 gives a NaN row.
+ * The prefill operator tt::flash_mla_prefill (custom_ops.py:223-378) is served by the same
+ * entry point: query row i of a sequence is a user at position i (see tt_xla_amd/custom_ops.py).
+ */
+size_t ttpa_paged_mla_decode_workspace_bytes(int32_t users, int32_t q_heads, int32_t kv_heads,
+                                             int32_t head_dim_v);
+
+int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t out_head_stride,
+                          const void *q, int64_t q_user_stride, int64_t q_head_stride,
+                          const void *k_cache, const void *v_cache, const int32_t *page_table,
+                          int64_t page_table_row_stride, const void *cur_pos, int cur_pos_is_i64,
+                          int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
+                          int32_t head_dim_v, int32_t block_size, int32_t table_width,
+                          int32_t num_blocks, float scale, const float *attention_sink,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Measurement hook, no reference counterpart: the NEXT attention call made by this host
  * thread (decode or prefill) records `before` and `after` (hipEvent_t, as void*) on its
  * stream immediately around its dominant kernel (the split-K main kernel for decode, the

@@ -21,6 +21,11 @@ What pins each function (see tests/test_oracle_*.py):
                          assignments, checked element by element, and the library SDPA
                          with the reference's own additive mask, checked against the fp32
                          loop and against the paged oracle on an identity page table
+  flash_mla_prefill / paged_flash_mla_decode
+                         the latent-attention forms (custom_ops.py:343-357, 551-610): the
+                         library SDPA on gathered K with V = key[..., :head_dim_v]; checked
+                         against an fp32 loop with separate QK / V widths and against the
+                         grouped decode oracle when V is given explicitly
   paged_sdpa_decode_windowed / sdpa_windowed
                          PARITY UNPINNED against the reference: its CPU branches ignore
                          `sliding_window_size` and `attention_sink`
@@ -442,3 +447,35 @@ def sdpa_decode_static(query, key, value, cur_pos_tensor, scale=None):
         mask[b, ..., int(cur_pos_tensor[b]) + 1 :] = float("-inf")
     out = F.scaled_dot_product_attention(q, key, value, mask, is_causal=False, scale=scale, enable_gqa=True)
     return out.reshape(1, batch, heads, d)
+
+
+# --------------------------------------------------------------------------- #
+# latent (MLA) attention
+# --------------------------------------------------------------------------- #
+def flash_mla_prefill(query, key, head_dim_v, value=None, attn_mask=None, is_causal=True, scale=None):
+    """custom_ops.py:343-357: V defaults to the leading head_dim_v features of K."""
+    if value is None:
+        value = key[..., :head_dim_v]
+    return F.scaled_dot_product_attention(query, key, value, attn_mask, is_causal=is_causal,
+                                          scale=scale, enable_gqa=True)
+
+
+def paged_flash_mla_decode(query, key, head_dim_v, page_table, value=None, cur_pos_tensor=None, scale=None):
+    """custom_ops.py:551-610, causal form: gather each user's blocks, additive mask to the right
+    of cur_pos, library SDPA with grouped heads, in the query's dtype."""
+    block_size, nkv, dh = key.shape[-2], key.shape[-3], key.shape[-1]
+    users, hq = query.shape[1], query.shape[2]
+    max_seq = page_table.shape[1] * block_size
+    index = page_table.long()
+    gk = key[index].permute(0, 2, 1, 3, 4).reshape(users, nkv, max_seq, dh)
+    if value is not None:
+        gv = value[index].permute(0, 2, 1, 3, 4).reshape(users, nkv, max_seq, value.shape[-1])
+    else:
+        gv = gk[..., :head_dim_v]
+    q = query.reshape(users, hq, 1, dh)
+    mask = torch.zeros(users, 1, 1, max_seq, dtype=query.dtype)
+    for i in range(users):
+        mask[i, :, :, int(cur_pos_tensor[i]) + 1 :] = float("-inf")
+    scale_val = 1.0 / (dh**0.5) if scale is None else scale
+    out = F.scaled_dot_product_attention(q, gk, gv, mask, is_causal=False, scale=scale_val, enable_gqa=True)
+    return out.reshape(1, users, hq, head_dim_v)

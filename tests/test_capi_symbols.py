@@ -78,3 +78,14 @@ def test_ops_are_registered_and_refuse_cpu_tensors(native):
     with pytest.raises(NotImplementedError):  # no CPU implementation, and no fallback
         torch.ops.tt.paged_update_cache(cache, fill, torch.zeros(1, dtype=torch.int32),
                                         torch.zeros(1, 2, dtype=torch.int32))
+
+
+def test_latent_decode_entry_refuses_to_launch():
+    """The latent (MLA) decode kernel is switched off after faulting on the device: the entry
+    point must answer TTPA_ERR_UNSUPPORTED before touching any argument (no GPU needed)."""
+    from tt_xla_amd import _native as N
+
+    rc = N.lib().ttpa_paged_mla_decode(None, 0, 0, None, 0, 0, None, None, None, 0, None, 0, 1, 16, 1, 576,
+                                       512, 32, 1, 1, 1.0, None, None, 0, None)
+    assert rc == -2
+    assert b"switched off" in N.lib().ttpa_last_error()

@@ -96,4 +96,42 @@ __device__ __forceinline__ float bfp8_group_scale(uint32_t e) {
   return __builtin_ldexpf(1.0f, static_cast<int>(e) - 133);
 }
 
+// Byte address inside the workgroup's LDS allocation of a __shared__ object.  LDS-DMA
+// destinations are absolute LDS addresses: when a kernel also has static __shared__ arrays the
+// dynamic segment does not start at 0.
+__device__ __forceinline__ uint32_t lds_address(const void *shared_ptr) {
+  return (uint32_t)reinterpret_cast<uintptr_t>(
+      (const __attribute__((address_space(3))) unsigned char *)shared_ptr);
+}
+
+// 64 lanes x 16 bytes, global memory -> 1 KiB of LDS starting at byte address `lds_addr`
+// (wavefront-uniform, passed in M0); lane l's 16 bytes land at lds_addr + 16 l.  Written as
+// assembly so that the compiler does not make every later LDS read wait for these loads: the
+// kernels wait for them themselves (vmcnt(0)) before the barrier that publishes a tile.  Lanes
+// switched off by the execution mask transfer nothing.
+__device__ __forceinline__ void dma16(const void *uniform_base, uint32_t lane_bytes, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(lane_bytes), "s"(uniform_base), "s"(lds_addr)
+               : "memory");
+}
+// The same for callers whose base / LDS address the compiler cannot prove uniform: both are
+// read from the first active lane.  readfirstlane returns a signed int: each half of the
+// pointer goes through uint32_t before widening, or a low half with bit 31 set would smear
+// ones over the high half.
+__device__ __forceinline__ void dma16_uniform(const void *uniform_base, uint32_t lane_bytes, uint32_t lds_addr) {
+  const uint64_t ub = reinterpret_cast<uint64_t>(uniform_base);
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)ub);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(ub >> 32));
+  dma16(reinterpret_cast<const void *>(((uint64_t)hi << 32) | (uint64_t)lo), lane_bytes,
+        (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr));
+}
+__device__ __forceinline__ void dma16_lane(const void *lane_ptr, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(lane_ptr), "s"(lds_addr)
+               : "memory");
+}
+
+
 }  // namespace ttpa

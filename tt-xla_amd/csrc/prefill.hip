@@ -84,23 +84,6 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   return d;
 }
 
-// 64 lanes x 16 bytes, global memory -> 1 KiB of LDS starting at byte address `lds_addr`
-// (wavefront-uniform, passed in M0); lane l's 16 bytes land at lds_addr + 16 l.  Written as
-// assembly so that the compiler does not make every later LDS read wait for these loads: the
-// kernel waits for them itself (vmcnt(0)) before the barrier that publishes the tile.
-__device__ __forceinline__ void dma16(const void *uniform_base, uint32_t lane_bytes, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :
-               : "v"(lane_bytes), "s"(uniform_base), "s"(lds_addr)
-               : "memory");
-}
-__device__ __forceinline__ void dma16_lane(const void *lane_ptr, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-               :
-               : "v"(lane_ptr), "s"(lds_addr)
-               : "memory");
-}
-
 // MODE 0: dense K/V; 1: paged, block_size a multiple of 64 (a tile lies in one block);
 // 2: paged, any block size (per-row table lookups).
 //
@@ -191,7 +174,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
   auto issue = [&](const uint16_t *src, const uint32_t (&ld)[T::NI], bool is_v, int kt, int buf) {
     const int key0 = kt * kKeysPerTile;
     const int last = a.skv - 1 - key0;  // last valid key of this tile, relative (>= 0)
-    const uint32_t lds_base = (uint32_t)(buf * T::STAGE_BYTES + (is_v ? T::TILE_BYTES : 0));
+    const uint32_t lds_base = lds_address(smem) + (uint32_t)(buf * T::STAGE_BYTES + (is_v ? T::TILE_BYTES : 0));
     const char *base = nullptr;  // uniform address of the tile (modes 0 and 1)
     if constexpr (MODE == 0) {
       base = reinterpret_cast<const char *>(src + b * a.kv_bs + hk * a.kv_hs + (int64_t)key0 * a.kv_ts);

@@ -450,6 +450,167 @@ def _(query, key, value, page_table, chunk_start_idx_tensor, scale=None):
 
 
 # --------------------------------------------------------------------------- #
+# latent (MLA) attention
+# --------------------------------------------------------------------------- #
+_MLA_MAX_USERS = 1024  # users per launch of the latent decode kernel
+
+
+def _mla_decode_launch(out, q, key, value, page_table, cur, head_dim_v, scale, sink):
+    """out [users, heads, dv] / q [users, heads, dh] by strides; caches in the paged layout.
+
+    The entry point below currently answers TTPA_ERR_UNSUPPORTED (its kernel is switched off
+    until a fix for a device fault has been verified), which surfaces here as TtpaError."""
+    nb, nkv, bs, dh = key.shape
+    users, hq = q.shape[0], q.shape[1]
+    for u0 in range(0, users, _MLA_MAX_USERS):
+        n = min(_MLA_MAX_USERS, users - u0)
+        ws_bytes = N.lib().ttpa_paged_mla_decode_workspace_bytes(n, hq, nkv, head_dim_v)
+        if ws_bytes == 0:
+            raise NotImplementedError(
+                f"latent attention with {hq} query heads over {nkv} KV heads is not built "
+                "(heads per KV head: up to 32 or a multiple of 32)"
+            )
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+        qs, os_, pts, curs = q[u0 : u0 + n], out[u0 : u0 + n], page_table[u0 : u0 + n], cur[u0 : u0 + n]
+        N.call(
+            "ttpa_paged_mla_decode",
+            os_.data_ptr(), os_.stride(0), os_.stride(1), qs.data_ptr(), qs.stride(0), qs.stride(1),
+            key.data_ptr(), _ptr(value), pts.data_ptr(), pts.stride(0), curs.data_ptr(),
+            int(curs.dtype == torch.int64), n, hq, nkv, dh, head_dim_v, bs, pts.shape[1], nb,
+            float(scale), _ptr(sink), ws.data_ptr(), ws_bytes, _stream(),
+        )
+
+
+@torch.library.custom_op("tt::paged_flash_mla_decode", mutates_args=[], device_types=["cuda"])
+def paged_flash_mla_decode(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    head_dim_v: int,
+    page_table: torch.Tensor,
+    value: Optional[torch.Tensor] = None,
+    is_causal: bool = True,
+    attn_mask: Optional[torch.Tensor] = None,
+    cur_pos_tensor: Optional[torch.Tensor] = None,
+    attention_sink: Optional[torch.Tensor] = None,
+    scale: Optional[float] = None,
+) -> torch.Tensor:
+    """Paged decode over a latent KV cache (reference custom_ops.py:381-632): query
+    [1, users, nqh, dh_qk], key cache [blocks, nkv, block_size, dh_qk], optional value cache
+    [blocks, nkv, block_size, head_dim_v]; without it V is key[..., :head_dim_v]."""
+    assert len(query.shape) == 4, "query must be a 4D tensor: [1, num_users, nqh, dh_qk]."
+    assert len(key.shape) == 4, "key must be a 4D tensor: [max_num_blocks, nkv, block_size, dh_qk]."
+    assert len(page_table.shape) == 2, "page_table must be a 2D tensor: [num_users, num_blocks_per_user]."
+    assert query.shape[0] == 1, "query dim 0 must be 1 (decode processes one token per user)."
+    assert key.shape[-1] == query.shape[-1], "key and query must have the same head size (dh_qk)."
+    assert query.shape[2] % key.shape[1] == 0, "nqh must be divisible by nkv (GQA/MQA/MLA constraint)."
+    assert page_table.shape[0] == query.shape[1], "page_table number of users must match query number of users."
+    assert isinstance(head_dim_v, int) and head_dim_v > 0, f"head_dim_v must be a positive int, got {head_dim_v}."
+    if value is not None:
+        assert len(value.shape) == 4, "value must be a 4D tensor: [max_num_blocks, nkv, block_size, head_dim_v]."
+        assert value.shape[:3] == key.shape[:3], "value's block/head/block_size dims must match key's."
+        assert value.shape[-1] == head_dim_v, f"value's last dim ({value.shape[-1]}) must equal head_dim_v ({head_dim_v})."
+    else:
+        assert head_dim_v <= key.shape[-1], (
+            f"head_dim_v ({head_dim_v}) cannot exceed key's head dim ({key.shape[-1]}) when value is None."
+        )
+    if is_causal:
+        assert attn_mask is None, "attn_mask must be None when is_causal is True."
+        assert cur_pos_tensor is not None, "cur_pos_tensor must be provided when is_causal is True."
+    if attn_mask is not None:
+        assert not is_causal, "attn_mask requires is_causal to be False."
+    else:
+        assert is_causal, "is_causal must be True when attn_mask is not provided"
+    if not is_causal:
+        raise NotImplementedError("latent decode with an explicit attn_mask is not built")
+    assert len(cur_pos_tensor.shape) == 1, "cur_pos_tensor must be a 1D tensor: [num_users]."
+    assert cur_pos_tensor.shape[0] == query.shape[1], "cur_pos_tensor number of users must match query number of users."
+    if query.dtype != torch.bfloat16 or key.dtype != torch.bfloat16 or not key.is_contiguous():
+        raise ValueError("query and the key cache must be bfloat16, the cache contiguous")
+    if value is not None and (value.dtype != torch.bfloat16 or not value.is_contiguous()):
+        raise ValueError("the value cache must be contiguous bfloat16")
+    users, hq, dh = query.shape[1], query.shape[2], query.shape[3]
+    if scale is None:
+        scale = 1.0 / math.sqrt(dh)
+    q = _rows_contiguous(query)[0]
+    out = torch.empty((1, users, hq, head_dim_v), dtype=query.dtype, device=query.device)
+    sink = None
+    if attention_sink is not None:
+        if attention_sink.numel() != hq:
+            raise ValueError(f"attention_sink must hold one logit per query head ({hq})")
+        sink = attention_sink.reshape(hq).to(device=query.device, dtype=torch.float32).contiguous()
+    _mla_decode_launch(out[0], q, key, value, _table(page_table), _index_tensor(cur_pos_tensor),
+                       head_dim_v, scale, sink)
+    return out
+
+
+@paged_flash_mla_decode.register_fake
+def _(query, key, head_dim_v, page_table, value=None, is_causal=True, attn_mask=None,
+      cur_pos_tensor=None, attention_sink=None, scale=None):
+    return torch.empty((query.shape[0], query.shape[1], query.shape[2], head_dim_v),
+                       dtype=query.dtype, device=query.device)
+
+
+@torch.library.custom_op("tt::flash_mla_prefill", mutates_args=[], device_types=["cuda"])
+def flash_mla_prefill(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    head_dim_v: int,
+    value: Optional[torch.Tensor] = None,
+    attn_mask: Optional[torch.Tensor] = None,
+    is_causal: bool = True,
+    scale: Optional[float] = None,
+) -> torch.Tensor:
+    """Causal prefill over freshly built latent K (reference custom_ops.py:223-378): query
+    [b, nqh, s, dh_qk], key [b, nkv, s, dh_qk], optional value [b, nkv, s, head_dim_v].
+
+    Runs on the latent decode kernel: query row i of a sequence is a user at position i
+    whose cache is the sequence itself (one block of s tokens, a one-column page table)."""
+    assert len(query.shape) == 4, "query must be a 4D tensor: [b, nqh, s, dh_qk]."
+    assert len(key.shape) == 4, "key must be a 4D tensor: [b, nkv, s, dh_qk]."
+    assert key.shape[-1] == query.shape[-1], "key and query must have the same head size (dh_qk)."
+    assert query.shape[0] == key.shape[0], "query and key must have the same batch size."
+    assert query.shape[2] == key.shape[2], "query and key must have the same sequence length for MLA prefill."
+    assert query.shape[1] % key.shape[1] == 0, "nqh must be divisible by nkv (GQA/MQA/MLA constraint)."
+    assert query.shape[2] % 32 == 0, f"query sequence length must be divisible by 32 but got {query.shape[2]}."
+    assert isinstance(head_dim_v, int) and head_dim_v > 0, f"head_dim_v must be a positive int, got {head_dim_v}."
+    if value is not None:
+        assert len(value.shape) == 4, "value must be a 4D tensor: [b, nkv, s, head_dim_v]."
+        assert value.shape[:3] == key.shape[:3], "value's batch/head/seq dims must match key's."
+        assert value.shape[-1] == head_dim_v, f"value's last dim ({value.shape[-1]}) must equal head_dim_v ({head_dim_v})."
+    else:
+        assert head_dim_v <= key.shape[-1], (
+            f"head_dim_v ({head_dim_v}) cannot exceed key's head dim ({key.shape[-1]}) when value is None."
+        )
+    if attn_mask is not None:
+        assert is_causal == False, "is_causal cannot be True when attn_mask is provided."  # noqa: E712
+        assert attn_mask.shape[0] == query.shape[0], "attention mask batch size must match query batch size."
+        raise NotImplementedError("latent prefill with an explicit attn_mask is not built")
+    assert is_causal == True, "is_causal must be True if attn_mask is not provided"  # noqa: E712
+    if query.dtype != torch.bfloat16 or key.dtype != torch.bfloat16:
+        raise ValueError("query and key must be bfloat16")
+    b, hq, s, dh = query.shape
+    if scale is None:
+        scale = 1.0 / math.sqrt(dh)
+    q = _rows_contiguous(query)
+    k = key.contiguous()
+    v = value.contiguous() if value is not None else None
+    out = torch.empty((b, hq, s, head_dim_v), dtype=query.dtype, device=query.device)
+    table = torch.zeros((s, 1), dtype=torch.int32, device=query.device)
+    cur = torch.arange(s, dtype=torch.int32, device=query.device)
+    for i in range(b):
+        # [s, heads, d] views: token-major "users", the sequence as a single block of s tokens
+        _mla_decode_launch(out[i].transpose(0, 1), q[i].transpose(0, 1), k[i : i + 1],
+                           None if v is None else v[i : i + 1], table, cur, head_dim_v, scale, None)
+    return out
+
+
+@flash_mla_prefill.register_fake
+def _(query, key, head_dim_v, value=None, attn_mask=None, is_causal=True, scale=None):
+    return torch.empty((query.shape[0], query.shape[1], query.shape[2], head_dim_v),
+                       dtype=query.dtype, device=query.device)
+
+
+# --------------------------------------------------------------------------- #
 # non-paged (static) cache: [batch, kv_heads, max_seq_len, head_size]
 # --------------------------------------------------------------------------- #
 # A static cache is a paged cache whose block u is the whole sequence of user u: the same
