@@ -1,0 +1,107 @@
+"""Host-side model of the address arithmetic of the latent decode kernel
+(tt-xla_amd/csrc/decode_wide.hip): for each built shape, every global source range, LDS
+destination, LDS operand read and partial-slot write the kernel forms must stay inside the
+buffer it belongs to.  Pure integer arithmetic, no GPU: it restates the kernel's formulas, so
+it guards the geometry (strides, tile sizes, slot layout), not the generated code."""
+
+import itertools
+
+import pytest
+
+K_TILE = 64
+STATIC_LDS = 8224          # s_pref + s_len + s_wsum of the kernel
+LDS_PER_CU = 160 * 1024
+
+SHAPES = [
+    # head_size, head_dim_v, separate_v, heads, kv_heads, block_size, table_width, num_blocks, users
+    (576, 512, False, 16, 1, 32, 24, 96, 4),
+    (576, 512, False, 128, 1, 64, 12, 36, 3),
+    (192, 128, False, 16, 1, 32, 16, 128, 8),
+    (192, 128, False, 16, 4, 32, 16, 128, 8),
+    (128, 128, True, 8, 8, 32, 16, 128, 8),
+    (128, 64, True, 16, 1, 32, 16, 128, 8),
+    (192, 128, False, 8, 1, 1184, 1, 1, 1024),   # prefill mapping: one block of s tokens
+]
+
+
+def _geometry(hq, nkv):
+    g = hq // nkv
+    if g <= 32:
+        return 1, g
+    assert g % 32 == 0
+    return g // 32, 32
+
+
+@pytest.mark.parametrize("dqk,dv,sep_v,hq,nkv,bs,width,nb,users", SHAPES)
+def test_every_address_stays_in_bounds(dqk, dv, sep_v, hq, nkv, bs, width, nb, users):
+    dvw = 128 if dv % 128 == 0 else 64
+    n_slices = dv // dvw
+    assert dv % dvw == 0 and n_slices <= (2 if sep_v else 4)
+    nhb, gseg = _geometry(hq, nkv)
+    krow = 2 * dqk + 16
+    ktile = K_TILE * krow
+    vrow_max = 2 * 2 * dvw + 16
+    vtile = K_TILE * vrow_max if sep_v else 0
+    stage = ktile + vtile
+    assert STATIC_LDS + 2 * stage <= LDS_PER_CU, "two stages must fit the CU's LDS"
+    row_bytes = 2 * dqk
+    cache_bytes = nb * nkv * bs * dqk * 2
+    vcache_bytes = nb * nkv * bs * dv * 2
+    v_lds_row = 2 * dv + 16
+    assert v_lds_row <= vrow_max or not sep_v
+
+    cap = width * bs
+    for t in {0, (cap - 1) // K_TILE}:                      # first and last tile of a full table
+        for phys, kvh in itertools.product({0, nb - 1}, {0, nkv - 1}):
+            for r in (0, 15, 16, 63):                      # rows moved by different wavefronts
+                tk = t * K_TILE + r
+                col = tk // bs
+                p = phys if col < width else 0            # columns past the table read block 0
+                row = (p * nkv + kvh) * bs + (tk - col * bs)
+                src = row * dqk * 2
+                # the row index inside a block must be < block_size
+                assert 0 <= tk - col * bs < bs
+                assert 0 <= src and src + row_bytes <= cache_bytes
+                for buf in (0, 1):
+                    dst = STATIC_LDS + buf * stage + r * krow
+                    assert dst + row_bytes <= STATIC_LDS + buf * stage + ktile
+                    if sep_v:
+                        vsrc = row * dv * 2
+                        assert vsrc + 2 * dv <= vcache_bytes
+                        vdst = STATIC_LDS + buf * stage + ktile + r * v_lds_row
+                        assert vdst + 2 * dv <= STATIC_LDS + (buf + 1) * stage
+
+    # LDS operand reads of every lane
+    ksteps = dqk // 16
+    for lane in range(64):
+        n, h = lane & 31, lane >> 5
+        for kb in (0, 1):
+            for s in (0, ksteps - 1):
+                off = (32 * kb + n) * krow + 16 * h + 32 * s
+                assert off + 16 <= ktile and off + 16 <= (32 * kb + n) * krow + row_bytes
+        grp, a16 = lane >> 4, lane & 15
+        vstride = v_lds_row if sep_v else krow
+        for wave in range(n_slices):
+            base = (4 * (grp >> 1) + (a16 >> 2)) * vstride + 2 * (wave * dvw + 16 * (grp & 1) + 4 * (a16 & 3))
+            for kb, s, db, hi in itertools.product((0, 1), (0, 1), range(dvw // 32), (0, 1)):
+                off = base + (32 * kb + 16 * s) * vstride + 64 * db + hi * 8 * vstride
+                row = off // vstride
+                assert row < K_TILE
+                assert off % vstride + 8 <= 2 * dv, "V fragment must stay inside the value columns"
+
+    # partial slots and workspace
+    slot_floats = (gseg * dv + 2 * gseg + 3) // 4 * 4
+    for n in range(gseg):
+        for wave in range(n_slices):
+            for h in (0, 1):
+                last = n * dv + wave * dvw + 4 * h + 32 * (dvw // 32 - 1) + 8 * 3 + 3
+                assert last < gseg * dv
+        assert gseg * dv + gseg + n < slot_floats
+    segs = users * nkv * nhb
+    cus = 256
+    # slot index = workgroup + segment; workgroups that get work < cus
+    assert (cus - 1) + (segs - 1) < cus + segs
+    # head index of (segment, column) stays a query head
+    for seg_h in (0, nkv * nhb - 1):
+        assert seg_h * gseg + gseg - 1 < hq
+        assert seg_h // nhb < nkv
