@@ -20,10 +20,11 @@
  * integrations/vllm_plugin/vllm_tt/attention_impls/attention.py:104-112):
  *   TTPA_KV_BF16  bfloat16 [num_blocks, kv_heads, block_size, head_size]
  *   TTPA_KV_BFP8  uint8    [num_blocks, kv_heads, block_size + block_size/16, head_size]
- *                 rows 0..block_size-1: one byte (sign<<7 | 7-bit magnitude) per element;
+ *                 rows 0..block_size-1: one byte b = 128 + v per element, v the signed
+ *                 7-bit mantissa in [-127, 127] (offset binary);
  *                 the remaining bytes, read as [block_size][head_size/16], hold one
  *                 shared exponent byte per 16 consecutive head_size elements;
- *                 value = (-1)^s * m * 2^(e - 133).
+ *                 value = (b - 128) * 2^(e - 133).
  * K and V are two separate tensors of that layout.
  */
 #ifndef TTPA_H_

@@ -12,14 +12,18 @@ Format
 ------
 A group is 16 consecutive head-dim elements of one token.  Per group one byte ``e``
 (the largest biased bfloat16 exponent in the group) and per element one byte
-``s<<7 | m`` (sign, 7-bit magnitude).  The decoded value is
+``b = 128 + v`` with the signed 7-bit mantissa ``v`` in [-127, 127] (offset binary:
+one byte permute turns it into a half-precision number on the device, no sign
+handling).  The decoded value is
 
-    (-1)^s * m * 2^(e - 133)            (133 = 127 bias + 6 fraction bits)
+    (b - 128) * 2^(e - 133)             (133 = 127 bias + 6 fraction bits)
 
-so the largest element keeps its hidden bit plus 6 fraction bits.  Encoding a
+so the largest element keeps its hidden bit plus 6 fraction bits.  Byte 0 (v = -128)
+is never produced by the encoder but decodes by the same formula; a zero-filled,
+never written cache therefore reads as -2^-126 per element, not as 0.  Encoding a
 bfloat16 with exponent field ``ex`` and 8-bit significand ``sig = 128 | frac``:
-``m = min(127, rne(sig >> (e - ex + 1)))`` with round-half-to-even on the bits
-shifted out; ``ex == 0`` (zero / subnormal) encodes as m = 0.  Inf / NaN inputs are
+``|v| = min(127, rne(sig >> (e - ex + 1)))`` with round-half-to-even on the bits
+shifted out; ``ex == 0`` (zero / subnormal, either sign) encodes as v = 0.  Inf / NaN inputs are
 rejected here (the device kernel does not check).
 
 Cache layout
@@ -63,17 +67,16 @@ def quantize(x: torch.Tensor):
     half = 1 << (sh - 1)
     up = (rem > half) | ((rem == half) & ((q & 1) == 1))
     m = np.minimum(q + up.astype(np.int64), 127)
-    elem = ((sign << 7) | m).astype(np.uint8)
-    # a group of zeros / subnormals has e == 0 and all m == 0 already
+    elem = (128 + np.where(sign == 1, -m, m)).astype(np.uint8)
+    # a group of zeros / subnormals has e == 0 and all v == 0 already
     return elem, e.astype(np.uint8)
 
 
 def dequantize(elem: np.ndarray, exps: np.ndarray) -> np.ndarray:
     """(elem uint8 [..., D], exps uint8 [..., D//16]) -> float32 [..., D] (exact)."""
-    m = (elem & 0x7F).astype(np.float64)
-    s = np.where(elem & 0x80, -1.0, 1.0)
+    v = elem.astype(np.float64) - 128.0
     e = np.repeat(exps.astype(np.int64), GROUP, axis=-1)
-    return (s * np.ldexp(m, e - 133)).astype(np.float32)
+    return np.ldexp(v, e - 133).astype(np.float32)
 
 
 def pack_cache(cache: torch.Tensor) -> torch.Tensor:

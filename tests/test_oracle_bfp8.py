@@ -27,7 +27,7 @@ def _brute_encode_group(vals):
     out = []
     for v, x in zip(vals, ex):
         if x == 0:
-            out.append(0x80 if math.copysign(1.0, v) < 0 else 0)
+            out.append(128)
             continue
         r = Fraction(abs(v)) / (Fraction(2) ** (e - 133))
         fl = r.numerator // r.denominator
@@ -35,7 +35,7 @@ def _brute_encode_group(vals):
         if frac > Fraction(1, 2) or (frac == Fraction(1, 2) and fl % 2 == 1):
             fl += 1
         m = min(127, fl)
-        out.append((0x80 if v < 0 else 0) | m)
+        out.append(128 - m if v < 0 else 128 + m)
     return out, e
 
 
@@ -98,9 +98,9 @@ def test_zero_group_and_signs():
     x = torch.zeros(2, 32, dtype=torch.bfloat16)
     x[1, 16:] = torch.tensor([-1.0, 1.0] * 8, dtype=torch.bfloat16)
     elem, exps = C.quantize(x)
-    assert exps[0, 0] == 0 and exps[0, 1] == 0 and not elem[0].any()
+    assert exps[0, 0] == 0 and exps[0, 1] == 0 and (elem[0] == 128).all()
     assert exps[1, 1] == 127
-    assert list(elem[1, 16:18]) == [0x80 | 64, 64]
+    assert list(elem[1, 16:18]) == [128 - 64, 128 + 64]
     assert torch.equal(C.roundtrip(x), x.float())
 
 
@@ -112,7 +112,7 @@ def test_ties_round_to_even_and_top_clamps():
     assert torch.equal(x.float(), torch.tensor([vals]))
     elem, exps = C.quantize(x)
     assert exps[0, 0] == 127
-    assert list(elem[0, :7]) == [64, 0, 2, 2, 0, 1, 127]  # 127.5 -> 128 -> clamp 127
+    assert list(elem[0, :7]) == [128 + m for m in (64, 0, 2, 2, 0, 1, 127)]  # 127.5 -> 128 -> clamp 127
 
 
 def test_inf_nan_rejected():

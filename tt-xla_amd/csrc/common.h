@@ -59,6 +59,10 @@ __device__ __forceinline__ int64_t load_index(const void *p, int is_i64, int64_t
 }
 
 // ---- block-float-8 ---------------------------------------------------------
+// A group of 16 values shares the exponent byte e (largest biased bfloat16 exponent of the
+// group); an element byte is 128 + v with the signed mantissa v in [-127, 127] and decodes
+// to v * 2^(e - 133).  Offset binary is chosen for the readers: one byte permute makes a
+// half-precision number out of an element byte, with no sign handling.
 // Encodes 16 bfloat16 values held as 8 packed dwords (element 2j in the low half of
 // w[j]).  Returns the shared exponent; out[0..3] receive the 16 element bytes.
 __device__ __forceinline__ uint32_t bfp8_encode16(const uint32_t (&w)[8], uint32_t (&out)[4]) {
@@ -81,16 +85,15 @@ __device__ __forceinline__ uint32_t bfp8_encode16(const uint32_t (&w)[8], uint32
     uint32_t half = 1u << (sh - 1u);
     q += (rem > half || (rem == half && (q & 1u))) ? 1u : 0u;
     q = min(q, 127u);
-    uint32_t byte = ((h >> 8) & 0x80u) | q;
+    uint32_t byte = (h & 0x8000u) ? 128u - q : 128u + q;
     out[i >> 2] |= byte << (8 * (i & 3));
   }
   return emax;
 }
 
-// Decodes one element byte with shared exponent e to float: (-1)^s * m * 2^(e-133).
+// Decodes one element byte with shared exponent e to float: (byte - 128) * 2^(e-133).
 __device__ __forceinline__ float bfp8_decode(uint32_t byte, float group_scale) {
-  float m = static_cast<float>(byte & 0x7fu) * group_scale;
-  return (byte & 0x80u) ? -m : m;
+  return static_cast<float>(static_cast<int>(byte) - 128) * group_scale;
 }
 __device__ __forceinline__ float bfp8_group_scale(uint32_t e) {
   return __builtin_ldexpf(1.0f, static_cast<int>(e) - 133);

@@ -389,7 +389,6 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   a.scale_log2e = scale * 1.4426950408889634f;
   a.ws_seg = static_cast<int *>(workspace);
   a.ws_slots = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + header_bytes(users, kv_heads));
-  a.n_waves = waves_for_device(kv_format);
   a.slot_floats = slot_floats_for(g, head_size);
   a.kv_format = kv_format;
   a.window = sliding_window;
@@ -398,23 +397,33 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   hipStream_t st = static_cast<hipStream_t>(stream);
   // Kernel choice: the VALU kernel streams at the HBM ceiling up to 4 query heads per KV head;
   // beyond that its per-head VALU work becomes the limiter and the matrix-core kernel takes
-  // over (its cost per tile does not depend on the group width).  The block-float-8 cache is
-  // bound by the byte -> bfloat16 expansion in either kernel.  TTPA_DECODE_KERNEL=valu|mfma
-  // overrides the choice.
+  // over (its cost per tile does not depend on the group width).  The block-float-8 cache goes
+  // to a matrix-core kernel whenever one applies: there the byte expansion costs one VALU
+  // operation per element and the products none, while the VALU kernel pays for both; head
+  // size 128 with up to 16 heads per group has the 16x16x32 kernel with twice the occupancy.
+  // TTPA_DECODE_KERNEL=valu|mfma|mfma16 overrides the choice.
   static int forced = -1;
   if (forced < 0) {
     const char *e = getenv("TTPA_DECODE_KERNEL");
-    forced = !e ? 0 : (!strcmp(e, "valu") ? 1 : (!strcmp(e, "mfma") ? 2 : 0));
+    forced = !e ? 0 : (!strcmp(e, "valu") ? 1 : (!strcmp(e, "mfma") ? 2 : (!strcmp(e, "mfma16") ? 3 : 0)));
   }
   const bool mfma_ok = mfma_decode_supported(a, head_size, g);
-  bool use_mfma = mfma_ok && g >= 5;
-  if (forced == 1) use_mfma = false;
-  if (forced == 2) use_mfma = mfma_ok;
+  const bool mfma16_ok = mfma16_decode_supported(a, head_size, g);
+  bool use_mfma16 = mfma16_ok;
+  bool use_mfma = !use_mfma16 && mfma_ok && (g >= 5 || kv_format == TTPA_KV_BFP8);
+  if (forced == 1) use_mfma = use_mfma16 = false;
+  if (forced == 2) use_mfma = mfma_ok, use_mfma16 = false;
+  if (forced == 3) use_mfma16 = mfma16_ok, use_mfma = !mfma16_ok && use_mfma;
+  // the 32x32 matrix-core kernel runs one workgroup per CU whatever the cache format
+  a.n_waves = waves_for_device(use_mfma ? TTPA_KV_BF16 : kv_format);
   hipEvent_t ev0, ev1;
   take_profile_events(ev0, ev1);
   if (ev0) (void)hipEventRecord(ev0, st);
   int rc = TTPA_OK;
-  if (use_mfma) {
+  if (use_mfma16) {
+    if (!launch_mfma16_main(a, st))
+      rc = fail(TTPA_ERR_LAUNCH, "decode: cannot configure the 16x16 matrix-core kernel");
+  } else if (use_mfma) {
     if (!launch_mfma_main(a, head_size, st))
       rc = fail(TTPA_ERR_LAUNCH, "decode: cannot configure the matrix-core kernel");
   } else {

@@ -4,8 +4,8 @@
 // 64-token tiles cut into equal wavefront ranges, lane (r, c) holds elements c of token
 // 4 i + r for load i, reduce-scatter of q.k over the 16 lanes of a row, one online-softmax
 // stream per lane row.  What changes is the data: per token row the cache holds head_size
-// element bytes (sign << 7 | 7-bit magnitude) and head_size / 16 shared exponent bytes.
-//   * element bytes are expanded to exact bfloat16 integers (+-m) in registers;
+// element bytes (128 + signed 7-bit mantissa) and head_size / 16 shared exponent bytes.
+//   * element bytes are expanded to exact bfloat16 integers in registers;
 //   * for q.k the group scale 2^(e-133) multiplies the lane's partial dot product (all
 //     elements a lane holds for a load belong to one 16-element group);
 //   * for p.V the scale is folded into the probability (a power of two times a bfloat16 is
@@ -17,19 +17,15 @@ namespace ttpa {
 namespace decode {
 namespace {
 
-// 4 element bytes -> two packed bfloat16 pairs holding +-magnitude exactly.
+// 4 element bytes (128 + v) -> two packed bfloat16 pairs holding the integers v exactly.
 __device__ __forceinline__ void expand4(uint32_t w, uint32_t &p01, uint32_t &p23) {
-  const uint32_t mag = w & 0x7f7f7f7fu;
-  const float f0 = (float)(mag & 0xffu), f1 = (float)((mag >> 8) & 0xffu);
-  const float f2 = (float)((mag >> 16) & 0xffu), f3 = (float)(mag >> 24);
-  // high halves of the floats (a value below 256 is exact in 8 significand bits)
+  const float f0 = (float)(w & 0xffu) - 128.f, f1 = (float)((w >> 8) & 0xffu) - 128.f;
+  const float f2 = (float)((w >> 16) & 0xffu) - 128.f, f3 = (float)(w >> 24) - 128.f;
+  // high halves of the floats (an integer of magnitude <= 128 is exact in 8 significand bits)
   p01 = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f1), __builtin_bit_cast(uint32_t, f0),
                               0x07060302u);
   p23 = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f3), __builtin_bit_cast(uint32_t, f2),
                               0x07060302u);
-  // sign bits: byte k's bit 7 -> bit 15 (even element) / bit 31 (odd element)
-  p01 ^= __builtin_amdgcn_perm(w, w, 0x010c000cu) & 0x80008000u;
-  p23 ^= __builtin_amdgcn_perm(w, w, 0x030c020cu) & 0x80008000u;
 }
 
 // 2^(e - 133) for a shared exponent byte; exponents below 7 (|x| < 2^-120) read as zero.

@@ -91,6 +91,37 @@ typedef uint32_t __attribute__((may_alias)) lds_u32;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
+typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+// Largest value of v over the wavefront, as a wavefront-uniform number.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kDppXor1, 0xf, 0xf, true));
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kDppXor2, 0xf, 0xf, true));
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kDppHalfMirror, 0xf, 0xf, true));
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kDppMirror, 0xf, 0xf, true));
+  const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)v, 0);
+  const uint32_t r1 = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+  const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane((int)v, 32);
+  const uint32_t r3 = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+  return max(max(r0, r1), max(r2, r3));
+}
+
+// 4 element bytes (128 + v) -> two half pairs holding v * s, given s2 = (s, s) and
+// c2 = (-1152 s, -1152 s) for a power of two s: (1024 + b) * s - 1152 s = (b - 128) * s.
+__device__ __forceinline__ void expand4_half(uint32_t w, halfx2 s2, halfx2 c2, uint32_t &p01,
+                                             uint32_t &p23) {
+  const uint32_t m01 = __builtin_amdgcn_perm(0x64646464u, w, 0x04010400u);
+  const uint32_t m23 = __builtin_amdgcn_perm(0x64646464u, w, 0x04030402u);
+  p01 = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(halfx2, m01), s2, c2));
+  p23 = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(halfx2, m23), s2, c2));
+}
+// two floats -> packed half pair, round to nearest even
+__device__ __forceinline__ uint32_t pack_half2(float lo, float hi) {
+  floatx2 f = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, halfx2));
+}
+
 // Streaming (non-temporal) load of DW dwords: K/V are read once per launch, so they
 // should not displace anything in L2 / MALL.
 // `ubase` is wavefront-uniform and `lane_bytes` a 32-bit per-lane offset, which lets the
@@ -345,6 +376,10 @@ bool launch_bfp8_main(const DecodeArgs &a, int head_size, int g, hipStream_t st)
 // Matrix-core main kernel (decode_mfma.hip) for wide head groups and block-float-8.
 bool mfma_decode_supported(const DecodeArgs &a, int head_size, int g);
 bool launch_mfma_main(const DecodeArgs &a, int head_size, hipStream_t st);
+// Matrix-core main kernel for the block-float-8 cache with head size 128 and up to 16 query
+// heads per KV head (decode_mfma16.hip): two workgroups per CU.
+bool mfma16_decode_supported(const DecodeArgs &a, int head_size, int g);
+bool launch_mfma16_main(const DecodeArgs &a, hipStream_t st);
 
 }  // namespace decode
 }  // namespace ttpa

@@ -7,13 +7,24 @@
 // on every tile (dot products, cross-lane reduction, softmax), which stops hiding behind
 // the HBM stream at 8 query heads per KV head, and the block-float-8 cache adds a byte ->
 // bfloat16 expansion on top.  Here a tile goes global -> registers -> wave-private LDS
-// (expanded to bfloat16 on the way for block-float-8), and the two products run on
-// v_mfma_f32_32x32x16_bf16 with the G query heads of the group as the 32-wide N dimension:
+// and the two products run on v_mfma_f32_32x32x16_bf16 with the G query heads of the group as
+// the 32-wide N dimension:
 //   S^T[key, head] = K[key, :] . Q[head, :]        A = K rows from LDS, B = Q in registers
 //   O^T[d, head]  += V^T[d, key] . P^T[key, head]  A = V through the transposing LDS load
 // Each lane owns one head column, so softmax statistics are per-lane scalars and the
 // probabilities are already the B operand of the second product.  Cost per tile is
 // independent of G (up to 32 heads per KV head).
+//
+// Block-float-8 cache: the tile is expanded to half precision on its way into LDS and the
+// products run on v_mfma_f32_32x32x16_f16.  An element byte b = 128 + v becomes the half
+// 0x6400 | b = 1024 + b with one byte permute per element pair, and one packed fma per pair
+// turns it into v * 2^(e - eref) exactly (e the group's exponent byte, eref the largest
+// exponent byte of the tile; groups more than 2^24 below it flush to zero).  The tile's K
+// factor 2^(eref - 133) joins the softmax scale.  V tiles are brought to a running largest
+// exponent of the segment the way scores are brought to a running maximum: the tile's factor
+// multiplies the probabilities, a raised reference rescales the accumulator, and the segment's
+// partial is multiplied by 2^(reference - 133) when it is written.  Q is converted to half
+// precision once per segment, scaled by a power of two so that its largest element is in [1, 2).
 //
 // LDS: 37 KiB per wavefront (K rows padded to 68 dwords, V rows to 80), four wavefronts
 // per workgroup, one workgroup per CU.
@@ -30,21 +41,16 @@ typedef short shortx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kMaxUsersMfma = 1024;
 
-// 4 element bytes with shared scale -> two packed bfloat16 pairs (exact).
-__device__ __forceinline__ void expand4_scaled(uint32_t w, float scale, uint32_t &p01,
-                                               uint32_t &p23) {
-  const uint32_t mag = w & 0x7f7f7f7fu;
-  const float f0 = (float)(mag & 0xffu) * scale, f1 = (float)((mag >> 8) & 0xffu) * scale;
-  const float f2 = (float)((mag >> 16) & 0xffu) * scale, f3 = (float)(mag >> 24) * scale;
-  p01 = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f1), __builtin_bit_cast(uint32_t, f0),
-                              0x07060302u);
-  p23 = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f3), __builtin_bit_cast(uint32_t, f2),
-                              0x07060302u);
-  p01 ^= __builtin_amdgcn_perm(w, w, 0x010c000cu) & 0x80008000u;
-  p23 ^= __builtin_amdgcn_perm(w, w, 0x030c020cu) & 0x80008000u;
-}
-__device__ __forceinline__ float group_scale(uint32_t e) {
-  return e >= 7u ? __builtin_bit_cast(float, (e - 6u) << 23) : 0.f;
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+
+template <bool F16>
+__device__ __forceinline__ floatx16 mma(const u32x4 &x, const u32x4 &y, const floatx16 &c) {
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, x),
+                                                  __builtin_bit_cast(halfx8, y), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x),
+                                                   __builtin_bit_cast(bf16x8, y), c, 0, 0, 0);
 }
 
 template <int D, bool BFP8, bool BIG>
@@ -120,24 +126,27 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
       }
     }
   };
-  // registers -> LDS tile (rows past `nvalid` are cleared when `clear` is set)
+  // registers -> LDS tile (rows past `nvalid` are cleared when `clear` is set); `eref` is the
+  // tile's reference exponent (block-float-8)
   auto stage = [&](uint16_t *dst, int stride, const u32x4 (&raw)[NL], const uint32_t (&ex)[NL],
-                   int nvalid, bool clear) {
+                   int eref, int nvalid, bool clear) {
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
       const int row = RPL * i + sr;
       const bool keep = !clear || row < nvalid;
       if constexpr (BFP8) {
-        const float gs = keep ? group_scale(ex[i]) : 0.f;
+        // 2^(e - eref) as a half: through the float with exponent field e - eref + 127; the
+        // conversion is exact down to 2^-24 and gives zero below
+        const int field = max((int)ex[i] - (eref - 127), 0);
+        const float sf = keep ? __builtin_bit_cast(float, (uint32_t)min(field, 127) << 23) : 0.f;
+        const _Float16 sh = (_Float16)sf;
+        const halfx2 s2 = {sh, sh};
+        const halfx2 c2 = s2 * halfx2{(_Float16)-1152.f, (_Float16)-1152.f};
         uint32_t o[8];
-        expand4_scaled(raw[i].x, gs, o[0], o[1]);
-        expand4_scaled(raw[i].y, gs, o[2], o[3]);
-        expand4_scaled(raw[i].z, gs, o[4], o[5]);
-        expand4_scaled(raw[i].w, gs, o[6], o[7]);
-        if (!keep) {
-#pragma unroll
-          for (int j = 0; j < 8; ++j) o[j] = 0;  // -0 from a cleared scale is harmless, but be exact
-        }
+        expand4_half(raw[i].x, s2, c2, o[0], o[1]);
+        expand4_half(raw[i].y, s2, c2, o[2], o[3]);
+        expand4_half(raw[i].z, s2, c2, o[4], o[5]);
+        expand4_half(raw[i].w, s2, c2, o[6], o[7]);
         uint4 *p = reinterpret_cast<uint4 *>(dst + row * stride + sc * 16);
         p[0] = make_uint4(o[0], o[1], o[2], o[3]);
         p[1] = make_uint4(o[4], o[5], o[6], o[7]);
@@ -147,14 +156,41 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
       }
     }
   };
-  // Q fragments: B operand, lane n = head of the group (zero beyond G)
-  auto load_q = [&](const Cursor &cu, bf16x8 (&qf)[KSTEPS]) {
+  // largest exponent byte of the tile's attended rows (block-float-8)
+  auto tile_exponent = [&](const uint32_t (&ex)[NL], int nvalid, bool partial) {
+    uint32_t e = 0;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const bool ok = !partial || RPL * i + sr < nvalid;
+      e = max(e, ok ? ex[i] : 0u);
+    }
+    return (int)wave_max_u32(e);
+  };
+  // Q fragments: B operand, lane n = head of the group (zero beyond G).  Block-float-8: half
+  // precision, scaled by 2^(127 - eq) with eq the largest exponent field of the segment's Q.
+  int eq = 0;
+  auto load_q = [&](const Cursor &cu, u32x4 (&qf)[KSTEPS]) {
     const uint16_t *qp = a.q + cu.u * a.q_us + (int64_t)(cu.h * G + min(n, G - 1)) * a.q_hs + 8 * h;
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
       uint4 t = *reinterpret_cast<const uint4 *>(qp + 16 * s);
       if (n >= G) t = make_uint4(0, 0, 0, 0);
-      qf[s] = __builtin_bit_cast(bf16x8, t);
+      qf[s] = u32x4{t.x, t.y, t.z, t.w};
+    }
+    if constexpr (BFP8) {
+      uint32_t em = 0;
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          em = max(em, max((qf[s][j] >> 7) & 0xffu, (qf[s][j] >> 23) & 0xffu));
+      eq = (int)min(wave_max_u32(em), 253u);
+      const float qs = __builtin_bit_cast(float, (uint32_t)(254 - eq) << 23);
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          qf[s][j] = pack_half2(bf16_lo(qf[s][j]) * qs, bf16_hi(qf[s][j]) * qs);
     }
   };
 
@@ -162,7 +198,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
   int64_t eo[NOFF], xo[NOFF];
   u32x4 kraw[NL], vraw[NL];
   uint32_t kex[NL], vex[NL];
-  bf16x8 qf[KSTEPS];
+  u32x4 qf[KSTEPS];
   tile_offsets(cur, eo, xo);
   fetch(a.k, eo, xo, kraw, kex);
   fetch(a.v, eo, xo, vraw, vex);
@@ -175,6 +211,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
+  int ev_run = 0;  // block-float-8: reference exponent of the V accumulator
 
   auto process_tile = [&](auto has_next_tag) {
     constexpr bool has_next = decltype(has_next_tag)::value;
@@ -197,20 +234,23 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
         fetch(a.v, eo, xo, vraw, vex);
       }
     };
+    int eref_k = 0, eref_v = 0;
     if constexpr (BFP8) {
-      // expansion is long: move the raw tile to a second register set so that the loads of
-      // the next tile are in flight while this one is expanded and staged
+      // move the raw tile to a second register set so that the loads of the next tile are in
+      // flight while this one is expanded and staged
       u32x4 kcur[NL], vcur[NL];
       uint32_t kexc[NL], vexc[NL];
 #pragma unroll
       for (int i = 0; i < NL; ++i) kcur[i] = kraw[i], vcur[i] = vraw[i], kexc[i] = kex[i], vexc[i] = vex[i];
       prefetch_next();
       __builtin_amdgcn_sched_barrier(0);
-      stage(ks, KS, kcur, kexc, nvalid, false);
-      stage(vs, VS, vcur, vexc, nvalid, partial);
+      eref_k = tile_exponent(kexc, nvalid, partial);
+      eref_v = tile_exponent(vexc, nvalid, partial);
+      stage(ks, KS, kcur, kexc, eref_k, nvalid, partial);
+      stage(vs, VS, vcur, vexc, eref_v, nvalid, partial);
     } else {
-      stage(ks, KS, kraw, kex, nvalid, false);
-      stage(vs, VS, vraw, vex, nvalid, partial);  // unattended V rows must not carry Inf / NaN
+      stage(ks, KS, kraw, kex, 0, nvalid, false);
+      stage(vs, VS, vraw, vex, 0, nvalid, partial);  // unattended V rows must not carry Inf / NaN
       prefetch_next();
     }
 
@@ -223,8 +263,8 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
       const uint16_t *krow = ks + (32 * kb + n) * KS + 8 * h;
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
-        bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(krow + 16 * s));
-        st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], st[kb], 0, 0, 0);
+        const uint4 kq = *reinterpret_cast<const uint4 *>(krow + 16 * s);
+        st[kb] = mma<BFP8>(u32x4{kq.x, kq.y, kq.z, kq.w}, qf[s], st[kb]);
       }
     }
     // ---- online softmax, one head per lane --------------------------------------------------
@@ -241,7 +281,9 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
 #pragma unroll
     for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(st[0][r], st[1][r]));
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-    const float scale = a.scale_log2e;  // > 0 or < 0: the maximum is tracked on scaled scores
+    // > 0 or < 0: the maximum is tracked on scaled scores.  Block-float-8: the factors taken
+    // out of the K tile and out of Q come back here.
+    const float scale = BFP8 ? __builtin_ldexpf(a.scale_log2e, eref_k + eq - 260) : a.scale_log2e;
     mloc *= scale;
     // a negative scale would turn the max into a min; scores are scaled before comparing then
     if (scale < 0.f) {
@@ -257,24 +299,47 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
     m_run = m_new;
     float lsum = 0.f;
-    bf16x8 pf[2][2];
+    u32x4 pf[2][2];
+    float alpha_acc = alpha;
+    if constexpr (BFP8) {
+      // bring this tile's V factor and the accumulator to the larger reference exponent
+      const int ev_new = max(ev_run, eref_v);
+      const float pscale = __builtin_ldexpf(1.f, eref_v - ev_new);
+      alpha_acc = alpha * __builtin_ldexpf(1.f, ev_run - ev_new);
+      ev_run = ev_new;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
+        for (int s = 0; s < 2; ++s)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float p = __builtin_amdgcn_exp2f(fmaf(st[kb][8 * s + e], scale, -m_safe));
-          __bf16 pb = (__bf16)p;
-          lsum += (float)pb;  // the normaliser sums the weights that multiply V
-          pf[kb][s][e] = pb;
+          for (int e = 0; e < 8; e += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(st[kb][8 * s + e], scale, -m_safe));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(st[kb][8 * s + e + 1], scale, -m_safe));
+            lsum += p0 + p1;  // half-precision rounding of the weights is 2^-12: not tracked
+            pf[kb][s][e >> 1] = pack_half2(p0 * pscale, p1 * pscale);
+          }
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          bf16x8 pb8;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            float p = __builtin_amdgcn_exp2f(fmaf(st[kb][8 * s + e], scale, -m_safe));
+            __bf16 pb = (__bf16)p;
+            lsum += (float)pb;  // the normaliser sums the weights that multiply V
+            pb8[e] = pb;
+          }
+          pf[kb][s] = __builtin_bit_cast(u32x4, pb8);
         }
+    }
     l_run = l_run * alpha + lsum;
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+    if (__builtin_amdgcn_ballot_w64(alpha_acc != 1.0f) != 0) {
 #pragma unroll
       for (int i = 0; i < DBLK; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][r] *= alpha;
+        for (int r = 0; r < 16; ++r) acc[i][r] *= alpha_acc;
     }
     // ---- O^T += V^T . P^T (V^T fragments through the transposing LDS load) -------------------
     const int grp = lane >> 4, a16 = lane & 15;
@@ -289,11 +354,8 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
           typedef __attribute__((address_space(3))) shortx4 *lds_v4;
           shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk + 32 * db));
           shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk + 8 * VS + 32 * db));
-          bf16x8 vf;
-          bf16x4 l4 = __builtin_bit_cast(bf16x4, lo), h4 = __builtin_bit_cast(bf16x4, hi);
-          vf[0] = l4[0], vf[1] = l4[1], vf[2] = l4[2], vf[3] = l4[3];
-          vf[4] = h4[0], vf[5] = h4[1], vf[6] = h4[2], vf[7] = h4[3];
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kb][s], acc[db], 0, 0, 0);
+          const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+          acc[db] = mma<BFP8>(u32x4{l2.x, l2.y, h2.x, h2.y}, pf[kb][s], acc[db]);
         }
       }
 
@@ -301,6 +363,14 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
     if (!same_seg) {
       float *slot = a.ws_slots + ((int64_t)wave + (int64_t)cur.u * a.hkv + cur.h) * a.slot_floats;
       const float l_tot = l_run + __shfl_xor(l_run, 32);
+      if constexpr (BFP8) {
+        const float vout = __builtin_ldexpf(1.f, ev_run - 133);
+#pragma unroll
+        for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][r] *= vout;
+        ev_run = 0;
+      }
       if (n < G) {
         float *dst = slot + n * D + 4 * h;
 #pragma unroll

@@ -1,0 +1,387 @@
+// Paged decode attention over a block-float-8 KV cache on the 16x16x32 matrix-core shape:
+// head size 128, up to 16 query heads per KV head, two workgroups (eight wavefronts) per CU.
+//
+// Work decomposition, partial slots and merge kernel are those of decode.hip.  Inside a
+// wavefront a 64-token tile of K, then of V, goes global -> registers -> half precision in a
+// 16 KiB wave-private LDS buffer that both tensors use in turn:
+//   stage K(t) | prefetch K(t+1) | S^T = K Q^T | softmax | stage V(t) | prefetch V(t+1) | O^T += V^T P^T
+// so every global load has three quarters of a tile period to arrive, and the second
+// wavefront of the SIMD fills what is left.  The byte -> half expansion is the one of
+// decode_mfma.hip (one permute and one packed fma per element pair, exponents relative to the
+// tile's largest, running reference exponent for the V accumulator).
+//
+// v_mfma_f32_16x16x32_f16 with the heads as the 16-wide N dimension:
+//   S^T block b (16 keys):  A = K rows 16 b + lane%16, 8 elements per lane and k-step
+//                           B = Q, lane%16 = head;   C: lane (head, quad) holds keys 16 b + 4 quad + r
+//   O^T block db (16 d):    the 32 k slots of a step are the keys lane (., quad) already holds
+//                           from blocks 2 s and 2 s + 1, so the probabilities are the B operand
+//                           as they are; A = V^T through two transposing LDS loads (4 keys each)
+// Compared with the 32x32x16 kernel, a lane carries half the scores and half the
+// accumulator, and the matrix pipe is busy half as long per tile.
+//
+// LDS tile: 64 rows of 256 bytes, unpadded, sixteen 16-byte chunks per row stored at
+// chunk ^ (row & 15) for K (A-operand reads: 16 rows, one chunk column) and at
+// chunk ^ (2 y | y & 1), y = row & 3, for V (transposing reads: 4 rows x 2 chunks); both make
+// the staging writes of two neighbouring rows land in different banks as well.
+#include "decode_common.h"
+
+namespace ttpa {
+namespace decode {
+namespace {
+
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kMaxUsers16 = 1024;
+constexpr int kTileBytes = kTile * 256;
+
+__device__ __forceinline__ floatx4 mma16(const u32x4 &x, const u32x4 &y, const floatx4 &c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, x),
+                                                __builtin_bit_cast(halfx8, y), c, 0, 0, 0);
+}
+
+// Maximum over the four lanes that share lane%16.  v_permlane16_swap exchanges the odd rows
+// of its first operand with the even rows of its second, v_permlane32_swap the upper half of
+// the first with the lower half of the second; fed with two copies of a value, the two
+// results hold the value of either partner.  Written as assembly: through the builtins the
+// compiler takes the two results for equal.
+__device__ __forceinline__ float max_over_quads(float v) {
+  float x = v, y = v;
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+  float m = fmaxf(x, y);
+  x = m, y = m;
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+  return fmaxf(x, y);
+}
+__device__ __forceinline__ float sum_over_quads(float v) {
+  float x = v, y = v;
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+  float m = x + y;
+  x = m, y = m;
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+  return x + y;
+}
+
+template <bool BIG>
+__global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
+    DecodeArgs a, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
+  constexpr int D = 128;
+  constexpr int KSTEPS = D / 32, DBLK = D / 16;
+  // staging geometry: a load instruction covers 8 whole token rows, 16 element bytes per lane
+  constexpr int LPR = 8, RPL = 8, NL = kTile / RPL, GPR = D / 16;
+  constexpr int NOFF = BIG ? 1 : NL;
+
+  __shared__ int s_pref[kMaxUsers16 + 1];
+  __shared__ int s_len[kMaxUsers16];
+  __shared__ int s_wsum[kWavesPerBlock];
+  extern __shared__ __attribute__((aligned(16))) uint8_t tiles[];
+
+  build_prefix(a, cur_pos, s_pref, s_len, s_wsum);
+
+  const int lane = threadIdx.x & 63;
+  const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n = lane & 15, quad = lane >> 4;
+  const int wave = blockIdx.x * kWavesPerBlock + wib;
+  const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
+  const int64_t total = (int64_t)total_tiles * a.hkv;
+  const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);
+  if (total == 0 || wave >= n_eff) {
+    publish_segment_row(a, s_pref, total, n_eff);
+    return;
+  }
+  int64_t x = (int64_t)wave * total / n_eff;
+  const int64_t x_hi = (int64_t)(wave + 1) * total / n_eff;
+  uint8_t *tile = tiles + wib * kTileBytes;
+  const int G = a.hq / a.hkv;
+
+  // staging lane mapping and swizzled write positions
+  const int sr = lane / LPR, sc = lane % LPR;
+  const uint32_t lane_bytes = (uint32_t)(sr * D + sc * 16);
+  const uint32_t lane_exp = (uint32_t)(sr * GPR + sc);
+  const int64_t slab = (int64_t)(a.bs + a.bs / 16) * D;  // bytes of one (block, head)
+  // K: row 8 i + sr has row & 15 = 8 (i & 1) + sr
+  const uint32_t kw_even = (uint32_t)(sr * 256 + (((2 * sc) ^ sr) << 4));
+  const uint32_t kw_odd = (uint32_t)(sr * 256 + (((2 * sc) ^ (8 + sr)) << 4));
+  // V: row & 3 = sr & 3
+  const int vy = sr & 3;
+  const uint32_t vw = (uint32_t)(sr * 256 + (((2 * sc) ^ ((2 * vy) | (vy & 1))) << 4));
+  // A-operand reads of K: row 16 b + n, chunk 4 s + quad
+  uint32_t kr[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) kr[s] = (uint32_t)(n * 256 + (((4 * s + quad) ^ n) << 4));
+  // transposing reads of V: lane addresses row 4 quad + n / 4 (+ 16 per key block), the 8 bytes
+  // at element 16 db + 4 (n & 3)
+  uint32_t vr[DBLK];
+  {
+    const int y = n >> 2, xx = (n & 3) >> 1;
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db)
+      vr[db] = (uint32_t)((4 * quad + y) * 256 + ((((2 * db + xx) ^ ((2 * y) | (y & 1)))) << 4) +
+                          8 * (n & 1));
+  }
+
+  auto locate = [&](int64_t xx) { return locate_unit(a, s_pref, s_len, xx); };
+  auto tile_offsets = [&](const Cursor &cu, int64_t (&eo)[NOFF], int64_t (&xo)[NOFF]) {
+    const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
+    const int tok0 = cu.t * kTile;
+#pragma unroll
+    for (int i = 0; i < NOFF; ++i) {
+      const int tk = tok0 + RPL * i;
+      const int col = tk / a.bs;
+      int phys = (col < a.w) ? __builtin_amdgcn_readfirstlane(pt_row[col]) : 0;
+      if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+      const int64_t base = ((int64_t)phys * a.hkv + cu.h) * slab;
+      const int row = tk - col * a.bs;
+      eo[i] = base + (int64_t)row * D;
+      xo[i] = base + (int64_t)a.bs * D + (int64_t)row * GPR;
+    }
+  };
+  auto fetch = [&](const uint8_t *base, const int64_t (&eo)[NOFF], const int64_t (&xo)[NOFF],
+                   u32x4 (&raw)[NL], uint32_t (&ex)[NL]) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const uint8_t *erow = BIG ? base + eo[0] + i * (RPL * D) : base + eo[BIG ? 0 : i];
+      raw[i] = __builtin_nontemporal_load(
+          reinterpret_cast<const u32x4 *>(erow + static_cast<uint64_t>(lane_bytes)));
+      const uint8_t *xrow = BIG ? base + xo[0] + i * (RPL * GPR) : base + xo[BIG ? 0 : i];
+      ex[i] = __builtin_nontemporal_load(xrow + static_cast<uint64_t>(lane_exp));
+    }
+  };
+  // largest exponent byte of the tile's attended rows
+  auto tile_exponent = [&](const uint32_t (&ex)[NL], int nvalid, bool partial) {
+    uint32_t e = 0;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const bool ok = !partial || RPL * i + sr < nvalid;
+      e = max(e, ok ? ex[i] : 0u);
+    }
+    return (int)wave_max_u32(e);
+  };
+  // registers -> LDS, expanded to half precision relative to the exponent `eref`; rows past
+  // `nvalid` of a partial tile are written as zeros
+  auto stage = [&](bool is_v, const u32x4 (&raw)[NL], const uint32_t (&ex)[NL], int eref,
+                   int nvalid, bool partial) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const bool keep = !partial || RPL * i + sr < nvalid;
+      // 2^(e - eref) as a half: through the float with exponent field e - eref + 127; the
+      // conversion is exact down to 2^-24 and gives zero below
+      const int field = max((int)ex[i] - (eref - 127), 0);
+      const float sf = keep ? __builtin_bit_cast(float, (uint32_t)min(field, 127) << 23) : 0.f;
+      const _Float16 sh = (_Float16)sf;
+      const halfx2 s2 = {sh, sh};
+      const halfx2 c2 = s2 * halfx2{(_Float16)-1152.f, (_Float16)-1152.f};
+      uint32_t o[8];
+      expand4_half(raw[i].x, s2, c2, o[0], o[1]);
+      expand4_half(raw[i].y, s2, c2, o[2], o[3]);
+      expand4_half(raw[i].z, s2, c2, o[4], o[5]);
+      expand4_half(raw[i].w, s2, c2, o[6], o[7]);
+      const uint32_t w0 = (is_v ? vw : ((i & 1) ? kw_odd : kw_even)) + (uint32_t)(i * RPL * 256);
+      *reinterpret_cast<uint4 *>(tile + w0) = make_uint4(o[0], o[1], o[2], o[3]);
+      *reinterpret_cast<uint4 *>(tile + (w0 ^ 16u)) = make_uint4(o[4], o[5], o[6], o[7]);
+    }
+  };
+  // Q fragments: B operand, lane%16 = head of the group (zero beyond G), half precision,
+  // scaled by 2^(127 - eq) with eq the largest exponent field of the segment's Q
+  int eq = 0;
+  auto load_q = [&](const Cursor &cu, u32x4 (&qf)[KSTEPS]) {
+    const uint16_t *qp =
+        a.q + cu.u * a.q_us + (int64_t)(cu.h * G + min(n, G - 1)) * a.q_hs + 8 * quad;
+    uint32_t em = 0;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      uint4 t = *reinterpret_cast<const uint4 *>(qp + 32 * s);
+      if (n >= G) t = make_uint4(0, 0, 0, 0);
+      qf[s] = u32x4{t.x, t.y, t.z, t.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        em = max(em, max((qf[s][j] >> 7) & 0xffu, (qf[s][j] >> 23) & 0xffu));
+    }
+    eq = (int)min(wave_max_u32(em), 253u);
+    const float qs = __builtin_bit_cast(float, (uint32_t)(254 - eq) << 23);
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        qf[s][j] = pack_half2(bf16_lo(qf[s][j]) * qs, bf16_hi(qf[s][j]) * qs);
+  };
+
+  Cursor cur = locate(x);
+  int64_t eo[NOFF], xo[NOFF];
+  u32x4 kraw[NL], vraw[NL];
+  uint32_t kex[NL], vex[NL];
+  u32x4 qf[KSTEPS];
+  tile_offsets(cur, eo, xo);
+  fetch(a.k, eo, xo, kraw, kex);
+  fetch(a.v, eo, xo, vraw, vex);
+  load_q(cur, qf);
+  publish_segment_row(a, s_pref, total, n_eff);
+
+  floatx4 acc[DBLK];
+#pragma unroll
+  for (int i = 0; i < DBLK; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+  int ev_run = 0;  // reference exponent of the V accumulator
+
+  auto process_tile = [&](auto has_next_tag) {
+    constexpr bool has_next = decltype(has_next_tag)::value;
+    const int nvalid = cur.len - cur.t * kTile;
+    const bool partial = nvalid < kTile;
+    const int nbelow = cur.lo - cur.t * kTile;  // sliding window: > 0 only in a segment's first tile
+    const bool same_seg = has_next && cur.tiles_left > 1;
+    Cursor nxt = cur;
+
+    // ---- K: registers -> LDS, then the next tile's K: global -> registers -------------------
+    const int eref_k = tile_exponent(kex, nvalid, partial);
+    stage(false, kraw, kex, eref_k, nvalid, partial);
+    if constexpr (has_next) {
+      if (same_seg) {
+        nxt.t = cur.t + 1;
+        nxt.tiles_left = cur.tiles_left - 1;
+      } else {
+        nxt = locate(x + 1);
+      }
+      tile_offsets(nxt, eo, xo);
+      fetch(a.k, eo, xo, kraw, kex);
+    }
+
+    // ---- S^T = K . Q^T ------------------------------------------------------------------------
+    floatx4 st[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      st[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {
+        const uint4 kq = *reinterpret_cast<const uint4 *>(tile + kr[s] + b * (16 * 256));
+        st[b] = mma16(u32x4{kq.x, kq.y, kq.z, kq.w}, qf[s], st[b]);
+      }
+    }
+    // ---- online softmax: lane (head, quad) holds keys 16 b + 4 quad + r ------------------------
+    if (partial || nbelow > 0) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int key = 16 * b + 4 * quad + r;
+          if (key >= nvalid || key < nbelow) st[b][r] = -INFINITY;
+        }
+    }
+    // the factors taken out of the K tile and out of Q come back in the scale
+    const float scale = __builtin_ldexpf(a.scale_log2e, eref_k + eq - 260);
+    float mloc = -INFINITY;
+    if (scale >= 0.f) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mloc = fmaxf(mloc, st[b][r]);
+      mloc *= scale;
+    } else {  // a negative scale turns the maximum into a minimum: compare scaled scores
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mloc = fmaxf(mloc, st[b][r] * scale);
+    }
+    mloc = max_over_quads(mloc);
+    const float m_new = fmaxf(m_run, mloc);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
+    m_run = m_new;
+
+    // ---- V: registers -> LDS (the K tile has been consumed), next tile's V -> registers -------
+    const int eref_v = tile_exponent(vex, nvalid, partial);
+    stage(true, vraw, vex, eref_v, nvalid, partial);
+    if constexpr (has_next) fetch(a.v, eo, xo, vraw, vex);
+
+    // bring this tile's V factor and the accumulator to the larger reference exponent
+    const int ev_new = max(ev_run, eref_v);
+    const float pscale = __builtin_ldexpf(1.f, eref_v - ev_new);
+    const float alpha_acc = alpha * __builtin_ldexpf(1.f, ev_run - ev_new);
+    ev_run = ev_new;
+    float lsum = 0.f;
+    u32x4 pf[2];
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int r = 0; r < 4; r += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(fmaf(st[b][r], scale, -m_safe));
+        const float p1 = __builtin_amdgcn_exp2f(fmaf(st[b][r + 1], scale, -m_safe));
+        lsum += p0 + p1;  // half-precision rounding of the weights is 2^-12: not tracked
+        pf[b >> 1][2 * (b & 1) + (r >> 1)] = pack_half2(p0 * pscale, p1 * pscale);
+      }
+    l_run = l_run * alpha + lsum;
+    if (__builtin_amdgcn_ballot_w64(alpha_acc != 1.0f) != 0) {
+#pragma unroll
+      for (int i = 0; i < DBLK; ++i) acc[i] *= alpha_acc;
+    }
+    // ---- O^T += V^T . P^T ------------------------------------------------------------------------
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int db = 0; db < DBLK; ++db) {
+        typedef __attribute__((address_space(3))) shortx4 *lds_v4;
+        const uint8_t *vp = tile + vr[db] + s * (32 * 256);
+        shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vp));
+        shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vp + 16 * 256));
+        const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+        acc[db] = mma16(u32x4{l2.x, l2.y, h2.x, h2.y}, pf[s], acc[db]);
+      }
+
+    // ---- close the segment --------------------------------------------------------------------
+    if (!same_seg) {
+      float *slot = a.ws_slots + ((int64_t)wave + (int64_t)cur.u * a.hkv + cur.h) * a.slot_floats;
+      const float l_tot = sum_over_quads(l_run);
+      const float vout = __builtin_ldexpf(1.f, ev_run - 133);
+      if (n < G) {
+        float *dst = slot + n * D + 4 * quad;
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db)
+          *reinterpret_cast<float4 *>(dst + 16 * db) = make_float4(
+              acc[db][0] * vout, acc[db][1] * vout, acc[db][2] * vout, acc[db][3] * vout);
+        if (quad == 0) {
+          slot[G * D + n] = m_run;
+          slot[G * D + G + n] = l_tot;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < DBLK; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+      m_run = -INFINITY;
+      l_run = 0.f;
+      ev_run = 0;
+      if constexpr (has_next) load_q(nxt, qf);
+    }
+    cur = nxt;
+    ++x;
+  };
+  while (x + 1 < x_hi) process_tile(std::true_type{});
+  process_tile(std::false_type{});
+}
+
+template <bool BIG>
+bool launch(const DecodeArgs &a, hipStream_t st) {
+  const int blocks = a.n_waves / kWavesPerBlock;
+  const size_t lds = (size_t)kWavesPerBlock * kTileBytes;
+  static bool once = false;
+  if (!once) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&paged_decode_bfp8_mfma_kernel<BIG>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return false;
+    once = true;
+  }
+  paged_decode_bfp8_mfma_kernel<BIG><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
+  return true;
+}
+
+}  // namespace
+
+bool mfma16_decode_supported(const DecodeArgs &a, int head_size, int g) {
+  return a.kv_format == TTPA_KV_BFP8 && head_size == 128 && g <= 16 && a.users <= kMaxUsers16 &&
+         a.bs % 8 == 0;
+}
+
+bool launch_mfma16_main(const DecodeArgs &a, hipStream_t st) {
+  return a.bs % kTile == 0 ? launch<true>(a, st) : launch<false>(a, st);
+}
+
+}  // namespace decode
+}  // namespace ttpa
