@@ -41,7 +41,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 # to the default seed and shapes of the workload it is keyed by.
 MEASURED_TRAFFIC_BYTES = {"config2": 306301 * 1024}
 DECODE_KERNEL_NAME = {"config2": "paged_decode_kernel", "config4": "paged_decode_mfma_kernel",
-                      "config5": "paged_decode_bfp8_kernel"}
+                      "config5": "paged_decode_bfp8_mfma_kernel"}
 CPU_THREADS_CAP = 16        # host cores a one-GPU box grants, whatever os.cpu_count() says
 
 

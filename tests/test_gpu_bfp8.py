@@ -118,3 +118,71 @@ def test_decode_bfp8_config5_reduced_and_property():
     wl = workloads.decode_config5(users=8, num_blocks=600)
     out = _decode_vs_roundtrip(wl, wl.name + " (8 users)")
     assert torch.isfinite(out).all()
+
+
+@pytest.mark.parametrize("kernel", ["valu", "mfma", "mfma16"])
+@pytest.mark.parametrize("users,hq,hkv,d,bs,ctx", [
+    (4, 32, 8, 128, 64, [5, 64, 200, 700]),
+    (3, 12, 4, 128, 16, [15, 16, 100]),
+])
+def test_decode_bfp8_every_kernel(monkeypatch, kernel, users, hq, hkv, d, bs, ctx):
+    """The three main kernels that can serve a block-float-8 cache (VALU, 32x32x16 and 16x16x32
+    matrix-core), each forced in turn on the same data."""
+    from tt_xla_amd import workloads
+
+    monkeypatch.setenv("TTPA_DECODE_KERNEL", kernel)
+    name = f"bfp8 decode [{kernel}] b{users} h{hq}x{hkv} d{d} bs{bs} ctx{ctx}"
+    print(name, flush=True)
+    nb = sum((c + 1 + bs - 1) // bs for c in ctx) + 3
+    wl = workloads.decode_ragged(name, hq + d + bs, users, hq, hkv, d, bs, nb, ctx)
+    workloads.add_outlier_channels(wl, 9, fraction=0.02)
+    _decode_vs_roundtrip(wl, name)
+
+
+@pytest.mark.parametrize("kernel", ["valu", "mfma", "mfma16"])
+def test_decode_bfp8_several_tiles_per_wavefront(monkeypatch, kernel):
+    """A grid of one wavefront per CU over ~1000 tiles: every wavefront walks several tiles and
+    crosses segment boundaries, so the running maximum, the running V exponent, the partial
+    hand-over and the Q reload are all exercised."""
+    from tt_xla_amd import workloads
+
+    monkeypatch.setenv("TTPA_DECODE_KERNEL", kernel)
+    monkeypatch.setenv("TTPA_DECODE_WAVES_PER_CU", "1")
+    ctx = [1990, 2047, 1500, 2300]
+    name = f"bfp8 decode [{kernel}] one wavefront per CU ctx{ctx}"
+    print(name, flush=True)
+    nb = sum((c + 1 + 63) // 64 for c in ctx) + 3
+    wl = workloads.decode_ragged(name, 77, 4, 32, 8, 128, 64, nb, ctx)
+    workloads.add_outlier_channels(wl, 9, fraction=0.02)
+    _decode_vs_roundtrip(wl, name)
+
+
+@pytest.mark.parametrize("kernel", ["mfma", "mfma16"])
+def test_decode_bfp8_exponent_spread(monkeypatch, kernel):
+    """K / V magnitudes that change by large powers of two from tile to tile and from group to
+    group, and a large Q: the matrix-core kernels expand a tile relative to its largest
+    exponent byte and carry a running exponent for the V accumulator; both have to follow."""
+    from tt_xla_amd import workloads
+
+    monkeypatch.setenv("TTPA_DECODE_KERNEL", kernel)
+    monkeypatch.setenv("TTPA_DECODE_WAVES_PER_CU", "1")
+    ctx = [700, 1023, 1500, 640]
+    name = f"bfp8 decode [{kernel}] exponent spread ctx{ctx}"
+    print(name, flush=True)
+    nb = sum((c + 1 + 63) // 64 for c in ctx) + 3
+    wl = workloads.decode_ragged(name, 78, 4, 32, 8, 128, 64, nb, ctx)
+    g = torch.Generator().manual_seed(5)
+    # per physical block (= tile) and per 16-element group a power of two
+    nblk = wl.k_cache.shape[0]
+    # (the 16x16x32 kernel writes a group more than 2^14 below its tile's largest as zeros, the
+    # 32x32x16 kernel one more than 2^24 below: the spread inside a tile stays within 2^10 here)
+    for cache, lo, hi in ((wl.k_cache, -10, -4), (wl.v_cache, -12, 2)):
+        e_blk = torch.randint(lo, hi + 1, (nblk, 1, 1, 1), generator=g).float()
+        e_grp = torch.randint(-10, 1, (1, cache.shape[1], 1, 8), generator=g).float()
+        e_grp = e_grp.repeat_interleave(16, dim=-1)
+        cache.copy_((cache.float() * torch.exp2(e_blk) * torch.exp2(e_grp)).to(torch.bfloat16))
+    wl.k_cache[1] = 0  # a block of zeros
+    wl.v_cache[2] = 0
+    wl.q.copy_((wl.q.float() * 2.0**8).to(torch.bfloat16))
+    wl.q[0, 1] *= 2.0**-30  # one user with a tiny query
+    _decode_vs_roundtrip(wl, name)

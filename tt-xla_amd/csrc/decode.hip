@@ -280,11 +280,10 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
 }
 
 int waves_for_device(int kv_format) {
-  static int override_waves = -1;
-  if (override_waves < 0) {
-    const char *e = getenv("TTPA_DECODE_WAVES_PER_CU");
-    override_waves = e ? atoi(e) : 0;
-  }
+  // TTPA_DECODE_WAVES_PER_CU (read on every call) overrides the grid size: tests use a small
+  // grid to give every wavefront several tiles and segments
+  const char *e = getenv("TTPA_DECODE_WAVES_PER_CU");
+  const int override_waves = e ? atoi(e) : 0;
   int per_cu = override_waves > 0 ? override_waves : (kv_format == TTPA_KV_BFP8 ? 8 : 4);
   int cus = device_cus();
   if (cus <= 0) cus = 256;
@@ -402,11 +401,13 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   // operation per element and the products none, while the VALU kernel pays for both; head
   // size 128 with up to 16 heads per group has the 16x16x32 kernel with twice the occupancy.
   // TTPA_DECODE_KERNEL=valu|mfma|mfma16 overrides the choice.
-  static int forced = -1;
-  if (forced < 0) {
-    const char *e = getenv("TTPA_DECODE_KERNEL");
-    forced = !e ? 0 : (!strcmp(e, "valu") ? 1 : (!strcmp(e, "mfma") ? 2 : (!strcmp(e, "mfma16") ? 3 : 0)));
-  }
+  // read on every call (a getenv is negligible next to a launch) so that a process can
+  // exercise every kernel
+  const char *forced_name = getenv("TTPA_DECODE_KERNEL");
+  const int forced = !forced_name ? 0
+                     : !strcmp(forced_name, "valu") ? 1
+                     : !strcmp(forced_name, "mfma") ? 2
+                     : !strcmp(forced_name, "mfma16") ? 3 : 0;
   const bool mfma_ok = mfma_decode_supported(a, head_size, g);
   const bool mfma16_ok = mfma16_decode_supported(a, head_size, g);
   bool use_mfma16 = mfma16_ok;
@@ -414,8 +415,10 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   if (forced == 1) use_mfma = use_mfma16 = false;
   if (forced == 2) use_mfma = mfma_ok, use_mfma16 = false;
   if (forced == 3) use_mfma16 = mfma16_ok, use_mfma = !mfma16_ok && use_mfma;
-  // the 32x32 matrix-core kernel runs one workgroup per CU whatever the cache format
-  a.n_waves = waves_for_device(use_mfma ? TTPA_KV_BF16 : kv_format);
+  // The matrix-core kernels get one workgroup per CU whatever the cache format: the 32x32 kernel
+  // fills the CU's LDS with one, and the 16x16 kernel streams as fast with one as with the two
+  // that would fit, while twice the partials cost the merge kernel more.
+  a.n_waves = waves_for_device((use_mfma || use_mfma16) ? TTPA_KV_BF16 : kv_format);
   hipEvent_t ev0, ev1;
   take_profile_events(ev0, ev1);
   if (ev0) (void)hipEventRecord(ev0, st);

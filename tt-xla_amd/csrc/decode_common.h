@@ -377,7 +377,7 @@ bool launch_bfp8_main(const DecodeArgs &a, int head_size, int g, hipStream_t st)
 bool mfma_decode_supported(const DecodeArgs &a, int head_size, int g);
 bool launch_mfma_main(const DecodeArgs &a, int head_size, hipStream_t st);
 // Matrix-core main kernel for the block-float-8 cache with head size 128 and up to 16 query
-// heads per KV head (decode_mfma16.hip): two workgroups per CU.
+// heads per KV head (decode_mfma16.hip).
 bool mfma16_decode_supported(const DecodeArgs &a, int head_size, int g);
 bool launch_mfma16_main(const DecodeArgs &a, hipStream_t st);
 

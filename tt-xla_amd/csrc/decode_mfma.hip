@@ -94,7 +94,11 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
   // staging lane mapping
   const int sr = lane / LPR, sc = lane % LPR;
   const uint32_t lane_bytes = (uint32_t)(sr * D * BPE + sc * 16);
-  const uint32_t lane_exp = (uint32_t)(sr * GPR + sc);  // block-float-8: one group per lane
+  // block-float-8: one group per lane; its exponent byte is fetched inside its aligned dword
+  // and cut out when the tile is staged (a byte load is widened where it is issued, which
+  // makes the loop wait for the load at once)
+  const uint32_t lane_exp = (uint32_t)((sr * GPR + sc) & ~3);
+  const uint32_t exp_shift = (uint32_t)(8 * ((sr * GPR + sc) & 3));
   const int64_t slab = BFP8 ? (int64_t)(a.bs + a.bs / 16) * D : (int64_t)a.bs * D * 2;  // bytes
 
   auto locate = [&](int64_t xx) { return locate_unit(a, s_pref, s_len, xx); };
@@ -122,7 +126,8 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
           reinterpret_cast<const u32x4 *>(erow + static_cast<uint64_t>(lane_bytes)));
       if constexpr (BFP8) {
         const uint8_t *xrow = BIG ? base + xo[0] + i * (RPL * GPR) : base + xo[BIG ? 0 : i];
-        ex[i] = __builtin_nontemporal_load(xrow + static_cast<uint64_t>(lane_exp));
+        ex[i] = __builtin_nontemporal_load(
+            reinterpret_cast<const uint32_t *>(xrow + static_cast<uint64_t>(lane_exp)));
       }
     }
   };
@@ -137,7 +142,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
       if constexpr (BFP8) {
         // 2^(e - eref) as a half: through the float with exponent field e - eref + 127; the
         // conversion is exact down to 2^-24 and gives zero below
-        const int field = max((int)ex[i] - (eref - 127), 0);
+        const int field = max((int)((ex[i] >> exp_shift) & 0xffu) - (eref - 127), 0);
         const float sf = keep ? __builtin_bit_cast(float, (uint32_t)min(field, 127) << 23) : 0.f;
         const _Float16 sh = (_Float16)sf;
         const halfx2 s2 = {sh, sh};
@@ -162,7 +167,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
       const bool ok = !partial || RPL * i + sr < nvalid;
-      e = max(e, ok ? ex[i] : 0u);
+      e = max(e, ok ? (ex[i] >> exp_shift) & 0xffu : 0u);
     }
     return (int)wave_max_u32(e);
   };

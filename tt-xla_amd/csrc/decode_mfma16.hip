@@ -1,12 +1,11 @@
 // Paged decode attention over a block-float-8 KV cache on the 16x16x32 matrix-core shape:
-// head size 128, up to 16 query heads per KV head, two workgroups (eight wavefronts) per CU.
+// head size 128, up to 16 query heads per KV head, 72 KiB of LDS per workgroup.
 //
 // Work decomposition, partial slots and merge kernel are those of decode.hip.  Inside a
 // wavefront a 64-token tile of K, then of V, goes global -> registers -> half precision in a
 // 16 KiB wave-private LDS buffer that both tensors use in turn:
 //   stage K(t) | prefetch K(t+1) | S^T = K Q^T | softmax | stage V(t) | prefetch V(t+1) | O^T += V^T P^T
-// so every global load has three quarters of a tile period to arrive, and the second
-// wavefront of the SIMD fills what is left.  The byte -> half expansion is the one of
+// so every global load has three quarters of a tile period to arrive.  The byte -> half expansion is the one of
 // decode_mfma.hip (one permute and one packed fma per element pair, exponents relative to the
 // tile's largest, running reference exponent for the V accumulator).
 //
@@ -21,8 +20,8 @@
 //
 // LDS tile: 64 rows of 256 bytes, unpadded, sixteen 16-byte chunks per row stored at
 // chunk ^ (row & 15) for K (A-operand reads: 16 rows, one chunk column) and at
-// chunk ^ (2 y | y & 1), y = row & 3, for V (transposing reads: 4 rows x 2 chunks); both make
-// the staging writes of two neighbouring rows land in different banks as well.
+// chunk ^ (2 y | y & 1), y = row & 7, for V (transposing reads: 32 lanes cover 8 rows x 2
+// chunks); both make the staging writes of two neighbouring rows land in different banks too.
 #include "decode_common.h"
 
 namespace ttpa {
@@ -98,14 +97,17 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
   // staging lane mapping and swizzled write positions
   const int sr = lane / LPR, sc = lane % LPR;
   const uint32_t lane_bytes = (uint32_t)(sr * D + sc * 16);
-  const uint32_t lane_exp = (uint32_t)(sr * GPR + sc);
+  // the lane's exponent byte (row sr, group sc) is fetched inside its aligned dword and cut
+  // out when the tile is staged: a byte load is widened where it is issued, which would make
+  // the loop wait for the next tile's exponents at the end of every iteration
+  const uint32_t lane_exp = (uint32_t)((sr * GPR + sc) & ~3);
+  const uint32_t exp_shift = (uint32_t)(8 * (sc & 3));
   const int64_t slab = (int64_t)(a.bs + a.bs / 16) * D;  // bytes of one (block, head)
   // K: row 8 i + sr has row & 15 = 8 (i & 1) + sr
   const uint32_t kw_even = (uint32_t)(sr * 256 + (((2 * sc) ^ sr) << 4));
   const uint32_t kw_odd = (uint32_t)(sr * 256 + (((2 * sc) ^ (8 + sr)) << 4));
-  // V: row & 3 = sr & 3
-  const int vy = sr & 3;
-  const uint32_t vw = (uint32_t)(sr * 256 + (((2 * sc) ^ ((2 * vy) | (vy & 1))) << 4));
+  // V: row & 7 = sr
+  const uint32_t vw = (uint32_t)(sr * 256 + (((2 * sc) ^ ((2 * sr) | (sr & 1))) << 4));
   // A-operand reads of K: row 16 b + n, chunk 4 s + quad
   uint32_t kr[KSTEPS];
 #pragma unroll
@@ -115,9 +117,10 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
   uint32_t vr[DBLK];
   {
     const int y = n >> 2, xx = (n & 3) >> 1;
+    const int y7 = (4 * quad + y) & 7;  // row & 7: key blocks start at multiples of 16
 #pragma unroll
     for (int db = 0; db < DBLK; ++db)
-      vr[db] = (uint32_t)((4 * quad + y) * 256 + ((((2 * db + xx) ^ ((2 * y) | (y & 1)))) << 4) +
+      vr[db] = (uint32_t)((4 * quad + y) * 256 + ((((2 * db + xx) ^ ((2 * y7) | (y7 & 1)))) << 4) +
                           8 * (n & 1));
   }
 
@@ -145,32 +148,31 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
       raw[i] = __builtin_nontemporal_load(
           reinterpret_cast<const u32x4 *>(erow + static_cast<uint64_t>(lane_bytes)));
       const uint8_t *xrow = BIG ? base + xo[0] + i * (RPL * GPR) : base + xo[BIG ? 0 : i];
-      ex[i] = __builtin_nontemporal_load(xrow + static_cast<uint64_t>(lane_exp));
+      ex[i] = __builtin_nontemporal_load(
+          reinterpret_cast<const uint32_t *>(xrow + static_cast<uint64_t>(lane_exp)));
     }
   };
-  // largest exponent byte of the tile's attended rows
-  auto tile_exponent = [&](const uint32_t (&ex)[NL], int nvalid, bool partial) {
+  // Cuts the lane's exponent bytes out of the fetched dwords (zero for rows past `nvalid` of a
+  // partial tile, which stages them as zeros) and returns the largest of the tile.
+  auto tile_exponent = [&](uint32_t (&ex)[NL], int nvalid, bool partial) {
     uint32_t e = 0;
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-      const bool ok = !partial || RPL * i + sr < nvalid;
-      e = max(e, ok ? ex[i] : 0u);
+      ex[i] = (ex[i] >> exp_shift) & 0xffu;
+      if (partial && RPL * i + sr >= nvalid) ex[i] = 0;
+      e = max(e, ex[i]);
     }
     return (int)wave_max_u32(e);
   };
-  // registers -> LDS, expanded to half precision relative to the exponent `eref`; rows past
-  // `nvalid` of a partial tile are written as zeros
-  auto stage = [&](bool is_v, const u32x4 (&raw)[NL], const uint32_t (&ex)[NL], int eref,
-                   int nvalid, bool partial) {
+  // registers -> LDS, expanded to half precision relative to the exponent `eref`: the group
+  // scale 2^(e - eref) is the half with exponent field e - eref + 15; groups more than 2^14
+  // below the tile's largest (field <= 0) are written as zeros
+  auto stage = [&](bool is_v, const u32x4 (&raw)[NL], const uint32_t (&ex)[NL], int eref) {
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-      const bool keep = !partial || RPL * i + sr < nvalid;
-      // 2^(e - eref) as a half: through the float with exponent field e - eref + 127; the
-      // conversion is exact down to 2^-24 and gives zero below
-      const int field = max((int)ex[i] - (eref - 127), 0);
-      const float sf = keep ? __builtin_bit_cast(float, (uint32_t)min(field, 127) << 23) : 0.f;
-      const _Float16 sh = (_Float16)sf;
-      const halfx2 s2 = {sh, sh};
+      const uint32_t field = (uint32_t)max((int)ex[i] - (eref - 15), 0);
+      const uint32_t sbits = field << 10;
+      const halfx2 s2 = __builtin_bit_cast(halfx2, sbits | (sbits << 16));
       const halfx2 c2 = s2 * halfx2{(_Float16)-1152.f, (_Float16)-1152.f};
       uint32_t o[8];
       expand4_half(raw[i].x, s2, c2, o[0], o[1]);
@@ -188,12 +190,12 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
   auto load_q = [&](const Cursor &cu, u32x4 (&qf)[KSTEPS]) {
     const uint16_t *qp =
         a.q + cu.u * a.q_us + (int64_t)(cu.h * G + min(n, G - 1)) * a.q_hs + 8 * quad;
+    const uint32_t qmask = n < G ? 0xffffffffu : 0u;  // no branch: a branch would wait for every load in flight
     uint32_t em = 0;
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
-      uint4 t = *reinterpret_cast<const uint4 *>(qp + 32 * s);
-      if (n >= G) t = make_uint4(0, 0, 0, 0);
-      qf[s] = u32x4{t.x, t.y, t.z, t.w};
+      const uint4 t = *reinterpret_cast<const uint4 *>(qp + 32 * s);
+      qf[s] = u32x4{t.x & qmask, t.y & qmask, t.z & qmask, t.w & qmask};
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         em = max(em, max((qf[s][j] >> 7) & 0xffu, (qf[s][j] >> 23) & 0xffu));
@@ -234,7 +236,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
 
     // ---- K: registers -> LDS, then the next tile's K: global -> registers -------------------
     const int eref_k = tile_exponent(kex, nvalid, partial);
-    stage(false, kraw, kex, eref_k, nvalid, partial);
+    stage(false, kraw, kex, eref_k);
     if constexpr (has_next) {
       if (same_seg) {
         nxt.t = cur.t + 1;
@@ -290,7 +292,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
 
     // ---- V: registers -> LDS (the K tile has been consumed), next tile's V -> registers -------
     const int eref_v = tile_exponent(vex, nvalid, partial);
-    stage(true, vraw, vex, eref_v, nvalid, partial);
+    stage(true, vraw, vex, eref_v);
     if constexpr (has_next) fetch(a.v, eo, xo, vraw, vex);
 
     // bring this tile's V factor and the accumulator to the larger reference exponent
