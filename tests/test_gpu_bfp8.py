@@ -25,6 +25,15 @@ def _bf(gen, *shape):
     return torch.randn(*shape, generator=gen).to(torch.bfloat16)
 
 
+def test_empty_cache_decodes_to_zero():
+    from tt_xla_amd import custom_ops as ops
+
+    c = ops.bfp8_empty_cache(3, 2, 32, 64, "cuda")
+    assert c.shape == ops.bfp8_cache_shape(3, 2, 32, 64)
+    assert torch.count_nonzero(C.unpack_cache(c.cpu(), 32)) == 0
+    assert torch.count_nonzero(ops.bfp8_unpack_cache(c).float()) == 0
+
+
 def test_pack_unpack_kernels_bit_exact():
     from tt_xla_amd import custom_ops as ops
 

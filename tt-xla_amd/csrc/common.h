@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "ttpa.h"
 
 namespace ttpa {
@@ -17,6 +19,11 @@ int device_cus();
 // Events armed by ttpa_profile_next_attention(); take_profile_events() hands them to the
 // launcher that brackets its dominant kernel and disarms them.
 void take_profile_events(hipEvent_t &before, hipEvent_t &after);
+
+// Raises the dynamic-LDS limit of `kernel` to `bytes` on the current device, once per device:
+// `done_devices` is the call site's own record (one bit per device ordinal; ordinals from 64
+// on are set on every call).  Returns false when the runtime refuses.
+bool ensure_dynamic_lds(const void *kernel, size_t bytes, std::atomic<uint64_t> &done_devices);
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -37,6 +37,19 @@ int device_cus() {
   return cached_cus;
 }
 
+bool ensure_dynamic_lds(const void *kernel, size_t bytes, std::atomic<uint64_t> &done_devices) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  const uint64_t bit = (dev >= 0 && dev < 64) ? (uint64_t{1} << dev) : 0;
+  if (bit && (done_devices.load(std::memory_order_acquire) & bit)) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  if (bit) done_devices.fetch_or(bit, std::memory_order_release);
+  return true;
+}
+
 static thread_local hipEvent_t g_ev_before = nullptr, g_ev_after = nullptr;
 
 void take_profile_events(hipEvent_t &before, hipEvent_t &after) {

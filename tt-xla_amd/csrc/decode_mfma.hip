@@ -409,22 +409,14 @@ bool launch(const DecodeArgs &a, hipStream_t st) {
   const int blocks = a.n_waves / kWavesPerBlock;
   const size_t lds = (size_t)kWavesPerBlock * kTile * ((D + 8) + (D + 32)) * 2;
   if (a.bs % kTile == 0) {
-    static bool once = false;
-    if (!once) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void *>(&paged_decode_mfma_kernel<D, BFP8, true>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-        return false;
-      once = true;
-    }
+    static std::atomic<uint64_t> lds_ready{0};
+    if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_mfma_kernel<D, BFP8, true>), lds, lds_ready))
+      return false;
     paged_decode_mfma_kernel<D, BFP8, true><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
   } else {
-    static bool once = false;
-    if (!once) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void *>(&paged_decode_mfma_kernel<D, BFP8, false>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-        return false;
-      once = true;
-    }
+    static std::atomic<uint64_t> lds_ready{0};
+    if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_mfma_kernel<D, BFP8, false>), lds, lds_ready))
+      return false;
     paged_decode_mfma_kernel<D, BFP8, false><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
   }
   return true;

@@ -363,13 +363,9 @@ template <bool BIG>
 bool launch(const DecodeArgs &a, hipStream_t st) {
   const int blocks = a.n_waves / kWavesPerBlock;
   const size_t lds = (size_t)kWavesPerBlock * kTileBytes;
-  static bool once = false;
-  if (!once) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&paged_decode_bfp8_mfma_kernel<BIG>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return false;
-    once = true;
-  }
+  static std::atomic<uint64_t> lds_ready{0};
+  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_bfp8_mfma_kernel<BIG>), lds, lds_ready))
+    return false;
   paged_decode_bfp8_mfma_kernel<BIG><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
   return true;
 }

@@ -294,13 +294,10 @@ template <int DQK, int DVW, bool SHARED_V>
 bool launch(const DecodeArgs &a, const WideArgs &w, hipStream_t st) {
   using L = WideLds<DQK, DVW, SHARED_V>;
   const size_t lds = 2 * (size_t)L::STAGE;
-  static bool once = false;
-  if (!once) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&paged_decode_wide_kernel<DQK, DVW, SHARED_V>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return false;
-    once = true;
-  }
+  static std::atomic<uint64_t> lds_ready{0};
+  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_wide_kernel<DQK, DVW, SHARED_V>), lds,
+                          lds_ready))
+    return false;
   paged_decode_wide_kernel<DQK, DVW, SHARED_V><<<dim3(a.n_waves), dim3(256), lds, st>>>(a, w, a.pt, a.cur);
   return true;
 }

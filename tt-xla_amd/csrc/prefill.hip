@@ -420,13 +420,9 @@ int launch_mode(const PrefillArgs &a, hipStream_t st) {
   constexpr int ROWS = kRowsPerWave;
   const int nqt = (a.sq + ROWS * RPW - 1) / (ROWS * RPW);
   const size_t lds = 2 * Tile<D>::STAGE_BYTES;  // two stages
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&prefill_kernel<D, HPW, MODE>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return fail(TTPA_ERR_LAUNCH, "prefill: cannot reserve %zu bytes of LDS", lds);
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ready{0};
+  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&prefill_kernel<D, HPW, MODE>), lds, lds_ready))
+    return fail(TTPA_ERR_LAUNCH, "prefill: cannot reserve %zu bytes of LDS", lds);
   hipEvent_t ev0, ev1;
   take_profile_events(ev0, ev1);
   if (ev0) (void)hipEventRecord(ev0, st);

@@ -86,6 +86,16 @@ def bfp8_cache_shape(num_blocks: int, num_kv_heads: int, block_size: int, head_s
     return (num_blocks, num_kv_heads, block_size + block_size // _BFP8_GROUP, head_size)
 
 
+def bfp8_empty_cache(num_blocks: int, num_kv_heads: int, block_size: int, head_size: int, device):
+    """A block-float-8 cache that decodes to zeros everywhere: element bytes 128 (offset binary
+    zero), exponent bytes 0.  An all-zero tensor is a valid cache too, but its never-written
+    positions decode to -2^-126 rather than 0."""
+    cache = torch.zeros(bfp8_cache_shape(num_blocks, num_kv_heads, block_size, head_size),
+                        dtype=torch.uint8, device=device)
+    cache[:, :, :block_size, :] = 128
+    return cache
+
+
 # --------------------------------------------------------------------------- #
 # cache writes
 # --------------------------------------------------------------------------- #
