@@ -52,6 +52,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--rotate", type=int, default=3, help="independent workload copies cycled through")
     ap.add_argument("--launch", choices=["graph", "eager"], default="graph")
+    ap.add_argument("--steps-per-graph", type=int, default=6,
+                    help="consecutive steps captured in one graph (a decode forward replays one "
+                         "attention step per layer inside one graph); 1 = one graph launch per step")
     ap.add_argument("--workload", choices=["config2", "config3", "config4", "config5"], default="config2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-users", type=int, default=0, help="users in the CPU sample (0 = auto)")
@@ -122,37 +125,70 @@ def prefill_step(impl, w, out):
 
 
 # --------------------------------------------------------------------------- timing helpers
-def build_launchers(fns, use_graph):
+class StepRunner:
+    """Runs steps over the rotating workload copies (step i uses copy i % n).  In graph mode a
+    graph holds `per_graph` consecutive steps (rounded up to a multiple of n so the rotation
+    continues across replays), the way the decode forward of a model replays one attention step
+    per layer inside a single graph; a shorter graph covers the remainder so that run(k)
+    executes exactly k steps."""
+
+    def __init__(self, fns, use_graph, per_graph):
+        import torch
+
+        self.fns, self.n, self.use_graph = fns, len(fns), use_graph
+        self.per_graph = max(1, (max(1, per_graph) + self.n - 1) // self.n * self.n)
+        self.graphs, self.keep = {}, []
+        if use_graph:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for f in fns:  # warm allocator and kernels outside capture
+                    f()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+
+    def _graph(self, length):
+        import torch
+
+        if length not in self.graphs:
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                for i in range(length):
+                    self.keep.append(self.fns[i % self.n]())
+            self.graphs[length] = gr
+        return self.graphs[length]
+
+    def prepare(self, steps):
+        if self.use_graph:
+            full, rem = divmod(steps, self.per_graph)
+            if full:
+                self._graph(self.per_graph)
+            if rem:
+                self._graph(rem)
+
+    def run(self, steps):
+        if not self.use_graph:
+            for i in range(steps):
+                self.fns[i % self.n]()
+            return
+        full, rem = divmod(steps, self.per_graph)
+        if full:
+            gr = self._graph(self.per_graph)
+            for _ in range(full):
+                gr.replay()
+        if rem:
+            self._graph(rem).replay()
+
+
+def time_steps(runner, steps, warmup):
     import torch
 
-    if not use_graph:
-        return fns, None
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        for f in fns:  # warm allocator and kernels outside capture
-            f()
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    graphs, keep = [], []
-    for f in fns:
-        gr = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(gr):
-            keep.append(f())
-        graphs.append(gr)
-    return [gr.replay for gr in graphs], keep
-
-
-def time_steps(launchers, steps, warmup):
-    import torch
-
-    n = len(launchers)
-    for i in range(warmup):
-        launchers[i % n]()
+    runner.prepare(steps)
+    runner.prepare(warmup)
+    runner.run(warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(steps):
-        launchers[i % n]()
+    runner.run(steps)
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) * 1e3 / steps
 
@@ -326,8 +362,8 @@ def run_decode(args):
     dec_bytes = [c.decode_bytes(e_kv) for c in copies]
     step_bytes = [b + c.update_bytes() for b, c in zip(dec_bytes, copies)]
     fns = [(lambda c=c: decode_step(c)) for c in copies]
-    launchers, _keep = build_launchers(fns, args.launch == "graph")
-    ms = time_steps(launchers, args.steps, args.warmup)
+    runner = StepRunner(fns, args.launch == "graph", args.steps_per_graph)
+    ms = time_steps(runner, args.steps, args.warmup)
     n = len(copies)
     avg_step_bytes = sum(step_bytes[i % n] for i in range(args.steps)) / args.steps
     durs = time_decode_kernel_direct(copies, min(args.steps, 100))
@@ -344,7 +380,8 @@ def run_decode(args):
         "config": {
             "workload": wl.name,
             "step": "K + V cache update (one launch) + paged decode attention, one layer, one token per sequence",
-            "launch": args.launch, "rotating_copies": n, **shape,
+            "launch": args.launch, "steps_per_graph": runner.per_graph if args.launch == "graph" else None,
+            "rotating_copies": n, **shape,
             "mean_context": float(wl.cache_position.float().mean()),
         },
         "tokens_per_s": shape["users"] / (ms * 1e-3),
@@ -364,8 +401,7 @@ def run_decode(args):
         impl = make_prefill_impl(w)
         outbuf = torch.empty_like(w.q)
         chunk = [lambda: prefill_step(impl, w, outbuf)]
-        cl, _k2 = build_launchers(chunk, args.launch == "graph")
-        cms = time_steps(cl, min(args.steps, 50), 5)
+        cms = time_steps(StepRunner(chunk, args.launch == "graph", args.steps_per_graph), min(args.steps, 50), 5)
         cd = time_dominant_kernel(chunk, 20)
         ck = sum(x for x, _ in cd) / len(cd)
         out["chunk_pass"] = {
@@ -386,9 +422,9 @@ def run_prefill(args):
     impls = [make_prefill_impl(w) for w in copies]
     outs = [torch.empty_like(w.q) for w in copies]
     fns = [(lambda i=i: prefill_step(impls[i], copies[i], outs[i])) for i in range(len(copies))]
-    launchers, _keep = build_launchers(fns, args.launch == "graph")
+    runner = StepRunner(fns, args.launch == "graph", args.steps_per_graph)
     steps = min(args.steps, 100)
-    ms = time_steps(launchers, steps, min(args.warmup, 10))
+    ms = time_steps(runner, steps, min(args.warmup, 10))
     w = copies[0]
     flops = w.useful_flops()
     durs = time_dominant_kernel(fns, min(steps, 50))
@@ -404,7 +440,8 @@ def run_prefill(args):
         "config": {
             "workload": w.name,
             "step": "K fill + V fill through the fill page table + causal attention on the fresh K/V",
-            "launch": args.launch, "rotating_copies": len(copies), "users": w.users,
+            "launch": args.launch, "steps_per_graph": runner.per_graph if args.launch == "graph" else None,
+            "rotating_copies": len(copies), "users": w.users,
             "tokens_per_user": w.seq, "q_heads": w.q_heads, "kv_heads": w.kv_heads,
             "head_size": w.head_size, "block_size": 64,
         },
