@@ -39,9 +39,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 # of this script scaled by a plain copy of known size (profiles/decode_kernel_hbm_traffic_config2.md).
 # A counter run cannot share a process with the timed run, so the figure is carried here; it belongs
 # to the default seed and shapes of the workload it is keyed by.
-MEASURED_TRAFFIC_BYTES = {"config2": 306301 * 1024}
-DECODE_KERNEL_NAME = {"config2": "paged_decode_kernel", "config4": "paged_decode_mfma_kernel",
-                      "config5": "paged_decode_bfp8_mfma_kernel"}
+MEASURED_TRAFFIC_BYTES = {"config2": 306207 * 1024}
+DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
+                      "config5": "paged_decode_mfma16_kernel"}
 CPU_THREADS_CAP = 16        # host cores a one-GPU box grants, whatever os.cpu_count() says
 
 

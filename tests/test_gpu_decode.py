@@ -166,3 +166,43 @@ def test_config2_full_size():
         g.q[:, perm.cuda()], k, v, g.page_table[perm.cuda()], True, None,
         g.cache_position[perm.cuda()], None, wl.scale).cpu()
     torch.testing.assert_close(out_p.float(), got[:, perm].float(), atol=4e-3, rtol=4e-3)
+
+
+@pytest.mark.parametrize("kernel", ["valu", "mfma", "mfma16"])
+@pytest.mark.parametrize("users,hq,hkv,d,bs,ctx", [
+    (4, 32, 8, 128, 64, [5, 64, 200, 700]),
+    (2, 64, 8, 128, 64, [1000, 257]),
+    (3, 16, 8, 128, 16, [15, 16, 100]),
+    (3, 12, 4, 128, 32, [100, 17, 450]),
+])
+def test_decode_every_kernel(monkeypatch, kernel, users, hq, hkv, d, bs, ctx):
+    """The dot-product kernel and the two matrix-core kernels, each forced in turn on the same
+    bfloat16 cache (a kernel that does not cover a shape leaves it to the default choice)."""
+    from tt_xla_amd import workloads
+
+    monkeypatch.setenv("TTPA_DECODE_KERNEL", kernel)
+    name = f"decode [{kernel}] b{users} h{hq}x{hkv} d{d} bs{bs} ctx{ctx}"
+    print(name, flush=True)
+    nb = sum((c + 1 + bs - 1) // bs for c in ctx) + 3
+    wl = workloads.decode_ragged(name, hq * 7 + d + bs, users, hq, hkv, d, bs, nb, ctx)
+    got, k, v = _run(wl)
+    _check(name, got,
+           O.textbook_decode_fp32(wl.q, k.cpu(), v.cpu(), wl.page_table, wl.cache_position, wl.scale))
+
+
+@pytest.mark.parametrize("kernel,hq", [("valu", 32), ("mfma", 64), ("mfma16", 64), ("mfma16", 32)])
+def test_decode_several_tiles_per_wavefront(monkeypatch, kernel, hq):
+    """A grid of one wavefront per CU over ~1000 tiles: every wavefront walks several tiles and
+    crosses segment boundaries (running maximum, partial hand-over, Q reload)."""
+    from tt_xla_amd import workloads
+
+    monkeypatch.setenv("TTPA_DECODE_KERNEL", kernel)
+    monkeypatch.setenv("TTPA_DECODE_WAVES_PER_CU", "1")
+    ctx = [1990, 2047, 1500, 2300]
+    name = f"decode [{kernel}] h{hq}x8 one wavefront per CU ctx{ctx}"
+    print(name, flush=True)
+    nb = sum((c + 1 + 63) // 64 for c in ctx) + 3
+    wl = workloads.decode_ragged(name, 91, 4, hq, 8, 128, 64, nb, ctx)
+    got, k, v = _run(wl)
+    _check(name, got,
+           O.textbook_decode_fp32(wl.q, k.cpu(), v.cpu(), wl.page_table, wl.cache_position, wl.scale))

@@ -61,6 +61,31 @@ def test_decode_window_and_sink(users, hq, hkv, d, bs, ctx, window, with_sink):
     _check(name, out.cpu(), want)
 
 
+@pytest.mark.parametrize("kernel", ["mfma", "mfma16"])
+def test_decode_window_and_sink_matrix_core_kernels(monkeypatch, kernel):
+    """Window edge inside a tile, sink, short and long users on each matrix-core kernel, with a
+    small grid so that wavefronts cross from one windowed segment into the next."""
+    from tt_xla_amd import workloads
+
+    monkeypatch.setenv("TTPA_DECODE_KERNEL", kernel)
+    monkeypatch.setenv("TTPA_DECODE_WAVES_PER_CU", "1")
+    users, hq, hkv, d, bs, ctx, window = 4, 64, 8, 128, 64, [1990, 30, 1500, 2300], 1000
+    name = f"decode [{kernel}] b{users} h{hq}x{hkv} ctx{ctx} window{window} sink"
+    print(name, flush=True)
+    nb = sum((c + 1 + bs - 1) // bs for c in ctx) + 3
+    wl = workloads.decode_ragged(name, 93, users, hq, hkv, d, bs, nb, ctx)
+    g = torch.Generator().manual_seed(3)
+    sink = (torch.randn(hq, generator=g) * 2).to(torch.bfloat16)
+    dev = wl.to("cuda")
+    out = torch.ops.tt.paged_scaled_dot_product_attention_decode(
+        dev.q, dev.k_cache, dev.v_cache, dev.page_table, is_causal=True,
+        cur_pos_tensor=dev.cache_position, scale=wl.scale, sliding_window_size=window,
+        attention_sink=sink.cuda())
+    want = O.paged_sdpa_decode_windowed(wl.q, wl.k_cache, wl.v_cache, wl.page_table,
+                                        wl.cache_position, wl.scale, window, sink)
+    _check(name, out.cpu(), want)
+
+
 def test_decode_sink_only_and_padded_row():
     from tt_xla_amd import workloads
 

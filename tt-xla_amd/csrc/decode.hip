@@ -394,12 +394,15 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   a.sink = attention_sink;
 
   hipStream_t st = static_cast<hipStream_t>(stream);
-  // Kernel choice: the VALU kernel streams at the HBM ceiling up to 4 query heads per KV head;
-  // beyond that its per-head VALU work becomes the limiter and the matrix-core kernel takes
-  // over (its cost per tile does not depend on the group width).  The block-float-8 cache goes
-  // to a matrix-core kernel whenever one applies: there the byte expansion costs one VALU
-  // operation per element and the products none, while the VALU kernel pays for both; head
-  // size 128 with up to 16 heads per group has the 16x16x32 kernel with twice the occupancy.
+  // Kernel choice.  The VALU kernel spends per-head work on every tile; the matrix-core kernels
+  // do not (their cost per tile does not depend on the group width).  Measured on bfloat16
+  // caches with head size 128: at 1 and 2 query heads per KV head the VALU kernel is 2 - 19 %
+  // faster (the larger figure on launches of a few tiles), at 4 the 16x16x32 kernel is 2 - 8 %
+  // faster, at 8 the VALU kernel is 2.5 times slower.  So: 16x16x32 kernel for head size 128 and
+  // 4 ... 16 heads per group, 32x32x16 kernel for the other wide groups (head size 64, up to 32
+  // heads), VALU kernel for the rest.  The block-float-8 cache goes to a matrix-core kernel
+  // whenever one applies: there the byte expansion costs one VALU operation per element and the
+  // products none, while the VALU kernel pays for both.
   // TTPA_DECODE_KERNEL=valu|mfma|mfma16 overrides the choice.
   // read on every call (a getenv is negligible next to a launch) so that a process can
   // exercise every kernel
@@ -410,7 +413,7 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
                      : !strcmp(forced_name, "mfma16") ? 3 : 0;
   const bool mfma_ok = mfma_decode_supported(a, head_size, g);
   const bool mfma16_ok = mfma16_decode_supported(a, head_size, g);
-  bool use_mfma16 = mfma16_ok;
+  bool use_mfma16 = mfma16_ok && (g >= 4 || kv_format == TTPA_KV_BFP8);
   bool use_mfma = !use_mfma16 && mfma_ok && (g >= 5 || kv_format == TTPA_KV_BFP8);
   if (forced == 1) use_mfma = use_mfma16 = false;
   if (forced == 2) use_mfma = mfma_ok, use_mfma16 = false;

@@ -1,15 +1,17 @@
-// Paged decode attention over a block-float-8 KV cache on the 16x16x32 matrix-core shape:
-// head size 128, up to 16 query heads per KV head, 72 KiB of LDS per workgroup.
+// Paged decode attention on the 16x16x32 matrix-core shape: head size 128, up to 16 query
+// heads per KV head, 72 KiB of LDS per workgroup; block-float-8 cache (expanded to half
+// precision) or bfloat16 cache.
 //
 // Work decomposition, partial slots and merge kernel are those of decode.hip.  Inside a
-// wavefront a 64-token tile of K, then of V, goes global -> registers -> half precision in a
-// 16 KiB wave-private LDS buffer that both tensors use in turn:
+// wavefront a 64-token tile of K, then of V, goes global -> registers -> a 16 KiB wave-private
+// LDS buffer of 16-bit elements that both tensors use in turn:
 //   stage K(t) | prefetch K(t+1) | S^T = K Q^T | softmax | stage V(t) | prefetch V(t+1) | O^T += V^T P^T
-// so every global load has three quarters of a tile period to arrive.  The byte -> half expansion is the one of
-// decode_mfma.hip (one permute and one packed fma per element pair, exponents relative to the
-// tile's largest, running reference exponent for the V accumulator).
+// so every global load has three quarters of a tile period to arrive.  The byte -> half
+// expansion of the block-float-8 cache is the one of decode_mfma.hip (one permute and one
+// packed fma per element pair, exponents relative to the tile's largest, running reference
+// exponent for the V accumulator).
 //
-// v_mfma_f32_16x16x32_f16 with the heads as the 16-wide N dimension:
+// v_mfma_f32_16x16x32_{f16,bf16} with the heads as the 16-wide N dimension:
 //   S^T block b (16 keys):  A = K rows 16 b + lane%16, 8 elements per lane and k-step
 //                           B = Q, lane%16 = head;   C: lane (head, quad) holds keys 16 b + 4 quad + r
 //   O^T block db (16 d):    the 32 k slots of a step are the keys lane (., quad) already holds
@@ -29,15 +31,22 @@ namespace decode {
 namespace {
 
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kMaxUsers16 = 1024;
 constexpr int kTileBytes = kTile * 256;
 
+template <bool F16>
 __device__ __forceinline__ floatx4 mma16(const u32x4 &x, const u32x4 &y, const floatx4 &c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, x),
-                                                __builtin_bit_cast(halfx8, y), c, 0, 0, 0);
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, x),
+                                                  __builtin_bit_cast(halfx8, y), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x),
+                                                   __builtin_bit_cast(bf16x8, y), c, 0, 0, 0);
 }
 
 // Maximum over the four lanes that share lane%16.  v_permlane16_swap exchanges the odd rows
@@ -62,13 +71,18 @@ __device__ __forceinline__ float sum_over_quads(float v) {
   return x + y;
 }
 
-template <bool BIG>
-__global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
+template <bool BFP8, bool BIG>
+__global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     DecodeArgs a, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
   constexpr int D = 128;
   constexpr int KSTEPS = D / 32, DBLK = D / 16;
-  // staging geometry: a load instruction covers 8 whole token rows, 16 element bytes per lane
-  constexpr int LPR = 8, RPL = 8, NL = kTile / RPL, GPR = D / 16;
+  // staging geometry: 16 bytes per lane, so a load instruction covers 8 whole token rows of
+  // element bytes or 4 of bfloat16
+  constexpr int BPE = BFP8 ? 1 : 2;   // bytes per cache element
+  constexpr int LPR = D * BPE / 16;   // lanes per token row
+  constexpr int RPL = 64 / LPR;       // rows per load
+  constexpr int NL = kTile / RPL;     // loads per tile and tensor
+  constexpr int GPR = D / 16;         // exponent bytes per row (block-float-8)
   constexpr int NOFF = BIG ? 1 : NL;
 
   __shared__ int s_pref[kMaxUsers16 + 1];
@@ -96,18 +110,29 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
 
   // staging lane mapping and swizzled write positions
   const int sr = lane / LPR, sc = lane % LPR;
-  const uint32_t lane_bytes = (uint32_t)(sr * D + sc * 16);
-  // the lane's exponent byte (row sr, group sc) is fetched inside its aligned dword and cut
-  // out when the tile is staged: a byte load is widened where it is issued, which would make
-  // the loop wait for the next tile's exponents at the end of every iteration
+  const uint32_t lane_bytes = (uint32_t)(sr * D * BPE + sc * 16);
+  // block-float-8: the lane's exponent byte (row sr, group sc) is fetched inside its aligned
+  // dword and cut out when the tile is staged: a byte load is widened where it is issued, which
+  // would make the loop wait for the next tile's exponents at the end of every iteration
   const uint32_t lane_exp = (uint32_t)((sr * GPR + sc) & ~3);
   const uint32_t exp_shift = (uint32_t)(8 * (sc & 3));
-  const int64_t slab = (int64_t)(a.bs + a.bs / 16) * D;  // bytes of one (block, head)
-  // K: row 8 i + sr has row & 15 = 8 (i & 1) + sr
-  const uint32_t kw_even = (uint32_t)(sr * 256 + (((2 * sc) ^ sr) << 4));
-  const uint32_t kw_odd = (uint32_t)(sr * 256 + (((2 * sc) ^ (8 + sr)) << 4));
-  // V: row & 7 = sr
-  const uint32_t vw = (uint32_t)(sr * 256 + (((2 * sc) ^ ((2 * sr) | (sr & 1))) << 4));
+  const int64_t slab = BFP8 ? (int64_t)(a.bs + a.bs / 16) * D : (int64_t)a.bs * D * 2;  // bytes
+  // A lane stages CPL chunks of 16 bytes (16-bit elements) per load, logical chunks CPL sc ...;
+  // load i holds row RPL i + sr, whose swizzle key repeats every 16 / RPL loads for K
+  // (row & 15) and every 8 / RPL (at least 1) loads for V (row & 7).
+  constexpr int CPL = BFP8 ? 2 : 1;
+  constexpr int KPAT = 16 / RPL, VPAT = RPL >= 8 ? 1 : 8 / RPL;
+  uint32_t kw[KPAT], vw[VPAT];
+#pragma unroll
+  for (int j = 0; j < KPAT; ++j) {
+    const int row = RPL * j + sr;
+    kw[j] = (uint32_t)(sr * 256 + (((CPL * sc) ^ (row & 15)) << 4));
+  }
+#pragma unroll
+  for (int j = 0; j < VPAT; ++j) {
+    const int y = (RPL * j + sr) & 7;
+    vw[j] = (uint32_t)(sr * 256 + (((CPL * sc) ^ ((2 * y) | (y & 1))) << 4));
+  }
   // A-operand reads of K: row 16 b + n, chunk 4 s + quad
   uint32_t kr[KSTEPS];
 #pragma unroll
@@ -136,7 +161,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
       if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
       const int64_t base = ((int64_t)phys * a.hkv + cu.h) * slab;
       const int row = tk - col * a.bs;
-      eo[i] = base + (int64_t)row * D;
+      eo[i] = base + (int64_t)row * D * BPE;
       xo[i] = base + (int64_t)a.bs * D + (int64_t)row * GPR;
     }
   };
@@ -144,12 +169,14 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
                    u32x4 (&raw)[NL], uint32_t (&ex)[NL]) {
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-      const uint8_t *erow = BIG ? base + eo[0] + i * (RPL * D) : base + eo[BIG ? 0 : i];
+      const uint8_t *erow = BIG ? base + eo[0] + i * (RPL * D * BPE) : base + eo[BIG ? 0 : i];
       raw[i] = __builtin_nontemporal_load(
           reinterpret_cast<const u32x4 *>(erow + static_cast<uint64_t>(lane_bytes)));
-      const uint8_t *xrow = BIG ? base + xo[0] + i * (RPL * GPR) : base + xo[BIG ? 0 : i];
-      ex[i] = __builtin_nontemporal_load(
-          reinterpret_cast<const uint32_t *>(xrow + static_cast<uint64_t>(lane_exp)));
+      if constexpr (BFP8) {
+        const uint8_t *xrow = BIG ? base + xo[0] + i * (RPL * GPR) : base + xo[BIG ? 0 : i];
+        ex[i] = __builtin_nontemporal_load(
+            reinterpret_cast<const uint32_t *>(xrow + static_cast<uint64_t>(lane_exp)));
+      }
     }
   };
   // Cuts the lane's exponent bytes out of the fetched dwords (zero for rows past `nvalid` of a
@@ -164,49 +191,65 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
     }
     return (int)wave_max_u32(e);
   };
-  // registers -> LDS, expanded to half precision relative to the exponent `eref`: the group
-  // scale 2^(e - eref) is the half with exponent field e - eref + 15; groups more than 2^14
-  // below the tile's largest (field <= 0) are written as zeros
-  auto stage = [&](bool is_v, const u32x4 (&raw)[NL], const uint32_t (&ex)[NL], int eref) {
+  // registers -> LDS.  Block-float-8: expanded to half precision relative to the exponent
+  // `eref`: the group scale 2^(e - eref) is the half with exponent field e - eref + 15; groups
+  // more than 2^14 below the tile's largest (field <= 0) are written as zeros.  bfloat16:
+  // copied; `clear` writes the rows past `nvalid` as zeros (unattended V rows must not carry
+  // Inf / NaN into the product).
+  auto stage = [&](bool is_v, const u32x4 (&raw)[NL], const uint32_t (&ex)[NL], int eref, int nvalid,
+                   bool clear) {
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-      const uint32_t field = (uint32_t)max((int)ex[i] - (eref - 15), 0);
-      const uint32_t sbits = field << 10;
-      const halfx2 s2 = __builtin_bit_cast(halfx2, sbits | (sbits << 16));
-      const halfx2 c2 = s2 * halfx2{(_Float16)-1152.f, (_Float16)-1152.f};
-      uint32_t o[8];
-      expand4_half(raw[i].x, s2, c2, o[0], o[1]);
-      expand4_half(raw[i].y, s2, c2, o[2], o[3]);
-      expand4_half(raw[i].z, s2, c2, o[4], o[5]);
-      expand4_half(raw[i].w, s2, c2, o[6], o[7]);
-      const uint32_t w0 = (is_v ? vw : ((i & 1) ? kw_odd : kw_even)) + (uint32_t)(i * RPL * 256);
-      *reinterpret_cast<uint4 *>(tile + w0) = make_uint4(o[0], o[1], o[2], o[3]);
-      *reinterpret_cast<uint4 *>(tile + (w0 ^ 16u)) = make_uint4(o[4], o[5], o[6], o[7]);
+      const uint32_t w0 = (is_v ? vw[i % VPAT] : kw[i % KPAT]) + (uint32_t)(i * RPL * 256);
+      if constexpr (BFP8) {
+        const uint32_t field = (uint32_t)max((int)ex[i] - (eref - 15), 0);
+        const uint32_t sbits = field << 10;
+        const halfx2 s2 = __builtin_bit_cast(halfx2, sbits | (sbits << 16));
+        const halfx2 c2 = s2 * halfx2{(_Float16)-1152.f, (_Float16)-1152.f};
+        uint32_t o[8];
+        expand4_half(raw[i].x, s2, c2, o[0], o[1]);
+        expand4_half(raw[i].y, s2, c2, o[2], o[3]);
+        expand4_half(raw[i].z, s2, c2, o[4], o[5]);
+        expand4_half(raw[i].w, s2, c2, o[6], o[7]);
+        *reinterpret_cast<uint4 *>(tile + w0) = make_uint4(o[0], o[1], o[2], o[3]);
+        *reinterpret_cast<uint4 *>(tile + (w0 ^ 16u)) = make_uint4(o[4], o[5], o[6], o[7]);
+      } else {
+        const bool keep = !clear || RPL * i + sr < nvalid;
+        *reinterpret_cast<uint4 *>(tile + w0) =
+            keep ? make_uint4(raw[i].x, raw[i].y, raw[i].z, raw[i].w) : make_uint4(0, 0, 0, 0);
+      }
     }
   };
-  // Q fragments: B operand, lane%16 = head of the group (zero beyond G), half precision,
-  // scaled by 2^(127 - eq) with eq the largest exponent field of the segment's Q
+  // Q fragments: B operand, lane%16 = head of the group (zero beyond G): as they are for a
+  // bfloat16 cache; half precision, scaled by 2^(127 - eq) with eq the largest exponent field of
+  // the segment's Q, for block-float-8.  (Requesting the next segment's Q rows early, ahead of
+  // the tile loads and inside the branch that detects the segment change, was measured slower:
+  // the wait-count pass then drains the tile loads in the steady-state loop.)
   int eq = 0;
   auto load_q = [&](const Cursor &cu, u32x4 (&qf)[KSTEPS]) {
     const uint16_t *qp =
         a.q + cu.u * a.q_us + (int64_t)(cu.h * G + min(n, G - 1)) * a.q_hs + 8 * quad;
     const uint32_t qmask = n < G ? 0xffffffffu : 0u;  // no branch: a branch would wait for every load in flight
-    uint32_t em = 0;
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
       const uint4 t = *reinterpret_cast<const uint4 *>(qp + 32 * s);
       qf[s] = u32x4{t.x & qmask, t.y & qmask, t.z & qmask, t.w & qmask};
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        em = max(em, max((qf[s][j] >> 7) & 0xffu, (qf[s][j] >> 23) & 0xffu));
     }
-    eq = (int)min(wave_max_u32(em), 253u);
-    const float qs = __builtin_bit_cast(float, (uint32_t)(254 - eq) << 23);
+    if constexpr (BFP8) {
+      uint32_t em = 0;
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s)
+      for (int s = 0; s < KSTEPS; ++s)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        qf[s][j] = pack_half2(bf16_lo(qf[s][j]) * qs, bf16_hi(qf[s][j]) * qs);
+        for (int j = 0; j < 4; ++j)
+          em = max(em, max((qf[s][j] >> 7) & 0xffu, (qf[s][j] >> 23) & 0xffu));
+      eq = (int)min(wave_max_u32(em), 253u);
+      const float qs = __builtin_bit_cast(float, (uint32_t)(254 - eq) << 23);
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          qf[s][j] = pack_half2(bf16_lo(qf[s][j]) * qs, bf16_hi(qf[s][j]) * qs);
+    }
   };
 
   Cursor cur = locate(x);
@@ -235,8 +278,9 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
     Cursor nxt = cur;
 
     // ---- K: registers -> LDS, then the next tile's K: global -> registers -------------------
-    const int eref_k = tile_exponent(kex, nvalid, partial);
-    stage(false, kraw, kex, eref_k);
+    int eref_k = 0, eref_v = 0;
+    if constexpr (BFP8) eref_k = tile_exponent(kex, nvalid, partial);
+    stage(false, kraw, kex, eref_k, nvalid, false);
     if constexpr (has_next) {
       if (same_seg) {
         nxt.t = cur.t + 1;
@@ -256,7 +300,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
         const uint4 kq = *reinterpret_cast<const uint4 *>(tile + kr[s] + b * (16 * 256));
-        st[b] = mma16(u32x4{kq.x, kq.y, kq.z, kq.w}, qf[s], st[b]);
+        st[b] = mma16<BFP8>(u32x4{kq.x, kq.y, kq.z, kq.w}, qf[s], st[b]);
       }
     }
     // ---- online softmax: lane (head, quad) holds keys 16 b + 4 quad + r ------------------------
@@ -270,7 +314,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
         }
     }
     // the factors taken out of the K tile and out of Q come back in the scale
-    const float scale = __builtin_ldexpf(a.scale_log2e, eref_k + eq - 260);
+    const float scale = BFP8 ? __builtin_ldexpf(a.scale_log2e, eref_k + eq - 260) : a.scale_log2e;
     float mloc = -INFINITY;
     if (scale >= 0.f) {
 #pragma unroll
@@ -291,26 +335,40 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
     m_run = m_new;
 
     // ---- V: registers -> LDS (the K tile has been consumed), next tile's V -> registers -------
-    const int eref_v = tile_exponent(vex, nvalid, partial);
-    stage(true, vraw, vex, eref_v);
+    if constexpr (BFP8) eref_v = tile_exponent(vex, nvalid, partial);
+    stage(true, vraw, vex, eref_v, nvalid, partial);
     if constexpr (has_next) fetch(a.v, eo, xo, vraw, vex);
 
-    // bring this tile's V factor and the accumulator to the larger reference exponent
-    const int ev_new = max(ev_run, eref_v);
-    const float pscale = __builtin_ldexpf(1.f, eref_v - ev_new);
-    const float alpha_acc = alpha * __builtin_ldexpf(1.f, ev_run - ev_new);
-    ev_run = ev_new;
-    float lsum = 0.f;
+    float lsum = 0.f, alpha_acc = alpha;
     u32x4 pf[2];
+    if constexpr (BFP8) {
+      // bring this tile's V factor and the accumulator to the larger reference exponent
+      const int ev_new = max(ev_run, eref_v);
+      const float pscale = __builtin_ldexpf(1.f, eref_v - ev_new);
+      alpha_acc = alpha * __builtin_ldexpf(1.f, ev_run - ev_new);
+      ev_run = ev_new;
 #pragma unroll
-    for (int b = 0; b < 4; ++b)
+      for (int b = 0; b < 4; ++b)
 #pragma unroll
-      for (int r = 0; r < 4; r += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(fmaf(st[b][r], scale, -m_safe));
-        const float p1 = __builtin_amdgcn_exp2f(fmaf(st[b][r + 1], scale, -m_safe));
-        lsum += p0 + p1;  // half-precision rounding of the weights is 2^-12: not tracked
-        pf[b >> 1][2 * (b & 1) + (r >> 1)] = pack_half2(p0 * pscale, p1 * pscale);
-      }
+        for (int r = 0; r < 4; r += 2) {
+          const float p0 = __builtin_amdgcn_exp2f(fmaf(st[b][r], scale, -m_safe));
+          const float p1 = __builtin_amdgcn_exp2f(fmaf(st[b][r + 1], scale, -m_safe));
+          lsum += p0 + p1;  // half-precision rounding of the weights is 2^-12: not tracked
+          pf[b >> 1][2 * (b & 1) + (r >> 1)] = pack_half2(p0 * pscale, p1 * pscale);
+        }
+    } else {
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; r += 2) {
+          const float p0 = __builtin_amdgcn_exp2f(fmaf(st[b][r], scale, -m_safe));
+          const float p1 = __builtin_amdgcn_exp2f(fmaf(st[b][r + 1], scale, -m_safe));
+          const floatx2 pp = {p0, p1};
+          const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, bf16x2));
+          lsum += bf16_lo(w) + bf16_hi(w);  // the normaliser sums the weights that multiply V
+          pf[b >> 1][2 * (b & 1) + (r >> 1)] = w;
+        }
+    }
     l_run = l_run * alpha + lsum;
     if (__builtin_amdgcn_ballot_w64(alpha_acc != 1.0f) != 0) {
 #pragma unroll
@@ -326,14 +384,14 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
         shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vp));
         shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vp + 16 * 256));
         const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
-        acc[db] = mma16(u32x4{l2.x, l2.y, h2.x, h2.y}, pf[s], acc[db]);
+        acc[db] = mma16<BFP8>(u32x4{l2.x, l2.y, h2.x, h2.y}, pf[s], acc[db]);
       }
 
     // ---- close the segment --------------------------------------------------------------------
     if (!same_seg) {
       float *slot = a.ws_slots + ((int64_t)wave + (int64_t)cur.u * a.hkv + cur.h) * a.slot_floats;
       const float l_tot = sum_over_quads(l_run);
-      const float vout = __builtin_ldexpf(1.f, ev_run - 133);
+      const float vout = BFP8 ? __builtin_ldexpf(1.f, ev_run - 133) : 1.f;
       if (n < G) {
         float *dst = slot + n * D + 4 * quad;
 #pragma unroll
@@ -359,26 +417,28 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_mfma_kernel(
   process_tile(std::false_type{});
 }
 
-template <bool BIG>
+template <bool BFP8, bool BIG>
 bool launch(const DecodeArgs &a, hipStream_t st) {
   const int blocks = a.n_waves / kWavesPerBlock;
   const size_t lds = (size_t)kWavesPerBlock * kTileBytes;
   static std::atomic<uint64_t> lds_ready{0};
-  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_bfp8_mfma_kernel<BIG>), lds, lds_ready))
+  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_mfma16_kernel<BFP8, BIG>), lds, lds_ready))
     return false;
-  paged_decode_bfp8_mfma_kernel<BIG><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
+  paged_decode_mfma16_kernel<BFP8, BIG><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
   return true;
 }
 
 }  // namespace
 
 bool mfma16_decode_supported(const DecodeArgs &a, int head_size, int g) {
-  return a.kv_format == TTPA_KV_BFP8 && head_size == 128 && g <= 16 && a.users <= kMaxUsers16 &&
-         a.bs % 8 == 0;
+  const int rows_per_load = a.kv_format == TTPA_KV_BFP8 ? 8 : 4;
+  return head_size == 128 && g <= 16 && a.users <= kMaxUsers16 && a.bs % rows_per_load == 0;
 }
 
 bool launch_mfma16_main(const DecodeArgs &a, hipStream_t st) {
-  return a.bs % kTile == 0 ? launch<true>(a, st) : launch<false>(a, st);
+  const bool big = a.bs % kTile == 0;
+  if (a.kv_format == TTPA_KV_BFP8) return big ? launch<true, true>(a, st) : launch<true, false>(a, st);
+  return big ? launch<false, true>(a, st) : launch<false, false>(a, st);
 }
 
 }  // namespace decode
