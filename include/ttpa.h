@@ -120,6 +120,11 @@ int ttpa_paged_fill_cache(void *cache, const void *fill, int64_t fill_user_strid
  * `workspace` holds split-K partial results: at least
  * ttpa_paged_decode_workspace_bytes(...) bytes, 256-byte aligned, private to this
  * call until the stream reaches its end.
+ * Built shapes (anything else returns TTPA_ERR_UNSUPPORTED): head_size 64, 128 or 256;
+ * block_size a multiple of 4; at most 2048 users; G = q_heads / kv_heads up to 8, and
+ * up to 32 for head_size 64 / 128 with at most 1024 users and block_size a multiple of
+ * 1024 / (bytes of a cache row) (8 rows for head_size 64, 4 for 128; block-float-8:
+ * 16 and 8).  TTPA_KV_BFP8: head_size 64 or 128, block_size a multiple of 16.
  */
 size_t ttpa_paged_decode_workspace_bytes(int32_t users, int32_t q_heads, int32_t kv_heads,
                                          int32_t head_size);

@@ -1,0 +1,104 @@
+"""Seeded random sweep of the paged decode operator over its shape envelope: head sizes,
+group widths on either side of every kernel-selection threshold, block sizes (whole tiles per
+block and not), ragged contexts with empty and padded rows, int32 / int64 positions, small and
+full grids, sliding windows, sinks, bfloat16 and block-float-8 caches.  Every case is
+compared with the plain fp32 loop oracle (windowed / sink cases with their own oracle) at
+atol = rtol = 2e-2; the case is printed before it runs."""
+
+import random
+
+import pytest
+import torch
+
+import __graft_entry__ as entry
+from oracle import bfp8_codec as C
+from oracle import paged_ops as O
+
+pytestmark = pytest.mark.gpu
+ATOL = RTOL = 2e-2
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _pkg():
+    entry.ensure_built()
+    import tt_xla_amd  # noqa: F401
+
+
+def _case(seed):
+    r = random.Random(seed)
+    d = r.choice([64, 128, 128, 128, 256])
+    hkv = r.choice([1, 2, 4, 8])
+    g = r.choice([1, 2, 3, 4, 5, 7, 8] if d == 256 else [1, 2, 3, 4, 4, 5, 6, 7, 8, 12, 16, 24, 32])
+    bfp8 = d in (64, 128) and r.random() < 0.35
+    bs = r.choice([16, 32, 64, 128] if bfp8 else [4, 8, 16, 32, 64, 128])
+    if g > 8:  # wide groups run on the matrix-core kernels only: whole 1 KiB loads per block
+        bs = max(bs, 1024 // (d * (1 if bfp8 else 2)))
+    users = r.randint(1, 9)
+    ctx = []
+    for _ in range(users):
+        kind = r.random()
+        if kind < 0.15:
+            ctx.append(0)
+        elif kind < 0.5:
+            ctx.append(r.randint(1, 130))
+        else:
+            ctx.append(r.randint(131, 900))
+    window = r.choice([0, 0, 1, 17, 64, 200, 5000])
+    sink = r.random() < 0.3
+    pad = [u for u in range(users) if r.random() < 0.12]          # rows with cur_pos = -1
+    i64 = r.random() < 0.3
+    small_grid = r.random() < 0.3  # one wavefront per CU: wavefronts walk several tiles / segments
+    if small_grid:
+        ctx = [x * 6 if x > 130 else x for x in ctx]
+    return dict(small_grid=small_grid, seed=seed, d=d, hkv=hkv, g=g, bfp8=bfp8, bs=bs, users=users, ctx=ctx,
+                window=window, sink=sink, pad=pad, i64=i64)
+
+
+@pytest.mark.parametrize("seed", range(96))
+def test_decode_random_case(monkeypatch, seed):
+    from tt_xla_amd import custom_ops as ops
+    from tt_xla_amd import workloads
+
+    c = _case(seed)
+    print("decode sweep", c, flush=True)
+    if c["small_grid"]:
+        monkeypatch.setenv("TTPA_DECODE_WAVES_PER_CU", "1")
+    d, hkv, g, bs, users, ctx = c["d"], c["hkv"], c["g"], c["bs"], c["users"], c["ctx"]
+    hq = hkv * g
+    nb = sum((x + 1 + bs - 1) // bs for x in ctx) + 3
+    wl = workloads.decode_ragged(f"sweep{seed}", 1000 + seed, users, hq, hkv, d, bs, nb, ctx)
+    if c["bfp8"]:
+        workloads.add_outlier_channels(wl, seed, fraction=0.02)
+    for u in c["pad"]:
+        wl.cache_position[u] = -1
+        wl.page_table[u] = 0
+    gen = torch.Generator().manual_seed(seed)
+    sink = (torch.randn(hq, generator=gen) * 2).to(torch.bfloat16) if c["sink"] else None
+    window = c["window"]
+
+    dev = wl.to("cuda")
+    kc, vc = dev.k_cache, dev.v_cache
+    k_ref, v_ref = wl.k_cache, wl.v_cache
+    if c["bfp8"]:
+        kc, vc = ops.bfp8_pack_cache(kc), ops.bfp8_pack_cache(vc)
+        k_ref = C.unpack_cache(kc.cpu(), bs).to(torch.bfloat16)  # exact: 8-bit integers times 2^k
+        v_ref = C.unpack_cache(vc.cpu(), bs).to(torch.bfloat16)
+    pos = dev.cache_position.long() if c["i64"] else dev.cache_position
+    out = torch.ops.tt.paged_scaled_dot_product_attention_decode(
+        dev.q, kc, vc, dev.page_table, is_causal=True, cur_pos_tensor=pos, scale=wl.scale,
+        sliding_window_size=window if window else None,
+        attention_sink=sink.cuda() if sink is not None else None).cpu().float()
+
+    if window or sink is not None:
+        want = O.paged_sdpa_decode_windowed(wl.q, k_ref, v_ref, wl.page_table, wl.cache_position,
+                                            wl.scale, window, sink).float()
+    else:
+        want = O.textbook_decode_fp32(wl.q, k_ref, v_ref, wl.page_table, wl.cache_position, wl.scale)
+    live = [u for u in range(users) if u not in c["pad"]]
+    for u in c["pad"]:
+        if sink is None:  # nothing attended and no sink: softmax over an empty set
+            assert torch.isnan(out[0, u]).all(), f"padded row {u} is not NaN"
+    if live:
+        err = (out[0, live] - want[0, live]).abs().max().item()
+        print(f"  max-abs error {err:.3e}", flush=True)
+        torch.testing.assert_close(out[0, live], want[0, live], atol=ATOL, rtol=RTOL)

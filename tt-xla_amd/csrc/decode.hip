@@ -319,7 +319,10 @@ int launch_g(const DecodeArgs &a, int g, hipStream_t st) {
     case 7: launch<D, 7>(a, st); break;
     case 8: launch<D, 8>(a, st); break;
     default:
-      return fail(TTPA_ERR_UNSUPPORTED, "query heads per KV head = %d; supported 1..8", g);
+      return fail(TTPA_ERR_UNSUPPORTED,
+                  "query heads per KV head = %d: more than 8 (up to 32) need head_size 64 / 128, at most "
+                  "1024 users and a block_size that is a multiple of 1024 / (bytes of a cache row)",
+                  g);
   }
   return TTPA_OK;
 }

@@ -425,8 +425,10 @@ bool launch(const DecodeArgs &a, hipStream_t st) {
 }  // namespace
 
 bool mfma_decode_supported(const DecodeArgs &a, int head_size, int g) {
-  return (head_size == 64 || head_size == 128) && g <= 32 && a.users <= kMaxUsersMfma &&
-         a.bs % 8 == 0;
+  if ((head_size != 64 && head_size != 128) || g > 32 || a.users > kMaxUsersMfma) return false;
+  // a load instruction covers 1 KiB of whole token rows, which must not straddle a block
+  const int row_bytes = head_size * (a.kv_format == TTPA_KV_BFP8 ? 1 : 2);
+  return a.bs % (1024 / row_bytes) == 0;
 }
 
 bool launch_mfma_main(const DecodeArgs &a, int head_size, hipStream_t st) {
