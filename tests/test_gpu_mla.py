@@ -125,3 +125,67 @@ def test_flash_mla_prefill(b, hq, s, dh, nkv, dv, has_value):
     _check(f"mla prefill b{b} h{hq} s{s} dh{dh} dv{dv}", got, want)
     with pytest.raises(NotImplementedError):
         torch.ops.tt.flash_mla_prefill(q.cuda(), k.cuda(), dv, None, torch.zeros(b, 1, s, s, dtype=torch.bfloat16).cuda(), False, 1.0)
+
+
+def test_mla_backend_prefill_then_decode():
+    """The serving backend (tt_xla_amd/attention_mla.py) end to end on the device at the
+    576 / 512 latent shape: prefill of 40 tokens per user, one decode step, output against a
+    dense fp32 computation and the latent cache position by position (the checks of
+    tests/integrations/vllm_plugin/oot_backends/test_mla_attention_impl.py:202-218, 317-333)."""
+    import types
+
+    from tt_xla_amd import attention_mla as M
+    from tt_xla_amd.attention import TTMetadata
+
+    n, p, r, lat, v, bs = 16, 128, 64, 512, 128, 32
+    users, s, nb, w = 2, 40, 12, 3
+    g = torch.Generator().manual_seed(7)
+    layer = types.SimpleNamespace(W_UK_T=(_bf(g, n, p, lat) / math.sqrt(p)).cuda(),
+                                  W_UV=(_bf(g, n, lat, v) / math.sqrt(lat)).cuda())
+    impl = M.TTMLAAttentionBackendImpl(
+        num_heads=n, head_size=lat + r, scale=1.0 / math.sqrt(p + r), num_kv_heads=1,
+        alibi_slopes=None, sliding_window=None, kv_cache_dtype="auto", logits_soft_cap=None,
+        attn_type="decoder", kv_sharing_target_layer_name=None, kv_lora_rank=lat,
+        qk_nope_head_dim=p, qk_rope_head_dim=r, qk_head_dim=p + r, v_head_dim=v)
+    table = (torch.randperm(nb - 1, generator=g)[: users * w] + 1).view(users, w).to(torch.int32)
+    cache = torch.zeros(nb, 1, bs, lat + r, dtype=torch.bfloat16, device="cuda")
+
+    def dense(q_nope, q_pe, ctx, positions):
+        q_lat = torch.cat([torch.einsum("bsnp,npl->bsnl", q_nope.float(), layer.W_UK_T.cpu().float())
+                           .to(torch.bfloat16).float(), q_pe.float()], dim=-1)
+        out = torch.zeros(q_nope.shape[0], q_nope.shape[1], n, v)
+        for u in range(q_nope.shape[0]):
+            for i in range(q_nope.shape[1]):
+                keys = ctx[u, : int(positions[u, i]) + 1].float()
+                wts = torch.softmax(q_lat[u, i] @ keys.T * impl.scale, dim=-1)
+                out[u, i] = torch.einsum("nl,nlv->nv", wts @ keys[:, :lat], layer.W_UV.cpu().float())
+        return out.reshape(-1, n * v)
+
+    q_nope, q_pe = _bf(g, users * s, n, p), _bf(g, users * s, n, r)
+    kv_c, k_pe = _bf(g, users * s, lat), _bf(g, users * s, 1, r)
+    meta = TTMetadata(cache_position=torch.full((users,), s - 1, dtype=torch.int32).cuda(),
+                      page_table=table.cuda(), fill_page_table=table.cuda(), is_causal=True)
+    out = torch.empty(users * s, n * v, dtype=torch.bfloat16, device="cuda")
+    impl.forward((q_nope.cuda(), q_pe.cuda()), kv_c.cuda(), k_pe.cuda(), cache, meta, layer, output=out)
+    k_lat = torch.cat([kv_c.view(users, s, lat), k_pe.view(users, s, r)], dim=-1)
+    _check("mla backend prefill", out.cpu(),
+           dense(q_nope.view(users, s, n, p), q_pe.view(users, s, n, r), k_lat,
+                 torch.arange(s).expand(users, s)))
+    host = cache.cpu()
+    for u in range(users):
+        for pos in range(s):
+            assert torch.equal(host[table[u, pos // bs], 0, pos % bs], k_lat[u, pos])
+
+    q1, qp1 = _bf(g, users, n, p), _bf(g, users, n, r)
+    c1, kp1 = _bf(g, users, lat), _bf(g, users, 1, r)
+    meta1 = TTMetadata(cache_position=torch.full((users,), s, dtype=torch.int32).cuda(),
+                       page_table=table.cuda(), is_causal=True)
+    out1 = torch.empty(users, n * v, dtype=torch.bfloat16, device="cuda")
+    impl.forward((q1.cuda(), qp1.cuda()), c1.cuda(), kp1.cuda(), cache, meta1, layer, output=out1)
+    k_new = torch.cat([c1, kp1.view(users, r)], dim=-1)
+    ctx = torch.cat([k_lat, k_new.view(users, 1, lat + r)], dim=1)
+    _check("mla backend decode", out1.cpu(),
+           dense(q1.view(users, 1, n, p), qp1.view(users, 1, n, r), ctx, torch.full((users, 1), s)))
+    host = cache.cpu()
+    for u in range(users):
+        assert torch.equal(host[table[u, s // bs], 0, s % bs], k_new[u])
