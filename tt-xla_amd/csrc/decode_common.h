@@ -316,8 +316,10 @@ __device__ __forceinline__ void write_partial(float *slot, int g, int G, int r, 
 }
 
 // Merges the partials of one (user, kv_head) segment and writes bfloat16 output.
-// Partials are read four at a time so that their loads overlap.  G and D are run-time values:
-// the matrix-core kernel serves any group width up to 32.
+// Partials are read eight at a time so that their loads overlap (with four wavefronts per CU
+// and at least one segment per CU, a segment has about five): the kernel is a chain of
+// dependent round trips, and this keeps it at two.  G and D are run-time values: the
+// matrix-core kernels serve any group width up to 32.
 __global__ inline __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a, int G, int D) {
   const int seg = blockIdx.x;
   const int u = seg / a.hkv, h = seg % a.hkv;
@@ -328,25 +330,28 @@ __global__ inline __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a
       out[(int64_t)(h * G + i / D) * a.out_hs + (i % D)] = 0x7fc0;
     return;
   }
+  constexpr int kBatch = 8;
   const float *base = a.ws_slots + (int64_t)first * a.slot_floats;
   for (int i = threadIdx.x; i < G * D; i += 256) {
     const int g = i / D;
     float mall = -INFINITY, num = 0.f, den = 0.f;
-    for (int w = 0; w < nw; w += 4) {
-      float mv[4], lv[4], av[4];
+    for (int w = 0; w < nw; w += kBatch) {
+      float mv[kBatch], lv[kBatch], av[kBatch];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < kBatch; ++j) {
         const float *sl = base + (int64_t)min(w + j, nw - 1) * a.slot_floats;
         mv[j] = (w + j < nw) ? sl[G * D + g] : -INFINITY;
         lv[j] = sl[G * D + G + g];
         av[j] = sl[i];
       }
-      float mnew = fmaxf(fmaxf(fmaxf(mv[0], mv[1]), fmaxf(mv[2], mv[3])), mall);
+      float mnew = mall;
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) mnew = fmaxf(mnew, mv[j]);
       float resc = __builtin_amdgcn_exp2f(mall - mnew);
       num *= resc;
       den *= resc;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < kBatch; ++j) {
         float wgt = __builtin_amdgcn_exp2f(mv[j] - mnew);  // 0 for the padding entries
         num = fmaf(wgt, av[j], num);
         den = fmaf(wgt, lv[j], den);
