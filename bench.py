@@ -39,7 +39,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 # of this script scaled by a plain copy of known size (profiles/decode_kernel_hbm_traffic_config2.md).
 # A counter run cannot share a process with the timed run, so the figure is carried here; it belongs
 # to the default seed and shapes of the workload it is keyed by.
-MEASURED_TRAFFIC_BYTES = {"config2": 306207 * 1024}
+MEASURED_TRAFFIC_BYTES = {"config2": 306650 * 1024}
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}
 CPU_THREADS_CAP = 16        # host cores a one-GPU box grants, whatever os.cpu_count() says
@@ -97,13 +97,10 @@ def make_decode(name, seed, device):
 def decode_step(g):
     import torch
 
-    # what the attention backend issues for a decode step: both cache scatters in one launch
-    torch.ops.tt.paged_update_kv_cache_(g.k_cache, g.v_cache, g.k_new, g.v_new, g.cache_position,
-                                        g.page_table)
-    return torch.ops.tt.paged_scaled_dot_product_attention_decode(
-        g.q, g.k_cache, g.v_cache, g.page_table, is_causal=True,
-        cur_pos_tensor=g.cache_position, scale=g.scale,
-    )
+    # what the attention backend issues for a decode step: the K / V cache update and the
+    # attention as one operator (the update runs inside the decode kernel)
+    return torch.ops.tt.paged_update_kv_decode_(
+        g.q, g.k_cache, g.v_cache, g.k_new, g.v_new, g.page_table, g.cache_position, scale=g.scale)
 
 
 def make_prefill_impl(w):
@@ -212,8 +209,8 @@ def time_dominant_kernel(fns, iters):
 
 
 def time_decode_kernel_direct(copies, iters):
-    """The decode kernel alone, driven through the C ABI with preallocated output and
-    workspace: the host enqueues far faster than the GPU executes, so the stream never runs
+    """The decode kernel alone (the one the step runs: cache update inside), driven through the
+    C ABI with preallocated output and workspace: the host enqueues far faster than the GPU executes, so the stream never runs
     dry and the armed event pair brackets the kernel the way a kernel trace does.  Returns
     [(milliseconds, copy index)]."""
     import torch
@@ -239,10 +236,11 @@ def time_decode_kernel_direct(copies, iters):
         a, b = ev.create(), ev.create()
         _native.call("ttpa_profile_next_attention", a, b)
         _native.call(
-            "ttpa_paged_sdpa_decode", out.data_ptr(), out.stride(1), out.stride(2),
+            "ttpa_paged_update_decode", out.data_ptr(), out.stride(1), out.stride(2),
             c.q.data_ptr(), c.q.stride(1), c.q.stride(2), c.k_cache.data_ptr(), c.v_cache.data_ptr(),
+            c.k_new.data_ptr(), c.v_new.data_ptr(), c.k_new.stride(1), c.k_new.stride(2),
             c.page_table.data_ptr(), c.page_table.stride(0), c.cache_position.data_ptr(), 0,
-            users, hq, hkv, d, bs, w, nb, float(c.scale), fmt, ws.data_ptr(), nbytes, stream)
+            users, hq, hkv, d, bs, w, nb, float(c.scale), fmt, 0, None, ws.data_ptr(), nbytes, stream)
         if i >= 10:
             pairs.append((a, b, i % n))
     torch.cuda.synchronize()
@@ -368,7 +366,9 @@ def run_decode(args):
     avg_step_bytes = sum(step_bytes[i % n] for i in range(args.steps)) / args.steps
     durs = time_decode_kernel_direct(copies, min(args.steps, 100))
     kern_ms = sum(d for d, _ in durs) / len(durs)
-    kern_bytes = sum(dec_bytes[w] for _, w in durs) / len(durs)
+    # with a bfloat16 cache the timed kernel also writes the new token (the update runs inside it)
+    per_launch = dec_bytes if args.workload == "config5" else step_bytes
+    kern_bytes = sum(per_launch[w] for _, w in durs) / len(durs)
     achieved = kern_bytes / (kern_ms * 1e-3) / 1e9
     out = {
         "metric": "paged_decode_attention_hbm_throughput",
@@ -379,7 +379,7 @@ def run_decode(args):
         "dtype": dtype, "data": "synthetic",
         "config": {
             "workload": wl.name,
-            "step": "K + V cache update (one launch) + paged decode attention, one layer, one token per sequence",
+            "step": "K + V cache update and paged decode attention as one operator (bfloat16 cache: the update runs inside the decode kernel; block-float-8: a launch of its own) + merge of the split-K partials, one layer, one token per sequence",
             "launch": args.launch, "steps_per_graph": runner.per_graph if args.launch == "graph" else None,
             "rotating_copies": n, **shape,
             "mean_context": float(wl.cache_position.float().mean()),

@@ -165,6 +165,33 @@ int ttpa_paged_sdpa_decode_windowed(void *out, int64_t out_user_stride, int64_t 
                                     size_t workspace_bytes, void *stream);
 
 /*
+ * The decode step of the attention backend in one call: the cache update
+ * (ttpa_paged_update_cache_kv with update_indices = cur_pos: the new token of user u goes to
+ * position cur_pos[u]) followed by ttpa_paged_sdpa_decode_windowed on the updated caches
+ * (vllm_tt/attention_impls/attention.py:473-483 followed by :634-668).  Results, in the
+ * caches and in `out`, are those of the two calls in that order.  k_new / v_new are the
+ * [1, users, >= kv_heads, head_size] bfloat16 operands of the update, addressed through
+ * new_user_stride / new_head_stride.  Where the 16x16x32 decode kernel serves the shape
+ * (bfloat16 cache, head_size 128, 4 ... 16 query heads per KV head) the update runs
+ * inside it: the wavefront that owns the tile of position cur_pos[u] takes the token from
+ * k_new / v_new and stores it into the cache; otherwise the library issues the two launches.
+ * The equivalence assumes that no user attends a cache row which ANOTHER user's token is
+ * written to in the same step (rows are owned by one user in a paged cache; the writes of
+ * padded rows go to the null block their zero table points to): inside one launch such a
+ * read is not ordered after that write.
+ * No counterpart as ONE operator in the reference, which issues the ops separately.
+ */
+int ttpa_paged_update_decode(
+    void *out, int64_t out_user_stride, int64_t out_head_stride, const void *q,
+    int64_t q_user_stride, int64_t q_head_stride, void *k_cache, void *v_cache, const void *k_new,
+    const void *v_new, int64_t new_user_stride, int64_t new_head_stride,
+    const int32_t *page_table, int64_t page_table_row_stride, const void *cur_pos,
+    int cur_pos_is_i64, int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
+    int32_t block_size, int32_t table_width, int32_t num_blocks, float scale, int32_t kv_format,
+    int32_t sliding_window, const float *attention_sink, void *workspace, size_t workspace_bytes,
+    void *stream);
+
+/*
  * Paged decode attention for latent-style (multi-head latent attention) caches.
  * Replaces the device branch of tt::paged_flash_mla_decode
  * (python_package/tt_torch/custom_ops.py:381-632; CPU semantics :551-610), causal form:

@@ -348,7 +348,9 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
                        int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
                        int32_t block_size, int32_t table_width, int32_t num_blocks, float scale,
                        int32_t kv_format, int32_t sliding_window, const float *attention_sink,
-                       void *workspace, size_t workspace_bytes, void *stream) {
+                       void *workspace, size_t workspace_bytes, void *stream,
+                       const void *k_new = nullptr, const void *v_new = nullptr,
+                       int64_t new_user_stride = 0, int64_t new_head_stride = 0) {
   TTPA_REQUIRE(sliding_window >= 0, "decode: sliding_window %d is negative", sliding_window);
   TTPA_REQUIRE(out && q && k_cache && v_cache && page_table && cur_pos, "null pointer argument");
   TTPA_REQUIRE(users > 0 && q_heads > 0 && kv_heads > 0 && head_size > 0 && block_size > 0 &&
@@ -395,6 +397,8 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   a.kv_format = kv_format;
   a.window = sliding_window;
   a.sink = attention_sink;
+  a.k_new = a.v_new = nullptr;
+  a.new_us = a.new_hs = 0;
 
   hipStream_t st = static_cast<hipStream_t>(stream);
   // Kernel choice.  The VALU kernel spends per-head work on every tile; the matrix-core kernels
@@ -425,6 +429,27 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   // fills the CU's LDS with one, and the 16x16 kernel streams as fast with one as with the two
   // that would fit, while twice the partials cost the merge kernel more.
   a.n_waves = waves_for_device((use_mfma || use_mfma16) ? TTPA_KV_BF16 : kv_format);
+  // one thread of the main grid per segment publishes the segment's partial slots
+  if ((int64_t)users * kv_heads > (int64_t)a.n_waves * kWave)
+    return fail(TTPA_ERR_UNSUPPORTED, "decode: %d x %d segments need a grid of more than %d wavefronts",
+                users, kv_heads, a.n_waves);
+  if (k_new) {
+    // The step's cache update: inside the 16x16 kernel when that is the kernel of this shape
+    // (bfloat16 caches), as a launch of its own in front of the attention otherwise.
+    const bool vec_ok = aligned16(k_new) && aligned16(v_new) && new_user_stride % 8 == 0 &&
+                        new_head_stride % 8 == 0;
+    if (use_mfma16 && vec_ok && kv_format == TTPA_KV_BF16) {
+      a.k_new = static_cast<const uint16_t *>(k_new);
+      a.v_new = static_cast<const uint16_t *>(v_new);
+      a.new_us = new_user_stride, a.new_hs = new_head_stride;
+    } else if (int rc = ttpa_paged_update_cache_kv(
+                   const_cast<void *>(k_cache), const_cast<void *>(v_cache), k_new, v_new,
+                   new_user_stride, new_head_stride, cur_pos, cur_pos_is_i64, page_table,
+                   page_table_row_stride, users, kv_heads, block_size, head_size, table_width,
+                   num_blocks, kv_format, stream)) {
+      return rc;
+    }
+  }
   hipEvent_t ev0, ev1;
   take_profile_events(ev0, ev1);
   if (ev0) (void)hipEventRecord(ev0, st);
@@ -475,4 +500,21 @@ extern "C" int ttpa_paged_sdpa_decode_windowed(
                      v_cache, page_table, page_table_row_stride, cur_pos, cur_pos_is_i64, users,
                      q_heads, kv_heads, head_size, block_size, table_width, num_blocks, scale,
                      kv_format, sliding_window, attention_sink, workspace, workspace_bytes, stream);
+}
+
+extern "C" int ttpa_paged_update_decode(
+    void *out, int64_t out_user_stride, int64_t out_head_stride, const void *q,
+    int64_t q_user_stride, int64_t q_head_stride, void *k_cache, void *v_cache, const void *k_new,
+    const void *v_new, int64_t new_user_stride, int64_t new_head_stride,
+    const int32_t *page_table, int64_t page_table_row_stride, const void *cur_pos,
+    int cur_pos_is_i64, int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
+    int32_t block_size, int32_t table_width, int32_t num_blocks, float scale, int32_t kv_format,
+    int32_t sliding_window, const float *attention_sink, void *workspace, size_t workspace_bytes,
+    void *stream) {
+  TTPA_REQUIRE(k_new && v_new, "update + decode: null fresh K / V pointer");
+  return decode_impl(out, out_user_stride, out_head_stride, q, q_user_stride, q_head_stride, k_cache,
+                     v_cache, page_table, page_table_row_stride, cur_pos, cur_pos_is_i64, users,
+                     q_heads, kv_heads, head_size, block_size, table_width, num_blocks, scale,
+                     kv_format, sliding_window, attention_sink, workspace, workspace_bytes, stream,
+                     k_new, v_new, new_user_stride, new_head_stride);
 }

@@ -33,6 +33,10 @@ struct DecodeArgs {
   int kv_format;
   int window;         // > 0: only the last `window` positions up to cur_pos are attended
   const float *sink;  // [q_heads] extra logit per head in the softmax denominator, or null
+  // Fused cache update (16x16x32 kernel only): the token at cur_pos of every user is taken from
+  // k_new / v_new [users][>= hkv heads][head_size] instead of the cache, and written to it.
+  const uint16_t *k_new, *v_new;
+  int64_t new_us, new_hs;
 };
 
 // First attended position of a user whose attended range ends at `len` (exclusive).

@@ -11,6 +11,17 @@
 // packed fma per element pair, exponents relative to the tile's largest, running reference
 // exponent for the V accumulator).
 //
+// FUSED: the kernel also performs the decode step's cache update.  The token at cur_pos of a
+// user sits in the last tile of each of its segments, and that tile belongs to exactly one
+// wavefront: it takes the token's K / V rows from the fresh activations instead of the cache
+// and stores them into the cache, so nobody depends on a separate update launch (bfloat16
+// caches; with block-float-8 the in-kernel quantiser cost the steady-state loop its scalar
+// registers, 64 spills, and the launch saved was lost again, so that format keeps two launches).  The fresh rows of the next tile's (user, head) are
+// requested with every tile, unconditionally: a conditional request in the steady-state loop
+// makes the wait-count pass drain the tile loads.  Users whose position is negative (padded
+// rows) attend nothing; their write follows the update operator's rule for negative positions
+// and is done by the thread that publishes their segment.
+//
 // v_mfma_f32_16x16x32_{f16,bf16} with the heads as the 16-wide N dimension:
 //   S^T block b (16 keys):  A = K rows 16 b + lane%16, 8 elements per lane and k-step
 //                           B = Q, lane%16 = head;   C: lane (head, quad) holds keys 16 b + 4 quad + r
@@ -71,9 +82,36 @@ __device__ __forceinline__ float sum_over_quads(float v) {
   return x + y;
 }
 
-template <bool BFP8, bool BIG>
+// The cache write of a user whose position is negative, by one thread per (user, kv head):
+// position -k counts from the end of the user's table (the update operator's floor rule:
+// column = floor(pos / bs) taken from the end once, row = pos mod bs); positions that still fall
+// outside the table and blocks outside the cache are skipped.
+__device__ inline void write_negative_position(const DecodeArgs &a, const int32_t *page_table,
+                                               const void *cur_pos, int seg) {
+  constexpr int D = 128;
+  if (seg >= a.users * a.hkv) return;
+  const int u = seg / a.hkv, h = seg - u * a.hkv;
+  const int64_t pos = load_index(cur_pos, a.cur_i64, u);
+  if (pos >= 0) return;
+  int64_t col = pos / a.bs, rem = pos - col * a.bs;
+  if (rem < 0) rem += a.bs, col -= 1;
+  col += a.w;
+  if (col < 0 || col >= a.w) return;
+  const int phys = page_table[(int64_t)u * a.pt_rs + col];
+  if ((unsigned)phys >= (unsigned)a.nb) return;
+  const uint16_t *src[2] = {a.k_new + u * a.new_us + h * a.new_hs, a.v_new + u * a.new_us + h * a.new_hs};
+  uint8_t *dst[2] = {const_cast<uint8_t *>(a.k), const_cast<uint8_t *>(a.v)};
+  for (int t = 0; t < 2; ++t) {
+    uint16_t *row = reinterpret_cast<uint16_t *>(dst[t]) + (((int64_t)phys * a.hkv + h) * a.bs + rem) * D;
+    for (int c = 0; c < D / 8; ++c)
+      *reinterpret_cast<uint4 *>(row + 8 * c) = *reinterpret_cast<const uint4 *>(src[t] + 8 * c);
+  }
+}
+
+template <bool BFP8, bool BIG, bool FUSED>
 __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     DecodeArgs a, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
+  static_assert(!(FUSED && BFP8), "the fused cache update is built for bfloat16 caches");
   constexpr int D = 128;
   constexpr int KSTEPS = D / 32, DBLK = D / 16;
   // staging geometry: 16 bytes per lane, so a load instruction covers 8 whole token rows of
@@ -99,6 +137,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
   const int64_t total = (int64_t)total_tiles * a.hkv;
   const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);
+  if constexpr (FUSED) write_negative_position(a, page_table, cur_pos, blockIdx.x * 256 + threadIdx.x);
   if (total == 0 || wave >= n_eff) {
     publish_segment_row(a, s_pref, total, n_eff);
     return;
@@ -179,6 +218,21 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
       }
     }
   };
+  // FUSED: the lane's 16-byte chunk of the fresh K or V row of (user, head).
+  auto fetch_fresh = [&](const uint16_t *src, const Cursor &cu) {
+    return *reinterpret_cast<const u32x4 *>(src + cu.u * a.new_us + cu.h * a.new_hs + 8 * sc);
+  };
+  // FUSED: puts the fresh row in place of row `r_star` of the fetched tile (registers) and
+  // stores it into the cache row `row` of the slab at byte offset `slab_base`.
+  auto patch_and_store = [&](uint8_t *cache, u32x4 (&raw)[NL], const u32x4 &fresh, int r_star,
+                             int64_t slab_base, int row) {
+    const int i_star = r_star / RPL;
+    const bool mine = sr == r_star % RPL;
+#pragma unroll
+    for (int i = 0; i < NL; ++i)
+      if (i == i_star && mine) raw[i] = fresh;
+    if (mine) *reinterpret_cast<u32x4 *>(cache + slab_base + (int64_t)row * (D * BPE) + 16 * sc) = fresh;
+  };
   // Cuts the lane's exponent bytes out of the fetched dwords (zero for rows past `nvalid` of a
   // partial tile, which stages them as zeros) and returns the largest of the tile.
   auto tile_exponent = [&](uint32_t (&ex)[NL], int nvalid, bool partial) {
@@ -257,9 +311,14 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   u32x4 kraw[NL], vraw[NL];
   uint32_t kex[NL], vex[NL];
   u32x4 qf[KSTEPS];
+  u32x4 kfresh = {0, 0, 0, 0}, vfresh = {0, 0, 0, 0};
   tile_offsets(cur, eo, xo);
   fetch(a.k, eo, xo, kraw, kex);
   fetch(a.v, eo, xo, vraw, vex);
+  if constexpr (FUSED) {
+    kfresh = fetch_fresh(a.k_new, cur);
+    vfresh = fetch_fresh(a.v_new, cur);
+  }
   load_q(cur, qf);
   publish_segment_row(a, s_pref, total, n_eff);
 
@@ -278,6 +337,27 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     Cursor nxt = cur;
 
     // ---- K: registers -> LDS, then the next tile's K: global -> registers -------------------
+    // FUSED: is this the tile that holds the token at cur_pos (the segment's last), and is that
+    // position inside the table and its block inside the cache?  Evaluated where it is used
+    // (once for K, once for V) rather than kept across the tile: it is all scalar work, and
+    // scalar registers are what this kernel is short of.
+    auto fresh_target = [&](int64_t &slab_off, int &row) -> bool {
+      if (cur.tiles_left != 1 || nvalid <= 0) return false;
+      const int pos = cur.len - 1;
+      const int col = pos / a.bs;
+      if (load_index(cur_pos, a.cur_i64, cur.u) != pos || col >= a.w) return false;  // cut short by the table
+      const int phys = __builtin_amdgcn_readfirstlane(page_table[(int64_t)cur.u * a.pt_rs + col]);
+      if ((unsigned)phys >= (unsigned)a.nb) return false;
+      slab_off = ((int64_t)phys * a.hkv + cur.h) * slab;
+      row = pos - col * a.bs;
+      return true;
+    };
+    if constexpr (FUSED) {
+      int64_t slab_off;
+      int row;
+      if (fresh_target(slab_off, row))
+        patch_and_store(const_cast<uint8_t *>(a.k), kraw, kfresh, nvalid - 1, slab_off, row);
+    }
     int eref_k = 0, eref_v = 0;
     if constexpr (BFP8) eref_k = tile_exponent(kex, nvalid, partial);
     stage(false, kraw, kex, eref_k, nvalid, false);
@@ -290,6 +370,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
       }
       tile_offsets(nxt, eo, xo);
       fetch(a.k, eo, xo, kraw, kex);
+      if constexpr (FUSED) kfresh = fetch_fresh(a.k_new, nxt);
     }
 
     // ---- S^T = K . Q^T ------------------------------------------------------------------------
@@ -335,9 +416,18 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     m_run = m_new;
 
     // ---- V: registers -> LDS (the K tile has been consumed), next tile's V -> registers -------
+    if constexpr (FUSED) {
+      int64_t slab_off;
+      int row;
+      if (fresh_target(slab_off, row))
+        patch_and_store(const_cast<uint8_t *>(a.v), vraw, vfresh, nvalid - 1, slab_off, row);
+    }
     if constexpr (BFP8) eref_v = tile_exponent(vex, nvalid, partial);
     stage(true, vraw, vex, eref_v, nvalid, partial);
-    if constexpr (has_next) fetch(a.v, eo, xo, vraw, vex);
+    if constexpr (has_next) {
+      fetch(a.v, eo, xo, vraw, vex);
+      if constexpr (FUSED) vfresh = fetch_fresh(a.v_new, nxt);
+    }
 
     float lsum = 0.f, alpha_acc = alpha;
     u32x4 pf[2];
@@ -417,15 +507,21 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   process_tile(std::false_type{});
 }
 
-template <bool BFP8, bool BIG>
+template <bool BFP8, bool BIG, bool FUSED>
 bool launch(const DecodeArgs &a, hipStream_t st) {
   const int blocks = a.n_waves / kWavesPerBlock;
   const size_t lds = (size_t)kWavesPerBlock * kTileBytes;
   static std::atomic<uint64_t> lds_ready{0};
-  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_mfma16_kernel<BFP8, BIG>), lds, lds_ready))
+  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_mfma16_kernel<BFP8, BIG, FUSED>), lds,
+                          lds_ready))
     return false;
-  paged_decode_mfma16_kernel<BFP8, BIG><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
+  paged_decode_mfma16_kernel<BFP8, BIG, FUSED><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
   return true;
+}
+
+template <bool BIG>
+bool launch_fused_or_not(const DecodeArgs &a, hipStream_t st) {
+  return a.k_new ? launch<false, BIG, true>(a, st) : launch<false, BIG, false>(a, st);
 }
 
 }  // namespace
@@ -435,10 +531,14 @@ bool mfma16_decode_supported(const DecodeArgs &a, int head_size, int g) {
   return head_size == 128 && g <= 16 && a.users <= kMaxUsers16 && a.bs % rows_per_load == 0;
 }
 
+// With a.k_new set (bfloat16 caches only), the launch also performs the cache update of the step.
 bool launch_mfma16_main(const DecodeArgs &a, hipStream_t st) {
   const bool big = a.bs % kTile == 0;
-  if (a.kv_format == TTPA_KV_BFP8) return big ? launch<true, true>(a, st) : launch<true, false>(a, st);
-  return big ? launch<false, true>(a, st) : launch<false, false>(a, st);
+  if (a.kv_format == TTPA_KV_BFP8) {
+    if (a.k_new) return false;
+    return big ? launch<true, true, false>(a, st) : launch<true, false, false>(a, st);
+  }
+  return big ? launch_fused_or_not<true>(a, st) : launch_fused_or_not<false>(a, st);
 }
 
 }  // namespace decode

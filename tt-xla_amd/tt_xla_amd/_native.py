@@ -51,6 +51,11 @@ SIGNATURES = {
         [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _i64, _p, _int, _i32, _i32, _i32, _i32, _i32,
          _i32, _i32, _f32, _i32, _i32, _p, _p, _sz, _p],
     ),
+    "ttpa_paged_update_decode": (
+        _int,
+        [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _int, _i32, _i32,
+         _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _p, _p, _sz, _p],
+    ),
     "ttpa_paged_mla_decode_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32]),
     "ttpa_paged_mla_decode": (
         _int,

@@ -11,8 +11,10 @@ surface.
 Differences from the reference, both invisible in results:
   * cache writes go through the in-place operators, so a decode step moves
     users x kv_heads x head_size elements instead of cloning and copying back the whole
-    cache (reference: functional op followed by ``kv_cache[i].copy_``, :473-515).
-    ``functional_cache_ops=True`` restores the reference's exact call sequence.
+    cache (reference: functional op followed by ``kv_cache[i].copy_``, :473-515), and a
+    causal decode step issues the write and the attention as one operator
+    (``tt::paged_update_kv_decode_``).  ``functional_cache_ops=True`` restores the reference's
+    exact call sequence.
   * ``get_page_size`` still answers 32 like the reference (:147-152); the kernels accept
     any block size that is a multiple of 4.
 """
@@ -244,18 +246,27 @@ class TTAttentionBackendImpl(_ImplBase):
 
         # a scalar placeholder stands in for the cache while vLLM profiles memory;
         # layers that share another layer's cache never write it
-        if (
+        writes_cache = (
             isinstance(kv_cache, (list, tuple))
             and kv_cache[0].numel() > 0
             and self.kv_sharing_target_layer_name is None
-        ):
+        )
+        # a causal decode step writes its token inside the attention call (one operator)
+        fused_step = (
+            writes_cache
+            and not inputs.is_prefill
+            and not self.functional_cache_ops
+            and attn_metadata.is_causal
+            and attn_metadata.attn_mask is None
+        )
+        if writes_cache and not fused_step:
             self._handle_paged_attention(inputs, kv_cache, attn_metadata)
 
         if inputs.is_prefill:
             assert self.sinks is None, "Attention sink is unsupported in SDPA prefill"
             attn_output = self._compute_full_attention(inputs, kv_cache, attn_metadata)
         else:
-            attn_output = self._compute_decode_attention(inputs, kv_cache, attn_metadata)
+            attn_output = self._compute_decode_attention(inputs, kv_cache, attn_metadata, fused_step)
 
         flat = attn_output.reshape(-1, self.num_heads * self.head_size)
         output.copy_(flat.reshape_as(output))
@@ -383,8 +394,16 @@ class TTAttentionBackendImpl(_ImplBase):
         g = g.view(users, width, hkv, bs, d).permute(0, 2, 1, 3, 4).contiguous()
         return g.reshape(users, hkv, -1, d)[:, :, :num_tokens, :]
 
-    def _compute_decode_attention(self, inputs, kv_cache, attn_metadata: TTMetadata) -> torch.Tensor:
+    def _compute_decode_attention(self, inputs, kv_cache, attn_metadata: TTMetadata,
+                                  fused_step: bool = False) -> torch.Tensor:
         q = inputs.query.transpose(0, 1)  # [1, users, Hq, D]
+        if fused_step:  # cache update (reference :473-483) and attention (:634-668) in one operator
+            out = torch.ops.tt.paged_update_kv_decode_(
+                q, kv_cache[0], kv_cache[1], inputs.key.transpose(0, 1), inputs.value.transpose(0, 1),
+                attn_metadata.page_table, attn_metadata.cache_position, attention_sink=self.sinks,
+                scale=self.scale, sliding_window_size=self.sliding_window,
+            )
+            return out.transpose(0, 1)
         kwargs = {
             "cur_pos_tensor": attn_metadata.cache_position,
             "is_causal": attn_metadata.is_causal,

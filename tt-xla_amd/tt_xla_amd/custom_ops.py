@@ -289,6 +289,14 @@ def paged_scaled_dot_product_attention_decode(
     scale: Optional[float] = None,
     sliding_window_size: Optional[int] = None,
 ) -> torch.Tensor:
+    return _decode(query, key, value, page_table, is_causal, attn_mask, cur_pos_tensor, attention_sink,
+                   scale, sliding_window_size, None, None)
+
+
+def _decode(query, key, value, page_table, is_causal, attn_mask, cur_pos_tensor, attention_sink, scale,
+            sliding_window_size, k_new, v_new):
+    """Checks and launch shared by the decode operator and the fused update + decode operator
+    (k_new / v_new given: the step's cache update happens in the same call)."""
     if is_causal:
         assert attn_mask is None, "attention_mask must be None when is_causal is True."
         assert cur_pos_tensor is not None, "cur_pos_tensor must be provided when is_causal is True."
@@ -326,15 +334,67 @@ def paged_scaled_dot_product_attention_decode(
         if attention_sink.numel() != hq:
             raise ValueError(f"attention_sink must hold one logit per query head ({hq})")
         sink = attention_sink.reshape(hq).to(device=query.device, dtype=torch.float32).contiguous()
+    if k_new is None:
+        N.call(
+            "ttpa_paged_sdpa_decode_windowed",
+            out.data_ptr(), out.stride(1), out.stride(2), q.data_ptr(), q.stride(1), q.stride(2),
+            key.data_ptr(), value.data_ptr(), pt.data_ptr(), pt.stride(0), cur.data_ptr(),
+            int(cur.dtype == torch.int64), users, hq, hkv, d, bs, pt.shape[1], nb, float(scale), fmt,
+            int(sliding_window_size or 0), sink.data_ptr() if sink is not None else None,
+            ws.data_ptr(), ws_bytes, _stream(),
+        )
+        return out
+    if k_new.shape != v_new.shape or k_new.dtype != torch.bfloat16 or v_new.dtype != torch.bfloat16:
+        raise ValueError("k_new and v_new must be bfloat16 tensors of one shape")
+    if (k_new.dim() != 4 or k_new.shape[0] != 1 or k_new.shape[1] != users or k_new.shape[2] < hkv
+            or k_new.shape[3] != d):
+        raise ValueError(f"k_new {tuple(k_new.shape)} does not match users={users}, kv_heads={hkv}, head_size={d}")
+    k_new, v_new = _rows_contiguous(k_new), _rows_contiguous(v_new)
+    if k_new.stride() != v_new.stride():
+        v_new = v_new.contiguous()
+        k_new = k_new.contiguous()
     N.call(
-        "ttpa_paged_sdpa_decode_windowed",
+        "ttpa_paged_update_decode",
         out.data_ptr(), out.stride(1), out.stride(2), q.data_ptr(), q.stride(1), q.stride(2),
-        key.data_ptr(), value.data_ptr(), pt.data_ptr(), pt.stride(0), cur.data_ptr(),
-        int(cur.dtype == torch.int64), users, hq, hkv, d, bs, pt.shape[1], nb, float(scale), fmt,
-        int(sliding_window_size or 0), sink.data_ptr() if sink is not None else None,
-        ws.data_ptr(), ws_bytes, _stream(),
+        key.data_ptr(), value.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), k_new.stride(1),
+        k_new.stride(2), pt.data_ptr(), pt.stride(0), cur.data_ptr(), int(cur.dtype == torch.int64),
+        users, hq, hkv, d, bs, pt.shape[1], nb, float(scale), fmt, int(sliding_window_size or 0),
+        sink.data_ptr() if sink is not None else None, ws.data_ptr(), ws_bytes, _stream(),
     )
     return out
+
+
+@torch.library.custom_op("tt::paged_update_kv_decode_", mutates_args=["k_cache", "v_cache"],
+                         device_types=["cuda"])
+def paged_update_kv_decode_(
+    query: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    k_new: torch.Tensor,
+    v_new: torch.Tensor,
+    page_table: torch.Tensor,
+    cur_pos_tensor: torch.Tensor,
+    attention_sink: Optional[torch.Tensor] = None,
+    scale: Optional[float] = None,
+    sliding_window_size: Optional[int] = None,
+) -> torch.Tensor:
+    """The decode step of the attention backend as one operator: ``paged_update_kv_cache_`` with
+    ``update_indices = cur_pos_tensor`` followed by the causal
+    ``paged_scaled_dot_product_attention_decode`` on the updated caches (reference
+    attention.py:473-483 and :634-668).  Same results in the caches and in the output as the
+    two operators; where the 16x16x32 decode kernel serves the shape it is one launch.  (The
+    equivalence assumes that no user attends a row that another user's token is written to in
+    the same step.)"""
+    return _decode(query, k_cache, v_cache, page_table, True, None, cur_pos_tensor, attention_sink,
+                   scale, sliding_window_size, k_new, v_new)
+
+
+@paged_update_kv_decode_.register_fake
+def _(query, k_cache, v_cache, k_new, v_new, page_table, cur_pos_tensor, attention_sink=None,
+      scale=None, sliding_window_size=None):
+    return torch.empty_like(query)
+
+
 
 
 @paged_scaled_dot_product_attention_decode.register_fake
