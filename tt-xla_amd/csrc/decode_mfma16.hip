@@ -11,16 +11,17 @@
 // packed fma per element pair, exponents relative to the tile's largest, running reference
 // exponent for the V accumulator).
 //
-// FUSED: the kernel also performs the decode step's cache update.  The token at cur_pos of a
-// user sits in the last tile of each of its segments, and that tile belongs to exactly one
-// wavefront: it takes the token's K / V rows from the fresh activations instead of the cache
-// and stores them into the cache, so nobody depends on a separate update launch (bfloat16
-// caches; with block-float-8 the in-kernel quantiser cost the steady-state loop its scalar
-// registers, 64 spills, and the launch saved was lost again, so that format keeps two launches).  The fresh rows of the next tile's (user, head) are
-// requested with every tile, unconditionally: a conditional request in the steady-state loop
-// makes the wait-count pass drain the tile loads.  Users whose position is negative (padded
-// rows) attend nothing; their write follows the update operator's rule for negative positions
-// and is done by the thread that publishes their segment.
+// FUSED (bfloat16 caches): the kernel also performs the decode step's cache update.  The token
+// at cur_pos of a user sits in the last tile of each of its segments, and that tile belongs to
+// exactly one wavefront: it takes the token's K / V rows from the fresh activations instead
+// of the cache and stores them into the cache, so nobody depends on a separate update launch.
+// The fresh rows of the next tile's (user, head) are requested with every tile,
+// unconditionally: a conditional request in the steady-state loop makes the wait-count pass
+// drain the tile loads.  Users whose position is negative (padded rows) attend nothing; their
+// write follows the update operator's rule for negative positions and is done by the thread
+// that publishes their segment.  With a block-float-8 cache the in-kernel quantiser cost the
+// steady-state loop its scalar registers (64 spills) and the launch saved was lost again, so
+// that format keeps the update as a launch of its own.
 //
 // v_mfma_f32_16x16x32_{f16,bf16} with the heads as the 16-wide N dimension:
 //   S^T block b (16 keys):  A = K rows 16 b + lane%16, 8 elements per lane and k-step
