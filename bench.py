@@ -366,9 +366,7 @@ def run_decode(args):
     avg_step_bytes = sum(step_bytes[i % n] for i in range(args.steps)) / args.steps
     durs = time_decode_kernel_direct(copies, min(args.steps, 100))
     kern_ms = sum(d for d, _ in durs) / len(durs)
-    # with a bfloat16 cache the timed kernel also writes the new token (the update runs inside it)
-    per_launch = dec_bytes if args.workload == "config5" else step_bytes
-    kern_bytes = sum(per_launch[w] for _, w in durs) / len(durs)
+    kern_bytes = sum(step_bytes[w] for _, w in durs) / len(durs)  # the kernel also writes the new token
     achieved = kern_bytes / (kern_ms * 1e-3) / 1e9
     out = {
         "metric": "paged_decode_attention_hbm_throughput",
@@ -379,7 +377,7 @@ def run_decode(args):
         "dtype": dtype, "data": "synthetic",
         "config": {
             "workload": wl.name,
-            "step": "K + V cache update and paged decode attention as one operator (bfloat16 cache: the update runs inside the decode kernel; block-float-8: a launch of its own) + merge of the split-K partials, one layer, one token per sequence",
+            "step": "K + V cache update and paged decode attention (one operator: the update runs inside the decode kernel) + merge of the split-K partials, one layer, one token per sequence",
             "launch": args.launch, "steps_per_graph": runner.per_graph if args.launch == "graph" else None,
             "rotating_copies": n, **shape,
             "mean_context": float(wl.cache_position.float().mean()),

@@ -83,16 +83,17 @@ __device__ __forceinline__ uint32_t bfp8_encode16(const uint32_t (&w)[8], uint32
   for (int j = 0; j < 4; ++j) out[j] = 0;
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
-    uint32_t h = (i & 1) ? (w[i >> 1] >> 16) : (w[i >> 1] & 0xffffu);
-    uint32_t ex = (h >> 7) & 0xffu;
-    uint32_t sig = ex ? (0x80u | (h & 0x7fu)) : 0u;
-    uint32_t sh = min(emax - ex + 1u, 16u);
-    uint32_t q = sig >> sh;
-    uint32_t rem = sig & ((1u << sh) - 1u);
-    uint32_t half = 1u << (sh - 1u);
-    q += (rem > half || (rem == half && (q & 1u))) ? 1u : 0u;
+    const uint32_t h = (i & 1) ? (w[i >> 1] >> 16) : (w[i >> 1] & 0xffffu);
+    const uint32_t ex = (h >> 7) & 0xffu;
+    const uint32_t sig = min(ex, 1u) * (0x80u | (h & 0x7fu));  // zero / subnormal: 0
+    const uint32_t sh = min(emax - ex + 1u, 16u);  // >= 1
+    // round to nearest even without comparisons (they would each cost a scalar mask register):
+    // add half an ulp minus one plus the bit that will become the last kept one, then shift
+    uint32_t q = (sig + ((1u << (sh - 1u)) - 1u) + ((sig >> sh) & 1u)) >> sh;
     q = min(q, 127u);
-    uint32_t byte = (h & 0x8000u) ? 128u - q : 128u + q;
+    // 128 + q for a positive, 128 - q for a negative element
+    const uint32_t neg = (h >> 15) & 1u;
+    const uint32_t byte = 128u + q - 2u * q * neg;
     out[i >> 2] |= byte << (8 * (i & 3));
   }
   return emax;

@@ -434,11 +434,11 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
     return fail(TTPA_ERR_UNSUPPORTED, "decode: %d x %d segments need a grid of more than %d wavefronts",
                 users, kv_heads, a.n_waves);
   if (k_new) {
-    // The step's cache update: inside the 16x16 kernel when that is the kernel of this shape
-    // (bfloat16 caches), as a launch of its own in front of the attention otherwise.
+    // The step's cache update: inside the 16x16 kernel when that is the kernel of this shape,
+    // as a launch of its own in front of the attention otherwise.
     const bool vec_ok = aligned16(k_new) && aligned16(v_new) && new_user_stride % 8 == 0 &&
                         new_head_stride % 8 == 0;
-    if (use_mfma16 && vec_ok && kv_format == TTPA_KV_BF16) {
+    if (use_mfma16 && vec_ok) {
       a.k_new = static_cast<const uint16_t *>(k_new);
       a.v_new = static_cast<const uint16_t *>(v_new);
       a.new_us = new_user_stride, a.new_hs = new_head_stride;

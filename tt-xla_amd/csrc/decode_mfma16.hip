@@ -11,17 +11,16 @@
 // packed fma per element pair, exponents relative to the tile's largest, running reference
 // exponent for the V accumulator).
 //
-// FUSED (bfloat16 caches): the kernel also performs the decode step's cache update.  The token
-// at cur_pos of a user sits in the last tile of each of its segments, and that tile belongs to
-// exactly one wavefront: it takes the token's K / V rows from the fresh activations instead
-// of the cache and stores them into the cache, so nobody depends on a separate update launch.
-// The fresh rows of the next tile's (user, head) are requested with every tile,
-// unconditionally: a conditional request in the steady-state loop makes the wait-count pass
-// drain the tile loads.  Users whose position is negative (padded rows) attend nothing; their
+// FUSED: the kernel also performs the decode step's cache update.  The token at cur_pos of a
+// user sits in the last tile of each of its segments, and that tile belongs to exactly one
+// wavefront: it takes the token's K / V rows from the fresh activations instead of the cache
+// (quantising them for a block-float-8 cache) and stores them into the cache, so nobody
+// depends on a separate update launch.  The fresh rows of a segment's (user, head) are
+// requested where its Q rows are, once per segment (that block has its own waits; a request
+// inside the per-tile path would make the wait-count pass drain the tile loads in the
+// steady-state loop).  Users whose position is negative (padded rows) attend nothing; their
 // write follows the update operator's rule for negative positions and is done by the thread
-// that publishes their segment.  With a block-float-8 cache the in-kernel quantiser cost the
-// steady-state loop its scalar registers (64 spills) and the launch saved was lost again, so
-// that format keeps the update as a launch of its own.
+// that publishes their segment.
 //
 // v_mfma_f32_16x16x32_{f16,bf16} with the heads as the 16-wide N dimension:
 //   S^T block b (16 keys):  A = K rows 16 b + lane%16, 8 elements per lane and k-step
@@ -87,6 +86,7 @@ __device__ __forceinline__ float sum_over_quads(float v) {
 // position -k counts from the end of the user's table (the update operator's floor rule:
 // column = floor(pos / bs) taken from the end once, row = pos mod bs); positions that still fall
 // outside the table and blocks outside the cache are skipped.
+template <bool BFP8>
 __device__ inline void write_negative_position(const DecodeArgs &a, const int32_t *page_table,
                                                const void *cur_pos, int seg) {
   constexpr int D = 128;
@@ -103,16 +103,28 @@ __device__ inline void write_negative_position(const DecodeArgs &a, const int32_
   const uint16_t *src[2] = {a.k_new + u * a.new_us + h * a.new_hs, a.v_new + u * a.new_us + h * a.new_hs};
   uint8_t *dst[2] = {const_cast<uint8_t *>(a.k), const_cast<uint8_t *>(a.v)};
   for (int t = 0; t < 2; ++t) {
-    uint16_t *row = reinterpret_cast<uint16_t *>(dst[t]) + (((int64_t)phys * a.hkv + h) * a.bs + rem) * D;
-    for (int c = 0; c < D / 8; ++c)
-      *reinterpret_cast<uint4 *>(row + 8 * c) = *reinterpret_cast<const uint4 *>(src[t] + 8 * c);
+    if constexpr (BFP8) {
+      uint8_t *slab = dst[t] + ((int64_t)phys * a.hkv + h) * (int64_t)(a.bs + a.bs / 16) * D;
+      for (int grp = 0; grp < D / 16; ++grp) {
+        const uint4 lo = *reinterpret_cast<const uint4 *>(src[t] + 16 * grp);
+        const uint4 hi = *reinterpret_cast<const uint4 *>(src[t] + 16 * grp + 8);
+        const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        uint32_t bytes[4];
+        const uint32_t e = bfp8_encode16(w, bytes);
+        *reinterpret_cast<uint4 *>(slab + rem * D + 16 * grp) = make_uint4(bytes[0], bytes[1], bytes[2], bytes[3]);
+        slab[(int64_t)a.bs * D + rem * (D / 16) + grp] = (uint8_t)e;
+      }
+    } else {
+      uint16_t *row = reinterpret_cast<uint16_t *>(dst[t]) + (((int64_t)phys * a.hkv + h) * a.bs + rem) * D;
+      for (int c = 0; c < D / 8; ++c)
+        *reinterpret_cast<uint4 *>(row + 8 * c) = *reinterpret_cast<const uint4 *>(src[t] + 8 * c);
+    }
   }
 }
 
 template <bool BFP8, bool BIG, bool FUSED>
 __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     DecodeArgs a, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
-  static_assert(!(FUSED && BFP8), "the fused cache update is built for bfloat16 caches");
   constexpr int D = 128;
   constexpr int KSTEPS = D / 32, DBLK = D / 16;
   // staging geometry: 16 bytes per lane, so a load instruction covers 8 whole token rows of
@@ -138,7 +150,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
   const int64_t total = (int64_t)total_tiles * a.hkv;
   const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);
-  if constexpr (FUSED) write_negative_position(a, page_table, cur_pos, blockIdx.x * 256 + threadIdx.x);
+  if constexpr (FUSED) write_negative_position<BFP8>(a, page_table, cur_pos, blockIdx.x * 256 + threadIdx.x);
   if (total == 0 || wave >= n_eff) {
     publish_segment_row(a, s_pref, total, n_eff);
     return;
@@ -219,20 +231,46 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
       }
     }
   };
-  // FUSED: the lane's 16-byte chunk of the fresh K or V row of (user, head).
-  auto fetch_fresh = [&](const uint16_t *src, const Cursor &cu) {
-    return *reinterpret_cast<const u32x4 *>(src + cu.u * a.new_us + cu.h * a.new_hs + 8 * sc);
+  // FUSED: the lane's part of the fresh K or V row of (user, head): the 16 bytes of its chunk
+  // for a bfloat16 cache, the 16 bfloat16 elements of its group for block-float-8.
+  constexpr int NF = BFP8 ? 2 : 1;
+  struct Fresh {
+    u32x4 part[NF];
   };
-  // FUSED: puts the fresh row in place of row `r_star` of the fetched tile (registers) and
-  // stores it into the cache row `row` of the slab at byte offset `slab_base`.
-  auto patch_and_store = [&](uint8_t *cache, u32x4 (&raw)[NL], const u32x4 &fresh, int r_star,
-                             int64_t slab_base, int row) {
+  auto fetch_fresh = [&](const uint16_t *src, const Cursor &cu) {
+    const uint16_t *p = src + cu.u * a.new_us + cu.h * a.new_hs + (BFP8 ? 16 : 8) * sc;
+    Fresh f;
+#pragma unroll
+    for (int j = 0; j < NF; ++j) f.part[j] = *reinterpret_cast<const u32x4 *>(p + 8 * j);
+    return f;
+  };
+  // FUSED: puts the fresh row (quantised here for block-float-8) in place of row `r_star` of
+  // the fetched tile (registers) and stores it into the cache row `row` of the slab at byte
+  // offset `slab_base`.
+  auto patch_and_store = [&](uint8_t *cache, u32x4 (&raw)[NL], uint32_t (&ex)[NL], const Fresh &fresh,
+                             int r_star, int64_t slab_base, int row) {
     const int i_star = r_star / RPL;
     const bool mine = sr == r_star % RPL;
+    u32x4 val = fresh.part[0];
+    uint32_t e = 0;
+    if constexpr (BFP8) {
+      const u32x4 lo = fresh.part[0], hi = fresh.part[NF - 1];
+      const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      uint32_t out[4];
+      e = bfp8_encode16(w, out);
+      val = u32x4{out[0], out[1], out[2], out[3]};
+    }
 #pragma unroll
     for (int i = 0; i < NL; ++i)
-      if (i == i_star && mine) raw[i] = fresh;
-    if (mine) *reinterpret_cast<u32x4 *>(cache + slab_base + (int64_t)row * (D * BPE) + 16 * sc) = fresh;
+      if (i == i_star && mine) {
+        raw[i] = val;
+        if constexpr (BFP8) ex[i] = e << exp_shift;
+      }
+    if (mine) {
+      uint8_t *slab_ptr = cache + slab_base;
+      *reinterpret_cast<u32x4 *>(slab_ptr + (int64_t)row * (D * BPE) + 16 * sc) = val;
+      if constexpr (BFP8) slab_ptr[(int64_t)a.bs * D + (int64_t)row * GPR + sc] = (uint8_t)e;
+    }
   };
   // Cuts the lane's exponent bytes out of the fetched dwords (zero for rows past `nvalid` of a
   // partial tile, which stages them as zeros) and returns the largest of the tile.
@@ -312,7 +350,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   u32x4 kraw[NL], vraw[NL];
   uint32_t kex[NL], vex[NL];
   u32x4 qf[KSTEPS];
-  u32x4 kfresh = {0, 0, 0, 0}, vfresh = {0, 0, 0, 0};
+  Fresh kfresh = {}, vfresh = {};
   tile_offsets(cur, eo, xo);
   fetch(a.k, eo, xo, kraw, kex);
   fetch(a.v, eo, xo, vraw, vex);
@@ -357,7 +395,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
       int64_t slab_off;
       int row;
       if (fresh_target(slab_off, row))
-        patch_and_store(const_cast<uint8_t *>(a.k), kraw, kfresh, nvalid - 1, slab_off, row);
+        patch_and_store(const_cast<uint8_t *>(a.k), kraw, kex, kfresh, nvalid - 1, slab_off, row);
     }
     int eref_k = 0, eref_v = 0;
     if constexpr (BFP8) eref_k = tile_exponent(kex, nvalid, partial);
@@ -371,7 +409,6 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
       }
       tile_offsets(nxt, eo, xo);
       fetch(a.k, eo, xo, kraw, kex);
-      if constexpr (FUSED) kfresh = fetch_fresh(a.k_new, nxt);
     }
 
     // ---- S^T = K . Q^T ------------------------------------------------------------------------
@@ -421,14 +458,11 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
       int64_t slab_off;
       int row;
       if (fresh_target(slab_off, row))
-        patch_and_store(const_cast<uint8_t *>(a.v), vraw, vfresh, nvalid - 1, slab_off, row);
+        patch_and_store(const_cast<uint8_t *>(a.v), vraw, vex, vfresh, nvalid - 1, slab_off, row);
     }
     if constexpr (BFP8) eref_v = tile_exponent(vex, nvalid, partial);
     stage(true, vraw, vex, eref_v, nvalid, partial);
-    if constexpr (has_next) {
-      fetch(a.v, eo, xo, vraw, vex);
-      if constexpr (FUSED) vfresh = fetch_fresh(a.v_new, nxt);
-    }
+    if constexpr (has_next) fetch(a.v, eo, xo, vraw, vex);
 
     float lsum = 0.f, alpha_acc = alpha;
     u32x4 pf[2];
@@ -499,7 +533,13 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
       m_run = -INFINITY;
       l_run = 0.f;
       ev_run = 0;
-      if constexpr (has_next) load_q(nxt, qf);
+      if constexpr (has_next) {
+        load_q(nxt, qf);
+        if constexpr (FUSED) {  // the fresh rows of the new segment, once per segment
+          kfresh = fetch_fresh(a.k_new, nxt);
+          vfresh = fetch_fresh(a.v_new, nxt);
+        }
+      }
     }
     cur = nxt;
     ++x;
@@ -520,9 +560,9 @@ bool launch(const DecodeArgs &a, hipStream_t st) {
   return true;
 }
 
-template <bool BIG>
+template <bool BFP8, bool BIG>
 bool launch_fused_or_not(const DecodeArgs &a, hipStream_t st) {
-  return a.k_new ? launch<false, BIG, true>(a, st) : launch<false, BIG, false>(a, st);
+  return a.k_new ? launch<BFP8, BIG, true>(a, st) : launch<BFP8, BIG, false>(a, st);
 }
 
 }  // namespace
@@ -532,14 +572,12 @@ bool mfma16_decode_supported(const DecodeArgs &a, int head_size, int g) {
   return head_size == 128 && g <= 16 && a.users <= kMaxUsers16 && a.bs % rows_per_load == 0;
 }
 
-// With a.k_new set (bfloat16 caches only), the launch also performs the cache update of the step.
+// With a.k_new set, the launch also performs the cache update of the step.
 bool launch_mfma16_main(const DecodeArgs &a, hipStream_t st) {
   const bool big = a.bs % kTile == 0;
-  if (a.kv_format == TTPA_KV_BFP8) {
-    if (a.k_new) return false;
-    return big ? launch<true, true, false>(a, st) : launch<true, false, false>(a, st);
-  }
-  return big ? launch_fused_or_not<true>(a, st) : launch_fused_or_not<false>(a, st);
+  if (a.kv_format == TTPA_KV_BFP8)
+    return big ? launch_fused_or_not<true, true>(a, st) : launch_fused_or_not<true, false>(a, st);
+  return big ? launch_fused_or_not<false, true>(a, st) : launch_fused_or_not<false, false>(a, st);
 }
 
 }  // namespace decode
