@@ -174,6 +174,9 @@ def test_config2_full_size():
     (2, 64, 8, 128, 64, [1000, 257]),
     (3, 16, 8, 128, 16, [15, 16, 100]),
     (3, 12, 4, 128, 32, [100, 17, 450]),
+    (3, 16, 8, 256, 32, [31, 32, 700]),          # head size 256: tiles of 32 tokens on the 16x16 kernel
+    (3, 24, 2, 256, 8, [100, 17, 450]),          # blocks smaller than a tile, 12 heads per group
+    (2, 16, 16, 256, 16, [63, 64]),              # one query head per KV head
 ])
 def test_decode_every_kernel(monkeypatch, kernel, users, hq, hkv, d, bs, ctx):
     """The dot-product kernel and the two matrix-core kernels, each forced in turn on the same
@@ -190,8 +193,9 @@ def test_decode_every_kernel(monkeypatch, kernel, users, hq, hkv, d, bs, ctx):
            O.textbook_decode_fp32(wl.q, k.cpu(), v.cpu(), wl.page_table, wl.cache_position, wl.scale))
 
 
-@pytest.mark.parametrize("kernel,hq", [("valu", 32), ("mfma", 64), ("mfma16", 64), ("mfma16", 32)])
-def test_decode_several_tiles_per_wavefront(monkeypatch, kernel, hq):
+@pytest.mark.parametrize("kernel,hq,d", [("valu", 32, 128), ("mfma", 64, 128), ("mfma16", 64, 128),
+                                          ("mfma16", 32, 128), ("mfma16", 32, 256), ("mfma16", 8, 256)])
+def test_decode_several_tiles_per_wavefront(monkeypatch, kernel, hq, d):
     """A grid of one wavefront per CU over ~1000 tiles: every wavefront walks several tiles and
     crosses segment boundaries (running maximum, partial hand-over, Q reload)."""
     from tt_xla_amd import workloads
@@ -199,10 +203,10 @@ def test_decode_several_tiles_per_wavefront(monkeypatch, kernel, hq):
     monkeypatch.setenv("TTPA_DECODE_KERNEL", kernel)
     monkeypatch.setenv("TTPA_DECODE_WAVES_PER_CU", "1")
     ctx = [1990, 2047, 1500, 2300]
-    name = f"decode [{kernel}] h{hq}x8 one wavefront per CU ctx{ctx}"
+    name = f"decode [{kernel}] h{hq}x8 d{d} one wavefront per CU ctx{ctx}"
     print(name, flush=True)
     nb = sum((c + 1 + 63) // 64 for c in ctx) + 3
-    wl = workloads.decode_ragged(name, 91, 4, hq, 8, 128, 64, nb, ctx)
+    wl = workloads.decode_ragged(name, 91, 4, hq, 8, d, 64, nb, ctx)
     got, k, v = _run(wl)
     _check(name, got,
            O.textbook_decode_fp32(wl.q, k.cpu(), v.cpu(), wl.page_table, wl.cache_position, wl.scale))

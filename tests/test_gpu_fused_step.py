@@ -33,7 +33,8 @@ CASES = [
     (4, 32, 8, 128, 64, [1990, 2047, 1500, 2300], True, 0, False, True),
     (3, 8, 8, 64, 32, [0, 62, 300], False, 0, False, False),            # not fused: two launches
     (2, 8, 4, 128, 32, [40, 333], False, 0, False, False),              # G = 2: dot-product kernel
-    (2, 16, 8, 256, 64, [130, 64], False, 0, False, False),
+    (2, 16, 8, 256, 64, [130, 64], False, 0, False, False),             # head size 256, fused
+    (4, 8, 4, 256, 16, [31, 32, 1000, 1500], False, 300, True, True),   # blocks smaller than its 32-token tiles
 ]
 
 

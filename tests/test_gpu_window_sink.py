@@ -61,16 +61,16 @@ def test_decode_window_and_sink(users, hq, hkv, d, bs, ctx, window, with_sink):
     _check(name, out.cpu(), want)
 
 
-@pytest.mark.parametrize("kernel", ["mfma", "mfma16"])
-def test_decode_window_and_sink_matrix_core_kernels(monkeypatch, kernel):
+@pytest.mark.parametrize("kernel,d", [("mfma", 128), ("mfma16", 128), ("mfma16", 256)])
+def test_decode_window_and_sink_matrix_core_kernels(monkeypatch, kernel, d):
     """Window edge inside a tile, sink, short and long users on each matrix-core kernel, with a
     small grid so that wavefronts cross from one windowed segment into the next."""
     from tt_xla_amd import workloads
 
     monkeypatch.setenv("TTPA_DECODE_KERNEL", kernel)
     monkeypatch.setenv("TTPA_DECODE_WAVES_PER_CU", "1")
-    users, hq, hkv, d, bs, ctx, window = 4, 64, 8, 128, 64, [1990, 30, 1500, 2300], 1000
-    name = f"decode [{kernel}] b{users} h{hq}x{hkv} ctx{ctx} window{window} sink"
+    users, hq, hkv, bs, ctx, window = 4, 64, 8, 64, [1990, 30, 1500, 2300], 1000
+    name = f"decode [{kernel}] b{users} h{hq}x{hkv} d{d} ctx{ctx} window{window} sink"
     print(name, flush=True)
     nb = sum((c + 1 + bs - 1) // bs for c in ctx) + 3
     wl = workloads.decode_ragged(name, 93, users, hq, hkv, d, bs, nb, ctx)

@@ -320,8 +320,9 @@ int launch_g(const DecodeArgs &a, int g, hipStream_t st) {
     case 8: launch<D, 8>(a, st); break;
     default:
       return fail(TTPA_ERR_UNSUPPORTED,
-                  "query heads per KV head = %d: more than 8 (up to 32) need head_size 64 / 128, at most "
-                  "1024 users and a block_size that is a multiple of 1024 / (bytes of a cache row)",
+                  "query heads per KV head = %d: more than 8 (up to 32 with head_size 64 / 128, up to 16 "
+                  "with 256) need at most 1024 users and a block_size that is a multiple of 1024 / (bytes "
+                  "of a cache row)",
                   g);
   }
   return TTPA_OK;
@@ -405,9 +406,11 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   // do not (their cost per tile does not depend on the group width).  Measured on bfloat16
   // caches with head size 128: at 1 and 2 query heads per KV head the VALU kernel is 2 - 19 %
   // faster (the larger figure on launches of a few tiles), at 4 the 16x16x32 kernel is 2 - 8 %
-  // faster, at 8 the VALU kernel is 2.5 times slower.  So: 16x16x32 kernel for head size 128 and
-  // 4 ... 16 heads per group, 32x32x16 kernel for the other wide groups (head size 64, up to 32
-  // heads), VALU kernel for the rest.  The block-float-8 cache goes to a matrix-core kernel
+  // faster, at 8 the VALU kernel is 2.5 times slower.  With head size 256 the VALU kernel streams
+  // at 3.8 TB/s with one head per group and at 1.2 TB/s with eight, the 16x16x32 kernel at 5.3 -
+  // 5.6 TB/s with any.  So: 16x16x32 kernel for head size 128 and 4 ... 16 heads per group and
+  // for head size 256 (up to 16 heads), 32x32x16 kernel for the other wide groups (head size 64,
+  // up to 32 heads), VALU kernel for the rest.  The block-float-8 cache goes to a matrix-core kernel
   // whenever one applies: there the byte expansion costs one VALU operation per element and the
   // products none, while the VALU kernel pays for both.
   // TTPA_DECODE_KERNEL=valu|mfma|mfma16 overrides the choice.
@@ -420,11 +423,12 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
                      : !strcmp(forced_name, "mfma16") ? 3 : 0;
   const bool mfma_ok = mfma_decode_supported(a, head_size, g);
   const bool mfma16_ok = mfma16_decode_supported(a, head_size, g);
-  bool use_mfma16 = mfma16_ok && (g >= 4 || kv_format == TTPA_KV_BFP8);
+  bool use_mfma16 = mfma16_ok && (g >= 4 || kv_format == TTPA_KV_BFP8 || head_size == 256);
   bool use_mfma = !use_mfma16 && mfma_ok && (g >= 5 || kv_format == TTPA_KV_BFP8);
-  if (forced == 1) use_mfma = use_mfma16 = false;
-  if (forced == 2) use_mfma = mfma_ok, use_mfma16 = false;
-  if (forced == 3) use_mfma16 = mfma16_ok, use_mfma = !mfma16_ok && use_mfma;
+  // a forced kernel that is not built for the shape leaves the default choice in place
+  if (forced == 1 && g <= 8) use_mfma = use_mfma16 = false;
+  if (forced == 2 && mfma_ok) use_mfma = true, use_mfma16 = false;
+  if (forced == 3 && mfma16_ok) use_mfma16 = true, use_mfma = false;
   // The matrix-core kernels get one workgroup per CU whatever the cache format: the 32x32 kernel
   // fills the CU's LDS with one, and the 16x16 kernel streams as fast with one as with the two
   // that would fit, while twice the partials cost the merge kernel more.
@@ -455,7 +459,7 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   if (ev0) (void)hipEventRecord(ev0, st);
   int rc = TTPA_OK;
   if (use_mfma16) {
-    if (!launch_mfma16_main(a, st))
+    if (!launch_mfma16_main(a, head_size, st))
       rc = fail(TTPA_ERR_LAUNCH, "decode: cannot configure the 16x16 matrix-core kernel");
   } else if (use_mfma) {
     if (!launch_mfma_main(a, head_size, st))

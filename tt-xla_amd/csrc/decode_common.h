@@ -44,19 +44,21 @@ __device__ __forceinline__ int window_lo(const DecodeArgs &a, int len) {
   return (a.window > 0 && len > a.window) ? len - a.window : 0;
 }
 
-// Attended positions of user u are [window_lo(len), len); returns the number of 64-token tiles
+// Attended positions of user u are [window_lo(len), len); returns the number of TILE-token tiles
 // they touch.
+template <int TILE = kTile>
 __device__ __forceinline__ int tiles_of_user(const DecodeArgs &a, const void *__restrict__ cur,
                                              int u, int &len) {
   int64_t cp = load_index(cur, a.cur_i64, u);
   int64_t cap = (int64_t)a.w * a.bs;
   int64_t l = cp < 0 ? 0 : (cp + 1 < cap ? cp + 1 : cap);
   len = (int)l;
-  return (int)((l + kTile - 1) / kTile) - window_lo(a, len) / kTile;
+  return (int)((l + TILE - 1) / TILE) - window_lo(a, len) / TILE;
 }
 
 // Exclusive prefix sum of per-user tile counts into pref[0..users] and attended lengths into
 // lens[0..users); all 256 threads.  Each position is read from global memory once.
+template <int TILE = kTile>
 __device__ inline void build_prefix(const DecodeArgs &a, const void *__restrict__ cur, int *pref,
                              int *lens, int *wave_sums) {
   const int tid = threadIdx.x;
@@ -66,7 +68,7 @@ __device__ inline void build_prefix(const DecodeArgs &a, const void *__restrict_
   int local = 0;
   for (int u = beg; u < end; ++u) {
     int len;
-    int nt = tiles_of_user(a, cur, u, len);
+    int nt = tiles_of_user<TILE>(a, cur, u, len);
     lens[u] = len;
     pref[u + 1] = nt;  // replaced by the running sum below
     local += nt;
@@ -228,13 +230,14 @@ struct Shape {
 
 // Position of a wavefront in the flat tile list.
 struct Cursor {
-  int u, h, t;      // user, kv head, absolute tile index (tile t covers positions 64 t ..)
+  int u, h, t;      // user, kv head, absolute tile index (tile t covers positions TILE t ..)
   int len, lo;      // user u attends positions [lo, len)
   int tiles_left;   // tiles of this segment from t on (including t)
 };
 
 // Finds the segment that owns unit `x` of the flat tile list (binary search over the
 // per-user prefix in LDS).  Everything is wavefront-uniform.
+template <int TILE = kTile>
 __device__ __forceinline__ Cursor locate_unit(const DecodeArgs &a, const int *s_pref,
                                               const int *s_len, int64_t x) {
   const int users = a.users, hkv = a.hkv;
@@ -254,7 +257,7 @@ __device__ __forceinline__ Cursor locate_unit(const DecodeArgs &a, const int *s_
   cu.tiles_left = nt - rel;
   cu.len = __builtin_amdgcn_readfirstlane(s_len[lo_u]);
   cu.lo = window_lo(a, cu.len);
-  cu.t = cu.lo / kTile + rel;
+  cu.t = cu.lo / TILE + rel;
   return cu;
 }
 
@@ -385,10 +388,10 @@ bool launch_bfp8_main(const DecodeArgs &a, int head_size, int g, hipStream_t st)
 // Matrix-core main kernel (decode_mfma.hip) for wide head groups and block-float-8.
 bool mfma_decode_supported(const DecodeArgs &a, int head_size, int g);
 bool launch_mfma_main(const DecodeArgs &a, int head_size, hipStream_t st);
-// Matrix-core main kernel for the block-float-8 cache with head size 128 and up to 16 query
-// heads per KV head (decode_mfma16.hip).
+// 16x16x32 matrix-core main kernel (decode_mfma16.hip): up to 16 query heads per KV head, head
+// size 128 (either cache format) or 256 (bfloat16 cache).
 bool mfma16_decode_supported(const DecodeArgs &a, int head_size, int g);
-bool launch_mfma16_main(const DecodeArgs &a, hipStream_t st);
+bool launch_mfma16_main(const DecodeArgs &a, int head_size, hipStream_t st);
 
 }  // namespace decode
 }  // namespace ttpa

@@ -1,10 +1,11 @@
-// Paged decode attention on the 16x16x32 matrix-core shape: head size 128, up to 16 query
-// heads per KV head, 72 KiB of LDS per workgroup; block-float-8 cache (expanded to half
-// precision) or bfloat16 cache.
+// Paged decode attention on the 16x16x32 matrix-core shape: up to 16 query heads per KV head,
+// 72 KiB of LDS per workgroup; head size 128 with a block-float-8 cache (expanded to half
+// precision) or a bfloat16 cache, head size 256 with a bfloat16 cache.
 //
-// Work decomposition, partial slots and merge kernel are those of decode.hip.  Inside a
-// wavefront a 64-token tile of K, then of V, goes global -> registers -> a 16 KiB wave-private
-// LDS buffer of 16-bit elements that both tensors use in turn:
+// Work decomposition, partial slots and merge kernel are those of decode.hip, with tiles of
+// 8192 / head_size tokens (64 or 32): 16 KiB of 16-bit elements whatever the head size.  Inside a
+// wavefront a tile of K, then of V, goes global -> registers -> a 16 KiB wave-private
+// LDS buffer that both tensors use in turn:
 //   stage K(t) | prefetch K(t+1) | S^T = K Q^T | softmax | stage V(t) | prefetch V(t+1) | O^T += V^T P^T
 // so every global load has three quarters of a tile period to arrive.  The byte -> half
 // expansion of the block-float-8 cache is the one of decode_mfma.hip (one permute and one
@@ -31,10 +32,11 @@
 // Compared with the 32x32x16 kernel, a lane carries half the scores and half the
 // accumulator, and the matrix pipe is busy half as long per tile.
 //
-// LDS tile: 64 rows of 256 bytes, unpadded, sixteen 16-byte chunks per row stored at
+// LDS tile: rows of 2 * head_size bytes, unpadded, 16-byte chunks stored at
 // chunk ^ (row & 15) for K (A-operand reads: 16 rows, one chunk column) and at
 // chunk ^ (2 y | y & 1), y = row & 7, for V (transposing reads: 32 lanes cover 8 rows x 2
 // chunks); both make the staging writes of two neighbouring rows land in different banks too.
+// (The exchange stays inside an aligned group of 16 chunks = 256 bytes = every bank once.)
 #include "decode_common.h"
 
 namespace ttpa {
@@ -48,7 +50,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kMaxUsers16 = 1024;
-constexpr int kTileBytes = kTile * 256;
+constexpr int kTileBytes = 16384;  // TILE tokens of head_size 16-bit elements
 
 template <bool F16>
 __device__ __forceinline__ floatx4 mma16(const u32x4 &x, const u32x4 &y, const floatx4 &c) {
@@ -86,10 +88,9 @@ __device__ __forceinline__ float sum_over_quads(float v) {
 // position -k counts from the end of the user's table (the update operator's floor rule:
 // column = floor(pos / bs) taken from the end once, row = pos mod bs); positions that still fall
 // outside the table and blocks outside the cache are skipped.
-template <bool BFP8>
+template <bool BFP8, int D>
 __device__ inline void write_negative_position(const DecodeArgs &a, const int32_t *page_table,
                                                const void *cur_pos, int seg) {
-  constexpr int D = 128;
   if (seg >= a.users * a.hkv) return;
   const int u = seg / a.hkv, h = seg - u * a.hkv;
   const int64_t pos = load_index(cur_pos, a.cur_i64, u);
@@ -122,17 +123,21 @@ __device__ inline void write_negative_position(const DecodeArgs &a, const int32_
   }
 }
 
-template <bool BFP8, bool BIG, bool FUSED>
+template <int D, bool BFP8, bool BIG, bool FUSED>
 __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     DecodeArgs a, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
-  constexpr int D = 128;
+  static_assert(D == 128 || (D == 256 && !BFP8), "shapes built");
+  constexpr int TILE = kTileBytes / (2 * D);  // tokens per tile
+  constexpr int ROWB = 2 * D;                 // bytes of a tile row in LDS
   constexpr int KSTEPS = D / 32, DBLK = D / 16;
-  // staging geometry: 16 bytes per lane, so a load instruction covers 8 whole token rows of
-  // element bytes or 4 of bfloat16
+  constexpr int KBLK = TILE / 16;     // score blocks (16 keys each) per tile
+  constexpr int PSTEPS = TILE / 32;   // k-steps of the second product per tile
+  // staging geometry: 16 bytes per lane, so a load instruction covers (head size 128) 8 whole
+  // token rows of element bytes or 4 of bfloat16
   constexpr int BPE = BFP8 ? 1 : 2;   // bytes per cache element
   constexpr int LPR = D * BPE / 16;   // lanes per token row
   constexpr int RPL = 64 / LPR;       // rows per load
-  constexpr int NL = kTile / RPL;     // loads per tile and tensor
+  constexpr int NL = TILE / RPL;      // loads per tile and tensor
   constexpr int GPR = D / 16;         // exponent bytes per row (block-float-8)
   constexpr int NOFF = BIG ? 1 : NL;
 
@@ -141,7 +146,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   __shared__ int s_wsum[kWavesPerBlock];
   extern __shared__ __attribute__((aligned(16))) uint8_t tiles[];
 
-  build_prefix(a, cur_pos, s_pref, s_len, s_wsum);
+  build_prefix<TILE>(a, cur_pos, s_pref, s_len, s_wsum);
 
   const int lane = threadIdx.x & 63;
   const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -150,7 +155,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
   const int64_t total = (int64_t)total_tiles * a.hkv;
   const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);
-  if constexpr (FUSED) write_negative_position<BFP8>(a, page_table, cur_pos, blockIdx.x * 256 + threadIdx.x);
+  if constexpr (FUSED) write_negative_position<BFP8, D>(a, page_table, cur_pos, blockIdx.x * 256 + threadIdx.x);
   if (total == 0 || wave >= n_eff) {
     publish_segment_row(a, s_pref, total, n_eff);
     return;
@@ -178,17 +183,17 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
 #pragma unroll
   for (int j = 0; j < KPAT; ++j) {
     const int row = RPL * j + sr;
-    kw[j] = (uint32_t)(sr * 256 + (((CPL * sc) ^ (row & 15)) << 4));
+    kw[j] = (uint32_t)(sr * ROWB + (((CPL * sc) ^ (row & 15)) << 4));
   }
 #pragma unroll
   for (int j = 0; j < VPAT; ++j) {
     const int y = (RPL * j + sr) & 7;
-    vw[j] = (uint32_t)(sr * 256 + (((CPL * sc) ^ ((2 * y) | (y & 1))) << 4));
+    vw[j] = (uint32_t)(sr * ROWB + (((CPL * sc) ^ ((2 * y) | (y & 1))) << 4));
   }
   // A-operand reads of K: row 16 b + n, chunk 4 s + quad
   uint32_t kr[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s) kr[s] = (uint32_t)(n * 256 + (((4 * s + quad) ^ n) << 4));
+  for (int s = 0; s < KSTEPS; ++s) kr[s] = (uint32_t)(n * ROWB + (((4 * s + quad) ^ n) << 4));
   // transposing reads of V: lane addresses row 4 quad + n / 4 (+ 16 per key block), the 8 bytes
   // at element 16 db + 4 (n & 3)
   uint32_t vr[DBLK];
@@ -197,14 +202,14 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     const int y7 = (4 * quad + y) & 7;  // row & 7: key blocks start at multiples of 16
 #pragma unroll
     for (int db = 0; db < DBLK; ++db)
-      vr[db] = (uint32_t)((4 * quad + y) * 256 + ((((2 * db + xx) ^ ((2 * y7) | (y7 & 1)))) << 4) +
+      vr[db] = (uint32_t)((4 * quad + y) * ROWB + ((((2 * db + xx) ^ ((2 * y7) | (y7 & 1)))) << 4) +
                           8 * (n & 1));
   }
 
-  auto locate = [&](int64_t xx) { return locate_unit(a, s_pref, s_len, xx); };
+  auto locate = [&](int64_t xx) { return locate_unit<TILE>(a, s_pref, s_len, xx); };
   auto tile_offsets = [&](const Cursor &cu, int64_t (&eo)[NOFF], int64_t (&xo)[NOFF]) {
     const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
-    const int tok0 = cu.t * kTile;
+    const int tok0 = cu.t * TILE;
 #pragma unroll
     for (int i = 0; i < NOFF; ++i) {
       const int tk = tok0 + RPL * i;
@@ -293,7 +298,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
                    bool clear) {
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-      const uint32_t w0 = (is_v ? vw[i % VPAT] : kw[i % KPAT]) + (uint32_t)(i * RPL * 256);
+      const uint32_t w0 = (is_v ? vw[i % VPAT] : kw[i % KPAT]) + (uint32_t)(i * RPL * ROWB);
       if constexpr (BFP8) {
         const uint32_t field = (uint32_t)max((int)ex[i] - (eref - 15), 0);
         const uint32_t sbits = field << 10;
@@ -369,9 +374,9 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
 
   auto process_tile = [&](auto has_next_tag) {
     constexpr bool has_next = decltype(has_next_tag)::value;
-    const int nvalid = cur.len - cur.t * kTile;
-    const bool partial = nvalid < kTile;
-    const int nbelow = cur.lo - cur.t * kTile;  // sliding window: > 0 only in a segment's first tile
+    const int nvalid = cur.len - cur.t * TILE;
+    const bool partial = nvalid < TILE;
+    const int nbelow = cur.lo - cur.t * TILE;  // sliding window: > 0 only in a segment's first tile
     const bool same_seg = has_next && cur.tiles_left > 1;
     Cursor nxt = cur;
 
@@ -412,20 +417,20 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     }
 
     // ---- S^T = K . Q^T ------------------------------------------------------------------------
-    floatx4 st[4];
+    floatx4 st[KBLK];
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
+    for (int b = 0; b < KBLK; ++b) {
       st[b] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
-        const uint4 kq = *reinterpret_cast<const uint4 *>(tile + kr[s] + b * (16 * 256));
+        const uint4 kq = *reinterpret_cast<const uint4 *>(tile + kr[s] + b * (16 * ROWB));
         st[b] = mma16<BFP8>(u32x4{kq.x, kq.y, kq.z, kq.w}, qf[s], st[b]);
       }
     }
     // ---- online softmax: lane (head, quad) holds keys 16 b + 4 quad + r ------------------------
     if (partial || nbelow > 0) {
 #pragma unroll
-      for (int b = 0; b < 4; ++b)
+      for (int b = 0; b < KBLK; ++b)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int key = 16 * b + 4 * quad + r;
@@ -437,13 +442,13 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     float mloc = -INFINITY;
     if (scale >= 0.f) {
 #pragma unroll
-      for (int b = 0; b < 4; ++b)
+      for (int b = 0; b < KBLK; ++b)
 #pragma unroll
         for (int r = 0; r < 4; ++r) mloc = fmaxf(mloc, st[b][r]);
       mloc *= scale;
     } else {  // a negative scale turns the maximum into a minimum: compare scaled scores
 #pragma unroll
-      for (int b = 0; b < 4; ++b)
+      for (int b = 0; b < KBLK; ++b)
 #pragma unroll
         for (int r = 0; r < 4; ++r) mloc = fmaxf(mloc, st[b][r] * scale);
     }
@@ -465,7 +470,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     if constexpr (has_next) fetch(a.v, eo, xo, vraw, vex);
 
     float lsum = 0.f, alpha_acc = alpha;
-    u32x4 pf[2];
+    u32x4 pf[PSTEPS];
     if constexpr (BFP8) {
       // bring this tile's V factor and the accumulator to the larger reference exponent
       const int ev_new = max(ev_run, eref_v);
@@ -473,7 +478,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
       alpha_acc = alpha * __builtin_ldexpf(1.f, ev_run - ev_new);
       ev_run = ev_new;
 #pragma unroll
-      for (int b = 0; b < 4; ++b)
+      for (int b = 0; b < KBLK; ++b)
 #pragma unroll
         for (int r = 0; r < 4; r += 2) {
           const float p0 = __builtin_amdgcn_exp2f(fmaf(st[b][r], scale, -m_safe));
@@ -483,7 +488,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
         }
     } else {
 #pragma unroll
-      for (int b = 0; b < 4; ++b)
+      for (int b = 0; b < KBLK; ++b)
 #pragma unroll
         for (int r = 0; r < 4; r += 2) {
           const float p0 = __builtin_amdgcn_exp2f(fmaf(st[b][r], scale, -m_safe));
@@ -501,13 +506,13 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     }
     // ---- O^T += V^T . P^T ------------------------------------------------------------------------
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
+    for (int s = 0; s < PSTEPS; ++s)
 #pragma unroll
       for (int db = 0; db < DBLK; ++db) {
         typedef __attribute__((address_space(3))) shortx4 *lds_v4;
-        const uint8_t *vp = tile + vr[db] + s * (32 * 256);
+        const uint8_t *vp = tile + vr[db] + s * (32 * ROWB);
         shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vp));
-        shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vp + 16 * 256));
+        shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vp + 16 * ROWB));
         const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
         acc[db] = mma16<BFP8>(u32x4{l2.x, l2.y, h2.x, h2.y}, pf[s], acc[db]);
       }
@@ -548,36 +553,40 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   process_tile(std::false_type{});
 }
 
-template <bool BFP8, bool BIG, bool FUSED>
+template <int D, bool BFP8, bool BIG, bool FUSED>
 bool launch(const DecodeArgs &a, hipStream_t st) {
   const int blocks = a.n_waves / kWavesPerBlock;
   const size_t lds = (size_t)kWavesPerBlock * kTileBytes;
   static std::atomic<uint64_t> lds_ready{0};
-  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_mfma16_kernel<BFP8, BIG, FUSED>), lds,
+  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_mfma16_kernel<D, BFP8, BIG, FUSED>), lds,
                           lds_ready))
     return false;
-  paged_decode_mfma16_kernel<BFP8, BIG, FUSED><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
+  paged_decode_mfma16_kernel<D, BFP8, BIG, FUSED><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
   return true;
 }
 
-template <bool BFP8, bool BIG>
+template <int D, bool BFP8, bool BIG>
 bool launch_fused_or_not(const DecodeArgs &a, hipStream_t st) {
-  return a.k_new ? launch<BFP8, BIG, true>(a, st) : launch<BFP8, BIG, false>(a, st);
+  return a.k_new ? launch<D, BFP8, BIG, true>(a, st) : launch<D, BFP8, BIG, false>(a, st);
 }
 
 }  // namespace
 
 bool mfma16_decode_supported(const DecodeArgs &a, int head_size, int g) {
-  const int rows_per_load = a.kv_format == TTPA_KV_BFP8 ? 8 : 4;
-  return head_size == 128 && g <= 16 && a.users <= kMaxUsers16 && a.bs % rows_per_load == 0;
+  const bool bfp8 = a.kv_format == TTPA_KV_BFP8;
+  if (!(head_size == 128 || (head_size == 256 && !bfp8))) return false;
+  const int rows_per_load = 1024 / (head_size * (bfp8 ? 1 : 2));  // a load covers whole rows of one block
+  return g <= 16 && a.users <= kMaxUsers16 && a.bs % rows_per_load == 0;
 }
 
 // With a.k_new set, the launch also performs the cache update of the step.
-bool launch_mfma16_main(const DecodeArgs &a, hipStream_t st) {
-  const bool big = a.bs % kTile == 0;
+bool launch_mfma16_main(const DecodeArgs &a, int head_size, hipStream_t st) {
+  const bool big = a.bs % (kTileBytes / (2 * head_size)) == 0;  // blocks hold whole tiles
+  if (head_size == 256)
+    return big ? launch_fused_or_not<256, false, true>(a, st) : launch_fused_or_not<256, false, false>(a, st);
   if (a.kv_format == TTPA_KV_BFP8)
-    return big ? launch_fused_or_not<true, true>(a, st) : launch_fused_or_not<true, false>(a, st);
-  return big ? launch_fused_or_not<false, true>(a, st) : launch_fused_or_not<false, false>(a, st);
+    return big ? launch_fused_or_not<128, true, true>(a, st) : launch_fused_or_not<128, true, false>(a, st);
+  return big ? launch_fused_or_not<128, false, true>(a, st) : launch_fused_or_not<128, false, false>(a, st);
 }
 
 }  // namespace decode
