@@ -100,10 +100,15 @@ def test_decode_random_case(monkeypatch, seed):
     kw = dict(scale=wl.scale, sliding_window_size=window if window else None,
               attention_sink=sink.cuda() if sink is not None else None)
     torch.ops.tt.paged_update_kv_cache_(k_seq, v_seq, dev.k_new, dev.v_new, pos, dev.page_table)
-    out_seq = torch.ops.tt.paged_scaled_dot_product_attention_decode(
-        dev.q, k_seq, v_seq, dev.page_table, is_causal=True, cur_pos_tensor=pos, **kw)
     out_fus = torch.ops.tt.paged_update_kv_decode_(
         dev.q, k_fus, v_fus, dev.k_new, dev.v_new, dev.page_table, pos, **kw)
+    # As a step, groups of 2 and 3 heads run on the 16x16x32 kernel, which the attention alone
+    # only picks from 4 up: ask for it here (ignored where it is not built for the shape), so
+    # that both sides run the same arithmetic and the outputs can be compared exactly.
+    if not c["bfp8"] and d == 128 and g in (2, 3):
+        monkeypatch.setenv("TTPA_DECODE_KERNEL", "mfma16")
+    out_seq = torch.ops.tt.paged_scaled_dot_product_attention_decode(
+        dev.q, k_seq, v_seq, dev.page_table, is_causal=True, cur_pos_tensor=pos, **kw)
     # several padded rows write different tokens to one row of the null block 0: which one
     # stays is unspecified on the reference too, so that block is left out of the comparison
     first = 1 if len(c["pad"]) > 1 else 0

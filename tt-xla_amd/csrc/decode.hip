@@ -423,7 +423,11 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
                      : !strcmp(forced_name, "mfma16") ? 3 : 0;
   const bool mfma_ok = mfma_decode_supported(a, head_size, g);
   const bool mfma16_ok = mfma16_decode_supported(a, head_size, g);
-  bool use_mfma16 = mfma16_ok && (g >= 4 || kv_format == TTPA_KV_BFP8 || head_size == 256);
+  // As a step (update + attention) the 16x16x32 kernel with the update inside already wins at 2
+  // and 3 heads per group (1 - 6 % and 2 - 11 % per step against update launch + VALU kernel; at
+  // 1 head the two are within 2.5 % of each other either way).
+  const int g_min16 = k_new ? 2 : 4;
+  bool use_mfma16 = mfma16_ok && (g >= g_min16 || kv_format == TTPA_KV_BFP8 || head_size == 256);
   bool use_mfma = !use_mfma16 && mfma_ok && (g >= 5 || kv_format == TTPA_KV_BFP8);
   // a forced kernel that is not built for the shape leaves the default choice in place
   if (forced == 1 && g <= 8) use_mfma = use_mfma16 = false;
