@@ -78,13 +78,20 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
       if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
       off[0] = (((int64_t)phys * a.hkv + cu.h) * a.bs + (tok0 % a.bs)) * D;
     } else {
+      // block_size is a multiple of 4, so the 4 rows of a load never cross a block: block and
+      // row advance without a division, and the table is read only where the block changes
+      int col = tok0 / a.bs, row = tok0 - col * a.bs;
+      int64_t base = 0;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        int tk = tok0 + 4 * i;
-        int col = tk / a.bs;
-        int phys = (col < a.w) ? __builtin_amdgcn_readfirstlane(pt_row[col]) : 0;
-        if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
-        off[i] = (((int64_t)phys * a.hkv + cu.h) * a.bs + (tk % a.bs)) * D;
+        if (i == 0 || row == 0) {
+          int phys = (col < a.w) ? __builtin_amdgcn_readfirstlane(pt_row[col]) : 0;
+          if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+          base = ((int64_t)phys * a.hkv + cu.h) * a.bs * D;
+        }
+        off[i] = base + (int64_t)row * D;
+        row += 4;
+        if (row >= a.bs) row = 0, ++col;
       }
     }
   };

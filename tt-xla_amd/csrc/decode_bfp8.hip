@@ -75,16 +75,21 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_kernel(
   auto tile_offsets = [&](const Cursor &cu, int64_t (&eo)[NOFF], int64_t (&xo)[NOFF]) {
     const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
     const int tok0 = cu.t * kTile;
+    // the 4 rows of a load never cross a block (block_size is a multiple of 16): block and row
+    // advance without a division, and the table is read only where the block changes
+    int col = tok0 / a.bs, row = tok0 - col * a.bs;
+    int64_t slab = 0;
 #pragma unroll
     for (int i = 0; i < NOFF; ++i) {
-      const int tk = tok0 + 4 * i;
-      const int col = tk / a.bs;
-      int phys = (col < a.w) ? __builtin_amdgcn_readfirstlane(pt_row[col]) : 0;
-      if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
-      const int64_t slab = ((int64_t)phys * a.hkv + cu.h) * slab_bytes;
-      const int row = tk - col * a.bs;
+      if (i == 0 || row == 0) {
+        int phys = (col < a.w) ? __builtin_amdgcn_readfirstlane(pt_row[col]) : 0;
+        if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+        slab = ((int64_t)phys * a.hkv + cu.h) * slab_bytes;
+      }
       eo[i] = slab + (int64_t)row * D;
       xo[i] = slab + (int64_t)a.bs * D + (int64_t)row * GPR;
+      row += 4;
+      if (row >= a.bs) row = 0, ++col;
     }
   };
   auto load_tile = [&](const uint8_t *base, const int64_t (&eo)[NOFF], const int64_t (&xo)[NOFF],

@@ -1,0 +1,13 @@
+// 16x16x32 matrix-core decode kernel, head size 128.
+#include "decode_mfma16_kernel.h"
+
+namespace ttpa {
+namespace decode {
+
+bool launch_mfma16_d128(const DecodeArgs &a, hipStream_t st) {
+  return a.kv_format == TTPA_KV_BFP8 ? launch_for_block_size<128, true>(a, st)
+                                     : launch_for_block_size<128, false>(a, st);
+}
+
+}  // namespace decode
+}  // namespace ttpa
