@@ -173,8 +173,8 @@ int ttpa_paged_sdpa_decode_windowed(void *out, int64_t out_user_stride, int64_t 
  * caches and in `out`, are those of the two calls in that order.  k_new / v_new are the
  * [1, users, >= kv_heads, head_size] bfloat16 operands of the update, addressed through
  * new_user_stride / new_head_stride.  Where the 16x16x32 decode kernel serves the shape
- * (head_size 128 with 2 ... 16 query heads per KV head or a block-float-8 cache; head_size 256
- * with up to 16 query heads per KV head; at most 1024 users) the update runs
+ * (head_size 64 / 128 with 2 ... 16 query heads per KV head or a block-float-8 cache; head_size
+ * 256 with up to 16 query heads per KV head; at most 1024 users) the update runs
  * inside it: the wavefront that owns the tile of position cur_pos[u] takes the token from
  * k_new / v_new and stores it into the cache; otherwise the library issues the two launches.
  * The equivalence assumes that no user attends a cache row which ANOTHER user's token is

@@ -415,9 +415,10 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   // faster (the larger figure on launches of a few tiles), at 4 the 16x16x32 kernel is 2 - 8 %
   // faster, at 8 the VALU kernel is 2.5 times slower.  With head size 256 the VALU kernel streams
   // at 3.8 TB/s with one head per group and at 1.2 TB/s with eight, the 16x16x32 kernel at 5.3 -
-  // 5.6 TB/s with any.  So: 16x16x32 kernel for head size 128 and 4 ... 16 heads per group and
-  // for head size 256 (up to 16 heads), 32x32x16 kernel for the other wide groups (head size 64,
-  // up to 32 heads), VALU kernel for the rest.  The block-float-8 cache goes to a matrix-core kernel
+  // 5.6 TB/s with any.  Head size 64 behaves like 128 (block size 32, 4 heads: 47.6 us on the
+  // 16x16x32 kernel, 50.0 us on the VALU kernel; block size 64: 47.5 and 46.7).  So: 16x16x32
+  // kernel for head sizes 64 / 128 and 4 ... 16 heads per group and for head size 256 (up to 16
+  // heads), 32x32x16 kernel for wider groups (up to 32 heads), VALU kernel for the rest.  The block-float-8 cache goes to a matrix-core kernel
   // whenever one applies: there the byte expansion costs one VALU operation per element and the
   // products none, while the VALU kernel pays for both.
   // TTPA_DECODE_KERNEL=valu|mfma|mfma16 overrides the choice.
