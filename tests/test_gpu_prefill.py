@@ -114,6 +114,10 @@ def test_chunked_reference_cases(hq, hkv, start):
     (2, 64, 8, 128, 64, 6, 192, 192),
     (1, 16, 8, 256, 64, 4, 64, 96),
     (2, 12, 4, 128, 16, 12, 96, 96),
+    (2, 8, 2, 64, 4, 40, 32, 100),        # block smaller than the rows of one load: per-lane lookups
+    (1, 4, 4, 128, 2, 100, 64, 70),
+    (2, 16, 8, 256, 8, 30, 32, 150),      # head size 256, block of 8: one lookup per load
+    (2, 8, 8, 64, 8, 40, 96, 130),        # head size 64, block of exactly one load
 ])
 def test_chunked_shapes(users, hq, hkv, d, bs, nbpu, start, lc):
     name = f"chunked u{users} h{hq}x{hkv} d{d} bs{bs} w{nbpu} start{start} lc{lc}"

@@ -53,9 +53,16 @@ struct PrefillArgs {
   const uint16_t *mask;
   int64_t mask_bs, mask_rs;
   int batch, hq, hkv, sq, skv, bs, w, nb, causal;
+  uint32_t bs_magic;  // floor(2^32 / bs) + 1: key / bs = mulhi(key, bs_magic) while key * bs < 2^32 (bs >= 2)
   int window;  // > 0 (causal only): row i attends keys offset + i - window < j <= offset + i
   float scale_log2e;
 };
+
+// key / block_size without a division instruction sequence (about 30 instructions each, and the
+// paged tile loads need several per tile).
+__device__ __forceinline__ int div_block(const PrefillArgs &a, int key) {
+  return a.bs == 1 ? key : (int)__umulhi((uint32_t)key, a.bs_magic);
+}
 
 // LDS geometry of one stage: the K tile (64 rows of D elements) followed by the V tile.
 // Chunk c (16 bytes) of row r is stored at chunk position c ^ swz(r).
@@ -85,7 +92,9 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
 }
 
 // MODE 0: dense K/V; 1: paged, block_size a multiple of 64 (a tile lies in one block);
-// 2: paged, any block size (per-row table lookups).
+// 3: paged, block_size a multiple of the rows one wavefront load covers (1 KiB: 8 / 4 / 2 rows
+// for head sizes 64 / 128 / 256): one wavefront-uniform table lookup per load; 2: paged, any
+// block size (per-lane table lookups).
 //
 // Per-tile schedule of a workgroup (LDS holds two K stages and two V stages):
 //   S^T = K(t) Q^T | barrier | issue loads of K(t+2) and V(t+1) | softmax | O^T += V(t)^T P^T
@@ -171,7 +180,22 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
   }
   // Issues the loads of one tile of one tensor.  Keys past the end of K/V are clamped to the
   // last row, whose scores are masked and whose V rows therefore carry weight 0.
-  auto issue = [&](const uint16_t *src, const uint32_t (&ld)[T::NI], bool is_v, int kt, int buf) {
+  // Modes 1 and 3 look their blocks up one tile ahead of the loads (below): NLK wavefront-
+  // uniform table entries per tile, one for the whole tile or one per load of this wavefront.
+  constexpr int NLK = MODE == 1 ? 1 : (MODE == 3 ? T::NI : 0);
+  struct Blocks {
+    int phys[NLK > 0 ? NLK : 1];
+  };
+  // first key of lookup j of tile kt
+  auto lookup_key = [&](int kt, int j) {
+    const int key0 = kt * kKeysPerTile;
+    if constexpr (MODE == 1) return key0;
+    // the rows of a load sit in one block; a load wholly past the last key reads the rows that
+    // hold the last key again (readable, and masked like any key past the end)
+    return key0 + min((4 * j + wave) * T::RPI, (a.skv - 1 - key0) / T::RPI * T::RPI);
+  };
+  auto issue = [&](const uint16_t *src, const uint32_t (&ld)[T::NI], bool is_v, int kt, int buf,
+                   const Blocks &blk) {
     const int key0 = kt * kKeysPerTile;
     const int last = a.skv - 1 - key0;  // last valid key of this tile, relative (>= 0)
     const uint32_t lds_base = lds_address(smem) + (uint32_t)(buf * T::STAGE_BYTES + (is_v ? T::TILE_BYTES : 0));
@@ -179,20 +203,27 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
     if constexpr (MODE == 0) {
       base = reinterpret_cast<const char *>(src + b * a.kv_bs + hk * a.kv_hs + (int64_t)key0 * a.kv_ts);
     } else if constexpr (MODE == 1) {
-      int phys = __builtin_amdgcn_readfirstlane(a.pt[(int64_t)b * a.pt_rs + key0 / a.bs]);
-      if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
-      base = reinterpret_cast<const char *>(src + (((int64_t)phys * a.hkv + hk) * a.bs + (key0 % a.bs)) * D);
+      base = reinterpret_cast<const char *>(
+          src + (((int64_t)blk.phys[0] * a.hkv + hk) * a.bs + (key0 - div_block(a, key0) * a.bs)) * D);
     }
     auto lds_dst = [&](int j) { return lds_base + (uint32_t)(4 * j + wave) * 1024u; };
     if constexpr (MODE == 2) {
 #pragma unroll
       for (int j = 0; j < T::NI; ++j) {
         const int key = key0 + min(ld_row[j], last);
-        const int col = key / a.bs;
+        const int col = div_block(a, key);
         int phys = a.pt[(int64_t)b * a.pt_rs + col];
         if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
         const int c = (lane % T::CPR) ^ (is_v ? T::swz_v(ld_row[j]) : T::swz_k(ld_row[j]));
         dma16_lane(src + (((int64_t)phys * a.hkv + hk) * a.bs + (key - col * a.bs)) * D + c * 8, lds_dst(j));
+      }
+    } else if constexpr (MODE == 3) {
+#pragma unroll
+      for (int j = 0; j < T::NI; ++j) {
+        const int key = lookup_key(kt, j);
+        const char *seg = reinterpret_cast<const char *>(
+            src + (((int64_t)blk.phys[j] * a.hkv + hk) * a.bs + (key - div_block(a, key) * a.bs)) * D);
+        dma16(seg, ld[j] - (uint32_t)((4 * j + wave) * T::RPI * T::RB), lds_dst(j));
       }
     } else if (MODE == 0 && last < kKeysPerTile - 1) {  // uniform: dense K/V ending inside the tile
 #pragma unroll
@@ -257,9 +288,41 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
 
   // ntiles >= 1 always (row 0 sees key 0).
   const int last_tile = ntiles - 1;
-  issue(a.k, ld_k, false, first_tile, first_tile & 1);
-  issue(a.v, ld_v, true, first_tile, first_tile & 1);
-  if (last_tile >= first_tile + 1) issue(a.k, ld_k, false, first_tile + 1, (first_tile + 1) & 1);
+  // Block-table entries are vector loads (the load-to-LDS instruction is opaque to the
+  // compiler, so it cannot prove the table unchanged and scalar), and waiting for one means
+  // waiting for every tile load in flight.  So the entries of tile t + 3 are requested right
+  // behind the loads issued in iteration t and read after the barrier of iteration t + 1, where
+  // everything in flight has landed anyway; K(t + 2) and, one iteration later, V(t + 2) use them.
+  struct Requested {
+    int raw[NLK > 0 ? NLK : 1];
+  };
+  auto request = [&](int kt) {
+    Requested r = {};
+    if constexpr (NLK > 0) {
+      const int t = min(kt, last_tile);  // past the end: any valid entry, never used
+#pragma unroll
+      for (int j = 0; j < NLK; ++j) r.raw[j] = a.pt[(int64_t)b * a.pt_rs + div_block(a, lookup_key(t, j))];
+    }
+    return r;
+  };
+  auto resolve = [&](const Requested &r) {
+    Blocks blk = {};
+    if constexpr (NLK > 0) {
+#pragma unroll
+      for (int j = 0; j < NLK; ++j) {
+        const int p = __builtin_amdgcn_readfirstlane(r.raw[j]);
+        blk.phys[j] = (unsigned)p >= (unsigned)a.nb ? 0 : p;
+      }
+    }
+    return blk;
+  };
+  Blocks blk_v = resolve(request(first_tile));     // blocks of the tile whose V is loaded next
+  Blocks blk_k = resolve(request(first_tile + 1));  // ... whose K is loaded next
+  Requested req = request(first_tile + 2);
+  issue(a.k, ld_k, false, first_tile, first_tile & 1, blk_v);
+  issue(a.v, ld_v, true, first_tile, first_tile & 1, blk_v);
+  if (last_tile >= first_tile + 1) issue(a.k, ld_k, false, first_tile + 1, (first_tile + 1) & 1, blk_k);
+  blk_v = blk_k;
   wait_loads_and_sync();
   // The first K fragments of a tile are read one tile ahead (K(t+1) has landed at the barrier
   // of tile t), so the score product starts without waiting for LDS.
@@ -293,8 +356,11 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
     }
     // K(kt+1) and V(kt) have landed for everyone; everyone is done with K(kt) and V(kt-1)
     wait_loads_and_sync();
-    if (kt + 2 <= last_tile) issue(a.k, ld_k, false, kt + 2, kt & 1);
-    if (kt + 1 <= last_tile) issue(a.v, ld_v, true, kt + 1, (kt + 1) & 1);
+    blk_k = resolve(req);  // blocks of tile kt + 2; blk_v holds those of tile kt + 1
+    if (kt + 2 <= last_tile) issue(a.k, ld_k, false, kt + 2, kt & 1, blk_k);
+    if (kt + 1 <= last_tile) issue(a.v, ld_v, true, kt + 1, (kt + 1) & 1, blk_v);
+    blk_v = blk_k;
+    req = request(kt + 3);
 
     if (compute) {
       bf16x8 vring[VPRE];
@@ -436,6 +502,7 @@ template <int D, int HPW>
 int launch(const PrefillArgs &a, hipStream_t st) {
   if (!a.pt) return launch_mode<D, HPW, 0>(a, st);
   if (a.bs % kKeysPerTile == 0) return launch_mode<D, HPW, 1>(a, st);
+  if (a.bs % Tile<D>::RPI == 0) return launch_mode<D, HPW, 3>(a, st);
   return launch_mode<D, HPW, 2>(a, st);
 }
 
@@ -477,6 +544,7 @@ static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_st
     TTPA_REQUIRE(block_size > 0 && table_width > 0 && num_blocks > 0,
                  "paged form needs block_size, table_width and num_blocks");
     kv_len = table_width * block_size;
+    TTPA_REQUIRE((int64_t)kv_len * block_size < (1ll << 32), "prefill: table_width * block_size^2 must stay below 2^32");
   } else {
     TTPA_REQUIRE(kv_len > 0, "dense form needs kv_len > 0");
     TTPA_REQUIRE(kv_batch_stride % 8 == 0 && kv_head_stride % 8 == 0 && kv_token_stride % 8 == 0,
@@ -507,6 +575,7 @@ static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_st
   a.bs = block_size, a.w = table_width, a.nb = num_blocks, a.causal = causal ? 1 : 0;
   a.window = sliding_window;
   a.scale_log2e = scale * 1.4426950408889634f;
+  a.bs_magic = block_size >= 2 ? (uint32_t)((1ull << 32) / (uint32_t)block_size) + 1u : 0u;
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (head_size) {
     case 64: return launch_d<64>(a, st);
