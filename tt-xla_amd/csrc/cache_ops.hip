@@ -105,35 +105,45 @@ struct FillArgs {
   const void *bidx;
   int bidx_i64;
   int fill_users, table_rows, hkv, s, bs, d, w, nb;
+  // floor(2^32 / divisor) + 1 for the two per-thread divisions (by the threads of a token row
+  // and by the block size), or 0 where the multiply-high quotient would not be exact
+  uint32_t tpr_magic, bs_magic;
 };
 
-__device__ __forceinline__ bool resolve_fill(const FillArgs &a, int i, int t, int &phys) {
+// x / d; a thread moves 16 bytes, so a division sequence (about 30 instructions) per quotient
+// would make these kernels instruction-bound.
+__device__ __forceinline__ int fast_div(int x, int d, uint32_t magic) {
+  return magic ? (int)__umulhi((uint32_t)x, magic) : x / d;
+}
+inline uint32_t magic_for(int64_t max_dividend, int d) {
+  return (d >= 2 && max_dividend * d < (1ll << 32)) ? (uint32_t)((1ull << 32) / (uint32_t)d) + 1u : 0u;
+}
+
+// Block of token t of fill row i, and the token's row inside it.
+__device__ __forceinline__ bool resolve_fill(const FillArgs &a, int i, int t, int &phys, int &off) {
   int64_t b = a.bidx ? load_index(a.bidx, a.bidx_i64, i) : 0;
   if (b < 0 || b >= a.table_rows) return false;
-  phys = a.pt[b * a.pt_rs + t / a.bs];
+  const int col = fast_div(t, a.bs, a.bs_magic);
+  off = t - col * a.bs;
+  phys = a.pt[b * a.pt_rs + col];
   return (unsigned)phys < (unsigned)a.nb;
 }
 
-// Thread order: chunk fastest, then token, then head, then user, so one (user, head,
-// block) destination slab of bs * D elements is written front to back by neighbouring
-// wavefronts while the source is read in whole 2*D-byte rows.
+// Grid: x over the (token, chunk) pairs of one (user, head), chunk fastest; y = KV head;
+// z = fill row.  One (user, head, block) destination slab of bs * D elements is written front
+// to back by neighbouring wavefronts while the source is read in whole 2*D-byte rows.
 template <int VEC>
 __global__ __launch_bounds__(256) void fill_bf16_kernel(FillArgs a) {
   const int cpr = a.d / VEC;
-  int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  int64_t total = (int64_t)a.fill_users * a.hkv * a.s * cpr;
-  if (gid >= total) return;
-  int chunk = (int)(gid % cpr);
-  int64_t r = gid / cpr;
-  int t = (int)(r % a.s);
-  r /= a.s;
-  int h = (int)(r % a.hkv);
-  int i = (int)(r / a.hkv);
-  int phys;
-  if (!resolve_fill(a, i, t, phys)) return;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= a.s * cpr) return;
+  const int t = fast_div(idx, cpr, a.tpr_magic), chunk = idx - t * cpr;
+  const int h = blockIdx.y, i = blockIdx.z;
+  int phys, off;
+  if (!resolve_fill(a, i, t, phys, off)) return;
   const uint16_t *src = a.fill + i * a.fill_us + h * a.fill_hs + t * a.fill_ts + chunk * VEC;
   uint16_t *dst = static_cast<uint16_t *>(a.cache) +
-                  (((int64_t)phys * a.hkv + h) * a.bs + (t % a.bs)) * a.d + chunk * VEC;
+                  (((int64_t)phys * a.hkv + h) * a.bs + off) * a.d + chunk * VEC;
   if constexpr (VEC == 8) {
     *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(src);
   } else {
@@ -143,24 +153,18 @@ __global__ __launch_bounds__(256) void fill_bf16_kernel(FillArgs a) {
 
 __global__ __launch_bounds__(256) void fill_bfp8_kernel(FillArgs a) {
   const int gpr = a.d / 16;
-  int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  int64_t total = (int64_t)a.fill_users * a.hkv * a.s * gpr;
-  if (gid >= total) return;
-  int grp = (int)(gid % gpr);
-  int64_t r = gid / gpr;
-  int t = (int)(r % a.s);
-  r /= a.s;
-  int h = (int)(r % a.hkv);
-  int i = (int)(r / a.hkv);
-  int phys;
-  if (!resolve_fill(a, i, t, phys)) return;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= a.s * gpr) return;
+  const int t = fast_div(idx, gpr, a.tpr_magic), grp = idx - t * gpr;
+  const int h = blockIdx.y, i = blockIdx.z;
+  int phys, off;
+  if (!resolve_fill(a, i, t, phys, off)) return;
   const uint4 *src = reinterpret_cast<const uint4 *>(a.fill + i * a.fill_us + h * a.fill_hs +
                                                      t * a.fill_ts + grp * 16);
   uint4 lo = src[0], hi = src[1];
   uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   uint32_t bytes[4];
   uint32_t e = bfp8_encode16(w, bytes);
-  int off = t % a.bs;
   uint8_t *slab = static_cast<uint8_t *>(a.cache) +
                   ((int64_t)phys * a.hkv + h) * (int64_t)(a.bs + a.bs / 16) * a.d;
   *reinterpret_cast<uint4 *>(slab + (int64_t)off * a.d + grp * 16) =
@@ -274,27 +278,30 @@ extern "C" int ttpa_paged_fill_cache(void *cache, const void *fill, int64_t fill
              page_table, page_table_row_stride,
              batch_idx,  batch_idx_is_i64,
              fill_users, table_rows, kv_heads, seq_len, block_size, head_size, table_width,
-             num_blocks};
+             num_blocks, 0u, 0u};
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool vec_ok = head_size % 8 == 0 && aligned16(cache) && aligned16(fill) &&
                       fill_user_stride % 8 == 0 && fill_head_stride % 8 == 0 &&
                       fill_token_stride % 8 == 0;
-  const int64_t rows = (int64_t)fill_users * kv_heads * seq_len;
-  int64_t threads;
+  int tpr;  // threads per token row
   if (kv_format == TTPA_KV_BFP8) {
     TTPA_REQUIRE(vec_ok, "block-float-8 fill needs 16-byte aligned fill rows");
-    threads = rows * (head_size / 16);
+    tpr = head_size / 16;
   } else {
-    threads = vec_ok ? rows * (head_size / 8) : rows * head_size;
+    tpr = vec_ok ? head_size / 8 : head_size;
   }
-  int64_t blocks = (threads + 255) / 256;
-  TTPA_REQUIRE(blocks < (int64_t)1 << 31, "fill too large for one launch");
+  const int64_t threads = (int64_t)seq_len * tpr;  // per (fill row, head)
+  TTPA_REQUIRE(threads < (int64_t)1 << 31 && fill_users <= 65535 && kv_heads <= 65535,
+               "fill too large for one launch");
+  a.tpr_magic = magic_for(threads, tpr);
+  a.bs_magic = magic_for(seq_len, block_size);
+  const dim3 grid((unsigned)((threads + 255) / 256), (unsigned)kv_heads, (unsigned)fill_users);
   if (kv_format == TTPA_KV_BFP8) {
-    fill_bfp8_kernel<<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a);
+    fill_bfp8_kernel<<<grid, dim3(256), 0, st>>>(a);
   } else if (vec_ok) {
-    fill_bf16_kernel<8><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a);
+    fill_bf16_kernel<8><<<grid, dim3(256), 0, st>>>(a);
   } else {
-    fill_bf16_kernel<1><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a);
+    fill_bf16_kernel<1><<<grid, dim3(256), 0, st>>>(a);
   }
   return check_launch("paged_fill_cache");
 }

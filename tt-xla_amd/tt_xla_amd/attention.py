@@ -262,14 +262,28 @@ class TTAttentionBackendImpl(_ImplBase):
         if writes_cache and not fused_step:
             self._handle_paged_attention(inputs, kv_cache, attn_metadata)
 
+        # The reference copies the operator's result into vLLM's output buffer (:330-336).  Where
+        # the buffer can be viewed as [users, tokens, heads, head_size] the operators write into
+        # it directly (their out-variants take any strides) and return None.
+        direct = None if self.functional_cache_ops else self._output_view(output, inputs)
         if inputs.is_prefill:
             assert self.sinks is None, "Attention sink is unsupported in SDPA prefill"
-            attn_output = self._compute_full_attention(inputs, kv_cache, attn_metadata)
+            attn_output = self._compute_full_attention(inputs, kv_cache, attn_metadata, direct)
         else:
-            attn_output = self._compute_decode_attention(inputs, kv_cache, attn_metadata, fused_step)
-
+            attn_output = self._compute_decode_attention(inputs, kv_cache, attn_metadata, fused_step, direct)
+        if attn_output is None:
+            return
         flat = attn_output.reshape(-1, self.num_heads * self.head_size)
         output.copy_(flat.reshape_as(output))
+
+    def _output_view(self, output: torch.Tensor, inputs) -> Optional[torch.Tensor]:
+        """``output`` as [users, tokens, heads, head_size] without a copy, or None."""
+        if output.dtype != torch.bfloat16 or not output.is_contiguous() or output.data_ptr() % 16:
+            return None
+        shape = (inputs.users, inputs.query_num_tokens, self.num_heads, self.head_size)
+        if output.numel() != shape[0] * shape[1] * shape[2] * shape[3] or self.head_size % 8:
+            return None
+        return output.view(shape)
 
     # ------------------------------------------------------------------ reshapes
     def _normalize_to_attention_format(
@@ -357,7 +371,8 @@ class TTAttentionBackendImpl(_ImplBase):
             ops.paged_fill_cache_(kv_cache[1], v_new, table, batch_idx=batch_idx)
 
     # ------------------------------------------------------------------ attention
-    def _compute_full_attention(self, inputs, kv_cache, attn_metadata: TTMetadata) -> torch.Tensor:
+    def _compute_full_attention(self, inputs, kv_cache, attn_metadata: TTMetadata,
+                                direct: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         has_paged_cache = (
             isinstance(kv_cache, (list, tuple)) and len(kv_cache) >= 2 and kv_cache[0].numel() > 0
         )
@@ -365,6 +380,12 @@ class TTAttentionBackendImpl(_ImplBase):
         q = inputs.query.transpose(-3, -2)  # [users, Hq, tokens, D]
         if attn_metadata.chunk_start_idx is not None and has_paged_cache and not shared_kv:
             # continuation chunk: keys come from the cache, prefix included
+            if direct is not None:
+                torch.ops.tt.chunked_scaled_dot_product_attention_out(
+                    q, kv_cache[0], kv_cache[1], attn_metadata.page_table,
+                    attn_metadata.chunk_start_idx, direct.transpose(-3, -2), scale=self.scale,
+                )
+                return None
             out = torch.ops.tt.chunked_scaled_dot_product_attention(
                 q, kv_cache[0], kv_cache[1], attn_metadata.page_table,
                 attn_metadata.chunk_start_idx, scale=self.scale,
@@ -383,6 +404,9 @@ class TTAttentionBackendImpl(_ImplBase):
         }
         if self.sliding_window is not None:
             kwargs["sliding_window_size"] = self.sliding_window
+        if direct is not None:
+            torch.ops.tt.scaled_dot_product_attention_out(q, k, v, direct.transpose(-3, -2), **kwargs)
+            return None
         out = torch.ops.tt.scaled_dot_product_attention(q, k, v, **kwargs)
         return out.transpose(-3, -2)  # [users, tokens, Hq, D]
 
@@ -395,9 +419,17 @@ class TTAttentionBackendImpl(_ImplBase):
         return g.reshape(users, hkv, -1, d)[:, :, :num_tokens, :]
 
     def _compute_decode_attention(self, inputs, kv_cache, attn_metadata: TTMetadata,
-                                  fused_step: bool = False) -> torch.Tensor:
+                                  fused_step: bool = False,
+                                  direct: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         q = inputs.query.transpose(0, 1)  # [1, users, Hq, D]
         if fused_step:  # cache update (reference :473-483) and attention (:634-668) in one operator
+            if direct is not None:
+                torch.ops.tt.paged_update_kv_decode_out_(
+                    q, kv_cache[0], kv_cache[1], inputs.key.transpose(0, 1), inputs.value.transpose(0, 1),
+                    attn_metadata.page_table, attn_metadata.cache_position, direct.transpose(0, 1),
+                    attention_sink=self.sinks, scale=self.scale, sliding_window_size=self.sliding_window,
+                )
+                return None
             out = torch.ops.tt.paged_update_kv_decode_(
                 q, kv_cache[0], kv_cache[1], inputs.key.transpose(0, 1), inputs.value.transpose(0, 1),
                 attn_metadata.page_table, attn_metadata.cache_position, attention_sink=self.sinks,

@@ -293,10 +293,21 @@ def paged_scaled_dot_product_attention_decode(
                    scale, sliding_window_size, None, None)
 
 
+def _check_out(out, shape, name):
+    """An output tensor handed in by the caller: bfloat16, the given shape, rows contiguous and
+    16-byte aligned, strides in whole 8-byte units (what the kernels' vector stores need)."""
+    if out.dtype != torch.bfloat16 or tuple(out.shape) != tuple(shape):
+        raise ValueError(f"{name}: out must be bfloat16 of shape {tuple(shape)}, got {out.dtype} {tuple(out.shape)}")
+    if out.stride(-1) != 1 or out.data_ptr() % 16 or any(st % 4 for st in out.stride()[:-1]):
+        raise ValueError(f"{name}: out needs contiguous 16-byte aligned rows and strides that are multiples of 4")
+    return out
+
+
 def _decode(query, key, value, page_table, is_causal, attn_mask, cur_pos_tensor, attention_sink, scale,
-            sliding_window_size, k_new, v_new):
+            sliding_window_size, k_new, v_new, out=None):
     """Checks and launch shared by the decode operator and the fused update + decode operator
-    (k_new / v_new given: the step's cache update happens in the same call)."""
+    (k_new / v_new given: the step's cache update happens in the same call).  ``out``
+    [1, users, heads, head_size]: written in place of a fresh tensor."""
     if is_causal:
         assert attn_mask is None, "attention_mask must be None when is_causal is True."
         assert cur_pos_tensor is not None, "cur_pos_tensor must be provided when is_causal is True."
@@ -326,7 +337,10 @@ def _decode(query, key, value, page_table, is_causal, attn_mask, cur_pos_tensor,
     q = _rows_contiguous(query)
     pt = _table(page_table)
     cur = _index_tensor(cur_pos_tensor)
-    out = torch.empty((1, users, hq, d), dtype=query.dtype, device=query.device)
+    if out is None:
+        out = torch.empty((1, users, hq, d), dtype=query.dtype, device=query.device)
+    else:
+        _check_out(out, (1, users, hq, d), "decode")
     ws_bytes = N.lib().ttpa_paged_decode_workspace_bytes(users, hq, hkv, d)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=query.device)
     sink = None
@@ -395,6 +409,29 @@ def _(query, k_cache, v_cache, k_new, v_new, page_table, cur_pos_tensor, attenti
     return torch.empty_like(query)
 
 
+@torch.library.custom_op("tt::paged_update_kv_decode_out_", mutates_args=["k_cache", "v_cache", "out"],
+                         device_types=["cuda"])
+def paged_update_kv_decode_out_(
+    query: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    k_new: torch.Tensor,
+    v_new: torch.Tensor,
+    page_table: torch.Tensor,
+    cur_pos_tensor: torch.Tensor,
+    out: torch.Tensor,
+    attention_sink: Optional[torch.Tensor] = None,
+    scale: Optional[float] = None,
+    sliding_window_size: Optional[int] = None,
+) -> None:
+    """``paged_update_kv_decode_`` writing into ``out`` [1, users, heads, head_size] (any user /
+    head strides): the attention backend hands its output buffer in, which saves the copy the
+    reference makes from the operator's result (attention.py:330-336)."""
+    _decode(query, k_cache, v_cache, page_table, True, None, cur_pos_tensor, attention_sink,
+            scale, sliding_window_size, k_new, v_new, out=out)
+
+
+
 
 
 @paged_scaled_dot_product_attention_decode.register_fake
@@ -406,12 +443,15 @@ def _(query, key, value, page_table, is_causal=False, attn_mask=None, cur_pos_te
 # --------------------------------------------------------------------------- #
 # prefill attention
 # --------------------------------------------------------------------------- #
-def _prefill(query, key, value, page_table, chunk_start, attn_mask, is_causal, scale, window=0):
+def _prefill(query, key, value, page_table, chunk_start, attn_mask, is_causal, scale, window=0, out=None):
     b, hq, s, d = query.shape
     if query.dtype != torch.bfloat16:
         raise ValueError("query must be bfloat16")
     q = _rows_contiguous(query)
-    out = torch.empty_like(q)  # keeps q's (possibly token-major) strides
+    if out is None:
+        out = torch.empty_like(q)  # keeps q's (possibly token-major) strides
+    else:
+        _check_out(out, (b, hq, s, d), "prefill")
     if scale is None:
         scale = 1.0 / math.sqrt(d)
     if page_table is None:
@@ -493,6 +533,33 @@ def _(query, key, value, attn_mask=None, is_causal=True, scale=None, sliding_win
     return torch.empty_like(query)
 
 
+@torch.library.custom_op("tt::scaled_dot_product_attention_out", mutates_args=["out"], device_types=["cuda"])
+def scaled_dot_product_attention_out(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    out: torch.Tensor,
+    attn_mask: Optional[torch.Tensor] = None,
+    is_causal: bool = True,
+    scale: Optional[float] = None,
+    sliding_window_size: Optional[int] = None,
+) -> None:
+    """``scaled_dot_product_attention`` writing into ``out`` [B, heads, q_len, head_size] (any
+    batch / head / token strides): the attention backend hands its output buffer in, which saves
+    the copy the reference makes from the operator's result (attention.py:330-336)."""
+    assert query.dim() == 4 and key.dim() == 4 and key.shape == value.shape
+    assert query.shape[2] % 32 == 0, f"query sequence length must be divisible by 32 but got {query.shape[2]}."
+    if attn_mask is not None:
+        assert is_causal == False, "is_causal attribute can't be True if attn_mask is available."  # noqa: E712
+    if sliding_window_size is not None:
+        if sliding_window_size <= 0:
+            raise ValueError("sliding_window_size must be positive")
+        if not is_causal:
+            raise NotImplementedError("sliding_window_size is built for the causal form only")
+    _prefill(query, key, value, None, None, attn_mask, is_causal, scale,
+             window=sliding_window_size or 0, out=out)
+
+
 @torch.library.custom_op(
     "tt::chunked_scaled_dot_product_attention", mutates_args=[], device_types=["cuda"]
 )
@@ -517,6 +584,30 @@ def chunked_scaled_dot_product_attention(
 @chunked_scaled_dot_product_attention.register_fake
 def _(query, key, value, page_table, chunk_start_idx_tensor, scale=None):
     return torch.empty_like(query)
+
+
+@torch.library.custom_op(
+    "tt::chunked_scaled_dot_product_attention_out", mutates_args=["out"], device_types=["cuda"]
+)
+def chunked_scaled_dot_product_attention_out(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    page_table: torch.Tensor,
+    chunk_start_idx_tensor: torch.Tensor,
+    out: torch.Tensor,
+    scale: Optional[float] = None,
+) -> None:
+    """``chunked_scaled_dot_product_attention`` writing into ``out`` (see
+    ``scaled_dot_product_attention_out``)."""
+    if query.dim() != 4:
+        raise ValueError("query must be [users, heads, chunk_len, head_size]")
+    if page_table.dim() != 2 or page_table.shape[0] != query.shape[0]:
+        raise ValueError("page_table must have one row per user")
+    start = chunk_start_idx_tensor.reshape(-1)
+    if start.dtype != torch.int32:
+        start = start.to(torch.int32)
+    _prefill(query, key, value, page_table, start, None, True, scale, out=out)
 
 
 # --------------------------------------------------------------------------- #
