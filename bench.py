@@ -111,7 +111,8 @@ def make_prefill_impl(w):
 
 def prefill_step(impl, w, out):
     """The backend's prefill pass: K fill + V fill + causal attention (dense on the fresh K/V
-    for a first chunk, paged with the cached prefix for a continuation chunk)."""
+    for a first chunk, where the backend issues all three as one operator; paged with the
+    cached prefix for a continuation chunk)."""
     from tt_xla_amd import TTMetadata
 
     md = TTMetadata(cache_position=None, page_table=w.page_table, num_users=w.users,
@@ -437,7 +438,8 @@ def run_prefill(args):
         "dtype": "bf16", "data": "synthetic",
         "config": {
             "workload": w.name,
-            "step": "K fill + V fill through the fill page table + causal attention on the fresh K/V",
+            "step": "K fill + V fill through the fill page table + causal attention on the fresh K/V "
+                    "(one operator, one launch: extra workgroups of the attention kernel copy the rows)",
             "launch": args.launch, "steps_per_graph": runner.per_graph if args.launch == "graph" else None,
             "rotating_copies": len(copies), "users": w.users,
             "tokens_per_user": w.seq, "q_heads": w.q_heads, "kv_heads": w.kv_heads,
@@ -451,7 +453,8 @@ def run_prefill(args):
             "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
             "kernel_us": kern_ms * 1e3, "kernel_us_min": min(d for d, _ in durs) * 1e3,
             "flops_per_launch": flops, "timed_launches": len(durs),
-            "note": "useful (causal) FLOPs only; the dense 4*B*Hq*S^2*D figure is twice this",
+            "note": "useful (causal) FLOPs only; the dense 4*B*Hq*S^2*D figure is twice this; the launch "
+                    "also carries the step's K / V cache fill (fill_bytes_per_step of traffic)",
         },
     }
 

@@ -279,6 +279,30 @@ int ttpa_sdpa_prefill_windowed(void *out, int64_t out_batch_stride, int64_t out_
                                int32_t sliding_window, void *stream);
 
 /*
+ * The backend's first-chunk prefill pass in one call: ttpa_paged_fill_cache on K and on V
+ * (attention.py:486-515: the prompt's keys and values go into the paged caches through the
+ * fill page table) and the dense-form ttpa_sdpa_prefill_windowed on the same k / v
+ * (attention.py:576-596).  Results, in the caches and in `out`, are those of the three calls;
+ * the attention reads the dense k / v and never the caches, so their order does not matter.
+ * k / v [batch, kv_heads, kv_len, head_size] by strides are both the attention's operands and
+ * the fill operands (batch entry i fills table row batch_idx[i]; batch_idx may be NULL for
+ * batch == 1; rows and blocks out of range are skipped, as in the fill).  bfloat16 caches
+ * only.  Inside the library this is ONE launch: extra workgroups behind the attention's copy
+ * the rows while the matrix pipes are busy.  No counterpart as one operator in the reference.
+ */
+int ttpa_sdpa_prefill_fill(void *out, int64_t out_batch_stride, int64_t out_head_stride,
+                           int64_t out_token_stride, const void *q, int64_t q_batch_stride,
+                           int64_t q_head_stride, int64_t q_token_stride, const void *k,
+                           const void *v, int64_t kv_batch_stride, int64_t kv_head_stride,
+                           int64_t kv_token_stride, int32_t batch, int32_t q_heads,
+                           int32_t kv_heads, int32_t q_len, int32_t kv_len, int32_t head_size,
+                           int32_t causal, float scale, int32_t sliding_window, void *k_cache,
+                           void *v_cache, const int32_t *fill_page_table,
+                           int64_t fill_page_table_row_stride, const void *batch_idx,
+                           int batch_idx_is_i64, int32_t table_rows, int32_t block_size,
+                           int32_t table_width, int32_t num_blocks, void *stream);
+
+/*
  * Block-float-8 codec on flat arrays (n_elems % 16 == 0), for tests and cache
  * conversion.  No reference counterpart: the reference forwards
  * experimental_kv_cache_dtype="bfp_bf8" to an un-vendored compiler

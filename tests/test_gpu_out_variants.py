@@ -105,3 +105,79 @@ def test_backend_falls_back_to_the_copy_for_a_strided_output_buffer():
     torch.cuda.synchronize()
     assert torch.equal(wide[:, : hq * d], plain)
     assert (wide[:, hq * d:] == 0).all()
+
+
+@pytest.mark.parametrize("b,hq,hkv,s,d,bs,window", [
+    (4, 32, 8, 256, 128, 64, 0),      # Llama-3-8B heads
+    (3, 8, 4, 96, 128, 32, 0),        # two heads per wavefront group, 96 tokens (not a multiple of a tile)
+    (2, 4, 4, 320, 64, 16, 50),       # one head per group, sliding window, more rows than one fill chunk
+    (2, 16, 8, 64, 256, 32, 0),       # head size 256
+    (1, 8, 2, 32, 128, 64, 0),        # single user without batch_idx
+])
+def test_prefill_pass_as_one_operator(b, hq, hkv, s, d, bs, window):
+    """tt::paged_fill_kv_prefill_out_ against fill K + fill V + dense attention: caches and
+    output bit for bit; table rows permuted through batch_idx, one fill row pointed outside the
+    table and one block id outside the cache (both skipped by the fill)."""
+    print(f"prefill pass b{b} h{hq}x{hkv} s{s} d{d} bs{bs} window{window}", flush=True)
+    g = torch.Generator().manual_seed(b * 7 + hq + s + d + bs)
+    q, k, v = _bf(g, b, hq, s, d), _bf(g, b, hkv, s, d), _bf(g, b, hkv, s, d)
+    w = (s + bs - 1) // bs + 1
+    rows = b + 2
+    nb = rows * w + 1
+    table = (torch.randperm(nb - 1, generator=g)[: rows * w] + 1).view(rows, w).to(torch.int32)
+    if b > 1:
+        table[1, 0] = nb + 5             # a block id outside the cache
+    bidx = None
+    if b > 1:
+        bidx = torch.randperm(rows, generator=g)[:b].to(torch.int32)
+        if b > 2:
+            bidx[2] = rows + 3           # a fill row outside the table
+        bidx = bidx.cuda()
+    table = table.cuda()
+    kc = torch.full((nb, hkv, bs, d), 3.0, dtype=torch.bfloat16, device="cuda")
+    vc = torch.full((nb, hkv, bs, d), -3.0, dtype=torch.bfloat16, device="cuda")
+    kw = dict(is_causal=True, sliding_window_size=window if window else None)
+
+    k_ref, v_ref = kc.clone(), vc.clone()
+    torch.ops.tt.paged_fill_cache_(k_ref, k, table, bidx)
+    torch.ops.tt.paged_fill_cache_(v_ref, v, table, bidx)
+    want = torch.ops.tt.scaled_dot_product_attention(q, k, v, **kw)
+
+    buf = torch.zeros(b, s, hq, d, dtype=torch.bfloat16, device="cuda")
+    # token-major operands, as the backend hands them in
+    qt, kt, vt = (x.transpose(1, 2).contiguous().transpose(1, 2) for x in (q, k, v))
+    torch.ops.tt.paged_fill_kv_prefill_out_(qt, kt, vt, kc, vc, table, bidx, buf.transpose(1, 2), **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(kc, k_ref), "K cache differs"
+    assert torch.equal(vc, v_ref), "V cache differs"
+    assert not torch.equal(kc, torch.full_like(kc, 3.0))
+    assert torch.equal(buf.transpose(1, 2), want)
+
+
+def test_backend_prefill_pass_equals_the_reference_sequence():
+    """TTAttentionBackendImpl.forward on a first-chunk prefill: the one-operator pass (default)
+    and the reference's sequence (functional_cache_ops=True) leave the same caches and output."""
+    from tt_xla_amd.attention import TTAttentionBackendImpl, TTMetadata
+
+    users, s, hq, hkv, d, bs = 3, 128, 32, 8, 128, 32
+    g = torch.Generator().manual_seed(11)
+    w = s // bs
+    nb = users * w + 1
+    table = (torch.randperm(nb - 1, generator=g)[: users * w] + 1).view(users, w).to(torch.int32).cuda()
+    q = _bf(g, users * s, hq * d)
+    k, v = _bf(g, users * s, hkv * d), _bf(g, users * s, hkv * d)
+    meta = TTMetadata(cache_position=None, page_table=table, num_users=users,
+                      batch_idx=torch.arange(users, dtype=torch.int32, device="cuda"),
+                      fill_page_table=table, chunk_start_idx=None)
+    results = []
+    for functional in (False, True):
+        impl = TTAttentionBackendImpl(hq, d, d**-0.5, hkv, functional_cache_ops=functional)
+        caches = [torch.zeros(nb, hkv, bs, d, dtype=torch.bfloat16, device="cuda") for _ in range(2)]
+        out = torch.empty(users * s, hq * d, dtype=torch.bfloat16, device="cuda")
+        impl.forward(None, q, k, v, caches, meta, output=out)
+        results.append((out, caches))
+    torch.cuda.synchronize()
+    (o1, c1), (o2, c2) = results
+    assert torch.equal(c1[0], c2[0]) and torch.equal(c1[1], c2[1])
+    assert c1[0].abs().sum() > 0
+    assert torch.equal(o1, o2)

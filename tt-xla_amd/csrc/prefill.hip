@@ -36,6 +36,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kKeysPerTile = 64;
 constexpr int kRowsPerWave = 32;
@@ -54,6 +55,18 @@ struct PrefillArgs {
   int64_t mask_bs, mask_rs;
   int batch, hq, hkv, sq, skv, bs, w, nb, causal;
   uint32_t bs_magic;  // floor(2^32 / bs) + 1: key / bs = mulhi(key, bs_magic) while key * bs < 2^32 (bs >= 2)
+  // Dense form with a cache fill in the same launch (fill_kc != null): k / v are also written
+  // to the paged caches through fill_pt, by workgroups n_attn ... of the grid.  bs / nb /
+  // bs_magic describe the caches; table row of batch entry i = fill_bidx[i] (or i == 0).
+  uint16_t *fill_kc, *fill_vc;
+  const int32_t *fill_pt;
+  int64_t fill_pt_rs;
+  const void *fill_bidx;
+  int fill_bidx_i64, fill_rows;
+  // Grid layout with a fill: fill_groups super-groups of (8 * attn_per_fill attention
+  // workgroups, then 8 fill workgroups), then the remaining attention workgroups.  Groups of 8
+  // keep an attention workgroup's index congruent to its hardware index modulo 8 (its XCD).
+  int fill_groups, attn_per_fill, n_fill;
   int window;  // > 0 (causal only): row i attends keys offset + i - window < j <= offset + i
   float scale_log2e;
 };
@@ -91,6 +104,54 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   return d;
 }
 
+// The cache fill that rides along with a dense prefill: workgroup f (counted from the end of
+// the attention workgroups) copies fill_rows_per_wg(D) token rows (128 KiB) of one (tensor, batch entry, KV head)
+// from the dense K / V operand into the paged cache, with the semantics of the fill operator
+// (rows whose table row or block is out of range are skipped).  Pure memory work that runs in
+// the shadow of the matrix-bound attention workgroups; nothing in this launch reads the caches.
+constexpr int kFillPasses = 32;  // 16-byte loads in flight per thread
+constexpr int fill_rows_per_wg(int d) { return kFillPasses * (256 / (d / 8)); }
+
+template <int D>
+__device__ __forceinline__ void fill_workgroup(const PrefillArgs &a, int f) {
+  constexpr int CPR = D / 8;        // 16-byte chunks per row
+  constexpr int RPP = 256 / CPR;    // rows per pass of the 256 threads
+  constexpr int NP = kFillPasses;
+  constexpr int kFillRows = fill_rows_per_wg(D);
+  const int chunks = (a.skv + kFillRows - 1) / kFillRows;
+  const int c0 = f % chunks;
+  int r = f / chunks;
+  const int h = r % a.hkv;
+  r /= a.hkv;
+  const int b = r % a.batch;
+  const bool is_v = r / a.batch != 0;
+  int64_t row = a.fill_bidx ? load_index(a.fill_bidx, a.fill_bidx_i64, b) : 0;
+  if (row < 0 || row >= a.fill_rows) return;
+  const uint16_t *src = (is_v ? a.v : a.k) + b * a.kv_bs + h * a.kv_hs;
+  uint16_t *cache = is_v ? a.fill_vc : a.fill_kc;
+  const int32_t *pt = a.fill_pt + row * a.fill_pt_rs;
+  const int t0 = c0 * kFillRows + (int)threadIdx.x / CPR, c = (int)threadIdx.x % CPR;
+  // every load (rows and table entries) is requested before the first store: the compiler
+  // cannot move a load across a store that might alias it, and a table entry per pass would
+  // otherwise cost a round trip each
+  u32x4 val[NP];
+  int phys[NP];
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int t = min(t0 + p * RPP, a.skv - 1);
+    val[p] = *reinterpret_cast<const u32x4 *>(src + (int64_t)t * a.kv_ts + 8 * c);
+    phys[p] = pt[div_block(a, t)];
+  }
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int t = t0 + p * RPP;
+    const int off = t - div_block(a, t) * a.bs;
+    // (no early exit from the loop: the arrays must stay in registers)
+    if (t < a.skv && (unsigned)phys[p] < (unsigned)a.nb)
+      *reinterpret_cast<u32x4 *>(cache + (((int64_t)phys[p] * a.hkv + h) * a.bs + off) * D + 8 * c) = val[p];
+  }
+}
+
 // MODE 0: dense K/V; 1: paged, block_size a multiple of 64 (a tile lies in one block);
 // 3: paged, block_size a multiple of the rows one wavefront load covers (1 KiB: 8 / 4 / 2 rows
 // for head sizes 64 / 128 / 256): one wavefront-uniform table lookup per load; 2: paged, any
@@ -112,6 +173,23 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
   using T = Tile<D>;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
+  int wg = blockIdx.x;  // index among the attention workgroups
+  if constexpr (MODE == 0) {
+    if (a.fill_kc != nullptr) {
+      const int per = 8 * (a.attn_per_fill + 1);
+      const int sg = wg / per, m = wg - sg * per;
+      if (sg < a.fill_groups) {
+        if (m >= 8 * a.attn_per_fill) {
+          const int f = sg * 8 + (m - 8 * a.attn_per_fill);
+          if (f < a.n_fill) fill_workgroup<D>(a, f);
+          return;
+        }
+        wg = sg * 8 * a.attn_per_fill + m;
+      } else {
+        wg -= 8 * a.fill_groups;
+      }
+    }
+  }
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -122,7 +200,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
   // while its query tiles stream through.
   const int nqt = (a.sq + ROWS * RPW - 1) / (ROWS * RPW);
   const int groups = a.hq / HPW;
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int xcd = wg & 7, slot = wg >> 3;
   const int yl = slot / nqt;
   const int y = yl * 8 + xcd;
   if (y >= a.batch * groups) return;  // grid is padded to a multiple of 8 groups
@@ -493,7 +571,22 @@ int launch_mode(const PrefillArgs &a, hipStream_t st) {
   take_profile_events(ev0, ev1);
   if (ev0) (void)hipEventRecord(ev0, st);
   const int ny8 = (a.batch * (a.hq / HPW) + 7) / 8;
-  prefill_kernel<D, HPW, MODE><<<dim3(nqt * ny8 * 8), dim3(256), lds, st>>>(a);
+  int grid = nqt * ny8 * 8;
+  PrefillArgs b = a;
+  if (MODE == 0 && a.fill_kc) {
+    // The fill workgroups are spread over the launch in groups of 8, one group behind every
+    // attn_per_fill groups of attention workgroups, so that their memory traffic runs while the
+    // neighbouring workgroups keep the matrix pipes busy (all of them at the end of the launch
+    // cost as much as two separate fills).
+    b.n_fill = 2 * a.batch * a.hkv * ((a.skv + fill_rows_per_wg(D) - 1) / fill_rows_per_wg(D));
+    const int fg = (b.n_fill + 7) / 8, ag = grid / 8;
+    b.fill_groups = fg;
+    b.attn_per_fill = ag >= fg ? ag / fg : 1;
+    // fewer attention groups than fill groups: one of each per super-group, and the attention
+    // slots past the last real one exit at once (the kernel's range check)
+    grid = ag >= fg ? grid + 8 * fg : 16 * fg;
+  }
+  prefill_kernel<D, HPW, MODE><<<dim3(grid), dim3(256), lds, st>>>(b);
   if (ev1) (void)hipEventRecord(ev1, st);
   return check_launch("sdpa_prefill");
 }
@@ -519,6 +612,15 @@ int launch_d(const PrefillArgs &a, hipStream_t st) {
 
 using namespace ttpa;
 
+// The cache fill that a dense prefill may carry along (ttpa_sdpa_prefill_fill).
+struct FillSpec {
+  void *k_cache, *v_cache;
+  const int32_t *pt;
+  int64_t pt_rs;
+  const void *bidx;
+  int bidx_i64, table_rows;
+};
+
 static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_stride,
                                  int64_t out_token_stride, const void *q, int64_t q_batch_stride,
                                  int64_t q_head_stride, int64_t q_token_stride, const void *k,
@@ -529,7 +631,8 @@ static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_st
                                  int64_t mask_row_stride, int32_t batch, int32_t q_heads,
                                  int32_t kv_heads, int32_t q_len, int32_t kv_len, int32_t head_size,
                                  int32_t block_size, int32_t table_width, int32_t num_blocks,
-                                 int32_t causal, float scale, int32_t sliding_window, void *stream) {
+                                 int32_t causal, float scale, int32_t sliding_window, void *stream,
+                                 const FillSpec *fill = nullptr) {
   TTPA_REQUIRE(out && q && k && v, "null pointer argument");
   TTPA_REQUIRE(sliding_window >= 0, "prefill: sliding_window %d is negative", sliding_window);
   TTPA_REQUIRE(sliding_window == 0 || causal, "prefill: a sliding window needs causal masking");
@@ -576,6 +679,14 @@ static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_st
   a.window = sliding_window;
   a.scale_log2e = scale * 1.4426950408889634f;
   a.bs_magic = block_size >= 2 ? (uint32_t)((1ull << 32) / (uint32_t)block_size) + 1u : 0u;
+  a.fill_kc = a.fill_vc = nullptr;
+  a.fill_pt = nullptr, a.fill_pt_rs = 0, a.fill_bidx = nullptr, a.fill_bidx_i64 = 0, a.fill_rows = 0;
+  a.fill_groups = a.attn_per_fill = a.n_fill = 0;
+  if (fill) {
+    a.fill_kc = static_cast<uint16_t *>(fill->k_cache), a.fill_vc = static_cast<uint16_t *>(fill->v_cache);
+    a.fill_pt = fill->pt, a.fill_pt_rs = fill->pt_rs;
+    a.fill_bidx = fill->bidx, a.fill_bidx_i64 = fill->bidx_i64, a.fill_rows = fill->table_rows;
+  }
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (head_size) {
     case 64: return launch_d<64>(a, st);
@@ -606,4 +717,30 @@ extern "C" int ttpa_sdpa_prefill(TTPA_PREFILL_PARAMS, void *stream) {
 
 extern "C" int ttpa_sdpa_prefill_windowed(TTPA_PREFILL_PARAMS, int32_t sliding_window, void *stream) {
   return prefill_impl(TTPA_PREFILL_ARGS, sliding_window, stream);
+}
+
+extern "C" int ttpa_sdpa_prefill_fill(
+    void *out, int64_t out_batch_stride, int64_t out_head_stride, int64_t out_token_stride,
+    const void *q, int64_t q_batch_stride, int64_t q_head_stride, int64_t q_token_stride,
+    const void *k, const void *v, int64_t kv_batch_stride, int64_t kv_head_stride,
+    int64_t kv_token_stride, int32_t batch, int32_t q_heads, int32_t kv_heads, int32_t q_len,
+    int32_t kv_len, int32_t head_size, int32_t causal, float scale, int32_t sliding_window,
+    void *k_cache, void *v_cache, const int32_t *fill_page_table, int64_t fill_page_table_row_stride,
+    const void *batch_idx, int batch_idx_is_i64, int32_t table_rows, int32_t block_size,
+    int32_t table_width, int32_t num_blocks, void *stream) {
+  TTPA_REQUIRE(k_cache && v_cache && fill_page_table, "prefill + fill: null cache / page_table pointer");
+  TTPA_REQUIRE(block_size > 0 && table_width > 0 && num_blocks > 0 && table_rows > 0,
+               "prefill + fill: non-positive cache geometry");
+  TTPA_REQUIRE(batch_idx != nullptr || batch <= 1, "batch_idx may only be omitted for a single-user fill");
+  TTPA_REQUIRE((int64_t)kv_len <= (int64_t)table_width * block_size,
+               "kv_len %d does not fit %d page-table columns of %d tokens", kv_len, table_width, block_size);
+  TTPA_REQUIRE((int64_t)kv_len * block_size < (1ll << 32), "prefill + fill: kv_len * block_size must stay below 2^32");
+  TTPA_REQUIRE(aligned16(k_cache) && aligned16(v_cache), "prefill + fill: caches must be 16-byte aligned");
+  const FillSpec fill{k_cache, v_cache, fill_page_table, fill_page_table_row_stride, batch_idx,
+                      batch_idx_is_i64, table_rows};
+  return prefill_impl(out, out_batch_stride, out_head_stride, out_token_stride, q, q_batch_stride,
+                      q_head_stride, q_token_stride, k, v, kv_batch_stride, kv_head_stride,
+                      kv_token_stride, nullptr, 0, nullptr, nullptr, 0, 0, batch, q_heads, kv_heads,
+                      q_len, kv_len, head_size, block_size, table_width, num_blocks, causal, scale,
+                      sliding_window, stream, &fill);
 }

@@ -72,6 +72,12 @@ SIGNATURES = {
         [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _i64, _p, _p,
          _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _p],
     ),
+    "ttpa_sdpa_prefill_fill": (
+        _int,
+        [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64,
+         _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32,
+         _p, _p, _p, _i64, _p, _int, _i32, _i32, _i32, _i32, _p],
+    ),
     "ttpa_bfp8_quantize": (_int, [_p, _p, _p, _i64, _p]),
     "ttpa_bfp8_dequantize": (_int, [_p, _p, _p, _i64, _p]),
 }

@@ -259,13 +259,38 @@ class TTAttentionBackendImpl(_ImplBase):
             and attn_metadata.is_causal
             and attn_metadata.attn_mask is None
         )
-        if writes_cache and not fused_step:
-            self._handle_paged_attention(inputs, kv_cache, attn_metadata)
-
         # The reference copies the operator's result into vLLM's output buffer (:330-336).  Where
         # the buffer can be viewed as [users, tokens, heads, head_size] the operators write into
         # it directly (their out-variants take any strides) and return None.
         direct = None if self.functional_cache_ops else self._output_view(output, inputs)
+        # a first-chunk prefill pass (fill K, fill V, dense attention on the fresh K / V) is one
+        # operator too: the attention does not read the caches, so the fills ride in its launch
+        fused_prefill = (
+            writes_cache
+            and inputs.is_prefill
+            and direct is not None
+            and attn_metadata.chunk_start_idx is None
+            and attn_metadata.attn_mask is None
+            and attn_metadata.is_causal
+            and self.sinks is None
+            and kv_cache[0].dtype == torch.bfloat16
+            and inputs.key.shape[0] == inputs.query.shape[0]
+            and inputs.query_num_tokens % 32 == 0
+        )
+        if fused_prefill:
+            batch_idx = attn_metadata.batch_idx
+            assert batch_idx is not None, "batch_idx must be provided for prefill."
+            if attn_metadata.dp_size > 1:
+                batch_idx = batch_idx % (inputs.key.shape[0] // attn_metadata.dp_size)
+            torch.ops.tt.paged_fill_kv_prefill_out_(
+                inputs.query.transpose(1, 2), inputs.key.transpose(1, 2), inputs.value.transpose(1, 2),
+                kv_cache[0], kv_cache[1], attn_metadata.fill_page_table, batch_idx, direct.transpose(1, 2),
+                is_causal=True, scale=self.scale, sliding_window_size=self.sliding_window,
+            )
+            return
+        if writes_cache and not fused_step:
+            self._handle_paged_attention(inputs, kv_cache, attn_metadata)
+
         if inputs.is_prefill:
             assert self.sinks is None, "Attention sink is unsupported in SDPA prefill"
             attn_output = self._compute_full_attention(inputs, kv_cache, attn_metadata, direct)

@@ -610,6 +610,75 @@ def chunked_scaled_dot_product_attention_out(
     _prefill(query, key, value, page_table, start, None, True, scale, out=out)
 
 
+@torch.library.custom_op("tt::paged_fill_kv_prefill_out_", mutates_args=["k_cache", "v_cache", "out"],
+                         device_types=["cuda"])
+def paged_fill_kv_prefill_out_(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    fill_page_table: torch.Tensor,
+    batch_idx: Optional[torch.Tensor],
+    out: torch.Tensor,
+    is_causal: bool = True,
+    scale: Optional[float] = None,
+    sliding_window_size: Optional[int] = None,
+) -> None:
+    """The first-chunk prefill pass of the attention backend as one operator:
+    ``paged_fill_cache_`` of ``key`` into ``k_cache`` and of ``value`` into ``v_cache`` through
+    ``fill_page_table`` / ``batch_idx`` (reference attention.py:486-515) and the dense
+    ``scaled_dot_product_attention_out`` on the same ``query`` / ``key`` / ``value``
+    [B, heads, tokens, head_size] (:576-596).  Same results in the caches and in ``out`` as the
+    three operators; one launch (the rows are copied by extra workgroups of the attention
+    kernel).  bfloat16 caches only."""
+    b, hq, s, d = query.shape
+    nb, hkv, bs, cd, fmt = _cache_geometry(k_cache)
+    if fmt != N.KV_BF16 or _cache_geometry(v_cache) != (nb, hkv, bs, cd, fmt):
+        raise ValueError("prefill + fill needs matching bfloat16 K / V caches")
+    if key.shape != value.shape or key.dim() != 4 or key.shape[0] != b or key.shape[1] != hkv or key.shape[3] != d or cd != d:
+        raise ValueError(f"key / value {tuple(key.shape)} do not match the query and the cache geometry")
+    if query.dtype != torch.bfloat16 or key.dtype != torch.bfloat16 or value.dtype != torch.bfloat16:
+        raise ValueError("query / key / value must be bfloat16")
+    if s % 32:
+        raise ValueError(f"query sequence length must be divisible by 32 but got {s}.")
+    if sliding_window_size is not None:
+        if sliding_window_size <= 0:
+            raise ValueError("sliding_window_size must be positive")
+        if not is_causal:
+            raise NotImplementedError("sliding_window_size is built for the causal form only")
+    if fill_page_table.dim() != 2:
+        raise ValueError("fill_page_table must be [users, blocks_per_user]")
+    skv = key.shape[2]
+    if skv > fill_page_table.shape[1] * bs:
+        raise ValueError(f"{skv} tokens do not fit {fill_page_table.shape[1]} page-table columns of {bs} tokens")
+    if batch_idx is None:
+        if b != 1:
+            raise ValueError("batch_idx is required when key holds more than one user")
+    else:
+        if batch_idx.numel() != b:
+            raise ValueError("batch_idx must have one entry per key row")
+        batch_idx = _index_tensor(batch_idx.reshape(-1))
+    q = _rows_contiguous(query)
+    k, v = _rows_contiguous(key), _rows_contiguous(value)
+    if k.stride() != v.stride():
+        k, v = k.contiguous(), v.contiguous()
+    _check_out(out, (b, hq, s, d), "prefill + fill")
+    pt = _table(fill_page_table)
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    N.call(
+        "ttpa_sdpa_prefill_fill",
+        out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
+        q.data_ptr(), q.stride(0), q.stride(1), q.stride(2),
+        k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), k.stride(2),
+        b, hq, hkv, s, skv, d, int(is_causal), float(scale), int(sliding_window_size or 0),
+        k_cache.data_ptr(), v_cache.data_ptr(), pt.data_ptr(), pt.stride(0), _ptr(batch_idx),
+        int(batch_idx is not None and batch_idx.dtype == torch.int64), pt.shape[0], bs, pt.shape[1], nb,
+        _stream(),
+    )
+
+
 # --------------------------------------------------------------------------- #
 # latent (MLA) attention
 # --------------------------------------------------------------------------- #
