@@ -122,10 +122,9 @@ int ttpa_paged_fill_cache(void *cache, const void *fill, int64_t fill_user_strid
  * call until the stream reaches its end.
  * Built shapes (anything else returns TTPA_ERR_UNSUPPORTED): head_size 64, 128 or 256;
  * block_size a multiple of 4; at most 2048 users; G = q_heads / kv_heads up to 8, and
- * up to 32 for head_size 64 / 128 (up to 16 for head_size 256) with at most 1024 users and
- * block_size a multiple of 1024 / (bytes of a cache row) (8 rows for head_size 64, 4 for 128,
- * 2 for 256; block-float-8: 16 and 8).  TTPA_KV_BFP8: head_size 64 or 128, block_size a
- * multiple of 16.
+ * up to 16 (head_size 64 / 128 with at most 1024 users: up to 32) with block_size a multiple
+ * of 1024 / (bytes of a cache row) (8 rows for head_size 64, 4 for 128, 2 for 256;
+ * block-float-8: 16 and 8).  TTPA_KV_BFP8: head_size 64 or 128, block_size a multiple of 16.
  */
 size_t ttpa_paged_decode_workspace_bytes(int32_t users, int32_t q_heads, int32_t kv_heads,
                                          int32_t head_size);
@@ -174,7 +173,7 @@ int ttpa_paged_sdpa_decode_windowed(void *out, int64_t out_user_stride, int64_t 
  * [1, users, >= kv_heads, head_size] bfloat16 operands of the update, addressed through
  * new_user_stride / new_head_stride.  Where the 16x16x32 decode kernel serves the shape
  * (head_size 64 / 128 with 2 ... 16 query heads per KV head or a block-float-8 cache; head_size
- * 256 with up to 16 query heads per KV head; at most 1024 users) the update runs
+ * 256 with up to 16 query heads per KV head) the update runs
  * inside it: the wavefront that owns the tile of position cur_pos[u] takes the token from
  * k_new / v_new and stores it into the cache; otherwise the library issues the two launches.
  * The equivalence assumes that no user attends a cache row which ANOTHER user's token is

@@ -210,3 +210,35 @@ def test_decode_several_tiles_per_wavefront(monkeypatch, kernel, hq, d):
     got, k, v = _run(wl)
     _check(name, got,
            O.textbook_decode_fp32(wl.q, k.cpu(), v.cpu(), wl.page_table, wl.cache_position, wl.scale))
+
+
+@pytest.mark.parametrize("bfp8", [False, True])
+def test_decode_more_than_1024_users_on_the_matrix_core_kernel(bfp8):
+    """1300 users (the library's limit is 2048) with 4 query heads per KV head: the 16x16x32
+    kernel's prefix tables hold them; contexts of 0 ... 40 tokens and a few padded rows."""
+    from tt_xla_amd import custom_ops as ops
+    from tt_xla_amd import workloads
+
+    users, hq, hkv, d, bs = 1300, 8, 2, 128, 16
+    import random
+    r = random.Random(5)
+    ctx = [r.randint(0, 40) for _ in range(users)]
+    nb = sum((c + 1 + bs - 1) // bs for c in ctx) + 3
+    name = f"decode b{users} h{hq}x{hkv} d{d} bs{bs} bfp8={bfp8}"
+    print(name, flush=True)
+    wl = workloads.decode_ragged(name, 77, users, hq, hkv, d, bs, nb, ctx)
+    for u in (3, 700, 1299):
+        wl.cache_position[u] = -1
+    dev = wl.to("cuda")
+    kc, vc, k_ref, v_ref = dev.k_cache, dev.v_cache, wl.k_cache, wl.v_cache
+    if bfp8:
+        from oracle import bfp8_codec as C
+        kc, vc = ops.bfp8_pack_cache(kc), ops.bfp8_pack_cache(vc)
+        k_ref = C.unpack_cache(kc.cpu(), bs).to(torch.bfloat16)
+        v_ref = C.unpack_cache(vc.cpu(), bs).to(torch.bfloat16)
+    got = torch.ops.tt.paged_scaled_dot_product_attention_decode(
+        dev.q, kc, vc, dev.page_table, is_causal=True, cur_pos_tensor=dev.cache_position, scale=wl.scale).cpu()
+    want = O.textbook_decode_fp32(wl.q, k_ref, v_ref, wl.page_table, wl.cache_position, wl.scale)
+    live = [u for u in range(users) if u not in (3, 700, 1299)]
+    assert torch.isnan(got[0, [3, 700, 1299]]).all()
+    _check(name, got[:, live], want[:, live])

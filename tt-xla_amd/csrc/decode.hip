@@ -327,9 +327,8 @@ int launch_g(const DecodeArgs &a, int g, hipStream_t st) {
     case 8: launch<D, 8>(a, st); break;
     default:
       return fail(TTPA_ERR_UNSUPPORTED,
-                  "query heads per KV head = %d: more than 8 (up to 32 with head_size 64 / 128, up to 16 "
-                  "with 256) need at most 1024 users and a block_size that is a multiple of 1024 / (bytes "
-                  "of a cache row)",
+                  "query heads per KV head = %d: more than 8 (up to 16; up to 32 with head_size 64 / 128 and "
+                  "at most 1024 users) need a block_size that is a multiple of 1024 / (bytes of a cache row)",
                   g);
   }
   return TTPA_OK;

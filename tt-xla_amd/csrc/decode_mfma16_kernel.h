@@ -1,5 +1,5 @@
 // Paged decode attention on the 16x16x32 matrix-core shape: up to 16 query heads per KV head,
-// 72 KiB of LDS per workgroup; head sizes 64 and 128 with a block-float-8 cache (expanded to
+// 80 KiB of LDS per workgroup; head sizes 64 and 128 with a block-float-8 cache (expanded to
 // half precision) or a bfloat16 cache, head size 256 with a bfloat16 cache.
 //
 // Work decomposition, partial slots and merge kernel are those of decode.hip, with tiles of
@@ -61,7 +61,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 
-constexpr int kMaxUsers16 = 1024;
+constexpr int kMaxUsers16 = kMaxUsers;  // the library-wide limit: 16 KiB of prefix tables
 constexpr int kTileBytes = 16384;  // TILE tokens of head_size 16-bit elements
 
 template <bool F16>
