@@ -109,6 +109,20 @@ int ttpa_paged_fill_cache(void *cache, const void *fill, int64_t fill_user_strid
                           int32_t num_blocks, int32_t kv_format, void *stream);
 
 /*
+ * ttpa_paged_fill_cache on the K cache and on the V cache in one launch: a prefill pass of
+ * the backend fills both with the same table and batch_idx (attention.py:500-511).  k_fill
+ * and v_fill share their strides.  Same result as the two calls.
+ */
+int ttpa_paged_fill_cache_kv(void *k_cache, void *v_cache, const void *k_fill, const void *v_fill,
+                             int64_t fill_user_stride, int64_t fill_head_stride,
+                             int64_t fill_token_stride, const int32_t *page_table,
+                             int64_t page_table_row_stride, const void *batch_idx,
+                             int batch_idx_is_i64, int32_t fill_users, int32_t table_rows,
+                             int32_t kv_heads, int32_t seq_len, int32_t block_size,
+                             int32_t head_size, int32_t table_width, int32_t num_blocks,
+                             int32_t kv_format, void *stream);
+
+/*
  * Causal paged decode attention, one query token per user.
  * Replaces the device branch of tt::paged_scaled_dot_product_attention_decode
  * (custom_ops.py:1198-1315; CPU semantics :1256-1312, grouped heads as in :551-610):

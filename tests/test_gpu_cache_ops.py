@@ -161,6 +161,37 @@ def test_fill_batched_backend_view(s):
                        key.transpose(1, 2))
 
 
+@pytest.mark.parametrize("fmt", ["bf16", "bfp8"])
+@pytest.mark.parametrize("s", [32, 50, 300])
+def test_fill_kv_single_launch_equals_two_fills(fmt, s):
+    """tt::paged_fill_kv_cache_ (one launch for K and V) against the oracle's batched fill applied
+    to each cache; one batch_idx entry points outside the table (its row is skipped)."""
+    from oracle import bfp8_codec as C
+
+    g = torch.Generator().manual_seed(100 + s)
+    users, hkv, bs, d = 4, 4, 32, 128
+    w = (s + bs - 1) // bs + 1
+    nb = users * w + 1
+    kc = torch.randn(nb, hkv, bs, d, generator=g).to(torch.bfloat16)
+    vc = torch.randn(nb, hkv, bs, d, generator=g).to(torch.bfloat16)
+    key = torch.randn(users, s, hkv, d, generator=g).to(torch.bfloat16)
+    val = torch.randn(users, s, hkv, d, generator=g).to(torch.bfloat16)
+    table = (_table(g, users, w) + 1).to(torch.int32)
+    bidx = torch.tensor([2, 0, 9, 1], dtype=torch.int32)
+    # the oracle takes rows inside the table: the skipped row is left out of its call
+    keep = [0, 1, 3]
+    k_want = O.paged_fill_cache_batched(kc, key[keep].transpose(1, 2), table, bidx[keep])
+    v_want = O.paged_fill_cache_batched(vc, val[keep].transpose(1, 2), table, bidx[keep])
+    if fmt == "bfp8":
+        k_dev, v_dev = C.pack_cache(kc).cuda(), C.pack_cache(vc).cuda()
+        k_want, v_want = C.pack_cache(k_want), C.pack_cache(v_want)
+    else:
+        k_dev, v_dev = kc.cuda(), vc.cuda()
+    torch.ops.tt.paged_fill_kv_cache_(k_dev, v_dev, key.cuda().transpose(1, 2), val.cuda().transpose(1, 2),
+                                      table.cuda(), batch_idx=bidx.cuda())
+    assert torch.equal(k_dev.cpu(), k_want) and torch.equal(v_dev.cpu(), v_want)
+
+
 def test_fill_rejects_sequence_longer_than_table():
     cache = torch.zeros(4, 1, 32, 64, dtype=torch.bfloat16).cuda()
     fill = torch.zeros(1, 1, 65, 64, dtype=torch.bfloat16).cuda()

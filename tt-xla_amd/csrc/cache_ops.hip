@@ -99,6 +99,10 @@ __global__ __launch_bounds__(256) void update_bfp8_kernel(UpdateArgs a) {
 struct FillArgs {
   void *cache;
   const uint16_t *fill;
+  // a second (cache, fill) pair written by the same launch (K and V of a prefill), or null:
+  // grid z = fill rows of the first pair, then those of the second
+  void *cache2;
+  const uint16_t *fill2;
   int64_t fill_us, fill_hs, fill_ts;
   const int32_t *pt;
   int64_t pt_rs;
@@ -138,11 +142,12 @@ __global__ __launch_bounds__(256) void fill_bf16_kernel(FillArgs a) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= a.s * cpr) return;
   const int t = fast_div(idx, cpr, a.tpr_magic), chunk = idx - t * cpr;
-  const int h = blockIdx.y, i = blockIdx.z;
+  const bool second = (int)blockIdx.z >= a.fill_users;
+  const int h = blockIdx.y, i = (int)blockIdx.z - (second ? a.fill_users : 0);
   int phys, off;
   if (!resolve_fill(a, i, t, phys, off)) return;
-  const uint16_t *src = a.fill + i * a.fill_us + h * a.fill_hs + t * a.fill_ts + chunk * VEC;
-  uint16_t *dst = static_cast<uint16_t *>(a.cache) +
+  const uint16_t *src = (second ? a.fill2 : a.fill) + i * a.fill_us + h * a.fill_hs + t * a.fill_ts + chunk * VEC;
+  uint16_t *dst = static_cast<uint16_t *>(second ? a.cache2 : a.cache) +
                   (((int64_t)phys * a.hkv + h) * a.bs + off) * a.d + chunk * VEC;
   if constexpr (VEC == 8) {
     *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(src);
@@ -156,16 +161,17 @@ __global__ __launch_bounds__(256) void fill_bfp8_kernel(FillArgs a) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= a.s * gpr) return;
   const int t = fast_div(idx, gpr, a.tpr_magic), grp = idx - t * gpr;
-  const int h = blockIdx.y, i = blockIdx.z;
+  const bool second = (int)blockIdx.z >= a.fill_users;
+  const int h = blockIdx.y, i = (int)blockIdx.z - (second ? a.fill_users : 0);
   int phys, off;
   if (!resolve_fill(a, i, t, phys, off)) return;
-  const uint4 *src = reinterpret_cast<const uint4 *>(a.fill + i * a.fill_us + h * a.fill_hs +
-                                                     t * a.fill_ts + grp * 16);
+  const uint4 *src = reinterpret_cast<const uint4 *>((second ? a.fill2 : a.fill) + i * a.fill_us +
+                                                     h * a.fill_hs + t * a.fill_ts + grp * 16);
   uint4 lo = src[0], hi = src[1];
   uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   uint32_t bytes[4];
   uint32_t e = bfp8_encode16(w, bytes);
-  uint8_t *slab = static_cast<uint8_t *>(a.cache) +
+  uint8_t *slab = static_cast<uint8_t *>(second ? a.cache2 : a.cache) +
                   ((int64_t)phys * a.hkv + h) * (int64_t)(a.bs + a.bs / 16) * a.d;
   *reinterpret_cast<uint4 *>(slab + (int64_t)off * a.d + grp * 16) =
       make_uint4(bytes[0], bytes[1], bytes[2], bytes[3]);
@@ -255,14 +261,14 @@ extern "C" int ttpa_paged_update_cache_kv(void *k_cache, void *v_cache, const vo
                        kv_heads, block_size, head_size, table_width, num_blocks, kv_format, stream);
 }
 
-extern "C" int ttpa_paged_fill_cache(void *cache, const void *fill, int64_t fill_user_stride,
-                                     int64_t fill_head_stride, int64_t fill_token_stride,
-                                     const int32_t *page_table, int64_t page_table_row_stride,
-                                     const void *batch_idx, int batch_idx_is_i64,
-                                     int32_t fill_users, int32_t table_rows, int32_t kv_heads,
-                                     int32_t seq_len, int32_t block_size, int32_t head_size,
-                                     int32_t table_width, int32_t num_blocks, int32_t kv_format,
-                                     void *stream) {
+// cache2 / fill2 non-null: both pairs in one launch.
+static int launch_fill(void *cache, void *cache2, const void *fill, const void *fill2,
+                       int64_t fill_user_stride, int64_t fill_head_stride, int64_t fill_token_stride,
+                       const int32_t *page_table, int64_t page_table_row_stride,
+                       const void *batch_idx, int batch_idx_is_i64, int32_t fill_users,
+                       int32_t table_rows, int32_t kv_heads, int32_t seq_len, int32_t block_size,
+                       int32_t head_size, int32_t table_width, int32_t num_blocks, int32_t kv_format,
+                       void *stream) {
   if (int rc = common_checks(cache, fill, page_table, kv_heads, block_size, head_size, table_width,
                              num_blocks, kv_format))
     return rc;
@@ -274,6 +280,7 @@ extern "C" int ttpa_paged_fill_cache(void *cache, const void *fill, int64_t fill
                block_size);
   if (fill_users == 0 || seq_len == 0) return TTPA_OK;
   FillArgs a{cache,      static_cast<const uint16_t *>(fill),
+             cache2,     static_cast<const uint16_t *>(fill2),
              fill_user_stride, fill_head_stride, fill_token_stride,
              page_table, page_table_row_stride,
              batch_idx,  batch_idx_is_i64,
@@ -281,6 +288,7 @@ extern "C" int ttpa_paged_fill_cache(void *cache, const void *fill, int64_t fill
              num_blocks, 0u, 0u};
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool vec_ok = head_size % 8 == 0 && aligned16(cache) && aligned16(fill) &&
+                      (!cache2 || (aligned16(cache2) && aligned16(fill2))) &&
                       fill_user_stride % 8 == 0 && fill_head_stride % 8 == 0 &&
                       fill_token_stride % 8 == 0;
   int tpr;  // threads per token row
@@ -291,11 +299,12 @@ extern "C" int ttpa_paged_fill_cache(void *cache, const void *fill, int64_t fill
     tpr = vec_ok ? head_size / 8 : head_size;
   }
   const int64_t threads = (int64_t)seq_len * tpr;  // per (fill row, head)
-  TTPA_REQUIRE(threads < (int64_t)1 << 31 && fill_users <= 65535 && kv_heads <= 65535,
+  const int pairs = cache2 ? 2 : 1;
+  TTPA_REQUIRE(threads < (int64_t)1 << 31 && fill_users * pairs <= 65535 && kv_heads <= 65535,
                "fill too large for one launch");
   a.tpr_magic = magic_for(threads, tpr);
   a.bs_magic = magic_for(seq_len, block_size);
-  const dim3 grid((unsigned)((threads + 255) / 256), (unsigned)kv_heads, (unsigned)fill_users);
+  const dim3 grid((unsigned)((threads + 255) / 256), (unsigned)kv_heads, (unsigned)(fill_users * pairs));
   if (kv_format == TTPA_KV_BFP8) {
     fill_bfp8_kernel<<<grid, dim3(256), 0, st>>>(a);
   } else if (vec_ok) {
@@ -304,4 +313,34 @@ extern "C" int ttpa_paged_fill_cache(void *cache, const void *fill, int64_t fill
     fill_bf16_kernel<1><<<grid, dim3(256), 0, st>>>(a);
   }
   return check_launch("paged_fill_cache");
+}
+
+extern "C" int ttpa_paged_fill_cache(void *cache, const void *fill, int64_t fill_user_stride,
+                                     int64_t fill_head_stride, int64_t fill_token_stride,
+                                     const int32_t *page_table, int64_t page_table_row_stride,
+                                     const void *batch_idx, int batch_idx_is_i64,
+                                     int32_t fill_users, int32_t table_rows, int32_t kv_heads,
+                                     int32_t seq_len, int32_t block_size, int32_t head_size,
+                                     int32_t table_width, int32_t num_blocks, int32_t kv_format,
+                                     void *stream) {
+  return launch_fill(cache, nullptr, fill, nullptr, fill_user_stride, fill_head_stride,
+                     fill_token_stride, page_table, page_table_row_stride, batch_idx,
+                     batch_idx_is_i64, fill_users, table_rows, kv_heads, seq_len, block_size,
+                     head_size, table_width, num_blocks, kv_format, stream);
+}
+
+extern "C" int ttpa_paged_fill_cache_kv(void *k_cache, void *v_cache, const void *k_fill,
+                                        const void *v_fill, int64_t fill_user_stride,
+                                        int64_t fill_head_stride, int64_t fill_token_stride,
+                                        const int32_t *page_table, int64_t page_table_row_stride,
+                                        const void *batch_idx, int batch_idx_is_i64,
+                                        int32_t fill_users, int32_t table_rows, int32_t kv_heads,
+                                        int32_t seq_len, int32_t block_size, int32_t head_size,
+                                        int32_t table_width, int32_t num_blocks, int32_t kv_format,
+                                        void *stream) {
+  TTPA_REQUIRE(v_cache && v_fill, "null V cache / fill pointer");
+  return launch_fill(k_cache, v_cache, k_fill, v_fill, fill_user_stride, fill_head_stride,
+                     fill_token_stride, page_table, page_table_row_stride, batch_idx,
+                     batch_idx_is_i64, fill_users, table_rows, kv_heads, seq_len, block_size,
+                     head_size, table_width, num_blocks, kv_format, stream);
 }

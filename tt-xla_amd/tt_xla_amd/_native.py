@@ -40,6 +40,11 @@ SIGNATURES = {
         [_p, _p, _i64, _i64, _i64, _p, _i64, _p, _int, _i32, _i32, _i32, _i32, _i32, _i32, _i32,
          _i32, _i32, _p],
     ),
+    "ttpa_paged_fill_cache_kv": (
+        _int,
+        [_p, _p, _p, _p, _i64, _i64, _i64, _p, _i64, _p, _int, _i32, _i32, _i32, _i32, _i32, _i32,
+         _i32, _i32, _i32, _p],
+    ),
     "ttpa_paged_decode_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32]),
     "ttpa_paged_sdpa_decode": (
         _int,

@@ -392,8 +392,7 @@ class TTAttentionBackendImpl(_ImplBase):
             kv_cache[0].copy_(ops.paged_fill_cache(kv_cache[0], k_new, table, batch_idx=batch_idx))
             kv_cache[1].copy_(ops.paged_fill_cache(kv_cache[1], v_new, table, batch_idx=batch_idx))
         else:
-            ops.paged_fill_cache_(kv_cache[0], k_new, table, batch_idx=batch_idx)
-            ops.paged_fill_cache_(kv_cache[1], v_new, table, batch_idx=batch_idx)
+            ops.paged_fill_kv_cache_(kv_cache[0], kv_cache[1], k_new, v_new, table, batch_idx=batch_idx)  # one launch
 
     # ------------------------------------------------------------------ attention
     def _compute_full_attention(self, inputs, kv_cache, attn_metadata: TTMetadata,

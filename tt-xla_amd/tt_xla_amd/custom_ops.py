@@ -202,7 +202,8 @@ def _(k_cache, v_cache, k_fill, v_fill, update_indices, page_table):
     return None
 
 
-def _fill_inplace(cache, fill_value, page_table, batch_idx):
+def _fill_inplace(cache, fill_value, page_table, batch_idx, cache2=None, fill_value2=None):
+    """cache2 / fill_value2 given: the second pair is written by the same launch."""
     nb, hkv, bs, d, fmt = _cache_geometry(cache)
     if fill_value.dim() != 4:
         raise ValueError("fill_value must be [users, heads, seq_len, head_size]")
@@ -230,6 +231,23 @@ def _fill_inplace(cache, fill_value, page_table, batch_idx):
         raise ValueError("fill_value dtype must match the cache (bfloat16 for block-float-8)")
     fill_value = _rows_contiguous(fill_value)
     pt = _table(page_table)
+    if cache2 is not None:
+        if _cache_geometry(cache2) != (nb, hkv, bs, d, fmt) or fill_value2.shape != (fu, fh, s, fd) \
+                or fill_value2.dtype != fill_value.dtype:
+            raise ValueError("K and V caches / fills must agree in shape and dtype")
+        fill_value2 = _rows_contiguous(fill_value2)
+        if fill_value2.stride() != fill_value.stride():
+            _fill_inplace(cache, fill_value, page_table, batch_idx)
+            _fill_inplace(cache2, fill_value2, page_table, batch_idx)
+            return
+        N.call(
+            "ttpa_paged_fill_cache_kv",
+            cache.data_ptr(), cache2.data_ptr(), fill_value.data_ptr(), fill_value2.data_ptr(),
+            fill_value.stride(0), fill_value.stride(1), fill_value.stride(2), pt.data_ptr(), pt.stride(0),
+            _ptr(batch_idx), int(batch_idx is not None and batch_idx.dtype == torch.int64),
+            fu, pt.shape[0], hkv, s, bs, d, pt.shape[1], nb, fmt, _stream(),
+        )
+        return
     N.call(
         "ttpa_paged_fill_cache",
         cache.data_ptr(), fill_value.data_ptr(), fill_value.stride(0), fill_value.stride(1),
@@ -269,6 +287,21 @@ def paged_fill_cache_(
 @paged_fill_cache_.register_fake
 def _(cache, fill_value, page_table, batch_idx=None):
     return None
+
+
+@torch.library.custom_op("tt::paged_fill_kv_cache_", mutates_args=["k_cache", "v_cache"],
+                         device_types=["cuda"])
+def paged_fill_kv_cache_(
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    k_fill: torch.Tensor,
+    v_fill: torch.Tensor,
+    page_table: torch.Tensor,
+    batch_idx: Optional[torch.Tensor] = None,
+) -> None:
+    """``paged_fill_cache_`` on the K cache and on the V cache in one launch (a prefill pass
+    always fills both through the same table and batch_idx, reference attention.py:500-511)."""
+    _fill_inplace(k_cache, k_fill, page_table, batch_idx, v_cache, v_fill)
 
 
 # --------------------------------------------------------------------------- #
