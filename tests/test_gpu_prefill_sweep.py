@@ -1,4 +1,4 @@
-"""Seeded random sweep of the prefill operators over their shape envelope: head sizes 64 /
+"""Seeded random sweep of the prefill operators (and of the one-operator prefill pass) over their shape envelope: head sizes 64 /
 128 / 256, group widths that select each heads-per-wavefront variant (4, 2, 1), query lengths
 from one 32-row block to several tiles, key lengths that end inside a tile, causal / additive
 mask / sliding window on the dense operator; block sizes on either side of the tile size,
@@ -88,3 +88,40 @@ def test_chunked_random_case(seed):
     got = torch.ops.tt.chunked_scaled_dot_product_attention(
         q.cuda(), key.cuda(), value.cuda(), table.cuda(), st.cuda()).cpu()
     _check(got, want)
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_prefill_pass_random_case(seed):
+    """The first-chunk prefill pass as one operator (tt::paged_fill_kv_prefill_out_) against
+    fill K + fill V + dense attention, caches and output bit for bit: head sizes, group widths,
+    prompt lengths from one 32-row block up, block sizes, sliding windows, permuted table rows,
+    and shapes with more fill workgroups than attention workgroups (many heads, short prompts)."""
+    r = random.Random(5000 + seed)
+    d = r.choice([64, 128, 128, 256])
+    g = r.choice([1, 1, 2, 4, 8])
+    hkv = r.choice([1, 2, 8, 16] if g == 1 else [1, 2, 4])
+    b = r.randint(1, 4)
+    s = 32 * r.choice([1, 1, 2, 3, 5, 9, 17])
+    bs = r.choice([16, 32, 64, 128])
+    window = r.choice([0, 0, 0, 40, 1000])
+    c = dict(seed=seed, b=b, hq=hkv * g, hkv=hkv, s=s, d=d, bs=bs, window=window)
+    print("prefill pass sweep", c, flush=True)
+    gen = torch.Generator().manual_seed(seed)
+    q, k, v = (_bf(gen, b, h, s, d).cuda() for h in (hkv * g, hkv, hkv))
+    w = (s + bs - 1) // bs + r.randint(0, 1)
+    rows = b + 1
+    nb = rows * w + 1
+    table = (torch.randperm(nb - 1, generator=gen)[: rows * w] + 1).view(rows, w).to(torch.int32).cuda()
+    bidx = torch.randperm(rows, generator=gen)[:b].to(torch.int32).cuda() if (b > 1 or r.random() < 0.5) else None
+    kc = _bf(gen, nb, hkv, bs, d).cuda()
+    vc = _bf(gen, nb, hkv, bs, d).cuda()
+    kw = dict(is_causal=True, sliding_window_size=window if window else None)
+    k_ref, v_ref = kc.clone(), vc.clone()
+    torch.ops.tt.paged_fill_kv_cache_(k_ref, v_ref, k, v, table, bidx)
+    want = torch.ops.tt.scaled_dot_product_attention(q, k, v, **kw)
+    out = torch.zeros(b, s, hkv * g, d, dtype=torch.bfloat16, device="cuda")
+    torch.ops.tt.paged_fill_kv_prefill_out_(q, k, v, kc, vc, table, bidx, out.transpose(1, 2), **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(kc, k_ref), "K cache differs"
+    assert torch.equal(vc, v_ref), "V cache differs"
+    assert torch.equal(out.transpose(1, 2), want)
