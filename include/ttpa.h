@@ -138,7 +138,8 @@ int ttpa_paged_fill_cache_kv(void *k_cache, void *v_cache, const void *k_fill, c
  * block_size a multiple of 4; at most 2048 users; G = q_heads / kv_heads up to 8, and
  * up to 16 (head_size 64 / 128 with at most 1024 users: up to 32) with block_size a multiple
  * of 1024 / (bytes of a cache row) (8 rows for head_size 64, 4 for 128, 2 for 256;
- * block-float-8: 16 and 8).  TTPA_KV_BFP8: head_size 64 or 128, block_size a multiple of 16.
+ * block-float-8: 16, 8 and 4).  TTPA_KV_BFP8: block_size a multiple of 16 (head_size 256: G up
+ * to 16).
  */
 size_t ttpa_paged_decode_workspace_bytes(int32_t users, int32_t q_heads, int32_t kv_heads,
                                          int32_t head_size);

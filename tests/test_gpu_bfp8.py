@@ -48,7 +48,7 @@ def test_pack_unpack_kernels_bit_exact():
     assert torch.equal(back.cpu().float(), C.unpack_cache(want, 32))
 
 
-@pytest.mark.parametrize("users,hkv,bs,d", [(8, 8, 32, 128), (5, 2, 64, 64), (16, 1, 128, 128)])
+@pytest.mark.parametrize("users,hkv,bs,d", [(8, 8, 32, 128), (5, 2, 64, 64), (16, 1, 128, 128), (6, 4, 16, 256)])
 def test_update_quantises_bit_exact(users, hkv, bs, d):
     g = torch.Generator().manual_seed(users + hkv + bs)
     w = 4
@@ -107,6 +107,10 @@ def _decode_vs_roundtrip(wl, name):
     (2, 64, 8, 128, 64, [1000, 257]),
     (3, 12, 4, 128, 16, [15, 16, 100]),
     (2, 8, 1, 128, 128, [127, 400]),
+    (3, 16, 8, 256, 32, [31, 32, 700]),           # head size 256: tiles of 32 tokens
+    (3, 24, 2, 256, 16, [100, 17, 450]),          # blocks smaller than a tile, 12 heads per group
+    (2, 4, 4, 256, 64, [63, 500]),                # one query head per KV head
+    (3, 16, 4, 64, 32, [0, 200, 2000]),           # head size 64: tiles of 128 tokens
 ])
 def test_decode_bfp8_shapes(users, hq, hkv, d, bs, ctx):
     from tt_xla_amd import workloads
@@ -133,6 +137,7 @@ def test_decode_bfp8_config5_reduced_and_property():
 @pytest.mark.parametrize("users,hq,hkv,d,bs,ctx", [
     (4, 32, 8, 128, 64, [5, 64, 200, 700]),
     (3, 12, 4, 128, 16, [15, 16, 100]),
+    (3, 16, 8, 256, 32, [31, 32, 700]),           # head size 256 is built on the 16x16x32 kernel only
 ])
 def test_decode_bfp8_every_kernel(monkeypatch, kernel, users, hq, hkv, d, bs, ctx):
     """The three main kernels that can serve a block-float-8 cache (VALU, 32x32x16 and 16x16x32

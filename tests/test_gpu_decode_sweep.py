@@ -30,7 +30,7 @@ def _case(seed):
     d = r.choice([64, 128, 128, 128, 256])
     hkv = r.choice([1, 2, 4, 8])
     g = r.choice([1, 2, 3, 4, 5, 7, 8, 12, 16] if d == 256 else [1, 2, 3, 4, 4, 5, 6, 7, 8, 12, 16, 24, 32])
-    bfp8 = d in (64, 128) and r.random() < 0.35
+    bfp8 = r.random() < 0.35 and (d != 256 or g <= 16)
     bs = r.choice([16, 32, 64, 128] if bfp8 else [4, 8, 16, 32, 64, 128])
     if g > 8:  # wide groups run on the matrix-core kernels only: whole 1 KiB loads per block
         bs = max(bs, 1024 // (d * (1 if bfp8 else 2)))

@@ -36,6 +36,8 @@ CASES = [
     (3, 8, 8, 128, 32, [40, 333, 64], False, 0, False, False),          # G = 1: dot-product kernel, two launches
     (2, 16, 8, 256, 64, [130, 64], False, 0, False, False),             # head size 256, fused
     (4, 8, 4, 256, 16, [31, 32, 1000, 1500], False, 300, True, True),   # blocks smaller than its 32-token tiles
+    (3, 16, 8, 256, 32, [31, 32, 700], True, 0, False, False),          # head size 256, block-float-8
+    (4, 4, 4, 256, 16, [15, 16, 1000, 1500], True, 300, True, True),
 ]
 
 

@@ -299,9 +299,9 @@ int waves_for_device(int kv_format) {
 }
 
 template <int D, int G>
-void launch(const DecodeArgs &a, hipStream_t st) {
+bool launch(const DecodeArgs &a, hipStream_t st) {
   if (a.kv_format == TTPA_KV_BFP8) {
-    launch_bfp8_main(a, D, G, st);
+    return launch_bfp8_main(a, D, G, st);
   } else {
     // With one workgroup per CU in the grid, a 64 KiB dynamic LDS request (unused) makes two
     // workgroups too large to share a CU, so the dispatcher has to spread them over all CUs.
@@ -312,25 +312,28 @@ void launch(const DecodeArgs &a, hipStream_t st) {
     else
       paged_decode_kernel<D, G, false><<<dim3(blocks), dim3(256), pad, st>>>(a, a.pt, a.cur);
   }
+  return true;
 }
 
 template <int D>
 int launch_g(const DecodeArgs &a, int g, hipStream_t st) {
+  bool ok = true;
   switch (g) {
-    case 1: launch<D, 1>(a, st); break;
-    case 2: launch<D, 2>(a, st); break;
-    case 3: launch<D, 3>(a, st); break;
-    case 4: launch<D, 4>(a, st); break;
-    case 5: launch<D, 5>(a, st); break;
-    case 6: launch<D, 6>(a, st); break;
-    case 7: launch<D, 7>(a, st); break;
-    case 8: launch<D, 8>(a, st); break;
+    case 1: ok = launch<D, 1>(a, st); break;
+    case 2: ok = launch<D, 2>(a, st); break;
+    case 3: ok = launch<D, 3>(a, st); break;
+    case 4: ok = launch<D, 4>(a, st); break;
+    case 5: ok = launch<D, 5>(a, st); break;
+    case 6: ok = launch<D, 6>(a, st); break;
+    case 7: ok = launch<D, 7>(a, st); break;
+    case 8: ok = launch<D, 8>(a, st); break;
     default:
       return fail(TTPA_ERR_UNSUPPORTED,
                   "query heads per KV head = %d: more than 8 (up to 16; up to 32 with head_size 64 / 128 and "
                   "at most 1024 users) need a block_size that is a multiple of 1024 / (bytes of a cache row)",
                   g);
   }
+  if (!ok) return fail(TTPA_ERR_UNSUPPORTED, "decode: the dot-product kernel is not built for this head size and cache format");
   return TTPA_OK;
 }
 
@@ -367,9 +370,11 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
                kv_heads);
   if (kv_format != TTPA_KV_BF16 && kv_format != TTPA_KV_BFP8)
     return fail(TTPA_ERR_INVALID_ARGUMENT, "decode: unknown kv_format %d", kv_format);
-  if (kv_format == TTPA_KV_BFP8 && ((head_size != 64 && head_size != 128) || block_size % 16))
+  if (kv_format == TTPA_KV_BFP8 && block_size % 16)
+    return fail(TTPA_ERR_UNSUPPORTED, "decode: a block-float-8 cache needs block_size %% 16 == 0");
+  if (kv_format == TTPA_KV_BFP8 && head_size == 256 && (q_heads / kv_heads > 16))
     return fail(TTPA_ERR_UNSUPPORTED,
-                "decode: block-float-8 is built for head_size 64 / 128 and block_size %% 16 == 0");
+                "decode: block-float-8 with head_size 256 is built for up to 16 query heads per KV head");
   if (users > kMaxUsers)
     return fail(TTPA_ERR_UNSUPPORTED, "decode: %d users exceeds the limit of %d", users, kMaxUsers);
   if (head_size != 64 && head_size != 128 && head_size != 256)
@@ -437,7 +442,7 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   bool use_mfma16 = mfma16_ok && (g >= g_min16 || kv_format == TTPA_KV_BFP8 || head_size == 256);
   bool use_mfma = !use_mfma16 && mfma_ok && (g >= 5 || kv_format == TTPA_KV_BFP8);
   // a forced kernel that is not built for the shape leaves the default choice in place
-  if (forced == 1 && g <= 8) use_mfma = use_mfma16 = false;
+  if (forced == 1 && g <= 8 && !(kv_format == TTPA_KV_BFP8 && head_size == 256)) use_mfma = use_mfma16 = false;
   if (forced == 2 && mfma_ok) use_mfma = true, use_mfma16 = false;
   if (forced == 3 && mfma16_ok) use_mfma16 = true, use_mfma = false;
   // The matrix-core kernels get one workgroup per CU whatever the cache format: the 32x32 kernel

@@ -11,7 +11,7 @@ bool launch_mfma16_d256(const DecodeArgs &a, hipStream_t st);
 
 bool mfma16_decode_supported(const DecodeArgs &a, int head_size, int g) {
   const bool bfp8 = a.kv_format == TTPA_KV_BFP8;
-  if (!(head_size == 64 || head_size == 128 || (head_size == 256 && !bfp8))) return false;
+  if (head_size != 64 && head_size != 128 && head_size != 256) return false;
   const int rows_per_load = 1024 / (head_size * (bfp8 ? 1 : 2));  // a load covers whole rows of one block
   return g <= 16 && a.users <= kMaxUsers && a.bs % rows_per_load == 0;
 }

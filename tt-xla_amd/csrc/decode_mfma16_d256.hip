@@ -5,7 +5,8 @@ namespace ttpa {
 namespace decode {
 
 bool launch_mfma16_d256(const DecodeArgs &a, hipStream_t st) {
-  return launch_for_block_size<256, false>(a, st);  // bfloat16 cache only
+  return a.kv_format == TTPA_KV_BFP8 ? launch_for_block_size<256, true>(a, st)
+                                     : launch_for_block_size<256, false>(a, st);
 }
 
 }  // namespace decode

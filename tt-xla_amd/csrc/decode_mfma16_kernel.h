@@ -1,6 +1,6 @@
 // Paged decode attention on the 16x16x32 matrix-core shape: up to 16 query heads per KV head,
-// 80 KiB of LDS per workgroup; head sizes 64 and 128 with a block-float-8 cache (expanded to
-// half precision) or a bfloat16 cache, head size 256 with a bfloat16 cache.
+// 80 KiB of LDS per workgroup; head sizes 64, 128 and 256 with a block-float-8 cache (expanded
+// to half precision) or a bfloat16 cache.
 //
 // Work decomposition, partial slots and merge kernel are those of decode.hip, with tiles of
 // 8192 / head_size tokens (128, 64 or 32): 16 KiB of 16-bit elements whatever the head size.  Inside a
@@ -139,7 +139,7 @@ __device__ inline void write_negative_position(const DecodeArgs &a, const int32_
 template <int D, bool BFP8, int RUNS, bool FUSED>
 __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     DecodeArgs a, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
-  static_assert(D == 64 || D == 128 || (D == 256 && !BFP8), "shapes built");
+  static_assert(D == 64 || D == 128 || D == 256, "shapes built");
   constexpr int TILE = kTileBytes / (2 * D);  // tokens per tile
   constexpr int ROWB = 2 * D;                 // bytes of a tile row in LDS
   constexpr int KSTEPS = D / 32, DBLK = D / 16;
