@@ -70,7 +70,9 @@ def test_ops_are_registered_and_refuse_cpu_tensors(native):
     for name in (
         "paged_update_cache", "paged_fill_cache", "paged_scaled_dot_product_attention_decode",
         "chunked_scaled_dot_product_attention", "scaled_dot_product_attention",
-        "paged_update_cache_", "paged_fill_cache_",
+        "paged_update_cache_", "paged_fill_cache_", "paged_update_kv_cache_", "paged_fill_kv_cache_",
+        "paged_update_kv_decode_", "paged_update_kv_decode_out_", "paged_fill_kv_prefill_out_",
+        "scaled_dot_product_attention_out", "chunked_scaled_dot_product_attention_out",
     ):
         assert hasattr(torch.ops.tt, name)
     cache = torch.zeros(2, 1, 32, 64, dtype=torch.bfloat16)
