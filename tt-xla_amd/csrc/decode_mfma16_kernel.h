@@ -41,8 +41,9 @@
 // banks and the keys are taken from row / 2: (row / 2) & 7 and y = (row / 2) & 3.
 //
 // Where a tile's rows sit in the cache (RUNS): one run of consecutive rows when a block holds
-// whole tiles; four runs of a quarter tile each when block_size is a multiple of a quarter tile
-// (block sizes 32 and 16 with head size 128; 64 and 32 with 64; 16 and 8 with 256); otherwise
+// whole tiles; two runs of half a tile when block_size is a multiple of half a tile (block size
+// 32 with head size 128, the serving default; 64 with 64; 16 with 256); four runs of a quarter
+// tile when it is a multiple of a quarter tile (16 with 128; 32 with 64; 8 with 256); otherwise
 // one run per load instruction.  A run costs a block-table lookup and a 64-bit base, which are
 // scalar registers, the resource this kernel is short of.
 //
@@ -135,7 +136,7 @@ __device__ inline void write_negative_position(const DecodeArgs &a, const int32_
   }
 }
 
-// RUNS: 1, 4, or 0 for one run per load.
+// RUNS: 1, 2, 4, or 0 for one run per load.
 template <int D, bool BFP8, int RUNS, bool FUSED>
 __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     DecodeArgs a, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
@@ -592,6 +593,7 @@ bool launch_for_block_size(const DecodeArgs &a, hipStream_t st) {
   constexpr int TILE = kTileBytes / (2 * D);
   const bool fused = a.k_new != nullptr;
   if (a.bs % TILE == 0) return fused ? launch<D, BFP8, 1, true>(a, st) : launch<D, BFP8, 1, false>(a, st);
+  if (a.bs % (TILE / 2) == 0) return fused ? launch<D, BFP8, 2, true>(a, st) : launch<D, BFP8, 2, false>(a, st);
   if (a.bs % (TILE / 4) == 0) return fused ? launch<D, BFP8, 4, true>(a, st) : launch<D, BFP8, 4, false>(a, st);
   return fused ? launch<D, BFP8, 0, true>(a, st) : launch<D, BFP8, 0, false>(a, st);
 }
