@@ -326,22 +326,26 @@ __device__ __forceinline__ void write_partial(float *slot, int g, int G, int r, 
 // Partials are read eight at a time so that their loads overlap (with four wavefronts per CU
 // and at least one segment per CU, a segment has about five): the kernel is a chain of
 // dependent round trips, and this keeps it at two.  G and D are run-time values: the
-// matrix-core kernels serve any group width up to 32.  D is a power of two (64, 128, 256).
+// matrix-core kernels serve any group width up to 32.  D is a power of two on the attention
+// paths (64, 128, 256: split by shift and mask); the latent path also has 384 (divided).
 __global__ inline __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a, int G, int D) {
   const int seg = blockIdx.x;
   const int u = seg / a.hkv, h = seg % a.hkv;
+  const bool pow2 = (D & (D - 1)) == 0;
   const int dshift = __builtin_ctz(D);
+  auto head_of = [&](int i) { return pow2 ? i >> dshift : i / D; };
+  auto elem_of = [&](int i) { return pow2 ? i & (D - 1) : i % D; };
   const int first = a.ws_seg[2 * seg], nw = a.ws_seg[2 * seg + 1];
   uint16_t *out = a.out + u * a.out_us;
   if (nw == 0) {  // padded row: no attended position -> NaN like softmax over nothing
     for (int i = threadIdx.x; i < G * D; i += 256)
-      out[(int64_t)(h * G + (i >> dshift)) * a.out_hs + (i & (D - 1))] = 0x7fc0;
+      out[(int64_t)(h * G + head_of(i)) * a.out_hs + elem_of(i)] = 0x7fc0;
     return;
   }
   constexpr int kBatch = 8;
   const float *base = a.ws_slots + (int64_t)first * a.slot_floats;
   for (int i = threadIdx.x; i < G * D; i += 256) {
-    const int g = i >> dshift;
+    const int g = head_of(i);
     float mall = -INFINITY, num = 0.f, den = 0.f;
     for (int w = 0; w < nw; w += kBatch) {
       float mv[kBatch], lv[kBatch], av[kBatch];
@@ -373,7 +377,7 @@ __global__ inline __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a
       num *= resc;
       den = den * resc + __builtin_amdgcn_exp2f(sk - mnew);
     }
-    out[(int64_t)(h * G + g) * a.out_hs + (i & (D - 1))] = (uint16_t)f32_to_bf16_bits(num / den);
+    out[(int64_t)(h * G + g) * a.out_hs + elem_of(i)] = (uint16_t)f32_to_bf16_bits(num / den);
   }
 }
 
