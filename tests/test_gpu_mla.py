@@ -51,6 +51,7 @@ DECODE = [
     (4, 16, 1, 576, 512, False, 32, 24, None),    # latent serving shape, 16 heads per rank
     (3, 128, 1, 576, 512, False, 64, 12, None),   # all 128 heads: four head blocks per user
     (2, 64, 2, 192, 128, False, 16, 40, 0.11),
+    (3, 16, 1, 576, 384, False, 32, 12, None),    # a value width that is not a power of two (merge kernel)
 ]
 
 
