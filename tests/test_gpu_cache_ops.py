@@ -112,6 +112,8 @@ FILL_GRID = [
     (8, 16, 1, 32, 128, 10), (8, 16, 8, 32, 128, 20), (16, 16, 8, 64, 128, 32),
     (8, 32, 32, 32, 128, 50), (16, 16, 8, 64, 128, 70), (8, 16, 8, 32, 128, 70),
     (8, 16, 8, 64, 128, 64), (4, 8, 8, 128, 256, 300), (2, 4, 2, 32, 64, 1),
+    (4, 8, 4, 48, 128, 200), (4, 16, 2, 20, 64, 131), (3, 40, 2, 1, 128, 33),   # block sizes off the powers of two, and 1
+    (2, 4, 2, 32, 40, 50),                                                     # head size with 5 chunks per row
 ]
 
 

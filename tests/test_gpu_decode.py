@@ -177,6 +177,10 @@ def test_config2_full_size():
     (3, 16, 8, 256, 32, [31, 32, 700]),          # head size 256: tiles of 32 tokens on the 16x16 kernel
     (3, 24, 2, 256, 8, [100, 17, 450]),          # blocks smaller than a tile, 12 heads per group
     (2, 16, 16, 256, 16, [63, 64]),              # one query head per KV head
+    (3, 32, 8, 128, 48, [47, 48, 700]),          # block sizes that are not powers of two: quarter-tile runs
+    (3, 32, 8, 128, 24, [23, 24, 700]),          # ... one run per load
+    (3, 16, 4, 64, 96, [95, 96, 1000]),
+    (2, 8, 2, 256, 12, [11, 300]),
 ])
 def test_decode_every_kernel(monkeypatch, kernel, users, hq, hkv, d, bs, ctx):
     """The dot-product kernel and the two matrix-core kernels, each forced in turn on the same

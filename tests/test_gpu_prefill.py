@@ -118,6 +118,9 @@ def test_chunked_reference_cases(hq, hkv, start):
     (1, 4, 4, 128, 2, 100, 64, 70),
     (2, 16, 8, 256, 8, 30, 32, 150),      # head size 256, block of 8: one lookup per load
     (2, 8, 8, 64, 8, 40, 96, 130),        # head size 64, block of exactly one load
+    (2, 16, 4, 128, 48, 6, 96, 100),      # block sizes that are not powers of two (multiply-high quotients)
+    (2, 8, 2, 128, 20, 12, 64, 70),
+    (1, 8, 8, 64, 24, 10, 32, 150),
 ])
 def test_chunked_shapes(users, hq, hkv, d, bs, nbpu, start, lc):
     name = f"chunked u{users} h{hq}x{hkv} d{d} bs{bs} w{nbpu} start{start} lc{lc}"
