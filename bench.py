@@ -52,9 +52,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--rotate", type=int, default=3, help="independent workload copies cycled through")
     ap.add_argument("--launch", choices=["graph", "eager"], default="graph")
-    ap.add_argument("--steps-per-graph", type=int, default=6,
-                    help="consecutive steps captured in one graph (a decode forward replays one "
-                         "attention step per layer inside one graph); 1 = one graph launch per step")
+    ap.add_argument("--steps-per-graph", type=int, default=32,
+                    help="consecutive steps captured in one graph: a decode forward replays one "
+                         "attention step per layer inside one graph, and Llama-3-8B has 32 layers; "
+                         "1 = one graph launch per step")
     ap.add_argument("--workload", choices=["config2", "config3", "config4", "config5"], default="config2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-users", type=int, default=0, help="users in the CPU sample (0 = auto)")
@@ -124,25 +125,29 @@ def prefill_step(impl, w, out):
 
 # --------------------------------------------------------------------------- timing helpers
 class StepRunner:
-    """Runs steps over the rotating workload copies (step i uses copy i % n).  In graph mode a
-    graph holds `per_graph` consecutive steps (rounded up to a multiple of n so the rotation
-    continues across replays), the way the decode forward of a model replays one attention step
-    per layer inside a single graph; a shorter graph covers the remainder so that run(k)
-    executes exactly k steps."""
+    """Runs steps over the rotating workload copies.  Eager: step i uses copy i % n.  In graph
+    mode a graph holds `per_graph` consecutive steps (step j of a graph uses copy j % n; the
+    length is chosen so that the last step of a replay and the first of the next use different
+    copies), the way the decode forward of a model replays one attention step per layer inside
+    one graph; a shorter graph covers the remainder so that run(k) executes exactly k steps.
+    sequence(k) lists the copies run(k) goes through."""
 
     def __init__(self, fns, use_graph, per_graph):
         import torch
 
         self.fns, self.n, self.use_graph = fns, len(fns), use_graph
-        self.per_graph = max(1, (max(1, per_graph) + self.n - 1) // self.n * self.n)
+        self.per_graph = max(1, per_graph)
+        if self.n > 1 and self.per_graph > 1 and (self.per_graph - 1) % self.n == 0:
+            self.per_graph += 1
         self.graphs, self.keep = {}, []
         if use_graph:
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
+            # warm-up and capture share one stream
+            self.side = torch.cuda.Stream()
+            self.side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(self.side):
                 for f in fns:  # warm allocator and kernels outside capture
                     f()
-            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.current_stream().wait_stream(self.side)
             torch.cuda.synchronize()
 
     def _graph(self, length):
@@ -150,7 +155,7 @@ class StepRunner:
 
         if length not in self.graphs:
             gr = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(gr):
+            with torch.cuda.graph(gr, stream=self.side):
                 for i in range(length):
                     self.keep.append(self.fns[i % self.n]())
             self.graphs[length] = gr
@@ -163,6 +168,12 @@ class StepRunner:
                 self._graph(self.per_graph)
             if rem:
                 self._graph(rem)
+
+    def sequence(self, steps):
+        if not self.use_graph:
+            return [i % self.n for i in range(steps)]
+        full, rem = divmod(steps, self.per_graph)
+        return [j % self.n for j in range(self.per_graph)] * full + [j % self.n for j in range(rem)]
 
     def run(self, steps):
         if not self.use_graph:
@@ -364,7 +375,7 @@ def run_decode(args):
     runner = StepRunner(fns, args.launch == "graph", args.steps_per_graph)
     ms = time_steps(runner, args.steps, args.warmup)
     n = len(copies)
-    avg_step_bytes = sum(step_bytes[i % n] for i in range(args.steps)) / args.steps
+    avg_step_bytes = sum(step_bytes[i] for i in runner.sequence(args.steps)) / args.steps
     durs = time_decode_kernel_direct(copies, min(args.steps, 100))
     kern_ms = sum(d for d, _ in durs) / len(durs)
     kern_bytes = sum(step_bytes[w] for _, w in durs) / len(durs)  # the kernel also writes the new token

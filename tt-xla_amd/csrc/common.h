@@ -124,7 +124,7 @@ __device__ __forceinline__ void dma16(const void *uniform_base, uint32_t lane_by
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :
                : "v"(lane_bytes), "s"(uniform_base), "s"(lds_addr)
-               : "memory");
+               : "memory", "m0");
 }
 // The same for callers whose base / LDS address the compiler cannot prove uniform: both are
 // read from the first active lane.  readfirstlane returns a signed int: each half of the
@@ -141,7 +141,7 @@ __device__ __forceinline__ void dma16_lane(const void *lane_ptr, uint32_t lds_ad
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
                : "v"(lane_ptr), "s"(lds_addr)
-               : "memory");
+               : "memory", "m0");
 }
 
 

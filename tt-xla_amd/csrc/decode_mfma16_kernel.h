@@ -3,9 +3,10 @@
 // to half precision) or a bfloat16 cache.
 //
 // Work decomposition, partial slots and merge kernel are those of decode.hip, with tiles of
-// 8192 / head_size tokens (128, 64 or 32): 16 KiB of 16-bit elements whatever the head size.  Inside a
-// wavefront a tile of K, then of V, goes global -> registers -> a 16 KiB wave-private
-// LDS buffer that both tensors use in turn:
+// 16 KiB of 16-bit elements (128, 64 or 32 tokens at head size 64, 128, 256; 8 KiB = 32 tokens
+// for a bfloat16 cache with head size 128, see tile_bytes).  Inside a wavefront a tile of K,
+// then of V, goes global -> registers -> a wave-private LDS buffer of that size that both
+// tensors use in turn:
 //   stage K(t) | prefetch K(t+1) | S^T = K Q^T | softmax | stage V(t) | prefetch V(t+1) | O^T += V^T P^T
 // so every global load has three quarters of a tile period to arrive.  The byte -> half
 // expansion of the block-float-8 cache is the one of decode_mfma.hip (one permute and one
@@ -63,7 +64,18 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kMaxUsers16 = kMaxUsers;  // the library-wide limit: 16 KiB of prefix tables
-constexpr int kTileBytes = 16384;  // TILE tokens of head_size 16-bit elements
+// Bytes of a tile's K (or V) rows as 16-bit elements, i.e. of a wavefront's LDS buffer: 16 KiB
+// (128 / 64 / 32 tokens at head size 64 / 128 / 256), except 8 KiB (32 tokens) for a bfloat16
+// cache with head size 128.  A wavefront has one tile of K and one of V in flight; the kernel
+// ends when the slowest wavefront has drained its last tile, and wavefronts of one launch finish
+// several microseconds apart (the XCDs do not get equal shares of the HBM bandwidth), so a
+// shorter tile shortens that tail: config 2's step 58.7 -> 57.8 us, config 4's 549 -> 543 us.
+// The block-float-8 cache moves half the bytes per token and loses with the shorter tile
+// (44.1 -> 46.2 us on config 5).
+template <int D, bool BFP8>
+constexpr int tile_bytes() {
+  return (D == 128 && !BFP8) ? 8192 : 16384;
+}
 
 template <bool F16>
 __device__ __forceinline__ floatx4 mma16(const u32x4 &x, const u32x4 &y, const floatx4 &c) {
@@ -141,6 +153,7 @@ template <int D, bool BFP8, int RUNS, bool FUSED>
 __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     DecodeArgs a, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
   static_assert(D == 64 || D == 128 || D == 256, "shapes built");
+  constexpr int kTileBytes = tile_bytes<D, BFP8>();
   constexpr int TILE = kTileBytes / (2 * D);  // tokens per tile
   constexpr int ROWB = 2 * D;                 // bytes of a tile row in LDS
   constexpr int KSTEPS = D / 32, DBLK = D / 16;
@@ -577,7 +590,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
 template <int D, bool BFP8, int RUNS, bool FUSED>
 bool launch(const DecodeArgs &a, hipStream_t st) {
   const int blocks = a.n_waves / kWavesPerBlock;
-  const size_t lds = (size_t)kWavesPerBlock * kTileBytes;
+  const size_t lds = (size_t)kWavesPerBlock * tile_bytes<D, BFP8>();
   static std::atomic<uint64_t> lds_ready{0};
   if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_mfma16_kernel<D, BFP8, RUNS, FUSED>), lds,
                           lds_ready))
@@ -590,7 +603,7 @@ bool launch(const DecodeArgs &a, hipStream_t st) {
 // cache update of the step).
 template <int D, bool BFP8>
 bool launch_for_block_size(const DecodeArgs &a, hipStream_t st) {
-  constexpr int TILE = kTileBytes / (2 * D);
+  constexpr int TILE = tile_bytes<D, BFP8>() / (2 * D);
   const bool fused = a.k_new != nullptr;
   if (a.bs % TILE == 0) return fused ? launch<D, BFP8, 1, true>(a, st) : launch<D, BFP8, 1, false>(a, st);
   if (a.bs % (TILE / 2) == 0) return fused ? launch<D, BFP8, 2, true>(a, st) : launch<D, BFP8, 2, false>(a, st);
