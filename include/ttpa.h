@@ -208,6 +208,31 @@ int ttpa_paged_update_decode(
     void *stream);
 
 /*
+ * ttpa_paged_update_decode for callers that cannot hold a workspace: code under HIP graph
+ * capture that may not call hipMalloc, tight serving loops, harnesses that forbid allocation.
+ * It has no counterpart in the reference.  The split-K partial results go to a static array
+ * inside the library's device image (ttpa_static_scratch_bytes() = 16 MiB per GPU the library
+ * runs on, held until the process ends) instead of a caller buffer; the call allocates nothing.
+ * Shapes whose ttpa_paged_decode_workspace_bytes(...) exceed that size are refused with
+ * TTPA_ERR_WORKSPACE (config 2 needs 4.8 MB, config 4 12.8 MB).  The array's device address is
+ * looked up once per device, at the first call on that device or by ttpa_static_scratch_init()
+ * (call it with the device current, outside graph capture, if the first call would be captured).
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two
+ * host threads) race; calls on one stream run in turn and need nothing cleared between them.
+ * Results equal ttpa_paged_update_decode's.
+ */
+size_t ttpa_static_scratch_bytes(void);
+int ttpa_static_scratch_init(void);
+int ttpa_paged_update_decode_static(
+    void *out, int64_t out_user_stride, int64_t out_head_stride, const void *q,
+    int64_t q_user_stride, int64_t q_head_stride, void *k_cache, void *v_cache, const void *k_new,
+    const void *v_new, int64_t new_user_stride, int64_t new_head_stride,
+    const int32_t *page_table, int64_t page_table_row_stride, const void *cur_pos,
+    int cur_pos_is_i64, int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
+    int32_t block_size, int32_t table_width, int32_t num_blocks, float scale, int32_t kv_format,
+    int32_t sliding_window, const float *attention_sink, void *stream);
+
+/*
  * Paged decode attention for latent-style (multi-head latent attention) caches.
  * Replaces the device branch of tt::paged_flash_mla_decode
  * (python_package/tt_torch/custom_ops.py:381-632; CPU semantics :551-610), causal form:

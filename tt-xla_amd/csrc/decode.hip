@@ -522,6 +522,71 @@ extern "C" int ttpa_paged_sdpa_decode_windowed(
                      kv_format, sliding_window, attention_sink, workspace, workspace_bytes, stream);
 }
 
+// ---- the entry point that allocates nothing ------------------------------------------------
+namespace {
+
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+// Workspace of ttpa_paged_update_decode_static.  In host code the name is only a handle for
+// hipGetSymbolAddress: the device address is looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (each GPU holds its own copy).
+int static_scratch(void **out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(TTPA_ERR_LAUNCH, "static scratch: no current device (ordinals up to %d)", kMaxDevices - 1);
+  void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return fail(TTPA_ERR_LAUNCH, "static scratch: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    }
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing first calls find the same address
+  }
+  *out = p;
+  return TTPA_OK;
+}
+
+}  // namespace
+
+extern "C" size_t ttpa_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int ttpa_static_scratch_init(void) {
+  void *p = nullptr;
+  return static_scratch(&p);
+}
+
+extern "C" int ttpa_paged_update_decode_static(
+    void *out, int64_t out_user_stride, int64_t out_head_stride, const void *q,
+    int64_t q_user_stride, int64_t q_head_stride, void *k_cache, void *v_cache, const void *k_new,
+    const void *v_new, int64_t new_user_stride, int64_t new_head_stride,
+    const int32_t *page_table, int64_t page_table_row_stride, const void *cur_pos,
+    int cur_pos_is_i64, int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
+    int32_t block_size, int32_t table_width, int32_t num_blocks, float scale, int32_t kv_format,
+    int32_t sliding_window, const float *attention_sink, void *stream) {
+  TTPA_REQUIRE(k_new && v_new, "update + decode: null fresh K / V pointer");
+  const size_t need = ttpa_paged_decode_workspace_bytes(users, q_heads, kv_heads, head_size);
+  if (need == 0) return fail(TTPA_ERR_INVALID_ARGUMENT, "update + decode: bad users / heads / head_size");
+  if (need > kStaticScratchBytes)
+    return fail(TTPA_ERR_WORKSPACE,
+                "update + decode without a workspace: this shape needs %zu bytes of partial results, the "
+                "library's static scratch holds %zu; use ttpa_paged_update_decode with a caller workspace",
+                need, kStaticScratchBytes);
+  void *ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  // nothing in the workspace has to start at zero: the segment table and every partial slot that
+  // the merge kernel reads are written by the main kernel of the same call
+  return decode_impl(out, out_user_stride, out_head_stride, q, q_user_stride, q_head_stride, k_cache,
+                     v_cache, page_table, page_table_row_stride, cur_pos, cur_pos_is_i64, users,
+                     q_heads, kv_heads, head_size, block_size, table_width, num_blocks, scale,
+                     kv_format, sliding_window, attention_sink, ws, kStaticScratchBytes, stream,
+                     k_new, v_new, new_user_stride, new_head_stride);
+}
+
 extern "C" int ttpa_paged_update_decode(
     void *out, int64_t out_user_stride, int64_t out_head_stride, const void *q,
     int64_t q_user_stride, int64_t q_head_stride, void *k_cache, void *v_cache, const void *k_new,

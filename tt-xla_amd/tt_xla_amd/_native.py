@@ -61,6 +61,13 @@ SIGNATURES = {
         [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _int, _i32, _i32,
          _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _p, _p, _sz, _p],
     ),
+    "ttpa_static_scratch_bytes": (_sz, []),
+    "ttpa_static_scratch_init": (_int, []),
+    "ttpa_paged_update_decode_static": (
+        _int,
+        [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _int, _i32, _i32,
+         _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _p, _p],
+    ),
     "ttpa_paged_mla_decode_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32]),
     "ttpa_paged_mla_decode": (
         _int,
