@@ -82,12 +82,11 @@ def test_ops_are_registered_and_refuse_cpu_tensors(native):
                                         torch.zeros(1, 2, dtype=torch.int32))
 
 
-def test_latent_decode_entry_refuses_to_launch():
-    """The latent (MLA) decode kernel is switched off after faulting on the device: the entry
-    point must answer TTPA_ERR_UNSUPPORTED before touching any argument (no GPU needed)."""
+def test_latent_decode_entry_validates_on_the_host():
+    """The latent (MLA) decode entry point rejects bad arguments before any launch (no GPU needed)."""
     from tt_xla_amd import _native as N
 
     rc = N.lib().ttpa_paged_mla_decode(None, 0, 0, None, 0, 0, None, None, None, 0, None, 0, 1, 16, 1, 576,
                                        512, 32, 1, 1, 1.0, None, None, 0, None)
-    assert rc == -2
-    assert b"switched off" in N.lib().ttpa_last_error()
+    assert rc == N.ERR_INVALID_ARGUMENT
+    assert b"null" in N.lib().ttpa_last_error()

@@ -1,12 +1,17 @@
 """Host-side model of the address arithmetic of the latent decode kernel
-(tt-xla_amd/csrc/decode_wide.hip): for each built shape, every global source range, LDS
-destination, LDS operand read and partial-slot write the kernel forms must stay inside the
-buffer it belongs to.  Pure integer arithmetic, no GPU: it restates the kernel's formulas, so
-it guards the geometry (strides, tile sizes, slot layout), not the generated code."""
+(tt-xla_amd/csrc/decode_wide.hip): for every shape that tests/test_gpu_mla.py runs, every global
+source range, LDS-DMA destination, LDS operand read and partial-slot write the kernel forms must
+stay inside the buffer it belongs to.  LDS-DMA destinations are modelled as the instruction takes
+them: ABSOLUTE byte addresses in the workgroup's LDS allocation (the static arrays come first, the
+dynamic stages behind them), 16-byte aligned, never inside the static arrays and never past the
+CU's LDS.  Pure integer arithmetic, no GPU: it restates the kernel's formulas, so it guards the
+geometry (strides, tile sizes, slot layout), not the generated code."""
 
 import itertools
 
 import pytest
+
+import test_gpu_mla as G
 
 K_TILE = 64
 STATIC_LDS = 8224          # s_pref + s_len + s_wsum of the kernel
@@ -21,7 +26,17 @@ SHAPES = [
     (128, 128, True, 8, 8, 32, 16, 128, 8),
     (128, 64, True, 16, 1, 32, 16, 128, 8),
     (192, 128, False, 8, 1, 1184, 1, 1, 1024),   # prefill mapping: one block of s tokens
+    (576, 512, False, 16, 1, 32, 8, 24, 3),      # test_mla_decode_padded_row_sink_and_errors
+    (576, 512, False, 16, 1, 32, 3, 12, 2),      # test_mla_backend_prefill_then_decode, decode step
+    (576, 512, False, 16, 1, 64, 1, 1, 64),      # ... its prefill (64 tokens per user)
 ]
+# every case of the GPU test's own lists
+SHAPES += [(dh, dv, has_v, hq, nkv, bs, width, width * users, users)
+           for users, hq, nkv, dh, dv, has_v, bs, width, _ in G.DECODE]
+# prefill runs on the decode kernel: query row i is a user, the sequence one block of s tokens,
+# at most 1024 users per launch
+SHAPES += [(dh, dv, has_v, hq, nkv, s, 1, 1, min(s, 1024)) for _, hq, s, dh, nkv, dv, has_v in G.PREFILL]
+SHAPES = sorted(set(SHAPES))
 
 
 def _geometry(hq, nkv):
@@ -62,14 +77,21 @@ def test_every_address_stays_in_bounds(dqk, dv, sep_v, hq, nkv, bs, width, nb, u
                 # the row index inside a block must be < block_size
                 assert 0 <= tk - col * bs < bs
                 assert 0 <= src and src + row_bytes <= cache_bytes
+                assert src % 16 == 0
                 for buf in (0, 1):
-                    dst = STATIC_LDS + buf * stage + r * krow
-                    assert dst + row_bytes <= STATIC_LDS + buf * stage + ktile
+                    dst = STATIC_LDS + buf * stage + r * krow      # absolute, as M0 carries it
+                    assert dst % 16 == 0 and dst >= STATIC_LDS
+                    assert dst + row_bytes <= STATIC_LDS + buf * stage + ktile <= LDS_PER_CU
+                    # the row moves as whole 1 KiB pieces (64 lanes x 16 bytes) plus a tail under a
+                    # lane mask: together exactly the row, nothing beyond it
+                    full, rem_lanes = row_bytes // 1024, (row_bytes % 1024) // 16
+                    assert full * 1024 + rem_lanes * 16 == row_bytes and rem_lanes < 64
                     if sep_v:
                         vsrc = row * dv * 2
                         assert vsrc + 2 * dv <= vcache_bytes
                         vdst = STATIC_LDS + buf * stage + ktile + r * v_lds_row
-                        assert vdst + 2 * dv <= STATIC_LDS + (buf + 1) * stage
+                        assert vdst % 16 == 0 and vsrc % 16 == 0 and 2 * dv <= 1024
+                        assert vdst + 2 * dv <= STATIC_LDS + (buf + 1) * stage <= LDS_PER_CU
 
     # LDS operand reads of every lane
     ksteps = dqk // 16

@@ -6,6 +6,7 @@
 
 #include <atomic>
 
+#include "pointer_words.h"
 #include "ttpa.h"
 
 namespace ttpa {
@@ -127,14 +128,12 @@ __device__ __forceinline__ void dma16(const void *uniform_base, uint32_t lane_by
                : "memory", "m0");
 }
 // The same for callers whose base / LDS address the compiler cannot prove uniform: both are
-// read from the first active lane.  readfirstlane returns a signed int: each half of the
-// pointer goes through uint32_t before widening, or a low half with bit 31 set would smear
-// ones over the high half.
+// read from the first active lane, the address word by word (address_from_words).
 __device__ __forceinline__ void dma16_uniform(const void *uniform_base, uint32_t lane_bytes, uint32_t lds_addr) {
   const uint64_t ub = reinterpret_cast<uint64_t>(uniform_base);
-  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)ub);
-  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(ub >> 32));
-  dma16(reinterpret_cast<const void *>(((uint64_t)hi << 32) | (uint64_t)lo), lane_bytes,
+  const int lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)ub);
+  const int hi = __builtin_amdgcn_readfirstlane((int)(uint32_t)(ub >> 32));
+  dma16(reinterpret_cast<const void *>(address_from_words(lo, hi)), lane_bytes,
         (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr));
 }
 __device__ __forceinline__ void dma16_lane(const void *lane_ptr, uint32_t lds_addr) {

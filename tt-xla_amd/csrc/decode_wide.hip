@@ -29,7 +29,6 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kMaxUsersWide = 1024;
-constexpr bool kLatentDecodeDisabled = true;
 
 struct WideArgs {
   int nkv;         // KV heads of the caches (DecodeArgs::hkv counts segments per user)
@@ -344,14 +343,6 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
                                      int32_t block_size, int32_t table_width, int32_t num_blocks,
                                      float scale, const float *attention_sink, void *workspace,
                                      size_t workspace_bytes, void *stream) {
-  // Switched off: the kernel's first two runs on the device ended in memory faults.  One cause
-  // has been found by reading the generated code (the wavefront-uniform copy of the source
-  // pointer sign-extended its low half) and is fixed in dma16_uniform; until a run on the
-  // device confirms that nothing else is wrong, the entry point refuses to launch.
-  if (kLatentDecodeDisabled)
-    return fail(TTPA_ERR_UNSUPPORTED,
-                "latent decode is switched off in this build: its kernel faulted on the device and the "
-                "fix has not been verified there yet");
   TTPA_REQUIRE(out && q && k_cache && page_table && cur_pos, "null pointer argument");
   TTPA_REQUIRE(users > 0 && q_heads > 0 && kv_heads > 0 && head_size > 0 && head_dim_v > 0 &&
                    block_size > 0 && table_width > 0 && num_blocks > 0,

@@ -22,8 +22,7 @@ Differences from the reference, invisible in results: the cache writes use the i
 operators (one batched fill instead of a per-user loop over functional fills followed by a
 copy of the whole cache); ``functional_cache_ops=True`` restores the reference's call sequence.
 
-The two latent attention operators sit on ``ttpa_paged_mla_decode``; while that entry point is
-switched off in the library they raise ``TtpaError`` and so does this backend.
+The two latent attention operators sit on ``ttpa_paged_mla_decode``.
 """
 
 from __future__ import annotations

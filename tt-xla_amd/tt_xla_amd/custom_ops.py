@@ -719,10 +719,7 @@ _MLA_MAX_USERS = 1024  # users per launch of the latent decode kernel
 
 
 def _mla_decode_launch(out, q, key, value, page_table, cur, head_dim_v, scale, sink):
-    """out [users, heads, dv] / q [users, heads, dh] by strides; caches in the paged layout.
-
-    The entry point below currently answers TTPA_ERR_UNSUPPORTED (its kernel is switched off
-    until a fix for a device fault has been verified), which surfaces here as TtpaError."""
+    """out [users, heads, dv] / q [users, heads, dh] by strides; caches in the paged layout."""
     nb, nkv, bs, dh = key.shape
     users, hq = q.shape[0], q.shape[1]
     for u0 in range(0, users, _MLA_MAX_USERS):
