@@ -137,3 +137,54 @@ def test_forward_errors():
         from tt_xla_amd import TTAttentionBackendImpl
 
         TTAttentionBackendImpl(HQ, D, 1.0, HKV, [0.1], None, "auto")
+
+
+def test_kv_shared_layer_prefill_reads_the_target_cache():
+    """A layer that shares another layer's KV cache (kv_sharing_target_layer_name set) never
+    writes the cache (reference attention.py:309-314) and its prefill attends over keys / values
+    gathered from it through the page table, block-major then in-block, cut to the pass's token
+    count (attention.py:562-574, 600-632)."""
+    from tt_xla_amd import TTMetadata
+
+    g = torch.Generator().manual_seed(5)
+    users, width, s = 2, 4, 96
+    table, kc, vc = _setup(g, users, width)
+    kv = [kc.cuda(), vc.cuda()]
+    q = _bf(g, users * s, HQ * D)
+    k, v = _bf(g, users * s, HKV * D), _bf(g, users * s, HKV * D)  # ignored: the layer owns no K / V
+    md = TTMetadata(cache_position=None, page_table=table.cuda(), num_users=users,
+                    batch_idx=torch.arange(users, dtype=torch.int32).cuda())
+    out = torch.empty(users * s, HQ * D, dtype=torch.bfloat16, device="cuda")
+    _impl(kv_sharing_target_layer_name="model.layers.0.self_attn").forward(
+        None, q.cuda(), k.cuda(), v.cuda(), kv, md, output=out)
+    assert torch.equal(kv[0].cpu(), kc) and torch.equal(kv[1].cpu(), vc), "a KV-shared layer wrote the cache"
+    k_dense = O.gather_paged_to_dense(kc, table)[:, :, :s]
+    v_dense = O.gather_paged_to_dense(vc, table)[:, :, :s]
+    assert k_dense.shape == (users, HKV, s, D)
+    # the gather order, spelled out: position p of user u is block table[u, p // BS], row p % BS
+    for u, p in ((0, 0), (1, 33), (1, s - 1)):
+        assert torch.equal(k_dense[u, :, p], kc[table[u, p // BS], :, p % BS])
+    want = O.sdpa(q.view(users, s, HQ, D).transpose(1, 2), k_dense, v_dense, None, True, D**-0.5)
+    torch.testing.assert_close(out.cpu().float(), want.transpose(1, 2).reshape(users * s, HQ * D).float(),
+                               atol=2e-2, rtol=2e-2)
+
+
+def test_kv_shared_layer_decode_reads_the_target_cache():
+    """The decode pass of a KV-shared layer attends over the target layer's cache as it is: no
+    update, not even of the position it is at (attention.py:309-314, 634-668)."""
+    from tt_xla_amd import TTMetadata
+
+    g = torch.Generator().manual_seed(6)
+    users, width = 3, 5
+    table, kc, vc = _setup(g, users, width)
+    pos = torch.tensor([7, 64, 159], dtype=torch.int32)
+    q, k, v = _bf(g, users, HQ * D), _bf(g, users, HKV * D), _bf(g, users, HKV * D)
+    kv = [kc.cuda(), vc.cuda()]
+    md = TTMetadata(cache_position=pos.cuda(), page_table=table.cuda(), num_users=users)
+    out = torch.empty(users, HQ * D, dtype=torch.bfloat16, device="cuda")
+    _impl(kv_sharing_target_layer_name="model.layers.0.self_attn").forward(
+        None, q.cuda(), k.cuda(), v.cuda(), kv, md, output=out)
+    assert torch.equal(kv[0].cpu(), kc) and torch.equal(kv[1].cpu(), vc)
+    want = O.paged_sdpa_decode(q.view(users, 1, HQ, D).transpose(0, 1), kc, vc, table, True, None, pos,
+                               None, D**-0.5).transpose(0, 1).reshape(users, HQ * D)
+    torch.testing.assert_close(out.cpu().float(), want.float(), atol=2e-2, rtol=2e-2)
