@@ -130,6 +130,9 @@ int ttpa_paged_fill_cache_kv(void *k_cache, void *v_cache, const void *k_fill, c
  *   over cache positions j = 0 .. min(cur_pos[u], table_width * block_size - 1),
  *   position j living in block page_table[u, j / block_size], row j % block_size.
  * cur_pos[u] < 0 (padded batch row) gives a NaN output row, as on the reference.
+ * (The operator's other form, is_causal = False with an additive attn_mask over all positions
+ * of the table, custom_ops.py:1299-1303, needs no entry point of its own: the host side gathers
+ * the user's blocks and calls ttpa_sdpa_prefill's masked dense form, see tt_xla_amd/custom_ops.py.)
  * Physical block ids outside [0, num_blocks) are read as block 0.
  * `workspace` holds split-K partial results: at least
  * ttpa_paged_decode_workspace_bytes(...) bytes, 256-byte aligned, private to this
@@ -283,7 +286,7 @@ int ttpa_profile_next_attention(void *before, void *after);
  *   is *chunk_start (device int32, may be NULL = 0) in the paged form and 0 in the
  *   dense form (the library routine's top-left aligned causal mask).  `mask` (may be
  *   NULL, requires causal == 0) is an additive bf16 mask [batch, 1, q_len, kv_len]
- *   addressed by mask_batch_stride / mask_row_stride.
+ *   addressed by mask_batch_stride / mask_row_stride.  `scale` must be positive.
  */
 int ttpa_sdpa_prefill(void *out, int64_t out_batch_stride, int64_t out_head_stride,
                       int64_t out_token_stride, const void *q, int64_t q_batch_stride,

@@ -12,7 +12,9 @@ What pins each function (see tests/test_oracle_*.py):
   paged_fill_cache       brute-force per-token loop over the reference's grid
                          (test_custom_ops.py:171-203), tail block kept intact
   paged_sdpa_decode      fp32 textbook attention over the first cur_pos+1 gathered
-                         tokens; GQA form against the chunked op with a 1-token chunk
+                         tokens; GQA form against the chunked op with a 1-token chunk;
+                         the masked form (is_causal=False) against the causal one with the
+                         causal mask handed in, and against an fp32 loop with a random mask
   chunked_sdpa           the reference's independent oracle and cases restated
                          (tests/torch/ops/test_chunked_sdpa_op_cpu.py:27-147)
   sdpa                   library routine (F.scaled_dot_product_attention)
@@ -241,17 +243,53 @@ def paged_sdpa_decode(
 ) -> torch.Tensor:
     """Operator-level entry with the reference's argument list
     (custom_ops.py:1203-1223).  ``attention_sink`` and ``sliding_window_size`` are
-    accepted and ignored, as on the reference's CPU branch.  Only the causal form
-    (the one the plugin issues, attention.py:646-664) is restated.
+    accepted and ignored, as on the reference's CPU branch.
     """
     if is_causal:
         assert attn_mask is None, "attention_mask must be None when is_causal is True."
         assert cur_pos_tensor is not None, "cur_pos_tensor must be provided when is_causal is True."
     else:
-        raise NotImplementedError("oracle restates the causal decode form only")
+        return paged_sdpa_decode_masked(query, key, value, page_table, attn_mask, scale)
     if query.shape[2] == key.shape[1]:
         return paged_sdpa_decode_mha(query, key, value, page_table, cur_pos_tensor, scale)
     return paged_sdpa_decode_gqa(query, key, value, page_table, cur_pos_tensor, scale)
+
+
+def paged_sdpa_decode_masked(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    page_table: torch.Tensor,
+    attn_mask: torch.Tensor,
+    scale: Optional[float] = None,
+) -> torch.Tensor:
+    """The decode operator with ``is_causal=False``: every position of the user's table is
+    attended, with the caller's additive ``attn_mask`` [B, 1, 1, W*bs] in place of the causal one.
+
+    Hq == Hkv follows the reference's branch op by op (custom_ops.py:1263-1311: the same dense
+    gather as the causal form, then ``attn_mask`` where the causal mask would go, :1299-1303, every
+    intermediate in the query dtype).  Grouped heads follow the reference-held form that runs
+    them, as in ``paged_sdpa_decode_gqa`` (custom_ops.py:551-610 with the caller's mask).
+    """
+    bs, hkv, d = key.shape[-2], key.shape[-3], key.shape[-1]
+    users, hq = query.shape[1], query.shape[2]
+    span = page_table.shape[1] * bs
+    idx = page_table.long()
+    gk = key[idx].permute(0, 2, 1, 3, 4).reshape(users, hkv, span, d)
+    gv = value[idx].permute(0, 2, 1, 3, 4).reshape(users, hkv, span, value.shape[-1])
+    if scale is None:
+        scale = 1 / d**0.5
+    if hq == hkv:
+        q = query.reshape(users, hkv, 1, d)
+        w_ = q @ gk.to(query.dtype).transpose(-2, -1) * scale
+        w_ += attn_mask
+        w_ = torch.softmax(w_, dim=-1)
+        return (w_ @ gv.to(query.dtype)).reshape(1, users, hkv, d)
+    out = F.scaled_dot_product_attention(
+        query.reshape(users, hq, 1, d), gk, gv, attn_mask.to(query.dtype), is_causal=False, scale=scale,
+        enable_gqa=True,
+    )
+    return out.reshape(1, users, hq, value.shape[-1])
 
 
 # --------------------------------------------------------------------------- #

@@ -246,3 +246,51 @@ def test_decode_more_than_1024_users_on_the_matrix_core_kernel(bfp8):
     live = [u for u in range(users) if u not in (3, 700, 1299)]
     assert torch.isnan(got[0, [3, 700, 1299]]).all()
     _check(name, got[:, live], want[:, live])
+
+
+@pytest.mark.parametrize("hq,hkv,d,bs,bfp8", [(8, 8, 64, 32, False), (32, 8, 128, 64, False), (16, 4, 128, 32, True)])
+def test_decode_with_explicit_mask(hq, hkv, d, bs, bfp8):
+    """is_causal=False with an additive attn_mask [users, 1, 1, W*bs] (reference CPU branch
+    custom_ops.py:1299-1311; the one-token pass of an encoder / pooling model) against the
+    oracle's masked form: every position of the table is attended, weighted by the mask.  A
+    boolean mask means "attend where True"."""
+    from oracle import bfp8_codec as C
+    from tt_xla_amd import custom_ops as ops
+
+    g = torch.Generator().manual_seed(hq + d)
+    users, w = 3, 5
+    span = w * bs
+    nb = users * w + 1
+    key = torch.randn(nb, hkv, bs, d, generator=g).to(torch.bfloat16)
+    value = torch.randn(nb, hkv, bs, d, generator=g).to(torch.bfloat16)
+    table = (torch.randperm(nb - 1, generator=g) + 1).view(users, w).to(torch.int32)
+    q = torch.randn(1, users, hq, d, generator=g).to(torch.bfloat16)
+    cur = torch.tensor([3, 40, span - 1], dtype=torch.int32)
+    mask = torch.randn(users, 1, 1, span, generator=g).to(torch.bfloat16)
+    keep = torch.rand(users, 1, 1, span, generator=g) > 0.4
+    keep[:, :, :, 0] = True
+    mask = mask.masked_fill(~keep, float("-inf"))
+    name = f"masked decode h{hq}x{hkv} d{d} bs{bs} bfp8={bfp8}"
+    print(name, flush=True)
+    if bfp8:
+        kd, vd = ops.bfp8_pack_cache(key.cuda()), ops.bfp8_pack_cache(value.cuda())
+        key, value = C.unpack_cache(kd.cpu(), bs).to(torch.bfloat16), C.unpack_cache(vd.cpu(), bs).to(torch.bfloat16)
+    else:
+        kd, vd = key.cuda(), value.cuda()
+    got = torch.ops.tt.paged_scaled_dot_product_attention_decode(
+        q.cuda(), kd, vd, table.cuda(), is_causal=False, attn_mask=mask.cuda(), cur_pos_tensor=cur.cuda(),
+        scale=0.11).cpu()
+    want = O.paged_sdpa_decode(q.float(), key.float(), value.float(), table, False, mask.float(), cur, None, 0.11)
+    err = (got.float() - want).abs().max().item()
+    print(f"{name}: max-abs error {err:.3e}", flush=True)
+    torch.testing.assert_close(got.float(), want, atol=ATOL, rtol=RTOL)
+    got_b = torch.ops.tt.paged_scaled_dot_product_attention_decode(
+        q.cuda(), kd, vd, table.cuda(), is_causal=False, attn_mask=keep.cuda(), cur_pos_tensor=cur.cuda(),
+        scale=0.11).cpu()
+    want_b = O.paged_sdpa_decode(q.float(), key.float(), value.float(), table, False,
+                                 torch.zeros(users, 1, 1, span).masked_fill(~keep, float("-inf")), cur, None, 0.11)
+    torch.testing.assert_close(got_b.float(), want_b, atol=ATOL, rtol=RTOL)
+    with pytest.raises(NotImplementedError):  # a mask per head
+        torch.ops.tt.paged_scaled_dot_product_attention_decode(
+            q.cuda(), kd, vd, table.cuda(), is_causal=False, attn_mask=mask.expand(users, hq, 1, span).cuda(),
+            cur_pos_tensor=cur.cuda())

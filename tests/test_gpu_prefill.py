@@ -153,3 +153,37 @@ def test_chunked_start0_equals_dense_causal_on_filled_cache():
     bb = torch.ops.tt.scaled_dot_product_attention(q.cuda(), k.cuda(), v.cuda())
     torch.testing.assert_close(a.float(), bb.float(), atol=4e-3, rtol=4e-3)
     _check("filled-cache vs oracle", a.cpu(), O.sdpa(q, k, v))
+
+
+def test_inputs_the_kernels_cannot_take_are_refused():
+    """A boolean mask means "attend where True" (the library routine's rule); float16 / float32
+    keys and values, a float16 cache under attention and a scale that is not positive raise
+    instead of being reinterpreted."""
+    g = torch.Generator().manual_seed(9)
+    b, hq, hkv, s, d = 2, 8, 4, 64, 64
+    q = torch.randn(b, hq, s, d, generator=g).to(torch.bfloat16)
+    k = torch.randn(b, hkv, s, d, generator=g).to(torch.bfloat16)
+    v = torch.randn(b, hkv, s, d, generator=g).to(torch.bfloat16)
+    keep = torch.rand(b, 1, s, s, generator=g) > 0.5
+    keep[:, :, :, 0] = True
+    got = torch.ops.tt.scaled_dot_product_attention(q.cuda(), k.cuda(), v.cuda(), attn_mask=keep.cuda(),
+                                                    is_causal=False).cpu()
+    want = O.sdpa(q.float(), k.float(), v.float(), keep, False, None)
+    torch.testing.assert_close(got.float(), want, atol=2e-2, rtol=2e-2)
+    with pytest.raises(ValueError, match="bfloat16"):
+        torch.ops.tt.scaled_dot_product_attention(q.cuda(), k.cuda().half(), v.cuda().half())
+    with pytest.raises(ValueError, match="bfloat16"):
+        torch.ops.tt.scaled_dot_product_attention(q.cuda(), k.cuda().float(), v.cuda().float())
+    with pytest.raises(ValueError, match="positive"):
+        torch.ops.tt.scaled_dot_product_attention(q.cuda(), k.cuda(), v.cuda(), scale=0.0)
+    with pytest.raises(ValueError, match="positive"):
+        torch.ops.tt.scaled_dot_product_attention(q.cuda(), k.cuda(), v.cuda(), scale=-0.125)
+    cache = torch.zeros(4, hkv, 32, d, dtype=torch.float16, device="cuda")
+    table = torch.zeros(b, 2, dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError, match="bfloat16 or block-float-8"):
+        torch.ops.tt.chunked_scaled_dot_product_attention(q.cuda(), cache, cache, table,
+                                                          torch.zeros(1, dtype=torch.int32, device="cuda"))
+    with pytest.raises(ValueError, match="bfloat16 or block-float-8"):
+        torch.ops.tt.paged_scaled_dot_product_attention_decode(
+            torch.zeros(1, 1, hq, d, dtype=torch.bfloat16, device="cuda"), cache, cache,
+            table[:1], is_causal=True, cur_pos_tensor=torch.zeros(1, dtype=torch.int32, device="cuda"))

@@ -197,3 +197,34 @@ def test_dense_sdpa_rejects_bad_shapes():
         O.sdpa(q, k, k)  # heads not divisible
     with pytest.raises(AssertionError):
         O.sdpa(torch.randn(1, 4, 32, 64), k, k, attn_mask=torch.zeros(1, 1, 32, 32), is_causal=True)
+
+
+@pytest.mark.parametrize("hq,hkv", [(8, 8), (8, 2)])
+def test_decode_masked_form(hq, hkv):
+    """is_causal=False with a caller mask (reference custom_ops.py:1299-1303).  With the causal
+    mask handed in it is the causal operator; with a random mask of 0 / -inf / finite biases it is
+    softmax(q K^T scale + mask) V over ALL positions of the table, computed here by a plain loop."""
+    g = torch.Generator().manual_seed(hq + hkv)
+    users, bs, d, w = 3, 32, 64, 4
+    span = w * bs
+    key, value = _cache(users * w, hkv, bs, d, seed=50)
+    table = torch.randperm(users * w, generator=g).view(users, w).to(torch.int32)
+    q = torch.randn(1, users, hq, d, generator=g)
+    cur = torch.tensor([0, 77, span - 1], dtype=torch.int32)
+    causal_mask = torch.zeros(users, 1, 1, span)
+    for u in range(users):
+        causal_mask[u, :, :, int(cur[u]) + 1:] = float("-inf")
+    torch.testing.assert_close(O.paged_sdpa_decode(q, key, value, table, False, causal_mask, cur),
+                               O.paged_sdpa_decode(q, key, value, table, True, None, cur), atol=1e-6, rtol=1e-6)
+    mask = torch.randn(users, 1, 1, span, generator=g)
+    mask[torch.rand(users, 1, 1, span, generator=g) < 0.3] = float("-inf")
+    mask[:, :, :, 5] = 0.0  # no row is masked out entirely
+    got = O.paged_sdpa_decode(q, key, value, table, False, mask, cur, None, 0.21)
+    grp = hq // hkv
+    for u in range(users):
+        pos = torch.arange(span)
+        blk, off = table[u, pos // bs].long(), pos % bs
+        for h in range(hq):
+            k, v = key[blk, h // grp, off], value[blk, h // grp, off]
+            p = torch.softmax((k @ q[0, u, h]) * 0.21 + mask[u, 0, 0], dim=0)
+            torch.testing.assert_close(got[0, u, h], p @ v, atol=1e-5, rtol=1e-5)

@@ -643,6 +643,9 @@ static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_st
   if (head_size != 64 && head_size != 128 && head_size != 256)
     return fail(TTPA_ERR_UNSUPPORTED, "prefill: head_size %d; supported 64, 128, 256", head_size);
   TTPA_REQUIRE(!(mask && causal), "an additive mask excludes causal masking");
+  // the running maximum is tracked on raw scores and the mask is brought to their units by a
+  // division: both need a positive scale
+  TTPA_REQUIRE(scale > 0.f, "prefill: scale %g must be positive", (double)scale);
   if (page_table) {
     TTPA_REQUIRE(block_size > 0 && table_width > 0 && num_blocks > 0,
                  "paged form needs block_size, table_width and num_blocks");

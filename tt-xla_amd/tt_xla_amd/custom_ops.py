@@ -80,6 +80,14 @@ def _cache_geometry(cache: torch.Tensor):
     return nb, hkv, bs, d, fmt
 
 
+def _attention_cache_geometry(cache: torch.Tensor):
+    """``_cache_geometry`` for the attention operators, which read the elements as numbers: a
+    bfloat16 or block-float-8 cache (the cache writers also move float16 caches: pure copies)."""
+    if cache.dtype not in (torch.bfloat16, torch.uint8):
+        raise ValueError(f"attention reads bfloat16 or block-float-8 (uint8) caches, got {cache.dtype}")
+    return _cache_geometry(cache)
+
+
 def bfp8_cache_shape(num_blocks: int, num_kv_heads: int, block_size: int, head_size: int):
     """Shape of the uint8 tensor that stores a block-float-8 cache."""
     assert block_size % _BFP8_GROUP == 0 and head_size % _BFP8_GROUP == 0
@@ -346,17 +354,17 @@ def _decode(query, key, value, page_table, is_causal, attn_mask, cur_pos_tensor,
         assert cur_pos_tensor is not None, "cur_pos_tensor must be provided when is_causal is True."
     if attn_mask is not None:
         assert not is_causal, "attention_mask must be None when is_causal is True."
-    if not is_causal:
-        raise NotImplementedError(
-            "paged decode with an explicit attn_mask is not built; the serving path always "
-            "issues the causal form"
-        )
     if sliding_window_size is not None and sliding_window_size <= 0:
         raise ValueError("sliding_window_size must be positive")
     if query.dim() != 4 or query.shape[0] != 1:
         raise ValueError("query must be [1, users, heads, head_size]")
-    nb, hkv, bs, d, fmt = _cache_geometry(key)
-    if _cache_geometry(value) != (nb, hkv, bs, d, fmt):
+    if not is_causal:
+        if k_new is not None:
+            raise ValueError("the fused update + decode step is causal")
+        return _decode_masked(query, key, value, page_table, attn_mask, attention_sink, scale,
+                              sliding_window_size, out)
+    nb, hkv, bs, d, fmt = _attention_cache_geometry(key)
+    if _attention_cache_geometry(value) != (nb, hkv, bs, d, fmt):
         raise ValueError("key and value caches must have the same shape and dtype")
     _, users, hq, qd = query.shape
     if qd != d or hq % hkv:
@@ -409,6 +417,57 @@ def _decode(query, key, value, page_table, is_causal, attn_mask, cur_pos_tensor,
         sink.data_ptr() if sink is not None else None, ws.data_ptr(), ws_bytes, _stream(),
     )
     return out
+
+
+def _decode_masked(query, key, value, page_table, attn_mask, attention_sink, scale, sliding_window_size, out):
+    """Decode with ``is_causal=False``: every position of the user's table is attended, weighted by
+    the additive ``attn_mask`` [users, 1, 1, table_width * block_size] (reference CPU branch
+    custom_ops.py:1296-1311; the one-token pass of a pooling / encoder model, never the
+    generative serving path).  Runs on the prefill kernel's masked dense form: the user's blocks
+    are gathered in table order (block-float-8 ones dequantised on the way) and the query token
+    is the first row of a 32-row tile.  A mask that differs between heads is not built."""
+    if attn_mask is None:
+        raise ValueError("attn_mask must be provided when is_causal is False")
+    if attention_sink is not None or sliding_window_size is not None:
+        raise NotImplementedError("attention_sink / sliding_window_size with an explicit attn_mask are not built")
+    nb, hkv, bs, d, fmt = _attention_cache_geometry(key)
+    if _attention_cache_geometry(value) != (nb, hkv, bs, d, fmt):
+        raise ValueError("key and value caches must have the same shape and dtype")
+    _, users, hq, qd = query.shape
+    if qd != d or hq % hkv or query.dtype != torch.bfloat16:
+        raise ValueError(f"query {tuple(query.shape)} {query.dtype} does not match the cache geometry")
+    width = page_table.shape[1]
+    skv = width * bs
+    if attn_mask.dim() != 4 or attn_mask.shape[0] != users or attn_mask.shape[2] != 1 or attn_mask.shape[3] != skv:
+        raise ValueError(f"attn_mask must be [users, 1, 1, {skv}], got {tuple(attn_mask.shape)}")
+    if attn_mask.shape[1] != 1:
+        raise NotImplementedError("a decode attn_mask that differs between heads is not built")
+
+    def dense(cache):
+        g = torch.index_select(cache, 0, page_table.reshape(-1).to(torch.int64))
+        if fmt == N.KV_BFP8:
+            g = bfp8_unpack_cache(g)
+        return g.view(users, width, hkv, bs, d).permute(0, 2, 1, 3, 4).reshape(users, hkv, skv, d)
+
+    rows = 32  # the prefill kernel's query tile
+    q = torch.zeros((users, hq, rows, d), dtype=torch.bfloat16, device=query.device)
+    q[:, :, 0] = query[0]
+    mask = _additive_mask(attn_mask).expand(users, 1, rows, skv).contiguous()
+    res = _prefill(q, dense(key), dense(value), None, None, mask, False, scale)[:, :, 0]  # [users, hq, d]
+    if out is None:
+        return res.unsqueeze(0).contiguous()
+    _check_out(out, (1, users, hq, d), "decode")
+    out[0].copy_(res)
+    return out
+
+
+def _additive_mask(attn_mask: torch.Tensor) -> torch.Tensor:
+    """The mask as the kernels add it to the scaled scores: bfloat16.  A boolean mask means
+    "attend where True" (torch.nn.functional.scaled_dot_product_attention's rule)."""
+    if attn_mask.dtype == torch.bool:
+        return torch.zeros(attn_mask.shape, dtype=torch.bfloat16, device=attn_mask.device).masked_fill(
+            ~attn_mask, float("-inf"))
+    return attn_mask if attn_mask.dtype == torch.bfloat16 else attn_mask.to(torch.bfloat16)
 
 
 @torch.library.custom_op("tt::paged_update_kv_decode_", mutates_args=["k_cache", "v_cache"],
@@ -487,7 +546,11 @@ def _prefill(query, key, value, page_table, chunk_start, attn_mask, is_causal, s
         _check_out(out, (b, hq, s, d), "prefill")
     if scale is None:
         scale = 1.0 / math.sqrt(d)
+    if not scale > 0:
+        raise ValueError(f"scale must be positive, got {scale}")
     if page_table is None:
+        if key.dtype != torch.bfloat16 or value.dtype != torch.bfloat16:
+            raise ValueError(f"key and value must be bfloat16, got {key.dtype} and {value.dtype}")
         hkv, skv = key.shape[1], key.shape[2]
         k = _rows_contiguous(key)
         v = _rows_contiguous(value)
@@ -497,8 +560,8 @@ def _prefill(query, key, value, page_table, chunk_start, attn_mask, is_causal, s
         bs = w = nb = 0
         pt_ptr, pt_rs = 0, 0
     else:
-        nb, hkv, bs, kd, fmt = _cache_geometry(key)
-        if fmt != N.KV_BF16 or _cache_geometry(value) != (nb, hkv, bs, kd, fmt) or kd != d:
+        nb, hkv, bs, kd, fmt = _attention_cache_geometry(key)
+        if fmt != N.KV_BF16 or _attention_cache_geometry(value) != (nb, hkv, bs, kd, fmt) or kd != d:
             raise ValueError("chunked attention needs matching bfloat16 K/V caches")
         k, v = key, value
         pt = _table(page_table)
@@ -508,9 +571,7 @@ def _prefill(query, key, value, page_table, chunk_start, attn_mask, is_causal, s
         pt_ptr, pt_rs = pt.data_ptr(), pt.stride(0)
     mask_ptr, mask_bs, mask_rs = 0, 0, 0
     if attn_mask is not None:
-        m = attn_mask
-        if m.dtype != torch.bfloat16:
-            m = m.to(torch.bfloat16)
+        m = _additive_mask(attn_mask)
         if m.dim() != 4 or m.shape[1] != 1 or m.shape[2] != s or m.shape[3] != skv:
             raise ValueError("attn_mask must be [batch, 1, q_len, kv_len]")
         if m.stride(-1) != 1:
