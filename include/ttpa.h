@@ -321,6 +321,28 @@ int ttpa_sdpa_prefill_windowed(void *out, int64_t out_batch_stride, int64_t out_
                                int32_t sliding_window, void *stream);
 
 /*
+ * ttpa_sdpa_prefill_windowed with the cache format as an argument: kv_format = TTPA_KV_BFP8
+ * (paged form only; block_size a multiple of 16) reads block-float-8 caches, expanding the
+ * element bytes to bfloat16 (exactly) on their way into LDS.  This is what
+ * tt::chunked_scaled_dot_product_attention runs when the plugin's
+ * experimental_kv_cache_dtype="bfp_bf8" option is on (vllm_tt/platform.py:165, 232-233; the
+ * reference's own test of the option is a chunked prefill,
+ * tests/integrations/vllm_plugin/generative/test_chunked_prefill.py:86-96).
+ * kv_format = TTPA_KV_BF16 is ttpa_sdpa_prefill_windowed.
+ */
+int ttpa_sdpa_prefill_format(void *out, int64_t out_batch_stride, int64_t out_head_stride,
+                             int64_t out_token_stride, const void *q, int64_t q_batch_stride,
+                             int64_t q_head_stride, int64_t q_token_stride, const void *k,
+                             const void *v, int64_t kv_batch_stride, int64_t kv_head_stride,
+                             int64_t kv_token_stride, const int32_t *page_table,
+                             int64_t page_table_row_stride, const int32_t *chunk_start,
+                             const void *mask, int64_t mask_batch_stride, int64_t mask_row_stride,
+                             int32_t batch, int32_t q_heads, int32_t kv_heads, int32_t q_len,
+                             int32_t kv_len, int32_t head_size, int32_t block_size,
+                             int32_t table_width, int32_t num_blocks, int32_t causal, float scale,
+                             int32_t sliding_window, int32_t kv_format, void *stream);
+
+/*
  * The backend's first-chunk prefill pass in one call: ttpa_paged_fill_cache on K and on V
  * (attention.py:486-515: the prompt's keys and values go into the paged caches through the
  * fill page table) and the dense-form ttpa_sdpa_prefill_windowed on the same k / v

@@ -251,3 +251,120 @@ def test_config5_full_size():
     out_q, _, _ = step(g.q, g.k_new, (g.v_new.float() * 0.25).to(torch.bfloat16), vp_q, g.page_table,
                        g.cache_position)
     torch.testing.assert_close(out_q.float() * 4, out.float(), atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("users,hq,hkv,d,bs,nbpu,start,lc", [
+    (2, 32, 8, 128, 32, 8, 128, 64),     # the serving default block size, a continuation chunk
+    (2, 8, 8, 64, 16, 12, 0, 96),        # first chunk through the paged operator, blocks of 16
+    (1, 16, 4, 128, 64, 6, 200, 128),    # a prefix that ends inside a block
+    (2, 8, 2, 256, 32, 6, 64, 64),       # head size 256
+    (3, 12, 4, 128, 48, 4, 100, 32),     # a block size that is no power of two
+])
+def test_chunked_prefill_over_a_bfp8_cache(users, hq, hkv, d, bs, nbpu, start, lc):
+    """tt::chunked_scaled_dot_product_attention on block-float-8 caches (the reference's one test
+    of the option is a chunked prefill, generative/test_chunked_prefill.py:86-96): against the
+    oracle's chunked operator on the codec round trip of the same caches."""
+    from tt_xla_amd import custom_ops as ops
+
+    g = torch.Generator().manual_seed(users + hq + d + bs)
+    nb = users * nbpu + 1
+    key = torch.randn(nb, hkv, bs, d, generator=g).to(torch.bfloat16)
+    value = torch.randn(nb, hkv, bs, d, generator=g).to(torch.bfloat16)
+    key[:, :, :, 5] *= 20   # an outlier channel
+    table = (torch.randperm(nb - 1, generator=g) + 1).view(users, nbpu).to(torch.int32)
+    q = (torch.randn(users, hq, lc, d, generator=g) * 0.5).to(torch.bfloat16)
+    cs = torch.tensor([start], dtype=torch.int32)
+    kp, vp = ops.bfp8_pack_cache(key.cuda()), ops.bfp8_pack_cache(value.cuda())
+    name = f"bfp8 chunked b{users} h{hq}x{hkv} d{d} bs{bs} start{start} lc{lc}"
+    print(name, flush=True)
+    got = torch.ops.tt.chunked_scaled_dot_product_attention(q.cuda(), kp, vp, table.cuda(), cs.cuda()).cpu()
+    k_rt = C.unpack_cache(kp.cpu(), bs).to(torch.bfloat16)
+    v_rt = C.unpack_cache(vp.cpu(), bs).to(torch.bfloat16)
+    want = O.chunked_sdpa(q.float(), k_rt.float(), v_rt.float(), table, cs, None)
+    err = (got.float() - want).abs().max().item()
+    print(f"{name}: max-abs error {err:.3e}", flush=True)
+    torch.testing.assert_close(got.float(), want, atol=2e-2, rtol=2e-2)
+
+
+def test_backend_flow_on_a_bfp8_cache():
+    """First chunk -> continuation chunk -> decode step through TTAttentionBackendImpl.forward on
+    uint8 block-float-8 caches (the flow of the reference's test of the option,
+    tests/integrations/vllm_plugin/generative/test_chunked_prefill.py:69-136): the caches after
+    every pass equal the quantised oracle writes bit for bit, and every output is within
+    atol = rtol = 2e-2 of the oracle's operator on the codec round trip of those caches."""
+    from tt_xla_amd import TTAttentionBackend, TTAttentionBackendImpl, TTMetadata
+    from tt_xla_amd import custom_ops as ops
+
+    hq, hkv, d, bs = 32, 8, 128, 32
+    users, width, s1, s2 = 2, 8, 128, 64
+    g = torch.Generator().manual_seed(21)
+    nb = users * width + 1
+    assert TTAttentionBackend.get_kv_cache_storage_shape(nb, bs, hkv, d, "bfp_bf8") == (nb, hkv, bs + bs // 16, d)
+    assert TTAttentionBackend.get_kv_cache_storage_shape(nb, bs, hkv, d) == (nb, hkv, bs, d)
+    table = (torch.randperm(nb - 1, generator=g) + 1).view(users, width).to(torch.int32)
+    kv = [ops.bfp8_empty_cache(nb, hkv, bs, d, "cuda"), ops.bfp8_empty_cache(nb, hkv, bs, d, "cuda")]
+    kc_ref = torch.zeros(nb, hkv, bs, d, dtype=torch.bfloat16)   # what the caches decode to
+    vc_ref = torch.zeros(nb, hkv, bs, d, dtype=torch.bfloat16)
+    impl = TTAttentionBackendImpl(hq, d, d**-0.5, hkv, None, None, "uint8")
+    bidx = torch.arange(users, dtype=torch.int32)
+    bf = lambda *shape: torch.randn(*shape, generator=g).to(torch.bfloat16)  # noqa: E731
+    rt = lambda t: C.roundtrip(t).to(torch.bfloat16)  # noqa: E731
+
+    def caches_match():
+        assert torch.equal(kv[0].cpu(), C.pack_cache(kc_ref)) and torch.equal(kv[1].cpu(), C.pack_cache(vc_ref))
+
+    # first chunk: quantising fills from column 0, dense causal attention on the fresh K / V
+    q1, k1, v1 = bf(users * s1, hq * d), bf(users * s1, hkv * d), bf(users * s1, hkv * d)
+    md = TTMetadata(cache_position=None, page_table=table.cuda(), num_users=users, batch_idx=bidx.cuda())
+    out1 = torch.empty(users * s1, hq * d, dtype=torch.bfloat16, device="cuda")
+    impl.forward(None, q1.cuda(), k1.cuda(), v1.cuda(), kv, md, output=out1)
+    k4, v4 = k1.view(users, s1, hkv, d).transpose(1, 2), v1.view(users, s1, hkv, d).transpose(1, 2)
+    kc_ref = rt(O.paged_fill_cache_batched(kc_ref, k4, table, bidx))
+    vc_ref = rt(O.paged_fill_cache_batched(vc_ref, v4, table, bidx))
+    caches_match()
+    want1 = O.sdpa(q1.view(users, s1, hq, d).transpose(1, 2), k4, v4, None, True, d**-0.5)
+    torch.testing.assert_close(out1.cpu().float(), want1.transpose(1, 2).reshape(users * s1, hq * d).float(),
+                               atol=2e-2, rtol=2e-2)
+
+    # continuation chunk: fill table rolled by the computed blocks, chunked attention over the cache
+    q2, k2, v2 = bf(users * s2, hq * d), bf(users * s2, hkv * d), bf(users * s2, hkv * d)
+    fill_table = torch.roll(table, -(s1 // bs), dims=1)
+    start = torch.tensor([s1], dtype=torch.int32)
+    md = TTMetadata(cache_position=None, page_table=table.cuda(), num_users=users, batch_idx=bidx.cuda(),
+                    fill_page_table=fill_table.cuda(), chunk_start_idx=start.cuda())
+    out2 = torch.empty(users * s2, hq * d, dtype=torch.bfloat16, device="cuda")
+    impl.forward(None, q2.cuda(), k2.cuda(), v2.cuda(), kv, md, output=out2)
+    kc_ref = rt(O.paged_fill_cache_batched(kc_ref, k2.view(users, s2, hkv, d).transpose(1, 2), fill_table, bidx))
+    vc_ref = rt(O.paged_fill_cache_batched(vc_ref, v2.view(users, s2, hkv, d).transpose(1, 2), fill_table, bidx))
+    caches_match()
+    want2 = O.chunked_sdpa(q2.view(users, s2, hq, d).transpose(1, 2).float(), kc_ref.float(), vc_ref.float(),
+                           table, start, d**-0.5)
+    torch.testing.assert_close(out2.cpu().float(), want2.transpose(1, 2).reshape(users * s2, hq * d),
+                               atol=2e-2, rtol=2e-2)
+
+    # one decode token on top
+    pos = torch.full((users,), s1 + s2, dtype=torch.int32)
+    q3, k3, v3 = bf(users, hq * d), bf(users, hkv * d), bf(users, hkv * d)
+    md = TTMetadata(cache_position=pos.cuda(), page_table=table.cuda(), num_users=users)
+    out3 = torch.empty(users, hq * d, dtype=torch.bfloat16, device="cuda")
+    impl.forward(None, q3.cuda(), k3.cuda(), v3.cuda(), kv, md, output=out3)
+    kc_ref = rt(O.paged_update_cache(kc_ref, k3.view(users, 1, hkv, d).transpose(0, 1), pos, table))
+    vc_ref = rt(O.paged_update_cache(vc_ref, v3.view(users, 1, hkv, d).transpose(0, 1), pos, table))
+    caches_match()
+    want3 = O.textbook_decode_fp32(q3.view(users, 1, hq, d).transpose(0, 1), kc_ref, vc_ref, table, pos, d**-0.5)
+    torch.testing.assert_close(out3.cpu().float(), want3.transpose(0, 1).reshape(users, hq * d),
+                               atol=2e-2, rtol=2e-2)
+
+    # a KV-shared layer's prefill gathers (and dequantises) the same caches
+    shared = TTAttentionBackendImpl(hq, d, d**-0.5, hkv, None, None, "uint8", kv_sharing_target_layer_name="l0")
+    s = s1 + s2
+    q4 = bf(users * 64, hq * d)
+    md = TTMetadata(cache_position=None, page_table=table.cuda(), num_users=users, batch_idx=bidx.cuda())
+    out4 = torch.empty(users * 64, hq * d, dtype=torch.bfloat16, device="cuda")
+    shared.forward(None, q4.cuda(), k2.cuda(), v2.cuda(), kv, md, output=out4)
+    caches_match()
+    k_d = O.gather_paged_to_dense(kc_ref, table)[:, :, :64]
+    v_d = O.gather_paged_to_dense(vc_ref, table)[:, :, :64]
+    want4 = O.sdpa(q4.view(users, 64, hq, d).transpose(1, 2), k_d, v_d, None, True, d**-0.5)
+    torch.testing.assert_close(out4.cpu().float(), want4.transpose(1, 2).reshape(users * 64, hq * d).float(),
+                               atol=2e-2, rtol=2e-2)

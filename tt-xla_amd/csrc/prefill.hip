@@ -69,6 +69,7 @@ struct PrefillArgs {
   int fill_groups, attn_per_fill, n_fill;
   int window;  // > 0 (causal only): row i attends keys offset + i - window < j <= offset + i
   float scale_log2e;
+  int kv_bfp8;  // paged form: the caches are block-float-8 (mode 4)
 };
 
 // key / block_size without a division instruction sequence (about 30 instructions each, and the
@@ -155,7 +156,12 @@ __device__ __forceinline__ void fill_workgroup(const PrefillArgs &a, int f) {
 // MODE 0: dense K/V; 1: paged, block_size a multiple of 64 (a tile lies in one block);
 // 3: paged, block_size a multiple of the rows one wavefront load covers (1 KiB: 8 / 4 / 2 rows
 // for head sizes 64 / 128 / 256): one wavefront-uniform table lookup per load; 2: paged, any
-// block size (per-lane table lookups).
+// block size (per-lane table lookups); 4: paged block-float-8 caches (block_size a multiple of
+// 16).  In mode 4 a tile goes global -> registers -> LDS: a thread fetches groups of 16 element
+// bytes with their exponent byte (D / 64 groups per tile and tensor) where the other modes issue
+// their LDS-DMA loads, and expands them to bfloat16 (exact: a 7-bit magnitude times a power of
+// two) into the same swizzled tile layout at the end of the iteration, one tile period before
+// the tile is used.  One workgroup per CU: the staging registers do not fit next to a second one.
 //
 // Per-tile schedule of a workgroup (LDS holds two K stages and two V stages):
 //   S^T = K(t) Q^T | barrier | issue loads of K(t+2) and V(t+1) | softmax | O^T += V(t)^T P^T
@@ -165,7 +171,7 @@ __device__ __forceinline__ void fill_workgroup(const PrefillArgs &a, int f) {
 // barrier too.  LDS operand reads run a few fragments ahead of the matrix instructions that
 // consume them.
 template <int D, int HPW, int MODE>
-__global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(PrefillArgs a) {
+__global__ __launch_bounds__(256, (D <= 128 && MODE != 4 ? 2 : 1)) void prefill_kernel(PrefillArgs a) {
   constexpr int RPW = 4 / HPW;            // wavefront row slots per workgroup
   constexpr int ROWS = kRowsPerWave;      // query rows per wavefront
   constexpr int KSTEPS = D / 16;          // MFMA k-steps over the head dimension
@@ -260,7 +266,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
   // last row, whose scores are masked and whose V rows therefore carry weight 0.
   // Modes 1 and 3 look their blocks up one tile ahead of the loads (below): NLK wavefront-
   // uniform table entries per tile, one for the whole tile or one per load of this wavefront.
-  constexpr int NLK = MODE == 1 ? 1 : (MODE == 3 ? T::NI : 0);
+  constexpr int GPR = D / 16;           // mode 4: 16-element groups (= exponent bytes) per row
+  constexpr int NG = D / 64;            // mode 4: groups per thread, tile and tensor
+  constexpr int NLK = MODE == 1 ? 1 : (MODE == 3 ? T::NI : (MODE == 4 ? NG : 0));
   struct Blocks {
     int phys[NLK > 0 ? NLK : 1];
   };
@@ -268,6 +276,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
   auto lookup_key = [&](int kt, int j) {
     const int key0 = kt * kKeysPerTile;
     if constexpr (MODE == 1) return key0;
+    if constexpr (MODE == 4) return key0 + min((tid + 256 * j) / GPR, a.skv - 1 - key0);  // per lane
     // the rows of a load sit in one block; a load wholly past the last key reads the rows that
     // hold the last key again (readable, and masked like any key past the end)
     return key0 + min((4 * j + wave) * T::RPI, (a.skv - 1 - key0) / T::RPI * T::RPI);
@@ -313,6 +322,54 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
     } else {
 #pragma unroll
       for (int j = 0; j < T::NI; ++j) dma16(base, ld[j], lds_dst(j));
+    }
+  };
+  // ---- mode 4: block-float-8 tiles through registers --------------------------------------
+  struct Staged {
+    u32x4 bytes[MODE == 4 ? NG : 1];
+    uint32_t ex[MODE == 4 ? NG : 1];
+  };
+  // group j of this thread: row (tid + 256 j) / GPR of the tile, 16 elements from 16 ((tid + 256 j) % GPR)
+  auto fetch_bfp8 = [&](const uint16_t *cache, int kt, const Blocks &blk) {
+    Staged st = {};
+    if constexpr (MODE == 4) {
+      const uint8_t *base = reinterpret_cast<const uint8_t *>(cache);
+      const int64_t slab = (int64_t)(a.bs + a.bs / 16) * D;
+#pragma unroll
+      for (int j = 0; j < NG; ++j) {
+        const int key = lookup_key(kt, j), c16 = (tid + 256 * j) % GPR;
+        const int rowin = key - div_block(a, key) * a.bs;
+        const uint8_t *sl = base + ((int64_t)blk.phys[j] * a.hkv + hk) * slab;
+        st.bytes[j] = *reinterpret_cast<const u32x4 *>(sl + rowin * D + 16 * c16);
+        st.ex[j] = sl[(int64_t)a.bs * D + rowin * GPR + c16];
+      }
+    }
+    return st;
+  };
+  // (b - 128) * 2^(e - 133) for the 16 bytes of a group, as 8 bfloat16 pairs; LDS chunks
+  // 2 c16 and 2 c16 + 1 of the row, at their swizzled positions
+  auto commit_bfp8 = [&](const Staged &st, bool is_v, int buf) {
+    if constexpr (MODE == 4) {
+      unsigned char *tile_base = smem + buf * T::STAGE_BYTES + (is_v ? T::TILE_BYTES : 0);
+#pragma unroll
+      for (int j = 0; j < NG; ++j) {
+        const int row = (tid + 256 * j) / GPR, c16 = (tid + 256 * j) % GPR;
+        const float sc = bfp8_group_scale(st.ex[j]), off = -128.f * sc;
+        uint32_t o[8];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t x = st.bytes[j][w];
+          const float f0 = fmaf((float)(x & 0xffu), sc, off), f1 = fmaf((float)((x >> 8) & 0xffu), sc, off);
+          const float f2 = fmaf((float)((x >> 16) & 0xffu), sc, off), f3 = fmaf((float)(x >> 24), sc, off);
+          // the products are exact in bfloat16: their upper halves are the elements
+          o[2 * w] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f1), __builtin_bit_cast(uint32_t, f0), 0x07060302u);
+          o[2 * w + 1] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f3), __builtin_bit_cast(uint32_t, f2), 0x07060302u);
+        }
+        const int sw = is_v ? T::swz_v(row) : T::swz_k(row);
+        unsigned char *rp = tile_base + row * T::RB;
+        *reinterpret_cast<uint4 *>(rp + 16 * ((2 * c16) ^ sw)) = make_uint4(o[0], o[1], o[2], o[3]);
+        *reinterpret_cast<uint4 *>(rp + 16 * ((2 * c16 + 1) ^ sw)) = make_uint4(o[4], o[5], o[6], o[7]);
+      }
     }
   };
   auto wait_loads_and_sync = [&]() {
@@ -388,7 +445,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
     if constexpr (NLK > 0) {
 #pragma unroll
       for (int j = 0; j < NLK; ++j) {
-        const int p = __builtin_amdgcn_readfirstlane(r.raw[j]);
+        const int p = MODE == 4 ? r.raw[j] : __builtin_amdgcn_readfirstlane(r.raw[j]);  // mode 4: per lane
         blk.phys[j] = (unsigned)p >= (unsigned)a.nb ? 0 : p;
       }
     }
@@ -397,9 +454,16 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
   Blocks blk_v = resolve(request(first_tile));     // blocks of the tile whose V is loaded next
   Blocks blk_k = resolve(request(first_tile + 1));  // ... whose K is loaded next
   Requested req = request(first_tile + 2);
-  issue(a.k, ld_k, false, first_tile, first_tile & 1, blk_v);
-  issue(a.v, ld_v, true, first_tile, first_tile & 1, blk_v);
-  if (last_tile >= first_tile + 1) issue(a.k, ld_k, false, first_tile + 1, (first_tile + 1) & 1, blk_k);
+  if constexpr (MODE == 4) {
+    commit_bfp8(fetch_bfp8(a.k, first_tile, blk_v), false, first_tile & 1);
+    commit_bfp8(fetch_bfp8(a.v, first_tile, blk_v), true, first_tile & 1);
+    if (last_tile >= first_tile + 1)
+      commit_bfp8(fetch_bfp8(a.k, first_tile + 1, blk_k), false, (first_tile + 1) & 1);
+  } else {
+    issue(a.k, ld_k, false, first_tile, first_tile & 1, blk_v);
+    issue(a.v, ld_v, true, first_tile, first_tile & 1, blk_v);
+    if (last_tile >= first_tile + 1) issue(a.k, ld_k, false, first_tile + 1, (first_tile + 1) & 1, blk_k);
+  }
   blk_v = blk_k;
   wait_loads_and_sync();
   // The first K fragments of a tile are read one tile ahead (K(t+1) has landed at the barrier
@@ -435,8 +499,14 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
     // K(kt+1) and V(kt) have landed for everyone; everyone is done with K(kt) and V(kt-1)
     wait_loads_and_sync();
     blk_k = resolve(req);  // blocks of tile kt + 2; blk_v holds those of tile kt + 1
-    if (kt + 2 <= last_tile) issue(a.k, ld_k, false, kt + 2, kt & 1, blk_k);
-    if (kt + 1 <= last_tile) issue(a.v, ld_v, true, kt + 1, (kt + 1) & 1, blk_v);
+    Staged k_staged = {}, v_staged = {};
+    if constexpr (MODE == 4) {
+      if (kt + 2 <= last_tile) k_staged = fetch_bfp8(a.k, kt + 2, blk_k);
+      if (kt + 1 <= last_tile) v_staged = fetch_bfp8(a.v, kt + 1, blk_v);
+    } else {
+      if (kt + 2 <= last_tile) issue(a.k, ld_k, false, kt + 2, kt & 1, blk_k);
+      if (kt + 1 <= last_tile) issue(a.v, ld_v, true, kt + 1, (kt + 1) & 1, blk_v);
+    }
     blk_v = blk_k;
     req = request(kt + 3);
 
@@ -531,6 +601,12 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void prefill_kernel(Prefil
         if (j + VPRE < NV) vring[j % VPRE] = read_v(cur, j + VPRE);
       }
     }
+    if constexpr (MODE == 4) {
+      // K(kt+2) takes the place of K(kt), V(kt+1) that of V(kt-1): nobody reads either any more
+      // (the barrier above), and the next barrier publishes what is written here
+      if (kt + 2 <= last_tile) commit_bfp8(k_staged, false, kt & 1);
+      if (kt + 1 <= last_tile) commit_bfp8(v_staged, true, (kt + 1) & 1);
+    }
     if (wave_active && kt + 1 < ntiles && key0 + kKeysPerTile <= wave_last_key &&
         key0 + 2 * kKeysPerTile > wave_first_key) {  // this wavefront computes tile kt + 1
       const unsigned char *nxt = smem + ((kt + 1) & 1) * T::STAGE_BYTES;
@@ -594,6 +670,7 @@ int launch_mode(const PrefillArgs &a, hipStream_t st) {
 template <int D, int HPW>
 int launch(const PrefillArgs &a, hipStream_t st) {
   if (!a.pt) return launch_mode<D, HPW, 0>(a, st);
+  if (a.kv_bfp8) return launch_mode<D, HPW, 4>(a, st);
   if (a.bs % kKeysPerTile == 0) return launch_mode<D, HPW, 1>(a, st);
   if (a.bs % Tile<D>::RPI == 0) return launch_mode<D, HPW, 3>(a, st);
   return launch_mode<D, HPW, 2>(a, st);
@@ -632,7 +709,7 @@ static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_st
                                  int32_t kv_heads, int32_t q_len, int32_t kv_len, int32_t head_size,
                                  int32_t block_size, int32_t table_width, int32_t num_blocks,
                                  int32_t causal, float scale, int32_t sliding_window, void *stream,
-                                 const FillSpec *fill = nullptr) {
+                                 const FillSpec *fill = nullptr, int32_t kv_format = TTPA_KV_BF16) {
   TTPA_REQUIRE(out && q && k && v, "null pointer argument");
   TTPA_REQUIRE(sliding_window >= 0, "prefill: sliding_window %d is negative", sliding_window);
   TTPA_REQUIRE(sliding_window == 0 || causal, "prefill: a sliding window needs causal masking");
@@ -681,6 +758,14 @@ static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_st
   a.bs = block_size, a.w = table_width, a.nb = num_blocks, a.causal = causal ? 1 : 0;
   a.window = sliding_window;
   a.scale_log2e = scale * 1.4426950408889634f;
+  if (kv_format != TTPA_KV_BF16 && kv_format != TTPA_KV_BFP8)
+    return fail(TTPA_ERR_INVALID_ARGUMENT, "prefill: unknown kv_format %d", kv_format);
+  a.kv_bfp8 = kv_format == TTPA_KV_BFP8;
+  if (a.kv_bfp8) {
+    TTPA_REQUIRE(page_table != nullptr, "prefill: a block-float-8 K / V is a paged cache");
+    if (block_size % 16)
+      return fail(TTPA_ERR_UNSUPPORTED, "prefill: a block-float-8 cache needs block_size %% 16 == 0");
+  }
   a.bs_magic = block_size >= 2 ? (uint32_t)((1ull << 32) / (uint32_t)block_size) + 1u : 0u;
   a.fill_kc = a.fill_vc = nullptr;
   a.fill_pt = nullptr, a.fill_pt_rs = 0, a.fill_bidx = nullptr, a.fill_bidx_i64 = 0, a.fill_rows = 0;
@@ -720,6 +805,11 @@ extern "C" int ttpa_sdpa_prefill(TTPA_PREFILL_PARAMS, void *stream) {
 
 extern "C" int ttpa_sdpa_prefill_windowed(TTPA_PREFILL_PARAMS, int32_t sliding_window, void *stream) {
   return prefill_impl(TTPA_PREFILL_ARGS, sliding_window, stream);
+}
+
+extern "C" int ttpa_sdpa_prefill_format(TTPA_PREFILL_PARAMS, int32_t sliding_window, int32_t kv_format,
+                                        void *stream) {
+  return prefill_impl(TTPA_PREFILL_ARGS, sliding_window, stream, nullptr, kv_format);
 }
 
 extern "C" int ttpa_sdpa_prefill_fill(

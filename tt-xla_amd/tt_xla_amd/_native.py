@@ -84,6 +84,11 @@ SIGNATURES = {
         [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _i64, _p, _p,
          _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _p],
     ),
+    "ttpa_sdpa_prefill_format": (
+        _int,
+        [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _i64, _p, _p,
+         _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _p],
+    ),
     "ttpa_sdpa_prefill_fill": (
         _int,
         [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64,

@@ -147,6 +147,23 @@ class TTAttentionBackend(_BackendBase):
         return (num_blocks, num_kv_heads, block_size, head_size)
 
     @staticmethod
+    def get_kv_cache_storage_shape(
+        num_blocks: int,
+        block_size: int,
+        num_kv_heads: int,
+        head_size: int,
+        cache_dtype_str: str = "auto",
+    ) -> tuple:
+        """Shape of the tensor that actually holds one cache.  As ``get_kv_cache_shape`` except
+        under the block-float-8 option (``experimental_kv_cache_dtype="bfp_bf8"``, reference
+        vllm_tt/platform.py:165, 232-233, where the reference keeps the logical shape and its
+        compiler picks the layout): a uint8 tensor with block_size / 16 more rows per block for
+        the shared exponents (``custom_ops.bfp8_cache_shape``)."""
+        if cache_dtype_str.lower().strip() in ("bfp_bf8", "bfp8"):
+            return custom_ops.bfp8_cache_shape(num_blocks, num_kv_heads, block_size, head_size)
+        return (num_blocks, num_kv_heads, block_size, head_size)
+
+    @staticmethod
     def swap_blocks(src_kv_cache, dst_kv_cache, src_to_dst) -> None:
         raise RuntimeError("swap_blocks is not used for the TPU backend.")
 
@@ -435,10 +452,13 @@ class TTAttentionBackendImpl(_ImplBase):
         return out.transpose(-3, -2)  # [users, tokens, Hq, D]
 
     def _gather_paged_to_dense(self, cache: torch.Tensor, page_table: torch.Tensor, num_tokens: int):
-        """[NB, Hkv, bs, D] -> [users, Hkv, num_tokens, D] in page-table order."""
+        """[NB, Hkv, bs, D] -> [users, Hkv, num_tokens, D] in page-table order (a block-float-8
+        cache comes out as the bfloat16 values it encodes)."""
         users, width = page_table.shape
-        _, hkv, bs, d = cache.shape
         g = torch.index_select(cache, 0, page_table.reshape(-1))
+        if cache.dtype == torch.uint8:
+            g = custom_ops.bfp8_unpack_cache(g)
+        _, hkv, bs, d = g.shape
         g = g.view(users, width, hkv, bs, d).permute(0, 2, 1, 3, 4).contiguous()
         return g.reshape(users, hkv, -1, d)[:, :, :num_tokens, :]
 

@@ -559,10 +559,11 @@ def _prefill(query, key, value, page_table, chunk_start, attn_mask, is_causal, s
         kv_strides = (k.stride(0), k.stride(1), k.stride(2))
         bs = w = nb = 0
         pt_ptr, pt_rs = 0, 0
+        fmt = N.KV_BF16
     else:
         nb, hkv, bs, kd, fmt = _attention_cache_geometry(key)
-        if fmt != N.KV_BF16 or _attention_cache_geometry(value) != (nb, hkv, bs, kd, fmt) or kd != d:
-            raise ValueError("chunked attention needs matching bfloat16 K/V caches")
+        if _attention_cache_geometry(value) != (nb, hkv, bs, kd, fmt) or kd != d:
+            raise ValueError("chunked attention needs K / V caches of one shape and format, head size as the query's")
         k, v = key, value
         pt = _table(page_table)
         w = pt.shape[1]
@@ -578,12 +579,12 @@ def _prefill(query, key, value, page_table, chunk_start, attn_mask, is_causal, s
             m = m.contiguous()
         mask_ptr, mask_bs, mask_rs = m.data_ptr(), m.stride(0), m.stride(2)
     N.call(
-        "ttpa_sdpa_prefill_windowed",
+        "ttpa_sdpa_prefill_format",
         out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
         q.data_ptr(), q.stride(0), q.stride(1), q.stride(2),
         k.data_ptr(), v.data_ptr(), *kv_strides, pt_ptr, pt_rs, _ptr(chunk_start),
         mask_ptr, mask_bs, mask_rs, b, hq, hkv, s, skv, d, bs, w, nb, int(is_causal),
-        float(scale), int(window), _stream(),
+        float(scale), int(window), fmt, _stream(),
     )
     return out
 
