@@ -36,13 +36,39 @@ for _p in (ROOT, os.path.join(ROOT, "tt-xla_amd")):
 HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs
-# of this script scaled by a plain copy of known size (profiles/decode_kernel_hbm_traffic_config2.md).
-# A counter run cannot share a process with the timed run, so the figure is carried here; it belongs
-# to the default seed and shapes of the workload it is keyed by.
-MEASURED_TRAFFIC_BYTES = {"config2": 306650 * 1024}
+# of this script scaled by a plain copy of known size (profiles/*_hbm_traffic_*.md).  A counter run
+# cannot share a process with the timed run, so the figures are carried here, each with the hash
+# of the kernel sources it was measured on (the first 16 hex digits of the SHA-256 over the files
+# listed): when the sources have changed since, `roofline.traffic` is null instead of stale.
+KERNEL_SOURCES = {
+    "paged_decode_mfma16_kernel": ["decode_mfma16_kernel.h", "decode_common.h", "common.h"],
+    "prefill_kernel": ["prefill.hip", "common.h"],
+}
+MEASURED_TRAFFIC = {
+    # workload: (kernel, hash of its sources, HBM bytes per launch)
+}
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}
 CPU_THREADS_CAP = 16        # host cores a one-GPU box grants, whatever os.cpu_count() says
+
+
+def kernel_source_hash(kernel):
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES[kernel]:
+        with open(os.path.join(ROOT, "tt-xla_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload, kernel):
+    """The counter-measured HBM bytes per launch for this workload, or None when there is no
+    measurement of the kernel as it is built now."""
+    rec = MEASURED_TRAFFIC.get(workload)
+    if rec is None or rec[0] != kernel or rec[1] != kernel_source_hash(kernel):
+        return None
+    return rec[2]
 
 
 def parse():
@@ -58,6 +84,8 @@ def parse():
                          "1 = one graph launch per step")
     ap.add_argument("--workload", choices=["config2", "config3", "config4", "config5"], default="config2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="config2 only: leave out the short config3 / config5 runs reported under 'secondary'")
     ap.add_argument("--cpu-users", type=int, default=0, help="users in the CPU sample (0 = auto)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 256 MiB device copies, so that a counter run of this "
@@ -399,7 +427,9 @@ def run_decode(args):
         "roofline": {
             "kernel": DECODE_KERNEL_NAME[args.workload],
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": measured_traffic(args.workload, DECODE_KERNEL_NAME[args.workload]),
+            "kernel_source_hash": kernel_source_hash(DECODE_KERNEL_NAME[args.workload]),
             "kernel_us": kern_ms * 1e3, "kernel_us_min": min(d for d, _ in durs) * 1e3,
             "bytes_per_launch": kern_bytes, "timed_launches": len(durs),
         },
@@ -461,13 +491,40 @@ def run_prefill(args):
         "roofline": {
             "kernel": "prefill_kernel", "bound": "mfma", "achieved": achieved,
             "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+            "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": measured_traffic("config3", "prefill_kernel"),
+            "kernel_source_hash": kernel_source_hash("prefill_kernel"),
             "kernel_us": kern_ms * 1e3, "kernel_us_min": min(d for d, _ in durs) * 1e3,
             "flops_per_launch": flops, "timed_launches": len(durs),
             "note": "useful (causal) FLOPs only; the dense 4*B*Hq*S^2*D figure is twice this; the launch "
                     "also carries the step's K / V cache fill (fill_bytes_per_step of traffic)",
         },
     }
+
+
+def secondary_runs(args):
+    """Short runs of the prefill workload (config3) and of the block-float-8 decode workload
+    (config5) in the headline's process, so that their figures come under the same clock: the
+    same functions as `--workload config3|config5`, fewer steps, only the key figures."""
+    import copy
+    import gc
+
+    import torch
+
+    out = {}
+    for wl, steps, warmup in (("config3", 30, 5), ("config5", 96, 12)):
+        gc.collect()
+        torch.cuda.empty_cache()
+        sub = copy.copy(args)
+        sub.workload, sub.steps, sub.warmup = wl, steps, warmup
+        r = run_prefill(sub) if wl == "config3" else run_decode(sub)
+        keep = {k: r[k] for k in ("metric", "value", "unit", "steps", "warmup", "ms_per_step", "dtype", "roofline")}
+        keep["workload"] = r["config"]["workload"]
+        if "pct_of_hbm_peak" in r:
+            keep["pct_of_hbm_peak"] = r["pct_of_hbm_peak"]
+        out[wl] = keep
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -493,6 +550,8 @@ def main():
             out["cpu_baseline"] = cpu_prefill_baseline(args)
     else:
         out = run_decode(args)
+        if args.workload == "config2" and not args.no_secondary:
+            out["secondary"] = secondary_runs(args)
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_decode_baseline(args)
     if args.calibrate_copy:

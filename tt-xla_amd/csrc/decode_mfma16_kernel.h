@@ -236,7 +236,10 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   }
 
   auto locate = [&](int64_t xx) { return locate_unit<TILE>(a, s_pref, s_len, xx); };
-  auto tile_offsets = [&](const Cursor &cu, int64_t (&eo)[NOFF], int64_t (&xo)[NOFF]) {
+  // `bad`: bit i set where run i's block lies outside the table or the cache (it reads block 0)
+  auto tile_offsets = [&](const Cursor &cu, int64_t (&eo)[NOFF], int64_t (&xo)[NOFF], uint32_t &bad) {
+    bad = 0;
+    bool base_bad = false;
     const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
     const int tok0 = cu.t * TILE;
     // a run never crosses a block (block_size is a multiple of the run length), so block and
@@ -246,10 +249,12 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
 #pragma unroll
     for (int i = 0; i < NOFF; ++i) {
       if (i == 0 || row == 0) {
-        int phys = (col < a.w) ? __builtin_amdgcn_readfirstlane(pt_row[col]) : 0;
-        if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+        int phys = (col < a.w) ? __builtin_amdgcn_readfirstlane(pt_row[col]) : -1;
+        base_bad = (unsigned)phys >= (unsigned)a.nb;
+        if (base_bad) phys = 0;
         base = ((int64_t)phys * a.hkv + cu.h) * slab;
       }
+      if (base_bad) bad |= 1u << i;
       eo[i] = base + (int64_t)row * D * BPE;
       xo[i] = base + (int64_t)a.bs * D + (int64_t)row * GPR;
       row += RPL * LPO;
@@ -287,7 +292,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   // the fetched tile (registers) and stores it into the cache row `row` of the slab at byte
   // offset `slab_base`.
   auto patch_and_store = [&](uint8_t *cache, u32x4 (&raw)[NL], uint32_t (&ex)[NL], const Fresh &fresh,
-                             int r_star, int64_t slab_base, int row) {
+                             int r_star, int64_t elem_off, int64_t exp_off) {
     const int i_star = r_star / RPL;
     const bool mine = sr == r_star % RPL;
     u32x4 val = fresh.part[0];
@@ -306,9 +311,8 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
         if constexpr (BFP8) ex[i] = e << exp_shift;
       }
     if (mine) {
-      uint8_t *slab_ptr = cache + slab_base;
-      *reinterpret_cast<u32x4 *>(slab_ptr + (int64_t)row * (D * BPE) + 16 * sc) = val;
-      if constexpr (BFP8) slab_ptr[(int64_t)a.bs * D + (int64_t)row * GPR + sc] = (uint8_t)e;
+      *reinterpret_cast<u32x4 *>(cache + elem_off + 16 * sc) = val;
+      if constexpr (BFP8) cache[exp_off + sc] = (uint8_t)e;
     }
   };
   // Cuts the lane's exponent bytes out of the fetched dwords (zero for rows past `nvalid` of a
@@ -390,7 +394,8 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   uint32_t kex[NL], vex[NL];
   u32x4 qf[KSTEPS];
   Fresh kfresh = {}, vfresh = {};
-  tile_offsets(cur, eo, xo);
+  uint32_t bad_cur = 0;  // the current tile's runs that read block 0 in place of a block out of range
+  tile_offsets(cur, eo, xo, bad_cur);
   fetch(a.k, eo, xo, kraw, kex);
   fetch(a.v, eo, xo, vraw, vex);
   if constexpr (FUSED) {
@@ -416,25 +421,28 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
 
     // ---- K: registers -> LDS, then the next tile's K: global -> registers -------------------
     // FUSED: is this the tile that holds the token at cur_pos (the segment's last), and is that
-    // position inside the table and its block inside the cache?  Evaluated where it is used
-    // (once for K, once for V) rather than kept across the tile: it is all scalar work, and
-    // scalar registers are what this kernel is short of.
-    auto fresh_target = [&](int64_t &slab_off, int &row) -> bool {
-      if (cur.tiles_left != 1 || nvalid <= 0) return false;
-      const int pos = cur.len - 1;
-      const int col = pos / a.bs;
-      if (load_index(cur_pos, a.cur_i64, cur.u) != pos || col >= a.w) return false;  // cut short by the table
-      const int phys = __builtin_amdgcn_readfirstlane(page_table[(int64_t)cur.u * a.pt_rs + col]);
-      if ((unsigned)phys >= (unsigned)a.nb) return false;
-      slab_off = ((int64_t)phys * a.hkv + cur.h) * slab;
-      row = pos - col * a.bs;
-      return true;
-    };
+    // position inside the table and its block inside the cache?  The row's place in the cache
+    // comes from the tile's own offsets: a second look at the position and the page table would
+    // be two round trips to memory in the middle of the tile, each waiting for every load in
+    // flight, and the wavefronts that end a segment are the ones a launch ends up waiting for.
+    bool fresh_ok = false;
+    int64_t fresh_eo = 0, fresh_xo = 0;
     if constexpr (FUSED) {
-      int64_t slab_off;
-      int row;
-      if (fresh_target(slab_off, row))
-        patch_and_store(const_cast<uint8_t *>(a.k), kraw, kex, kfresh, nvalid - 1, slab_off, row);
+      if (cur.tiles_left == 1 && nvalid > 0) {
+        // a length below the table's capacity is the position + 1; at the capacity it may have
+        // been cut short, and only then the position is read again
+        const int64_t cap = (int64_t)a.w * a.bs;
+        const bool exact = cur.len < cap || load_index(cur_pos, a.cur_i64, cur.u) == cur.len - 1;
+        constexpr int RUN_ROWS = RPL * LPO;
+        const int i_run = (nvalid - 1) / RUN_ROWS, rr = (nvalid - 1) % RUN_ROWS;
+        if (exact && !((bad_cur >> i_run) & 1u)) {
+          fresh_ok = true;
+#pragma unroll
+          for (int i = 0; i < NOFF; ++i)
+            if (i == i_run) fresh_eo = eo[i] + (int64_t)rr * D * BPE, fresh_xo = xo[i] + (int64_t)rr * GPR;
+        }
+      }
+      if (fresh_ok) patch_and_store(const_cast<uint8_t *>(a.k), kraw, kex, kfresh, nvalid - 1, fresh_eo, fresh_xo);
     }
     int eref_k = 0, eref_v = 0;
     if constexpr (BFP8) eref_k = tile_exponent(kex, nvalid, partial);
@@ -446,7 +454,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
       } else {
         nxt = locate(x + 1);
       }
-      tile_offsets(nxt, eo, xo);
+      tile_offsets(nxt, eo, xo, bad_cur);  // (of the next tile: this one's has been used above)
       fetch(a.k, eo, xo, kraw, kex);
     }
 
@@ -494,10 +502,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
 
     // ---- V: registers -> LDS (the K tile has been consumed), next tile's V -> registers -------
     if constexpr (FUSED) {
-      int64_t slab_off;
-      int row;
-      if (fresh_target(slab_off, row))
-        patch_and_store(const_cast<uint8_t *>(a.v), vraw, vex, vfresh, nvalid - 1, slab_off, row);
+      if (fresh_ok) patch_and_store(const_cast<uint8_t *>(a.v), vraw, vex, vfresh, nvalid - 1, fresh_eo, fresh_xo);
     }
     if constexpr (BFP8) eref_v = tile_exponent(vex, nvalid, partial);
     stage(true, vraw, vex, eref_v, nvalid, partial);
