@@ -42,10 +42,15 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 # listed): when the sources have changed since, `roofline.traffic` is null instead of stale.
 KERNEL_SOURCES = {
     "paged_decode_mfma16_kernel": ["decode_mfma16_kernel.h", "decode_common.h", "common.h"],
-    "prefill_kernel": ["prefill.hip", "common.h"],
+    "prefill_kernel": ["prefill.hip", "prefill_acc_regs.h", "common.h"],
 }
 MEASURED_TRAFFIC = {
-    # workload: (kernel, hash of its sources, HBM bytes per launch)
+    # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
+    # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
+    # the rotating workload copies; the summaries under profiles/ hold the runs)
+    "config2": ("paged_decode_mfma16_kernel", "a88126b215c90579", 311719985),
+    "config5": ("paged_decode_mfma16_kernel", "a88126b215c90579", 168854438),
+    "config3": ("prefill_kernel", "c9602929cb330d80", 234209088),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}
