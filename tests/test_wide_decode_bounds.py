@@ -127,3 +127,79 @@ def test_every_address_stays_in_bounds(dqk, dv, sep_v, hq, nkv, bs, width, nb, u
     for seg_h in (0, nkv * nhb - 1):
         assert seg_h * gseg + gseg - 1 < hq
         assert seg_h // nhb < nkv
+
+
+# ---- the 16-head form (every wavefront streams its own 16-token tiles) ---------------------------
+BUILT_16 = {(576, 512), (576, 384), (192, 128), (128, 128)}
+SHAPES_16 = [s for s in SHAPES
+             if not s[2] and s[3] // s[4] <= 16 and s[5] % 16 == 0 and (s[0], s[1]) in BUILT_16]
+
+
+def test_the_16_head_form_is_exercised():
+    assert len(SHAPES_16) >= 6
+    assert any(s[0] == 576 for s in SHAPES_16) and any(s[0] == 192 for s in SHAPES_16)
+
+
+def _position(row_bytes, r, c):
+    """LDS chunk position of chunk c of row r (the kernel's Latent16::position)."""
+    half_period = (row_bytes // 4) % 64 == 32
+    return c ^ ((r >> 1) & 7) if half_period else c ^ (r & 15)
+
+
+@pytest.mark.parametrize("dqk,dv,sep_v,hq,nkv,bs,width,nb,users", SHAPES_16)
+def test_every_address_of_the_16_head_form_stays_in_bounds(dqk, dv, sep_v, hq, nkv, bs, width, nb, users):
+    tile, waves = 16, 4
+    g = hq // nkv
+    row_bytes = 2 * dqk
+    cpr = row_bytes // 16
+    stage = tile * row_bytes
+    wave_lds = 2 * stage
+    ndma = stage // 1024
+    assert stage % 1024 == 0 and STATIC_LDS + waves * wave_lds <= LDS_PER_CU
+    assert (row_bytes // 4) % 64 in (0, 32) and cpr % (8 if (row_bytes // 4) % 64 == 32 else 16) == 0
+    cache_bytes = nb * nkv * bs * row_bytes
+    # the swizzle permutes the chunks of a row among themselves
+    for r in range(tile):
+        assert sorted(_position(row_bytes, r, c) for c in range(cpr)) == list(range(cpr))
+    cap = width * bs
+    for t in {0, (cap - 1) // tile}:
+        tok0 = t * tile
+        col = tok0 // bs
+        assert tok0 - col * bs + tile <= bs, "a tile lies inside one block"
+        for phys, kvh in itertools.product({0, nb - 1}, {0, nkv - 1}):
+            tile_base = ((phys * nkv + kvh) * bs + (tok0 - col * bs)) * row_bytes
+            assert tile_base % 16 == 0
+            seen = set()
+            for k in range(ndma):
+                for lane in range(64):
+                    pos = 64 * k + lane
+                    r, p = pos // cpr, pos % cpr
+                    off = r * row_bytes + 16 * _position(row_bytes, r, p)
+                    assert 0 <= off and off + 16 <= stage and tile_base + off + 16 <= cache_bytes
+                    seen.add(off)
+                for wib, buf in itertools.product(range(waves), (0, 1)):
+                    dst = STATIC_LDS + wib * wave_lds + buf * stage + 1024 * k     # absolute, as M0 carries it
+                    assert dst % 16 == 0 and dst + 1024 <= STATIC_LDS + wib * wave_lds + (buf + 1) * stage <= LDS_PER_CU
+            assert len(seen) == stage // 16, "every chunk of the tile is fetched exactly once"
+    ksteps, vb = dqk // 32, dv // 16
+    assert dqk % 32 == 0 and dv % 16 == 0 and dv <= dqk
+    for s in range(ksteps):
+        for quad in range(4):                                      # 16 lanes of an A-operand read: 16 bank quads
+            quads = {((n * row_bytes + 16 * _position(row_bytes, n, 4 * s + quad)) // 16) % 16 for n in range(16)}
+            assert len(quads) == 16
+    for lane in range(64):
+        n, quad = lane & 15, lane >> 4
+        for s in (0, ksteps - 1):
+            off = n * row_bytes + 16 * _position(row_bytes, n, 4 * s + quad)
+            assert off // row_bytes == n and off + 16 <= stage
+        rv, q = 4 * quad + (n >> 2), n & 3
+        for b in (0, vb - 1):
+            off = rv * row_bytes + 16 * _position(row_bytes, rv, 2 * b + (q >> 1)) + 8 * (q & 1)
+            assert off // row_bytes == rv and off + 8 <= stage
+        assert 8 * quad + 32 * (ksteps - 1) + 8 <= dqk
+        slot_floats = (g * dv + 2 * g + 3) // 4 * 4
+        if n < g:
+            assert n * dv + 4 * quad + 16 * (vb - 1) + 4 <= g * dv
+            assert g * dv + g + n < slot_floats
+    segs, cus = users * nkv, 256
+    assert (waves * cus - 1) + (segs - 1) < waves * cus + segs     # slot index = wavefront + segment

@@ -489,7 +489,7 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   }
   if (ev1) (void)hipEventRecord(ev1, st);
   if (rc) return rc;
-  decode_combine_kernel<<<dim3(users * kv_heads), dim3(256), 0, st>>>(a, g, head_size);
+  decode_combine_kernel<<<dim3(users * kv_heads, combine_pieces(g, head_size)), dim3(256), 0, st>>>(a, g, head_size);
   return check_launch("paged_sdpa_decode");
 }
 

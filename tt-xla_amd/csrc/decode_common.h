@@ -261,6 +261,28 @@ __device__ __forceinline__ Cursor locate_unit(const DecodeArgs &a, const int *s_
   return cu;
 }
 
+// Maximum over the four lanes that share lane%16.  v_permlane16_swap exchanges the odd rows
+// of its first operand with the even rows of its second, v_permlane32_swap the upper half of
+// the first with the lower half of the second; fed with two copies of a value, the two
+// results hold the value of either partner.  Written as assembly: through the builtins the
+// compiler takes the two results for equal.
+__device__ __forceinline__ float max_over_quads(float v) {
+  float x = v, y = v;
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+  float m = fmaxf(x, y);
+  x = m, y = m;
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+  return fmaxf(x, y);
+}
+__device__ __forceinline__ float sum_over_quads(float v) {
+  float x = v, y = v;
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+  float m = x + y;
+  x = m, y = m;
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+  return x + y;
+}
+
 // One thread per segment (the first blocks of the grid): publishes which partial slots the
 // merge kernel has to read for that segment.
 __device__ __forceinline__ void publish_segment_row(const DecodeArgs &a, const int *s_pref,
@@ -328,8 +350,16 @@ __device__ __forceinline__ void write_partial(float *slot, int g, int G, int r, 
 // dependent round trips, and this keeps it at two.  G and D are run-time values: the
 // matrix-core kernels serve any group width up to 32.  D is a power of two on the attention
 // paths (64, 128, 256: split by shift and mask); the latent path also has 384 (divided).
+// Grid: x = segment, y = piece of kCombinePiece of the segment's G * D output elements (one piece
+// for the plain decode shapes; a latent segment of 16 heads x 512 values is 16 pieces, and as one
+// workgroup per segment its merge took as long as the attention itself).
+constexpr int kCombinePiece = 512;
+inline int combine_pieces(int g, int d) { return (g * d + kCombinePiece - 1) / kCombinePiece; }
+
 __global__ inline __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a, int G, int D) {
   const int seg = blockIdx.x;
+  const int i_begin = blockIdx.y * kCombinePiece + threadIdx.x;
+  const int i_end = min(G * D, (int)(blockIdx.y + 1) * kCombinePiece);
   const int u = seg / a.hkv, h = seg % a.hkv;
   const bool pow2 = (D & (D - 1)) == 0;
   const int dshift = __builtin_ctz(D);
@@ -338,13 +368,13 @@ __global__ inline __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a
   const int first = a.ws_seg[2 * seg], nw = a.ws_seg[2 * seg + 1];
   uint16_t *out = a.out + u * a.out_us;
   if (nw == 0) {  // padded row: no attended position -> NaN like softmax over nothing
-    for (int i = threadIdx.x; i < G * D; i += 256)
+    for (int i = i_begin; i < i_end; i += 256)
       out[(int64_t)(h * G + head_of(i)) * a.out_hs + elem_of(i)] = 0x7fc0;
     return;
   }
   constexpr int kBatch = 8;
   const float *base = a.ws_slots + (int64_t)first * a.slot_floats;
-  for (int i = threadIdx.x; i < G * D; i += 256) {
+  for (int i = i_begin; i < i_end; i += 256) {
     const int g = head_of(i);
     float mall = -INFINITY, num = 0.f, den = 0.f;
     for (int w = 0; w < nw; w += kBatch) {

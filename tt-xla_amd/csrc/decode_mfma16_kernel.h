@@ -87,28 +87,6 @@ __device__ __forceinline__ floatx4 mma16(const u32x4 &x, const u32x4 &y, const f
                                                    __builtin_bit_cast(bf16x8, y), c, 0, 0, 0);
 }
 
-// Maximum over the four lanes that share lane%16.  v_permlane16_swap exchanges the odd rows
-// of its first operand with the even rows of its second, v_permlane32_swap the upper half of
-// the first with the lower half of the second; fed with two copies of a value, the two
-// results hold the value of either partner.  Written as assembly: through the builtins the
-// compiler takes the two results for equal.
-__device__ __forceinline__ float max_over_quads(float v) {
-  float x = v, y = v;
-  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
-  float m = fmaxf(x, y);
-  x = m, y = m;
-  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
-  return fmaxf(x, y);
-}
-__device__ __forceinline__ float sum_over_quads(float v) {
-  float x = v, y = v;
-  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
-  float m = x + y;
-  x = m, y = m;
-  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
-  return x + y;
-}
-
 // The cache write of a user whose position is negative, by one thread per (user, kv head):
 // position -k counts from the end of the user's table (the update operator's floor rule:
 // column = floor(pos / bs) taken from the end once, row = pos mod bs); positions that still fall

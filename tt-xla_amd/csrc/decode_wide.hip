@@ -289,6 +289,287 @@ __global__ __launch_bounds__(256, 1) void paged_decode_wide_kernel(
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Up to 16 query heads per KV head with V taken from K: the latent serving shape (16 heads of
+// 576 = 512 + 64 features on a rank, V = the 512 leading ones).  Here nothing is shared between
+// wavefronts, and nothing is computed twice: every wavefront streams its own range of 16-token
+// tiles, as in the 16x16x32 kernel of the plain decode shapes, with the group's heads as the
+// 16-wide N dimension:
+//   S^T[key, head]   = K[key, :] . Q[head, :]     v_mfma_f32_16x16x32_bf16, DQK / 32 steps
+//   O^T[d, head]    += V^T[d, key] . P^T[key, head]   v_mfma_f32_16x16x16_bf16 per 16 values
+// The C layout of the first (lane (head, quad) holds keys 4 quad + r) is the B layout of the
+// second.  A tile is 16 consecutive cache rows (block_size is a multiple of 16), so it goes
+// global -> LDS as whole 1 KiB LDS-DMA instructions (18 for rows of 1152 bytes; an instruction
+// holds the wavefront until the address unit has taken it, and one per row plus one per row tail
+// was 32), into one of two wave-private stages; the wavefront waits for its own loads only, there
+// is no barrier.  Rows are unpadded in LDS; bank conflicts are avoided by an XOR swizzle of the
+// 16-byte chunk position, applied on the global side (which chunk a lane fetches: every lane of
+// an LDS-DMA instruction supplies its own source address) and when fragments are read.  Rows of
+// 1152 or 384 bytes start 32 banks apart, so chunk ^ ((row >> 1) & 7) inside aligned groups of 8
+// chunks gives the sixteen rows of an A-operand read sixteen different bank quads; rows of 256
+// bytes start at the same bank and take chunk ^ (row & 15).  The arithmetic of a tile is an
+// order of magnitude below what its bytes cost in HBM time, so nothing here is scheduled by hand.
+template <int DQK, int DV>
+struct Latent16 {
+  static constexpr int TILE = 16;
+  static constexpr int ROW = 2 * DQK;            // bytes per row, in the cache and in LDS
+  static constexpr int CPR = ROW / 16;           // 16-byte chunks per row
+  static constexpr int STAGE = TILE * ROW;
+  static constexpr int WAVE_LDS = 2 * STAGE;
+  static constexpr int NDMA = STAGE / 1024;      // LDS-DMA instructions per tile
+  static constexpr bool HALF_PERIOD = (ROW / 4) % 64 == 32;
+  static_assert(STAGE % 1024 == 0 && (HALF_PERIOD ? CPR % 8 == 0 : ((ROW / 4) % 64 == 0 && CPR % 16 == 0)),
+                "row length the swizzle is not made for");
+  // position of chunk c of row r inside the row
+  __device__ static constexpr int position(int r, int c) {
+    return HALF_PERIOD ? (c ^ ((r >> 1) & 7)) : (c ^ (r & 15));
+  }
+};
+
+template <int DQK, int DV>
+__global__ __launch_bounds__(256, 1) void paged_decode_latent16_kernel(
+    DecodeArgs a, WideArgs w, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
+  using L = Latent16<DQK, DV>;
+  typedef float floatx4 __attribute__((ext_vector_type(4)));
+  constexpr int TILE = L::TILE, KSTEPS = DQK / 32, VB = DV / 16;
+  constexpr int ROW_BYTES = L::ROW;
+
+  __shared__ int s_pref[kMaxUsersWide + 1];
+  __shared__ int s_len[kMaxUsersWide];
+  __shared__ int s_wsum[kWavesPerBlock];
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  build_prefix<TILE>(a, cur_pos, s_pref, s_len, s_wsum);
+
+  const int lane = threadIdx.x & 63;
+  const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n = lane & 15, quad = lane >> 4;
+  // LDS-DMA instruction k fills chunk positions 64 k .. 64 k + 63 of the stage; this lane's is
+  // position p of row r, which holds chunk position(r, p): the source offset inside the tile
+  uint32_t src_off[L::NDMA];
+#pragma unroll
+  for (int k = 0; k < L::NDMA; ++k) {
+    const int P = 64 * k + lane, r = P / L::CPR, p = P % L::CPR;
+    src_off[k] = (uint32_t)(r * ROW_BYTES + 16 * L::position(r, p));
+  }
+  // Fragment addresses inside a stage: A operand of the score product (row n, chunk 4 s + quad)
+  // and the transposing read of the value columns (row 4 quad + n / 4, values 16 vb + 4 (n % 4) ..).
+  // The swizzle only touches the chunk index inside its aligned group of GC chunks, so a lane
+  // needs one address per chunk offset inside a group; the group itself is an immediate offset.
+  constexpr int GC = L::HALF_PERIOD ? 8 : 16;
+  constexpr int KB = GC / 4, VBASES = GC / 2;
+  uint32_t kbase[KB], vbase[VBASES];
+#pragma unroll
+  for (int i = 0; i < KB; ++i) kbase[i] = (uint32_t)(n * ROW_BYTES + 16 * L::position(n, 4 * i + quad));
+  {
+    const int rv = 4 * quad + (n >> 2), q = n & 3;
+#pragma unroll
+    for (int i = 0; i < VBASES; ++i)
+      vbase[i] = (uint32_t)(rv * ROW_BYTES + 16 * L::position(rv, 2 * i + (q >> 1)) + 8 * (q & 1));
+  }
+  auto read_k = [&](const unsigned char *stage, int s) {
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(stage + kbase[s % KB] + 16 * GC * (s / KB)));
+  };
+  auto read_v = [&](const unsigned char *stage, int vb) {
+    typedef __attribute__((address_space(3))) shortx4 *lds_v4;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(stage + vbase[vb % VBASES] + 16 * GC * (vb / VBASES)));
+  };
+  constexpr int KPRE = KSTEPS < 8 ? KSTEPS : 8;  // fragments in flight (an LDS read takes a few hundred cycles)
+  constexpr int VPRE = VB < 12 ? VB : 12;
+  const int wave = blockIdx.x * kWavesPerBlock + wib;
+  const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
+  const int64_t total = (int64_t)total_tiles * a.hkv;
+  const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);
+  if (total == 0 || wave >= n_eff) {
+    publish_segment_row(a, s_pref, total, n_eff);
+    return;
+  }
+  int64_t x = (int64_t)wave * total / n_eff;
+  const int64_t x_hi = (int64_t)(wave + 1) * total / n_eff;
+  const int G = w.gseg;
+  unsigned char *my_lds = smem + wib * L::WAVE_LDS;
+
+  // ---- tile load: block_size is a multiple of the tile, so a tile is 16 consecutive cache rows ----
+  auto issue_tile = [&](const Cursor &cu, int buf) {
+    const int tok0 = cu.t * TILE;
+    const int col = tok0 / a.bs;
+    int phys = (col < a.w) ? page_table[(int64_t)cu.u * a.pt_rs + col] : 0;
+    if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+    const int64_t row0 = ((int64_t)phys * w.nkv + cu.h) * a.bs + (tok0 - col * a.bs);
+    const uint64_t addr = reinterpret_cast<uint64_t>(a.k) + (uint64_t)row0 * ROW_BYTES;
+    const char *src = reinterpret_cast<const char *>(address_from_words(
+        __builtin_amdgcn_readfirstlane((int)(uint32_t)addr), __builtin_amdgcn_readfirstlane((int)(uint32_t)(addr >> 32))));
+    const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_address(my_lds) + (uint32_t)(buf * L::STAGE)));
+    const void *bases[4] = {src, src - 1024, src - 2048, src - 3072};
+#pragma unroll
+    for (int k = 0; k + 4 <= L::NDMA; k += 4) {
+      const uint32_t off[4] = {src_off[k], src_off[k + 1], src_off[k + 2], src_off[k + 3]};
+      dma16_quad(bases, off, dst + 1024u * k);
+    }
+#pragma unroll
+    for (int k = L::NDMA / 4 * 4; k < L::NDMA; ++k) dma16(src, src_off[k], dst + 1024u * k);
+  };
+  // Rows past the attended length may be cache rows nobody ever wrote: their scores are masked,
+  // but as V rows they would turn 0 * Inf into NaN, so they are cleared in LDS.
+  auto clear_unattended_rows = [&](unsigned char *stage, int nvalid) {
+    for (int r = nvalid; r < TILE; ++r) {
+      uint4 *row = reinterpret_cast<uint4 *>(stage + r * L::ROW);
+      for (int c = lane; c < ROW_BYTES / 16; c += 64) row[c] = make_uint4(0, 0, 0, 0);
+    }
+  };
+  // B operand of the score product: lane (head, quad) holds features 32 s + 8 quad .. + 7
+  auto load_q = [&](const Cursor &cu, bf16x8 (&qf)[KSTEPS]) {
+    const uint16_t *qp = a.q + cu.u * a.q_us + (int64_t)(cu.h * G + min(n, G - 1)) * a.q_hs + 8 * quad;
+    const uint32_t qmask = n < G ? 0xffffffffu : 0u;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      uint4 t = *reinterpret_cast<const uint4 *>(qp + 32 * s);
+      t.x &= qmask, t.y &= qmask, t.z &= qmask, t.w &= qmask;
+      qf[s] = __builtin_bit_cast(bf16x8, t);
+    }
+  };
+
+  Cursor cur = locate_unit<TILE>(a, s_pref, s_len, x);
+  bf16x8 qf[KSTEPS];
+  issue_tile(cur, 0);
+  load_q(cur, qf);
+  publish_segment_row(a, s_pref, total, n_eff);
+
+  floatx4 acc[VB];
+#pragma unroll
+  for (int i = 0; i < VB; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+
+  for (int it = 0; x < x_hi; ++x, ++it) {
+    const int buf = it & 1;
+    unsigned char *stage = my_lds + buf * L::STAGE;
+    const int nvalid = cur.len - cur.t * TILE;
+    const bool partial = nvalid < TILE;
+    const int nbelow = cur.lo - cur.t * TILE;
+    const bool has_next = x + 1 < x_hi;
+    const bool same_seg = has_next && cur.tiles_left > 1;
+
+    // The next tile is requested BEFORE this one is waited for (its stage has been idle since the
+    // previous iteration), so two tiles are in flight while the wavefront waits: with one, a
+    // tile took the memory latency plus its own issue and arithmetic, 3.9 us for 18 KiB.  Vector
+    // loads return in order: all but the NDMA newest done means this tile, and the Q rows
+    // requested before it, have landed.
+    Cursor nxt = cur;
+    if (has_next) {
+      if (same_seg) {
+        nxt.t = cur.t + 1;
+        nxt.tiles_left = cur.tiles_left - 1;
+      } else {
+        nxt = locate_unit<TILE>(a, s_pref, s_len, x + 1);
+      }
+      issue_tile(nxt, buf ^ 1);
+      __builtin_amdgcn_s_waitcnt((L::NDMA & 15) | 0x0F70 | ((L::NDMA >> 4) << 14));  // vmcnt(NDMA)
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    }
+    if (partial) clear_unattended_rows(stage, max(nvalid, 0));
+
+    // ---- S^T = K . Q^T ----------------------------------------------------------------------
+    floatx4 st = {0.f, 0.f, 0.f, 0.f};
+    {
+      bf16x8 ring[KPRE];
+#pragma unroll
+      for (int s = 0; s < KPRE; ++s) ring[s] = read_k(stage, s);
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {
+        st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % KPRE], qf[s], st, 0, 0, 0);
+        if (s + KPRE < KSTEPS) ring[s % KPRE] = read_k(stage, s + KPRE);
+      }
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {  // pin the order: one fragment read behind every matrix instruction
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (s + KPRE < KSTEPS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+    }
+    // ---- online softmax: lane (head, quad) holds keys 4 quad + r --------------------------------
+    const float scale = a.scale_log2e;
+    float sc[4], mloc = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int key = 4 * quad + r;
+      sc[r] = (key >= nvalid || key < nbelow) ? -INFINITY : st[r] * scale;
+      mloc = fmaxf(mloc, sc[r]);
+    }
+    mloc = max_over_quads(mloc);
+    // the running maximum moves only when a head's maximum grows by more than 2^8: rescaling the
+    // 4 VB accumulator registers costs more than the rest of the tile
+    const bool move = !(mloc - m_run <= 8.0f);  // also true from -inf
+    const float m_new = move ? mloc : m_run;
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = move ? __builtin_amdgcn_exp2f(m_run - m_safe) : 1.0f;
+    m_run = m_new;
+    float lsum = 0.f;
+    shortx4 pf;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float p = __builtin_amdgcn_exp2f(sc[r] - m_safe);
+      const __bf16 pb = (__bf16)p;
+      lsum += (float)pb;  // the normaliser sums the weights that multiply V
+      pf[r] = __builtin_bit_cast(short, pb);
+    }
+    l_run = l_run * alpha + lsum;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+      for (int i = 0; i < VB; ++i) acc[i] *= alpha;
+    }
+    // ---- O^T += V^T . P^T: lane (i, quad) of the transposing load addresses row 4 quad + i / 4,
+    //      values 16 vb + 4 (i % 4) .. + 3, and receives value 16 vb + i of rows 4 quad .. + 3 ------
+    {
+      shortx4 vring[VPRE];
+#pragma unroll
+      for (int vb = 0; vb < VPRE; ++vb) vring[vb] = read_v(stage, vb);
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb) {
+        acc[vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vring[vb % VPRE], pf, acc[vb], 0, 0, 0);
+        if (vb + VPRE < VB) vring[vb % VPRE] = read_v(stage, vb + VPRE);
+      }
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (vb + VPRE < VB) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+    }
+    // ---- close the segment ------------------------------------------------------------------------
+    if (!same_seg) {
+      float *slot = a.ws_slots + ((int64_t)wave + (int64_t)cur.u * a.hkv + cur.h) * a.slot_floats;
+      const float l_tot = sum_over_quads(l_run);
+      if (n < G) {
+        float *dst = slot + n * DV + 4 * quad;
+#pragma unroll
+        for (int vb = 0; vb < VB; ++vb)
+          *reinterpret_cast<float4 *>(dst + 16 * vb) = make_float4(acc[vb][0], acc[vb][1], acc[vb][2], acc[vb][3]);
+        if (quad == 0) {
+          slot[G * DV + n] = m_run;
+          slot[G * DV + G + n] = l_tot;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < VB; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+      m_run = -INFINITY;
+      l_run = 0.f;
+      if (has_next) load_q(nxt, qf);
+    }
+    cur = nxt;
+  }
+}
+
+template <int DQK, int DV>
+bool launch_latent16(const DecodeArgs &a, const WideArgs &w, hipStream_t st) {
+  using L = Latent16<DQK, DV>;
+  const size_t lds = (size_t)kWavesPerBlock * L::WAVE_LDS;
+  static std::atomic<uint64_t> lds_ready{0};
+  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_latent16_kernel<DQK, DV>), lds, lds_ready))
+    return false;
+  paged_decode_latent16_kernel<DQK, DV><<<dim3(a.n_waves / kWavesPerBlock), dim3(256), lds, st>>>(a, w, a.pt, a.cur);
+  return true;
+}
+
 template <int DQK, int DVW, bool SHARED_V>
 bool launch(const DecodeArgs &a, const WideArgs &w, hipStream_t st) {
   using L = WideLds<DQK, DVW, SHARED_V>;
@@ -331,7 +612,8 @@ extern "C" size_t ttpa_paged_mla_decode_workspace_bytes(int32_t users, int32_t q
   if (cus <= 0) cus = 256;
   const size_t segs = (size_t)users * kv_heads * nhb;
   const size_t slot = (size_t)slot_floats_for(gseg, head_dim_v) * sizeof(float);
-  return header_bytes(users, kv_heads * nhb) + ((size_t)cus + segs) * slot;
+  // one slot per range of the larger grid (four wavefront ranges per CU in the 16-head form)
+  return header_bytes(users, kv_heads * nhb) + ((size_t)cus * kWavesPerBlockHost + segs) * slot;
 }
 
 extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t out_head_stride,
@@ -400,6 +682,27 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
   if (ev0) (void)hipEventRecord(ev0, st);
   bool ok = false, built = true;
   const bool shared = v_cache == nullptr;
+  // The 16-head form: V taken from K, one head block of up to 16 heads, tiles inside one block.
+  // TTPA_LATENT_KERNEL=wide (read on every call) keeps such shapes on the workgroup-shared form.
+  const char *force = getenv("TTPA_LATENT_KERNEL");
+  const bool want16 = shared && nhb == 1 && gseg <= 16 && block_size % 16 == 0 && !(force && force[0] == 'w');
+  if (want16) {
+    a.n_waves = cus * kWavesPerBlockHost;
+    bool have = true;
+    if (head_size == 576 && head_dim_v == 512) ok = launch_latent16<576, 512>(a, w, st);
+    else if (head_size == 576 && head_dim_v == 384) ok = launch_latent16<576, 384>(a, w, st);
+    else if (head_size == 192 && head_dim_v == 128) ok = launch_latent16<192, 128>(a, w, st);
+    else if (head_size == 128 && head_dim_v == 128) ok = launch_latent16<128, 128>(a, w, st);
+    else have = false;
+    if (have) {
+      if (!ok) return fail(TTPA_ERR_LAUNCH, "latent decode: cannot configure the kernel");
+      if (ev1) (void)hipEventRecord(ev1, st);
+      if (int rc = check_launch("paged_mla_decode")) return rc;
+      decode_combine_kernel<<<dim3(users * kv_heads, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+      return check_launch("paged_mla_decode");
+    }
+    a.n_waves = cus;
+  }
 #define TTPA_WIDE_CASE(DQK, DVW)                                                                   \
   if (head_size == DQK && dvw == DVW)                                                              \
     ok = shared ? launch<DQK, DVW, true>(a, w, st) : launch<DQK, DVW, false>(a, w, st);            \
@@ -418,6 +721,6 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
   if (!ok) return fail(TTPA_ERR_LAUNCH, "latent decode: cannot configure the kernel");
   if (ev1) (void)hipEventRecord(ev1, st);
   if (int rc = check_launch("paged_mla_decode")) return rc;
-  decode_combine_kernel<<<dim3(users * kv_heads * nhb), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+  decode_combine_kernel<<<dim3(users * kv_heads * nhb, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
   return check_launch("paged_mla_decode");
 }
