@@ -42,6 +42,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 # listed): when the sources have changed since, `roofline.traffic` is null instead of stale.
 KERNEL_SOURCES = {
     "paged_decode_mfma16_kernel": ["decode_mfma16_kernel.h", "decode_common.h", "common.h"],
+    "paged_decode_latent16_kernel": ["decode_wide.hip", "decode_common.h", "common.h"],
     "prefill_kernel": ["prefill.hip", "prefill_acc_regs.h", "common.h"],
 }
 MEASURED_TRAFFIC = {
@@ -87,7 +88,7 @@ def parse():
                     help="consecutive steps captured in one graph: a decode forward replays one "
                          "attention step per layer inside one graph, and Llama-3-8B has 32 layers; "
                          "1 = one graph launch per step")
-    ap.add_argument("--workload", choices=["config2", "config3", "config4", "config5"], default="config2")
+    ap.add_argument("--workload", choices=["config2", "config3", "config4", "config5", "latent"], default="config2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true",
                     help="config2 only: leave out the short config3 / config5 runs reported under 'secondary'")
@@ -457,6 +458,63 @@ def run_decode(args):
     return out
 
 
+def run_latent(args):
+    """Latent (MLA) decode at the shape one rank of a latent-attention model serves: 16 query heads
+    over one latent KV head of 576 = 512 + 64 features, V = its 512 leading features; 128 users,
+    contexts uniform in [512, 8192], block 64.  The step is tt::paged_flash_mla_decode (attention +
+    merge of the split-K partials); the cache write of the step is the plain tt::paged_update_cache
+    on the latent cache and is not part of it."""
+    import torch
+
+    users, hq, dh, dv, bs, lo, hi = 128, 16, 576, 512, 64, 512, 8192
+    dev = "cuda:0"
+    copies = []
+    for i in range(max(1, min(args.rotate, 2))):
+        g = torch.Generator().manual_seed(11 + i)
+        ctx = torch.randint(lo, hi + 1, (users,), generator=g)
+        w = (hi + bs) // bs
+        nb = users * w + 1
+        key = torch.randn(nb, 1, bs, dh, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+        table = (torch.randperm(nb - 1, generator=g)[: users * w] + 1).view(users, w).to(torch.int32).to(dev)
+        q = torch.randn(1, users, hq, dh, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+        copies.append((q, key, table, ctx.to(torch.int32).to(dev), int((ctx + 1).sum())))
+    fns = [(lambda c=c: torch.ops.tt.paged_flash_mla_decode(c[0], c[1], dv, c[2], None, True, None, c[3], None, None))
+           for c in copies]
+    nbytes = [c[4] * dh * 2 + users * hq * (dh + dv) * 2 + users * (c[2].shape[1] * 4 + 4) for c in copies]
+    runner = StepRunner(fns, args.launch == "graph", args.steps_per_graph)
+    steps = min(args.steps, 100)
+    ms = time_steps(runner, steps, min(args.warmup, 10))
+    avg_bytes = sum(nbytes[i] for i in runner.sequence(steps)) / steps
+    durs = time_dominant_kernel(fns, min(steps, 50))
+    kern_ms = sum(d for d, _ in durs) / len(durs)
+    kern_bytes = sum(nbytes[w] for _, w in durs) / len(durs)
+    achieved = kern_bytes / (kern_ms * 1e-3) / 1e9
+    kernel = "paged_decode_latent16_kernel"
+    return {
+        "metric": "paged_decode_attention_hbm_throughput",
+        "value": avg_bytes / (ms * 1e-3) / 1e9, "unit": "GB/s",
+        "n_gpus": 1, "steps": steps, "warmup": min(args.warmup, 10), "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "workload": f"latent-decode-b{users}-h{hq}x1-d{dh}/{dv}-bs{bs}-ctx{lo}..{hi}",
+            "step": "paged latent decode attention + merge of the split-K partials, one layer, one token per sequence",
+            "launch": args.launch, "steps_per_graph": runner.per_graph if args.launch == "graph" else None,
+            "rotating_copies": len(copies), "users": users, "q_heads": hq, "kv_heads": 1, "head_size": dh,
+            "head_dim_v": dv, "block_size": bs,
+        },
+        "tokens_per_s": users / (ms * 1e-3),
+        "pct_of_hbm_peak": 100.0 * avg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "roofline": {
+            "kernel": kernel, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic("latent", kernel),
+            "kernel_source_hash": kernel_source_hash(kernel),
+            "kernel_us": kern_ms * 1e3, "kernel_us_min": min(d for d, _ in durs) * 1e3,
+            "bytes_per_launch": kern_bytes, "timed_launches": len(durs),
+        },
+    }
+
+
 def run_prefill(args):
     import torch
 
@@ -553,6 +611,8 @@ def main():
         out = run_prefill(args)
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_prefill_baseline(args)
+    elif args.workload == "latent":
+        out = run_latent(args)  # (no CPU leg: the headline workload carries it)
     else:
         out = run_decode(args)
         if args.workload == "config2" and not args.no_secondary:

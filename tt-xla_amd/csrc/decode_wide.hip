@@ -391,11 +391,18 @@ __global__ __launch_bounds__(256, 1) void paged_decode_latent16_kernel(
   unsigned char *my_lds = smem + wib * L::WAVE_LDS;
 
   // ---- tile load: block_size is a multiple of the tile, so a tile is 16 consecutive cache rows ----
+  // (the table entry of a block is read once, with the first of the block's tiles: the read is a
+  // trip to the L2 in front of the tile's loads)
+  int seen_user = -1, seen_col = -1, seen_phys = 0;
   auto issue_tile = [&](const Cursor &cu, int buf) {
     const int tok0 = cu.t * TILE;
     const int col = tok0 / a.bs;
-    int phys = (col < a.w) ? page_table[(int64_t)cu.u * a.pt_rs + col] : 0;
-    if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+    if (cu.u != seen_user || col != seen_col) {
+      int p = (col < a.w) ? page_table[(int64_t)cu.u * a.pt_rs + col] : 0;
+      if ((unsigned)p >= (unsigned)a.nb) p = 0;
+      seen_user = cu.u, seen_col = col, seen_phys = p;
+    }
+    const int phys = seen_phys;
     const int64_t row0 = ((int64_t)phys * w.nkv + cu.h) * a.bs + (tok0 - col * a.bs);
     const uint64_t addr = reinterpret_cast<uint64_t>(a.k) + (uint64_t)row0 * ROW_BYTES;
     const char *src = reinterpret_cast<const char *>(address_from_words(
@@ -405,10 +412,10 @@ __global__ __launch_bounds__(256, 1) void paged_decode_latent16_kernel(
 #pragma unroll
     for (int k = 0; k + 4 <= L::NDMA; k += 4) {
       const uint32_t off[4] = {src_off[k], src_off[k + 1], src_off[k + 2], src_off[k + 3]};
-      dma16_quad(bases, off, dst + 1024u * k);
+      dma16_streaming_quad(bases, off, dst + 1024u * k);
     }
 #pragma unroll
-    for (int k = L::NDMA / 4 * 4; k < L::NDMA; ++k) dma16(src, src_off[k], dst + 1024u * k);
+    for (int k = L::NDMA / 4 * 4; k < L::NDMA; ++k) dma16_streaming(src, src_off[k], dst + 1024u * k);
   };
   // Rows past the attended length may be cache rows nobody ever wrote: their scores are masked,
   // but as V rows they would turn 0 * Inf into NaN, so they are cleared in LDS.
