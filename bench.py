@@ -49,9 +49,10 @@ MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
     # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
     # the rotating workload copies; the summaries under profiles/ hold the runs)
-    "config2": ("paged_decode_mfma16_kernel", "a88126b215c90579", 311719985),
-    "config5": ("paged_decode_mfma16_kernel", "a88126b215c90579", 168854438),
-    "config3": ("prefill_kernel", "c9602929cb330d80", 234209088),
+    "config2": ("paged_decode_mfma16_kernel", "0ce82103339e6a76", 311711749),
+    "config5": ("paged_decode_mfma16_kernel", "0ce82103339e6a76", 168848210),
+    "config3": ("prefill_kernel", "0e6012ae2521a65c", 234204866),
+    "latent": ("paged_decode_latent16_kernel", "e9406c499974ed2e", 678500460),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}
