@@ -10,7 +10,8 @@ steps never touch the same cache lines.
 
 Other workloads (same JSON contract):
   config4  Llama-3-70B-shaped decode, batch 128, context 256..32768, fragmented pool
-           (its 4 x 512-token chunked-prefill pass is timed separately, see "chunk_pass")
+           (its 4 x 512-token chunked-prefill pass is timed separately, see "chunk_pass";
+           config5 carries one too: 4 x 512-token chunks over 2048 tokens of block-float-8 cache)
   config5  config2 with a block-float-8 KV cache (dequantised inside the decode kernel)
   config3  causal prefill, 4 x 2048 tokens: K fill + V fill + MFMA attention; value is
            useful TFLOP/s
@@ -139,10 +140,28 @@ def decode_step(g):
         g.q, g.k_cache, g.v_cache, g.k_new, g.v_new, g.page_table, g.cache_position, scale=g.scale)
 
 
-def make_prefill_impl(w):
+def make_prefill_impl(w, kv_cache_dtype="auto"):
     from tt_xla_amd import TTAttentionBackendImpl
 
-    return TTAttentionBackendImpl(w.q_heads, w.head_size, w.head_size**-0.5, w.kv_heads, None, None, "auto")
+    return TTAttentionBackendImpl(w.q_heads, w.head_size, w.head_size**-0.5, w.kv_heads, None, None, kv_cache_dtype)
+
+
+def time_chunk_pass(w, args, kv_cache_dtype="auto"):
+    """A chunked-prefill pass of the backend (fill of the chunk's K / V rows + attention over the cached
+    prefix and the chunk), timed as steps and as its attention kernel."""
+    import torch
+
+    impl = make_prefill_impl(w, kv_cache_dtype)
+    outbuf = torch.empty_like(w.q)
+    chunk = [lambda: prefill_step(impl, w, outbuf)]
+    cms = time_steps(StepRunner(chunk, args.launch == "graph", args.steps_per_graph), min(args.steps, 50), 5)
+    cd = time_dominant_kernel(chunk, 20)
+    ck = sum(x for x, _ in cd) / len(cd)
+    return {
+        "workload": w.name, "ms_per_pass": cms, "attention_kernel_us": ck * 1e3,
+        "useful_tflops": w.useful_flops() / (ck * 1e-3) / 1e12,
+        "frac_of_bf16_mfma_peak": w.useful_flops() / (ck * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+    }
 
 
 def prefill_step(impl, w, out):
@@ -444,18 +463,15 @@ def run_decode(args):
     if args.workload == "config4":
         from tt_xla_amd import workloads
 
-        w = workloads.prefill_config4_chunks(device=dev).to(dev)
-        impl = make_prefill_impl(w)
-        outbuf = torch.empty_like(w.q)
-        chunk = [lambda: prefill_step(impl, w, outbuf)]
-        cms = time_steps(StepRunner(chunk, args.launch == "graph", args.steps_per_graph), min(args.steps, 50), 5)
-        cd = time_dominant_kernel(chunk, 20)
-        ck = sum(x for x, _ in cd) / len(cd)
-        out["chunk_pass"] = {
-            "workload": w.name, "ms_per_pass": cms, "attention_kernel_us": ck * 1e3,
-            "useful_tflops": w.useful_flops() / (ck * 1e-3) / 1e12,
-            "frac_of_bf16_mfma_peak": w.useful_flops() / (ck * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-        }
+        out["chunk_pass"] = time_chunk_pass(workloads.prefill_config4_chunks(device=dev).to(dev), args)
+    if args.workload == "config5":
+        from tt_xla_amd import workloads
+
+        # the chunked-prefill pass over the same kind of cache: 4 x 512-token chunks on 2048 cached tokens
+        w = workloads.prefill_workload("config5-chunks-b4x512-start2048-h32x8-d128-bs64-bfp8", 55, 4, 512, 32, 8,
+                                       128, 64, 2048, dev).to(dev)
+        w.k_cache, w.v_cache = ops.bfp8_pack_cache(w.k_cache), ops.bfp8_pack_cache(w.v_cache)
+        out["chunk_pass"] = time_chunk_pass(w, args, "uint8")
     return out
 
 
@@ -583,8 +599,9 @@ def secondary_runs(args):
         r = run_prefill(sub) if wl == "config3" else run_decode(sub)
         keep = {k: r[k] for k in ("metric", "value", "unit", "steps", "warmup", "ms_per_step", "dtype", "roofline")}
         keep["workload"] = r["config"]["workload"]
-        if "pct_of_hbm_peak" in r:
-            keep["pct_of_hbm_peak"] = r["pct_of_hbm_peak"]
+        for extra in ("pct_of_hbm_peak", "chunk_pass"):
+            if extra in r:
+                keep[extra] = r[extra]
         out[wl] = keep
     gc.collect()
     torch.cuda.empty_cache()
