@@ -8,9 +8,14 @@
 //   a[16 k .. 16 k + 15], k = 0 .. 7    output accumulator k = half * DBLK + output block
 //   a[128 + 4 k .. + 3], k = 0 .. 15    Q fragment k = half * KSTEPS + k-step
 // The compiler never sees them as operands.  reserve_accumulation_registers() lists them as
-// clobbered once, which makes the kernel descriptor allocate them; nothing else in these
-// kernels lives in accumulation registers (they stay far below 256 vector registers, and
-// the build checks that the compiler emitted no accumulation-register move of its own).
+// clobbered once, which makes the kernel descriptor allocate them.  That reserves NOTHING: a
+// compiler short of vector registers parks its own values in accumulation registers, these
+// included, between two statements of the loop (seen in a 32-row variant of the loop built for
+// two wavefronts per SIMD, where a wavefront has 128 vector registers: wrong outputs, then a
+// memory fault from the addresses parked there).  The kernels of the 64-row form are safe because,
+// with 256 vector registers to themselves, the compiler generates no access to an accumulation
+// register of its own in them; tests/test_prefill_acc_regs.py checks exactly that on the
+// device assembly, and has to keep passing for every kernel that includes this file.
 // Every statement is `asm volatile`: they keep their order among themselves.
 #pragma once
 #include <cstdint>
