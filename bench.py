@@ -52,7 +52,7 @@ MEASURED_TRAFFIC = {
     # the rotating workload copies; the summaries under profiles/ hold the runs)
     "config2": ("paged_decode_mfma16_kernel", "0ce82103339e6a76", 311711749),
     "config5": ("paged_decode_mfma16_kernel", "0ce82103339e6a76", 168848210),
-    "config3": ("prefill_kernel", "0e6012ae2521a65c", 234204866),
+    "config3": ("prefill_kernel", "a709fcceeae2965a", 234132431),
     "latent": ("paged_decode_latent16_kernel", "e9406c499974ed2e", 678500460),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
