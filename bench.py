@@ -50,10 +50,10 @@ MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
     # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
     # the rotating workload copies; the summaries under profiles/ hold the runs)
-    "config2": ("paged_decode_mfma16_kernel", "0ce82103339e6a76", 311711749),
-    "config5": ("paged_decode_mfma16_kernel", "0ce82103339e6a76", 168848210),
+    "config2": ("paged_decode_mfma16_kernel", "de87f18b9bb9b272", 311087101),
+    "config5": ("paged_decode_mfma16_kernel", "de87f18b9bb9b272", 168848210),
     "config3": ("prefill_kernel", "a709fcceeae2965a", 234132431),
-    "latent": ("paged_decode_latent16_kernel", "e9406c499974ed2e", 678500460),
+    "latent": ("paged_decode_latent16_kernel", "427116ee0858dac2", 678500460),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}

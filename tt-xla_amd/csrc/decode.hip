@@ -286,15 +286,15 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   process_tile(std::false_type{});
 }
 
-int waves_for_device(int kv_format) {
-  // TTPA_DECODE_WAVES_PER_CU (read on every call) overrides the grid size: tests use a small
-  // grid to give every wavefront several tiles and segments
+int waves_for_device(double default_per_cu) {
+  // TTPA_DECODE_WAVES_PER_CU (read on every call, fractions allowed) overrides the grid size: tests
+  // use a small grid to give every wavefront several tiles and segments
   const char *e = getenv("TTPA_DECODE_WAVES_PER_CU");
-  const int override_waves = e ? atoi(e) : 0;
-  int per_cu = override_waves > 0 ? override_waves : (kv_format == TTPA_KV_BFP8 ? 8 : 4);
+  const double override_waves = e ? atof(e) : 0.0;
+  const double per_cu = override_waves > 0 ? override_waves : default_per_cu;
   int cus = device_cus();
   if (cus <= 0) cus = 256;
-  int waves = cus * per_cu;
+  const int waves = (int)(cus * per_cu + 0.5);
   return (waves + kWavesPerBlock - 1) / kWavesPerBlock * kWavesPerBlock;
 }
 
@@ -343,11 +343,14 @@ int launch_g(const DecodeArgs &a, int g, hipStream_t st) {
 using namespace ttpa;
 using namespace ttpa::decode;
 
+// wavefronts per CU of the largest grid a decode launch uses (the VALU kernel on a block-float-8 cache)
+static constexpr double kLargestGrid = 8.0;
+
 extern "C" size_t ttpa_paged_decode_workspace_bytes(int32_t users, int32_t q_heads,
                                                     int32_t kv_heads, int32_t head_size) {
   if (users <= 0 || q_heads <= 0 || kv_heads <= 0 || head_size <= 0 || q_heads % kv_heads) return 0;
   int g = q_heads / kv_heads;
-  size_t slots = (size_t)waves_for_device(TTPA_KV_BFP8) + (size_t)users * kv_heads;  // the larger grid
+  size_t slots = (size_t)waves_for_device(kLargestGrid) + (size_t)users * kv_heads;  // the larger grid
   return header_bytes(users, kv_heads) + slots * (size_t)slot_floats_for(g, head_size) * sizeof(float);
 }
 
@@ -445,10 +448,19 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   if (forced == 1 && g <= 8 && !(kv_format == TTPA_KV_BFP8 && head_size == 256)) use_mfma = use_mfma16 = false;
   if (forced == 2 && mfma_ok) use_mfma = true, use_mfma16 = false;
   if (forced == 3 && mfma16_ok) use_mfma16 = true, use_mfma = false;
-  // The matrix-core kernels get one workgroup per CU whatever the cache format: the 32x32 kernel
-  // fills the CU's LDS with one, and the 16x16 kernel streams as fast with one as with the two
-  // that would fit, while twice the partials cost the merge kernel more.
-  a.n_waves = waves_for_device((use_mfma || use_mfma16) ? TTPA_KV_BF16 : kv_format);
+  // The matrix-core kernels get at most one workgroup per CU whatever the cache format: the 32x32
+  // kernel fills the CU's LDS with one, and the 16x16 kernel streams as fast with one as with the
+  // two that would fit, while twice the partials cost the merge kernel more.  On a bfloat16 cache
+  // the 16x16 kernel is fastest with three quarters of the CUs (measured in one process, grids of
+  // 2.5 ... 4 wavefronts per CU: 56.0-56.9 us per step at 2.75 ... 3.75 against 57.3-57.7 at 4 on
+  // the 32-user workload, 531 against 544 us on the 128-user one: the streams of 192 workgroups
+  // already hold the memory system's latency in bytes, and every further wavefront is one more
+  // partial and one more share in the contention); on a block-float-8 cache it wants all of them
+  // (50.4 against 43.9 us).
+  a.n_waves = waves_for_device(use_mfma16 && kv_format == TTPA_KV_BF16 ? 3.0
+                               : (use_mfma || use_mfma16)               ? 4.0
+                               : kv_format == TTPA_KV_BFP8              ? kLargestGrid
+                                                                        : 4.0);
   // one thread of the main grid per segment publishes the segment's partial slots
   if ((int64_t)users * kv_heads > (int64_t)a.n_waves * kWave)
     return fail(TTPA_ERR_UNSUPPORTED, "decode: %d x %d segments need a grid of more than %d wavefronts",

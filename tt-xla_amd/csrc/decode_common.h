@@ -415,7 +415,7 @@ inline int slot_floats_for(int g, int d) { return ((g * d + 2 * g + 3) / 4) * 4;
 inline size_t header_bytes(int users, int hkv) { return (((size_t)users * hkv * 8 + 255) / 256) * 256; }
 
 
-int waves_for_device(int kv_format);
+int waves_for_device(double default_per_cu);
 constexpr int kWavesPerBlockHost = kWavesPerBlock;
 
 // Launches the block-float-8 VALU main kernel (decode_bfp8.hip); false = shape not built.
