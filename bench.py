@@ -42,7 +42,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 # of the kernel sources it was measured on (the first 16 hex digits of the SHA-256 over the files
 # listed): when the sources have changed since, `roofline.traffic` is null instead of stale.
 KERNEL_SOURCES = {
-    "paged_decode_mfma16_kernel": ["decode_mfma16_kernel.h", "decode_common.h", "common.h"],
+    "paged_decode_mfma16_kernel": ["decode_mfma16_kernel.h", "decode_common.h", "common.h", "decode.hip"],  # the grid rule is in decode.hip
     "paged_decode_latent16_kernel": ["decode_wide.hip", "decode_common.h", "common.h"],
     "prefill_kernel": ["prefill.hip", "prefill_acc_regs.h", "common.h"],
 }
@@ -50,8 +50,9 @@ MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
     # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
     # the rotating workload copies; the summaries under profiles/ hold the runs)
-    "config2": ("paged_decode_mfma16_kernel", "de87f18b9bb9b272", 311087101),
-    "config5": ("paged_decode_mfma16_kernel", "de87f18b9bb9b272", 168848210),
+    "config2": ("paged_decode_mfma16_kernel", "9922548835d1bf49", 311087101),
+    "config5": ("paged_decode_mfma16_kernel", "9922548835d1bf49", 168848210),
+    "config4": ("paged_decode_mfma16_kernel", "9922548835d1bf49", 3444648636),
     "config3": ("prefill_kernel", "a709fcceeae2965a", 234132431),
     "latent": ("paged_decode_latent16_kernel", "427116ee0858dac2", 678500460),
 }
