@@ -286,6 +286,12 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   process_tile(std::false_type{});
 }
 
+int segment_units(int default_units) {
+  const char *e = getenv("TTPA_DECODE_SEG_UNITS");
+  const int v = e ? atoi(e) : default_units;
+  return v < 0 ? 0 : (v > 64 ? 64 : v);
+}
+
 int waves_for_device(double default_per_cu) {
   // TTPA_DECODE_WAVES_PER_CU (read on every call, fractions allowed) overrides the grid size: tests
   // use a small grid to give every wavefront several tiles and segments
@@ -461,6 +467,13 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
                                : (use_mfma || use_mfma16)               ? 4.0
                                : kv_format == TTPA_KV_BFP8              ? kLargestGrid
                                                                         : 4.0);
+  // Ranges of the 16x16 kernel are equal in units of one tile, with one unit in front of every
+  // segment: a change of segment inside a range (partial, search, next Q rows) costs a wavefront
+  // about what a tile costs, and the slowest wavefront ends the launch.  Measured in one process,
+  // 0 / 1 / 2 units: 56.4 / 54.9 / 55.1 us per step on the 32-user workload, 44.4 / 42.3 / 42.9 on
+  // its block-float-8 form, 534 / 520 / 519 on the 128-user one.  TTPA_DECODE_SEG_UNITS (read on
+  // every call) overrides.
+  a.seg_units = use_mfma16 ? segment_units(1) : 0;
   // one thread of the main grid per segment publishes the segment's partial slots
   if ((int64_t)users * kv_heads > (int64_t)a.n_waves * kWave)
     return fail(TTPA_ERR_UNSUPPORTED, "decode: %d x %d segments need a grid of more than %d wavefronts",

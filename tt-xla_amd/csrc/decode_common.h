@@ -32,6 +32,11 @@ struct DecodeArgs {
   int slot_floats;
   int kv_format;
   int window;         // > 0: only the last `window` positions up to cur_pos are attended
+  // Units of the flat list that stand in front of the tiles of every non-empty segment and carry
+  // no work: they charge the wavefront that opens a segment inside its range for what a change
+  // of segment costs (its partial, the search, the next Q rows), so that equal ranges of units
+  // take about equal time.  0: the list holds tiles only.
+  int seg_units = 0;
   const float *sink;  // [q_heads] extra logit per head in the softmax denominator, or null
   // Fused cache update (16x16x32 kernel only): the token at cur_pos of every user is taken from
   // k_new / v_new [users][>= hkv heads][head_size] instead of the cache, and written to it.
@@ -56,11 +61,12 @@ __device__ __forceinline__ int tiles_of_user(const DecodeArgs &a, const void *__
   return (int)((l + TILE - 1) / TILE) - window_lo(a, len) / TILE;
 }
 
-// Exclusive prefix sum of per-user tile counts into pref[0..users] and attended lengths into
-// lens[0..users); all 256 threads.  Each position is read from global memory once.
+// Exclusive prefix sum of per-user unit counts (tiles, plus `extra` for a user that has any) into
+// pref[0..users] and attended lengths into lens[0..users); all 256 threads.  Each position is read
+// from global memory once.
 template <int TILE = kTile>
 __device__ inline void build_prefix(const DecodeArgs &a, const void *__restrict__ cur, int *pref,
-                             int *lens, int *wave_sums) {
+                             int *lens, int *wave_sums, int extra = 0) {
   const int tid = threadIdx.x;
   const int per = (a.users + 255) / 256;
   const int beg = tid * per;
@@ -69,6 +75,7 @@ __device__ inline void build_prefix(const DecodeArgs &a, const void *__restrict_
   for (int u = beg; u < end; ++u) {
     int len;
     int nt = tiles_of_user<TILE>(a, cur, u, len);
+    if (nt > 0) nt += extra;  // units per segment of this user
     lens[u] = len;
     pref[u + 1] = nt;  // replaced by the running sum below
     local += nt;
@@ -237,9 +244,12 @@ struct Cursor {
 
 // Finds the segment that owns unit `x` of the flat tile list (binary search over the
 // per-user prefix in LDS).  Everything is wavefront-uniform.
+// With `extra` leading units per segment, a unit among them stands for the segment's first tile;
+// `x_tile` receives the unit of the tile found.
 template <int TILE = kTile>
 __device__ __forceinline__ Cursor locate_unit(const DecodeArgs &a, const int *s_pref,
-                                              const int *s_len, int64_t x) {
+                                              const int *s_len, int64_t x, int extra = 0,
+                                              int64_t *x_tile = nullptr) {
   const int users = a.users, hkv = a.hkv;
   int lo_u = 0, hi_u = users - 1;
   while (lo_u < hi_u) {
@@ -250,10 +260,12 @@ __device__ __forceinline__ Cursor locate_unit(const DecodeArgs &a, const int *s_
   Cursor cu;
   cu.u = lo_u;
   const int pref_u = __builtin_amdgcn_readfirstlane(s_pref[lo_u]);
-  const int nt = __builtin_amdgcn_readfirstlane(s_pref[lo_u + 1]) - pref_u;
+  const int nv = __builtin_amdgcn_readfirstlane(s_pref[lo_u + 1]) - pref_u;  // units per segment
+  const int nt = nv - extra;
   const int rem = (int)(x - (int64_t)pref_u * hkv);
-  cu.h = rem / nt;
-  const int rel = rem - cu.h * nt;
+  cu.h = rem / nv;
+  const int rel = max(rem - cu.h * nv - extra, 0);
+  if (x_tile) *x_tile = (int64_t)pref_u * hkv + (int64_t)cu.h * nv + extra + rel;
   cu.tiles_left = nt - rel;
   cu.len = __builtin_amdgcn_readfirstlane(s_len[lo_u]);
   cu.lo = window_lo(a, cu.len);
@@ -286,15 +298,15 @@ __device__ __forceinline__ float sum_over_quads(float v) {
 // One thread per segment (the first blocks of the grid): publishes which partial slots the
 // merge kernel has to read for that segment.
 __device__ __forceinline__ void publish_segment_row(const DecodeArgs &a, const int *s_pref,
-                                                    int64_t total, int n_eff) {
+                                                    int64_t total, int n_eff, int extra = 0) {
   const int seg = blockIdx.x * 256 + threadIdx.x;
   if (seg >= a.users * a.hkv) return;
   const int su = seg / a.hkv, sh = seg - su * a.hkv;
-  const int snt = s_pref[su + 1] - s_pref[su];
+  const int snv = s_pref[su + 1] - s_pref[su];  // units per segment: `extra` in front of the tiles
   int first = 0, count = 0;
-  if (snt > 0) {
-    const int64_t x0 = (int64_t)s_pref[su] * a.hkv + (int64_t)sh * snt;
-    const int64_t x1 = x0 + snt - 1;
+  if (snv > 0) {
+    const int64_t x0 = (int64_t)s_pref[su] * a.hkv + (int64_t)sh * snv + extra;  // first tile
+    const int64_t x1 = x0 + (snv - extra) - 1;                                   // last tile
     // wave owning unit x: largest w with floor(w * total / n_eff) <= x; every wave in
     // [w0, w1] owns at least one unit of the segment because n_eff <= total
     const int w0 = (int)(((x0 + 1) * n_eff + total - 1) / total) - 1;
@@ -350,10 +362,12 @@ __device__ __forceinline__ void write_partial(float *slot, int g, int G, int r, 
 // dependent round trips, and this keeps it at two.  G and D are run-time values: the
 // matrix-core kernels serve any group width up to 32.  D is a power of two on the attention
 // paths (64, 128, 256: split by shift and mask); the latent path also has 384 (divided).
-// Grid: x = segment, y = piece of kCombinePiece of the segment's G * D output elements (one piece
-// for the plain decode shapes; a latent segment of 16 heads x 512 values is 16 pieces, and as one
-// workgroup per segment its merge took as long as the attention itself).
-constexpr int kCombinePiece = 512;
+// Grid: x = segment, y = piece of kCombinePiece of the segment's G * D output elements: one
+// element per thread, so a thread's loads are one batch in flight (two pieces for the Llama-3-8B
+// decode shape, whose step is 0.7 us shorter than with one piece of 512; a latent segment of
+// 16 heads x 512 values is 32 pieces, and as one workgroup per segment its merge took as long as
+// the attention itself).
+constexpr int kCombinePiece = 256;
 inline int combine_pieces(int g, int d) { return (g * d + kCombinePiece - 1) / kCombinePiece; }
 
 __global__ inline __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a, int G, int D) {
@@ -416,6 +430,8 @@ inline size_t header_bytes(int users, int hkv) { return (((size_t)users * hkv * 
 
 
 int waves_for_device(double default_per_cu);
+// Units in front of every segment of the flat list (TTPA_DECODE_SEG_UNITS overrides, 0 ... 64).
+int segment_units(int default_units);
 constexpr int kWavesPerBlockHost = kWavesPerBlock;
 
 // Launches the block-float-8 VALU main kernel (decode_bfp8.hip); false = shape not built.

@@ -153,22 +153,27 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   __shared__ int s_wsum[kWavesPerBlock];
   extern __shared__ __attribute__((aligned(16))) uint8_t tiles[];
 
-  build_prefix<TILE>(a, cur_pos, s_pref, s_len, s_wsum);
+  const int seg_units = a.seg_units;
+  build_prefix<TILE>(a, cur_pos, s_pref, s_len, s_wsum, seg_units);
 
   const int lane = threadIdx.x & 63;
   const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 15, quad = lane >> 4;
   const int wave = blockIdx.x * kWavesPerBlock + wib;
-  const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
-  const int64_t total = (int64_t)total_tiles * a.hkv;
-  const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);
+  // The flat list in units: per segment `seg_units` units that stand for the cost of opening it,
+  // then its tiles.  A range of more than seg_units units holds at least one tile.
+  const int total_units = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
+  const int64_t total = (int64_t)total_units * a.hkv;
+  const int64_t max_ranges = total / (seg_units + 1);
+  const int n_eff = (int)(max_ranges < a.n_waves ? max_ranges : a.n_waves);
   if constexpr (FUSED) write_negative_position<BFP8, D>(a, page_table, cur_pos, blockIdx.x * 256 + threadIdx.x);
   if (total == 0 || wave >= n_eff) {
-    publish_segment_row(a, s_pref, total, n_eff);
+    publish_segment_row(a, s_pref, total, n_eff, seg_units);
     return;
   }
-  int64_t x = (int64_t)wave * total / n_eff;
+  const int64_t x_lo = (int64_t)wave * total / n_eff;
   const int64_t x_hi = (int64_t)(wave + 1) * total / n_eff;
+  int64_t x = x_lo;  // set below to the unit of the first tile at or behind x_lo
   uint8_t *tile = tiles + wib * kTileBytes;
   const int G = a.hq / a.hkv;
 
@@ -213,7 +218,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
       vr[db] = (uint32_t)(vrow * ROWB + (((2 * db + xx) ^ vkey(vrow)) << 4) + 8 * (n & 1));
   }
 
-  auto locate = [&](int64_t xx) { return locate_unit<TILE>(a, s_pref, s_len, xx); };
+  auto locate = [&](int64_t xx) { return locate_unit<TILE>(a, s_pref, s_len, xx, seg_units); };
   // `bad`: bit i set where run i's block lies outside the table or the cache (it reads block 0)
   auto tile_offsets = [&](const Cursor &cu, int64_t (&eo)[NOFF], int64_t (&xo)[NOFF], uint32_t &bad) {
     bad = 0;
@@ -366,7 +371,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     }
   };
 
-  Cursor cur = locate(x);
+  Cursor cur = locate_unit<TILE>(a, s_pref, s_len, x_lo, seg_units, &x);
   int64_t eo[NOFF], xo[NOFF];
   u32x4 kraw[NL], vraw[NL];
   uint32_t kex[NL], vex[NL];
@@ -381,7 +386,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     vfresh = fetch_fresh(a.v_new, cur);
   }
   load_q(cur, qf);
-  publish_segment_row(a, s_pref, total, n_eff);
+  publish_segment_row(a, s_pref, total, n_eff, seg_units);
 
   floatx4 acc[DBLK];
 #pragma unroll
@@ -564,9 +569,11 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
       }
     }
     cur = nxt;
-    ++x;
+    x += same_seg ? 1 : 1 + seg_units;
   };
-  while (x + 1 < x_hi) process_tile(std::true_type{});
+  // the unit of the tile behind the current one: the next, or behind the next segment's leading units
+  auto next_tile_unit = [&]() { return x + (cur.tiles_left > 1 ? 1 : 1 + seg_units); };
+  while (next_tile_unit() < x_hi) process_tile(std::true_type{});
   process_tile(std::false_type{});
 }
 

@@ -340,7 +340,8 @@ __global__ __launch_bounds__(256, 1) void paged_decode_latent16_kernel(
   __shared__ int s_wsum[kWavesPerBlock];
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
-  build_prefix<TILE>(a, cur_pos, s_pref, s_len, s_wsum);
+  const int seg_units = a.seg_units;
+  build_prefix<TILE>(a, cur_pos, s_pref, s_len, s_wsum, seg_units);
 
   const int lane = threadIdx.x & 63;
   const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -378,15 +379,19 @@ __global__ __launch_bounds__(256, 1) void paged_decode_latent16_kernel(
   constexpr int KPRE = KSTEPS < 8 ? KSTEPS : 8;  // fragments in flight (an LDS read takes a few hundred cycles)
   constexpr int VPRE = VB < 12 ? VB : 12;
   const int wave = blockIdx.x * kWavesPerBlock + wib;
-  const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
-  const int64_t total = (int64_t)total_tiles * a.hkv;
-  const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);
+  // The flat list in units: per segment `seg_units` units that stand for the cost of opening it,
+  // then its tiles.  A range of more than seg_units units holds at least one tile.
+  const int total_units = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
+  const int64_t total = (int64_t)total_units * a.hkv;
+  const int64_t max_ranges = total / (seg_units + 1);
+  const int n_eff = (int)(max_ranges < a.n_waves ? max_ranges : a.n_waves);
   if (total == 0 || wave >= n_eff) {
-    publish_segment_row(a, s_pref, total, n_eff);
+    publish_segment_row(a, s_pref, total, n_eff, seg_units);
     return;
   }
-  int64_t x = (int64_t)wave * total / n_eff;
+  const int64_t x_lo = (int64_t)wave * total / n_eff;
   const int64_t x_hi = (int64_t)(wave + 1) * total / n_eff;
+  int64_t x = x_lo;  // set below to the unit of the first tile at or behind x_lo
   const int G = w.gseg;
   unsigned char *my_lds = smem + wib * L::WAVE_LDS;
 
@@ -437,24 +442,26 @@ __global__ __launch_bounds__(256, 1) void paged_decode_latent16_kernel(
     }
   };
 
-  Cursor cur = locate_unit<TILE>(a, s_pref, s_len, x);
+  Cursor cur = locate_unit<TILE>(a, s_pref, s_len, x_lo, seg_units, &x);
   bf16x8 qf[KSTEPS];
   issue_tile(cur, 0);
   load_q(cur, qf);
-  publish_segment_row(a, s_pref, total, n_eff);
+  publish_segment_row(a, s_pref, total, n_eff, seg_units);
 
   floatx4 acc[VB];
 #pragma unroll
   for (int i = 0; i < VB; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
 
-  for (int it = 0; x < x_hi; ++x, ++it) {
+  for (int it = 0; x < x_hi; ++it) {
     const int buf = it & 1;
     unsigned char *stage = my_lds + buf * L::STAGE;
     const int nvalid = cur.len - cur.t * TILE;
     const bool partial = nvalid < TILE;
     const int nbelow = cur.lo - cur.t * TILE;
-    const bool has_next = x + 1 < x_hi;
+    // the unit of the tile behind this one: the next, or behind the next segment's leading units
+    const int64_t x_next = x + (cur.tiles_left > 1 ? 1 : 1 + seg_units);
+    const bool has_next = x_next < x_hi;
     const bool same_seg = has_next && cur.tiles_left > 1;
 
     // The next tile is requested BEFORE this one is waited for (its stage has been idle since the
@@ -468,7 +475,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_latent16_kernel(
         nxt.t = cur.t + 1;
         nxt.tiles_left = cur.tiles_left - 1;
       } else {
-        nxt = locate_unit<TILE>(a, s_pref, s_len, x + 1);
+        nxt = locate_unit<TILE>(a, s_pref, s_len, x + 1, seg_units);
       }
       issue_tile(nxt, buf ^ 1);
       __builtin_amdgcn_s_waitcnt((L::NDMA & 15) | 0x0F70 | ((L::NDMA >> 4) << 14));  // vmcnt(NDMA)
@@ -563,6 +570,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_latent16_kernel(
       if (has_next) load_q(nxt, qf);
     }
     cur = nxt;
+    x = x_next;
   }
 }
 
@@ -619,7 +627,7 @@ extern "C" size_t ttpa_paged_mla_decode_workspace_bytes(int32_t users, int32_t q
   if (cus <= 0) cus = 256;
   const size_t segs = (size_t)users * kv_heads * nhb;
   const size_t slot = (size_t)slot_floats_for(gseg, head_dim_v) * sizeof(float);
-  // one slot per range of the larger grid (four wavefront ranges per CU in the 16-head form)
+  // one slot per range of the largest grid (at most four wavefront ranges per CU in the 16-head form)
   return header_bytes(users, kv_heads * nhb) + ((size_t)cus * kWavesPerBlockHost + segs) * slot;
 }
 
@@ -694,7 +702,13 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
   const char *force = getenv("TTPA_LATENT_KERNEL");
   const bool want16 = shared && nhb == 1 && gseg <= 16 && block_size % 16 == 0 && !(force && force[0] == 'w');
   if (want16) {
-    a.n_waves = cus * kWavesPerBlockHost;
+    // three wavefront ranges per CU: 131 us per step on the 128-user workload against 134 at four
+    // (fewer partials of 32 KiB each), 139 at 2.5 and 159 at two; TTPA_DECODE_WAVES_PER_CU overrides,
+    // up to the four per CU that the workspace is sized for
+    a.n_waves = std::min(cus * kWavesPerBlockHost, waves_for_device(3.0));
+    // three units in front of every segment of the flat list (a partial here is 32 KiB, a tile
+    // 18 KiB): 130 us per step against 131-134 with none
+    a.seg_units = segment_units(3);
     bool have = true;
     if (head_size == 576 && head_dim_v == 512) ok = launch_latent16<576, 512>(a, w, st);
     else if (head_size == 576 && head_dim_v == 384) ok = launch_latent16<576, 384>(a, w, st);
@@ -709,6 +723,7 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
       return check_launch("paged_mla_decode");
     }
     a.n_waves = cus;
+    a.seg_units = 0;
   }
 #define TTPA_WIDE_CASE(DQK, DVW)                                                                   \
   if (head_size == DQK && dvw == DVW)                                                              \
