@@ -50,11 +50,11 @@ MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
     # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
     # the rotating workload copies; the summaries under profiles/ hold the runs)
-    "config2": ("paged_decode_mfma16_kernel", "9922548835d1bf49", 311087101),
-    "config5": ("paged_decode_mfma16_kernel", "9922548835d1bf49", 168848210),
-    "config4": ("paged_decode_mfma16_kernel", "9922548835d1bf49", 3444648636),
+    "config2": ("paged_decode_mfma16_kernel", "2a8b24417a69da26", 311092795),
+    "config5": ("paged_decode_mfma16_kernel", "2a8b24417a69da26", 168807640),
+    "config4": ("paged_decode_mfma16_kernel", "2a8b24417a69da26", 3444653293),
     "config3": ("prefill_kernel", "a709fcceeae2965a", 234132431),
-    "latent": ("paged_decode_latent16_kernel", "427116ee0858dac2", 678500460),
+    "latent": ("paged_decode_latent16_kernel", "9d6f8cf3c9aed2fa", 668460502),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}
