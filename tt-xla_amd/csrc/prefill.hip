@@ -460,7 +460,7 @@ __device__ __forceinline__ void rows64_loop(const PrefillArgs &a,
 // as the LDS delivers in the time the matrix pipes need for that tile), and half as many
 // workgroups pay the start-up and the store.
 template <int RH>
-constexpr int prefill_wgs_per_cu(int d, int mode) { return RH == 1 && d <= 128 && mode != 4 ? 2 : 1; }
+constexpr int prefill_wgs_per_cu(int d, int mode) { return RH == 1 && d <= 128 ? 2 : 1; }
 
 template <int D, int HPW, int MODE, int RH>
 __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_kernel(PrefillArgs a) {
@@ -732,8 +732,12 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
 
   constexpr int NK = 2 * KSTEPS;  // K fragments per tile
   constexpr int NV = 4 * DBLK;    // V^T fragments per tile
-  constexpr int KPRE = 6;         // K fragments in flight
-  constexpr int VPRE = 4;         // V^T fragments in flight
+  // Fragments in flight.  Mode 4 holds a K and a V tile's bytes in registers across the iteration
+  // and keeps the rings short: with 6 and 4 it spills 17 registers at two workgroups per CU (head
+  // size 128), with 4 and 2 none, and the second workgroup is worth 224 -> 136 us on a pass of
+  // four 512-token chunks over 2048 cached tokens.
+  constexpr int KPRE = MODE == 4 ? 4 : 6;  // K fragments
+  constexpr int VPRE = MODE == 4 ? 2 : 4;  // V^T fragments
 
   // ntiles >= 1 always (row 0 sees key 0).
   const int last_tile = ntiles - 1;
