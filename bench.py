@@ -53,7 +53,7 @@ MEASURED_TRAFFIC = {
     "config2": ("paged_decode_mfma16_kernel", "2a8b24417a69da26", 311092795),
     "config5": ("paged_decode_mfma16_kernel", "2a8b24417a69da26", 168807640),
     "config4": ("paged_decode_mfma16_kernel", "2a8b24417a69da26", 3444653293),
-    "config3": ("prefill_kernel", "a709fcceeae2965a", 234132431),
+    "config3": ("prefill_kernel", "b3d3733fd88ea3b8", 234139507),
     "latent": ("paged_decode_latent16_kernel", "9d6f8cf3c9aed2fa", 668460502),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
