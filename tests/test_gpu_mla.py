@@ -68,6 +68,28 @@ def test_paged_flash_mla_decode(users, hq, nkv, dh, dv, has_value, bs, width, sc
     _check(f"mla decode u{users} h{hq}x{nkv} dh{dh} dv{dv} bs{bs}", got, want)
 
 
+@pytest.mark.parametrize("partials", ["f32", "bf16"])
+@pytest.mark.parametrize("dv", [512, 384])
+def test_mla_decode_16_heads_either_partial_format(monkeypatch, partials, dv):
+    """The 16-head latent kernel hands its partial outputs to the merge as bfloat16 by default and
+    as floats under TTPA_LATENT_PARTIALS=f32: both against the oracle, on a small grid (a quarter
+    wavefront per CU) so that every user's context is cut into several partials."""
+    monkeypatch.setenv("TTPA_LATENT_PARTIALS", partials)
+    monkeypatch.setenv("TTPA_DECODE_WAVES_PER_CU", "0.25")
+    users, hq, dh, bs, width = 5, 16, 576, 32, 40
+    print(f"case: mla decode partials={partials} u{users} h{hq} dh{dh} dv{dv} bs{bs} w{width}", flush=True)
+    g = torch.Generator().manual_seed(1000 + dv)
+    nb = width * users
+    q = _bf(g, 1, users, hq, dh)
+    key = _bf(g, nb, 1, bs, dh)
+    table = torch.randperm(nb, generator=g).view(users, width).to(torch.int32)
+    pos = torch.tensor([width * bs - 1, 700, 5, 1279, 64], dtype=torch.int32)
+    got = torch.ops.tt.paged_flash_mla_decode(q.cuda(), key.cuda(), dv, table.cuda(), None, True, None,
+                                              pos.cuda(), None, None).cpu()
+    want = O.paged_flash_mla_decode(q, key, dv, table, None, pos, None)
+    _check(f"mla decode partials={partials} dv{dv}", got, want)
+
+
 def test_mla_decode_padded_row_sink_and_errors():
     g = torch.Generator().manual_seed(3)
     users, hq, dh, dv, bs, width = 3, 16, 576, 512, 32, 8

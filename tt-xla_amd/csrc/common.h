@@ -53,6 +53,14 @@ __device__ __forceinline__ float bf16_hi(uint32_t w) {
   return __builtin_bit_cast(float, w & 0xffff0000u);
 }
 
+// two floats -> packed bfloat16 pair (lo in the low half), round to nearest even
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef float float_pair __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16_pair __attribute__((ext_vector_type(2)));
+  const float_pair f = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16_pair));
+}
+
 // float -> bfloat16 bits, round to nearest even (NaN stays NaN).
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   uint32_t u = __builtin_bit_cast(uint32_t, f);

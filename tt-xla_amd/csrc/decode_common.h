@@ -37,6 +37,9 @@ struct DecodeArgs {
   // of segment costs (its partial, the search, the next Q rows), so that equal ranges of units
   // take about equal time.  0: the list holds tiles only.
   int seg_units = 0;
+  // Partial outputs stored as bfloat16 (16-head latent kernel: a partial there is 16 heads x 512
+  // values): a slot is G * D bfloat16 values, then G running maxima and G running sums as floats.
+  int partial_bf16 = 0;
   const float *sink;  // [q_heads] extra logit per head in the softmax denominator, or null
   // Fused cache update (16x16x32 kernel only): the token at cur_pos of every user is taken from
   // k_new / v_new [users][>= hkv heads][head_size] instead of the cache, and written to it.
@@ -425,7 +428,63 @@ __global__ inline __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a
   }
 }
 
+// The same merge over partials whose values are bfloat16 (DecodeArgs::partial_bf16): a thread owns
+// two neighbouring output elements, one 32-bit word of every partial, and stores them as one word
+// (the caller checks that output rows start on 4-byte boundaries).  Grid: x = segment, y = piece
+// of kCombinePiece element pairs.
+__global__ inline __launch_bounds__(256) void decode_combine_bf16_kernel(DecodeArgs a, int G, int D) {
+  const int seg = blockIdx.x;
+  const int pairs = G * D / 2;
+  const int p = blockIdx.y * kCombinePiece + threadIdx.x;
+  if (p >= pairs) return;
+  const int u = seg / a.hkv, h = seg % a.hkv;
+  const int i = 2 * p, g = i / D, e = i - g * D;
+  const int first = a.ws_seg[2 * seg], nw = a.ws_seg[2 * seg + 1];
+  uint32_t *out = reinterpret_cast<uint32_t *>(a.out + u * a.out_us + (int64_t)(h * G + g) * a.out_hs + e);
+  if (nw == 0) {  // padded row: no attended position -> NaN like softmax over nothing
+    *out = 0x7fc07fc0u;
+    return;
+  }
+  constexpr int kBatch = 8;
+  const float *base = a.ws_slots + (int64_t)first * a.slot_floats;
+  float mall = -INFINITY, num0 = 0.f, num1 = 0.f, den = 0.f;
+  for (int w = 0; w < nw; w += kBatch) {
+    float mv[kBatch], lv[kBatch];
+    uint32_t av[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const float *sl = base + (int64_t)min(w + j, nw - 1) * a.slot_floats;
+      mv[j] = (w + j < nw) ? sl[pairs + g] : -INFINITY;
+      lv[j] = sl[pairs + G + g];
+      av[j] = reinterpret_cast<const uint32_t *>(sl)[p];
+    }
+    float mnew = mall;
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) mnew = fmaxf(mnew, mv[j]);
+    const float resc = __builtin_amdgcn_exp2f(mall - mnew);
+    num0 *= resc, num1 *= resc, den *= resc;
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const float wgt = __builtin_amdgcn_exp2f(mv[j] - mnew);  // 0 for the padding entries
+      num0 = fmaf(wgt, bf16_lo(av[j]), num0);
+      num1 = fmaf(wgt, bf16_hi(av[j]), num1);
+      den = fmaf(wgt, lv[j], den);
+    }
+    mall = mnew;
+  }
+  if (a.sink) {
+    const float sk = a.sink[h * G + g] * 1.4426950408889634f;
+    const float mnew = fmaxf(mall, sk);
+    const float resc = __builtin_amdgcn_exp2f(mall - mnew);
+    num0 *= resc, num1 *= resc;
+    den = den * resc + __builtin_amdgcn_exp2f(sk - mnew);
+  }
+  *out = f32_to_bf16_bits(num0 / den) | (f32_to_bf16_bits(num1 / den) << 16);
+}
+
 inline int slot_floats_for(int g, int d) { return ((g * d + 2 * g + 3) / 4) * 4; }
+// the same with the values as bfloat16 (g * d even)
+inline int slot_floats_bf16_for(int g, int d) { return ((g * d / 2 + 2 * g + 3) / 4) * 4; }
 inline size_t header_bytes(int users, int hkv) { return (((size_t)users * hkv * 8 + 255) / 256) * 256; }
 
 

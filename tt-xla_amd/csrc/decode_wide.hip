@@ -554,13 +554,25 @@ __global__ __launch_bounds__(256, 1) void paged_decode_latent16_kernel(
       float *slot = a.ws_slots + ((int64_t)wave + (int64_t)cur.u * a.hkv + cur.h) * a.slot_floats;
       const float l_tot = sum_over_quads(l_run);
       if (n < G) {
-        float *dst = slot + n * DV + 4 * quad;
+        if (a.partial_bf16) {  // wavefront-uniform
+          uint32_t *dst = reinterpret_cast<uint32_t *>(slot) + (n * DV + 4 * quad) / 2;
 #pragma unroll
-        for (int vb = 0; vb < VB; ++vb)
-          *reinterpret_cast<float4 *>(dst + 16 * vb) = make_float4(acc[vb][0], acc[vb][1], acc[vb][2], acc[vb][3]);
-        if (quad == 0) {
-          slot[G * DV + n] = m_run;
-          slot[G * DV + G + n] = l_tot;
+          for (int vb = 0; vb < VB; ++vb)
+            *reinterpret_cast<uint2 *>(dst + 8 * vb) =
+                make_uint2(pack_bf16x2(acc[vb][0], acc[vb][1]), pack_bf16x2(acc[vb][2], acc[vb][3]));
+          if (quad == 0) {
+            slot[G * DV / 2 + n] = m_run;
+            slot[G * DV / 2 + G + n] = l_tot;
+          }
+        } else {
+          float *dst = slot + n * DV + 4 * quad;
+#pragma unroll
+          for (int vb = 0; vb < VB; ++vb)
+            *reinterpret_cast<float4 *>(dst + 16 * vb) = make_float4(acc[vb][0], acc[vb][1], acc[vb][2], acc[vb][3]);
+          if (quad == 0) {
+            slot[G * DV + n] = m_run;
+            slot[G * DV + G + n] = l_tot;
+          }
         }
       }
 #pragma unroll
@@ -709,6 +721,13 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
     // three units in front of every segment of the flat list (a partial here is 32 KiB, a tile
     // 18 KiB): 130 us per step against 131-134 with none
     a.seg_units = segment_units(3);
+    // partials as bfloat16 (TTPA_LATENT_PARTIALS=f32, read on every call, keeps floats): half the
+    // bytes written here and read by the merge
+    const char *pf = getenv("TTPA_LATENT_PARTIALS");
+    // (the merge then stores output pairs as words: rows on 4-byte boundaries)
+    a.partial_bf16 = !(pf && pf[0] == 'f') && out_user_stride % 2 == 0 && out_head_stride % 2 == 0 &&
+                     reinterpret_cast<uintptr_t>(out) % 4 == 0;
+    if (a.partial_bf16) a.slot_floats = slot_floats_bf16_for(gseg, head_dim_v);
     bool have = true;
     if (head_size == 576 && head_dim_v == 512) ok = launch_latent16<576, 512>(a, w, st);
     else if (head_size == 576 && head_dim_v == 384) ok = launch_latent16<576, 384>(a, w, st);
@@ -719,11 +738,16 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
       if (!ok) return fail(TTPA_ERR_LAUNCH, "latent decode: cannot configure the kernel");
       if (ev1) (void)hipEventRecord(ev1, st);
       if (int rc = check_launch("paged_mla_decode")) return rc;
-      decode_combine_kernel<<<dim3(users * kv_heads, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+      if (a.partial_bf16)
+        decode_combine_bf16_kernel<<<dim3(users * kv_heads, combine_pieces(gseg, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+      else
+        decode_combine_kernel<<<dim3(users * kv_heads, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
       return check_launch("paged_mla_decode");
     }
     a.n_waves = cus;
     a.seg_units = 0;
+    a.partial_bf16 = 0;
+    a.slot_floats = slot_floats_for(gseg, head_dim_v);
   }
 #define TTPA_WIDE_CASE(DQK, DVW)                                                                   \
   if (head_size == DQK && dvw == DVW)                                                              \
