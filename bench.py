@@ -50,11 +50,11 @@ MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
     # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
     # the rotating workload copies; the summaries under profiles/ hold the runs)
-    "config2": ("paged_decode_mfma16_kernel", "e0544a1ba3466af1", 311092608),
-    "config5": ("paged_decode_mfma16_kernel", "e0544a1ba3466af1", 168806426),
-    "config4": ("paged_decode_mfma16_kernel", "e0544a1ba3466af1", 3444654255),
+    "config2": ("paged_decode_mfma16_kernel", "bcd1c63630416cb6", 311092057),
+    "config5": ("paged_decode_mfma16_kernel", "bcd1c63630416cb6", 168806756),
+    "config4": ("paged_decode_mfma16_kernel", "bcd1c63630416cb6", 3444655083),
     "config3": ("prefill_kernel", "6e6361ba6cb9745e", 234146442),
-    "latent": ("paged_decode_latent16_kernel", "489772a6bf7e481f", 654097976),
+    "latent": ("paged_decode_latent16_kernel", "489772a6bf7e481f", 654098077),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}

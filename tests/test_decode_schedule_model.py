@@ -1,5 +1,5 @@
 """Host-side model of the split-K schedule of the decode kernels (tt-xla_amd/csrc/decode_common.h:
-build_prefix, locate_unit, publish_segment_row; the range walk of decode_mfma16_kernel.h).
+build_prefix, locate_unit, publish_segment_row; the range walk that every decode kernel repeats).
 
 The flat list holds, per (user, kv head) segment with at least one tile, `extra` leading units that
 carry no work and then the segment's tiles; it is cut into n_eff equal ranges of units.  The model

@@ -218,21 +218,22 @@ def test_decode_several_tiles_per_wavefront(monkeypatch, kernel, hq, d):
 
 @pytest.mark.parametrize("seg_units", ["0", "1", "3"])
 @pytest.mark.parametrize("waves", ["0.25", "1", "3"])
-def test_decode_ranges_weighted_by_segment_changes(monkeypatch, seg_units, waves):
-    """The 16x16x32 kernel cuts the flat list into ranges of units, with `seg_units` units in front
+@pytest.mark.parametrize("kernel,hq", [("mfma16", 32), ("mfma", 64), ("valu", 8)])
+def test_decode_ranges_weighted_by_segment_changes(monkeypatch, seg_units, waves, kernel, hq):
+    """The decode kernels cut the flat list into ranges of units, with `seg_units` units in front
     of every segment's tiles (tests/test_decode_schedule_model.py holds the arithmetic): short and
     long segments, a padded user and one tile per user, on grids where a wavefront crosses many
     segments (a quarter wavefront per CU) and where most wavefronts hold a single tile."""
     from tt_xla_amd import workloads
 
-    monkeypatch.setenv("TTPA_DECODE_KERNEL", "mfma16")
+    monkeypatch.setenv("TTPA_DECODE_KERNEL", kernel)
     monkeypatch.setenv("TTPA_DECODE_WAVES_PER_CU", waves)
     monkeypatch.setenv("TTPA_DECODE_SEG_UNITS", seg_units)
     ctx = [5, 700, 31, 32, 33, 1200, 0, 64, 95, 257]
-    name = f"decode [mfma16] h32x8 d128 seg_units={seg_units} waves/CU={waves} ctx{ctx}"
+    name = f"decode [{kernel}] h{hq}x8 d128 seg_units={seg_units} waves/CU={waves} ctx{ctx}"
     print(name, flush=True)
     nb = sum((c + 1 + 63) // 64 for c in ctx) + 3
-    wl = workloads.decode_ragged(name, 93, len(ctx), 32, 8, 128, 64, nb, ctx)
+    wl = workloads.decode_ragged(name, 93, len(ctx), hq, 8, 128, 64, nb, ctx)
     got, k, v = _run(wl)
     _check(name, got,
            O.textbook_decode_fp32(wl.q, k.cpu(), v.cpu(), wl.page_table, wl.cache_position, wl.scale))

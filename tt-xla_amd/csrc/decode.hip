@@ -47,19 +47,24 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   // probabilities of one tile as bfloat16: [wave][lane row r][head g][16 loads]
   __shared__ __attribute__((aligned(16))) uint16_t s_p[kWavesPerBlock][4 * G * 16];
 
-  build_prefix(a, cur_pos, s_pref, s_len, s_wsum);
+  const int seg_units = a.seg_units;
+  build_prefix(a, cur_pos, s_pref, s_len, s_wsum, seg_units);
   const int lane = threadIdx.x & 63;
   const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane >> 4, c = lane & 15;
   const int wave = blockIdx.x * kWavesPerBlock + wib;
-  const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
-  const int64_t total = (int64_t)total_tiles * a.hkv;
-  const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);  // waves that get work
+  // The flat list in units: per segment `seg_units` units that stand for the cost of opening it,
+  // then its tiles.  A range of more than seg_units units holds at least one tile.
+  const int total_units = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
+  const int64_t total = (int64_t)total_units * a.hkv;
+  const int64_t max_ranges = total / (seg_units + 1);
+  const int n_eff = (int)(max_ranges < a.n_waves ? max_ranges : a.n_waves);  // wavefronts that get work
   if (total == 0 || wave >= n_eff) {  // idle wavefronts still do their share of the table
-    publish_segment_row(a, s_pref, total, n_eff);
+    publish_segment_row(a, s_pref, total, n_eff, seg_units);
     return;
   }
-  int64_t x = (int64_t)wave * total / n_eff;
+  const int64_t x_lo = (int64_t)wave * total / n_eff;
+  int64_t x = x_lo;  // set below to the unit of the first tile at or behind x_lo
   const int64_t x_hi = (int64_t)(wave + 1) * total / n_eff;
   lds_u16 *plds = s_p[wib];
   const int my_step = bitrev4(c);
@@ -68,7 +73,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
   const uint32_t lane_bytes = (uint32_t)(r * D + c * EPL) * 2u;
 
   // ---- helpers (all uniform across the wavefront) ---------------------------------
-  auto locate = [&](int64_t xx) { return locate_unit(a, s_pref, s_len, xx); };
+  auto locate = [&](int64_t xx) { return locate_unit(a, s_pref, s_len, xx, seg_units); };
   // element offset (relative to the cache base) of the first row of each 4-row load
   auto tile_offsets = [&](const Cursor &cu, int64_t (&off)[NOFF]) {
     const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
@@ -126,14 +131,14 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
                         q[g][hf]);
   };
 
-  Cursor cur = locate(x);
+  Cursor cur = locate_unit(a, s_pref, s_len, x_lo, seg_units, &x);
   int64_t off[NOFF];
   uint32_t kreg[NH][16][DW], q[G][NH][DW];
   tile_offsets(cur, off);
   load_tile(kb, off, kreg);
   load_q(cur, q);
 
-  publish_segment_row(a, s_pref, total, n_eff);  // hidden behind the first tile's latency
+  publish_segment_row(a, s_pref, total, n_eff, seg_units);  // hidden behind the first tile's latency
 
   float m[G], l[G], acc[G][NH][EPL];
 #pragma unroll
@@ -280,9 +285,11 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(
     cur = nxt;
 #pragma unroll
     for (int i = 0; i < NOFF; ++i) off[i] = noff[i];
-    ++x;
+    x += same_seg ? 1 : 1 + seg_units;
   };
-  while (x + 1 < x_hi) process_tile(std::true_type{});
+  // the unit of the tile behind the current one: the next, or behind the next segment's leading units
+  auto next_tile_unit = [&]() { return x + (cur.tiles_left > 1 ? 1 : 1 + seg_units); };
+  while (next_tile_unit() < x_hi) process_tile(std::true_type{});
   process_tile(std::false_type{});
 }
 
@@ -467,13 +474,15 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
                                : (use_mfma || use_mfma16)               ? 4.0
                                : kv_format == TTPA_KV_BFP8              ? kLargestGrid
                                                                         : 4.0);
-  // Ranges of the 16x16 kernel are equal in units of one tile, with one unit in front of every
+  // Ranges are equal in units of one tile, with units that carry no work in front of every
   // segment: a change of segment inside a range (partial, search, next Q rows) costs a wavefront
   // about what a tile costs, and the slowest wavefront ends the launch.  Measured in one process,
-  // 0 / 1 / 2 units: 56.4 / 54.9 / 55.1 us per step on the 32-user workload, 44.4 / 42.3 / 42.9 on
-  // its block-float-8 form, 534 / 520 / 519 on the 128-user one.  TTPA_DECODE_SEG_UNITS (read on
-  // every call) overrides.
-  a.seg_units = use_mfma16 ? segment_units(1) : 0;
+  // 0 / 1 / 2 units with the 16x16 kernel: 56.4 / 54.9 / 55.1 us per step on the 32-user workload,
+  // 44.4 / 42.3 / 42.9 on its block-float-8 form, 534 / 520 / 519 on the 128-user one.  The 32x32
+  // kernel wants two (32 users of 64 / 2 heads, contexts 512 ... 4096: 33.3 / 33.2 / 31.6 / 31.5 /
+  // 32.0 us at 0 / 1 / 2 / 3 / 4), the VALU kernels none (8 / 8 heads: 52.1 / 53.3 / 53.8 us at
+  // 0 / 1 / 2).  TTPA_DECODE_SEG_UNITS (read on every call) overrides.
+  a.seg_units = segment_units(use_mfma16 ? 1 : use_mfma ? 2 : 0);
   // one thread of the main grid per segment publishes the segment's partial slots
   if ((int64_t)users * kv_heads > (int64_t)a.n_waves * kWave)
     return fail(TTPA_ERR_UNSUPPORTED, "decode: %d x %d segments need a grid of more than %d wavefronts",

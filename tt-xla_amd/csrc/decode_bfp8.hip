@@ -48,20 +48,25 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_kernel(
   __shared__ int s_wsum[kWavesPerBlock];
   __shared__ __attribute__((aligned(16))) uint16_t s_p[kWavesPerBlock][4 * G * 16];
 
-  build_prefix(a, cur_pos, s_pref, s_len, s_wsum);
+  const int seg_units = a.seg_units;
+  build_prefix(a, cur_pos, s_pref, s_len, s_wsum, seg_units);
 
   const int lane = threadIdx.x & 63;
   const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane >> 4, c = lane & 15;
   const int wave = blockIdx.x * kWavesPerBlock + wib;
-  const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
-  const int64_t total = (int64_t)total_tiles * a.hkv;
-  const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);
+  // The flat list in units: per segment `seg_units` units that stand for the cost of opening it,
+  // then its tiles.  A range of more than seg_units units holds at least one tile.
+  const int total_units = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
+  const int64_t total = (int64_t)total_units * a.hkv;
+  const int64_t max_ranges = total / (seg_units + 1);
+  const int n_eff = (int)(max_ranges < a.n_waves ? max_ranges : a.n_waves);  // wavefronts that get work
   if (total == 0 || wave >= n_eff) {
-    publish_segment_row(a, s_pref, total, n_eff);
+    publish_segment_row(a, s_pref, total, n_eff, seg_units);
     return;
   }
-  int64_t x = (int64_t)wave * total / n_eff;
+  const int64_t x_lo = (int64_t)wave * total / n_eff;
+  int64_t x = x_lo;  // set below to the unit of the first tile at or behind x_lo
   const int64_t x_hi = (int64_t)(wave + 1) * total / n_eff;
   lds_u16 *plds = s_p[wib];
   const int my_step = bitrev4(c);
@@ -70,7 +75,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_kernel(
   const uint32_t lane_exp = (uint32_t)(r * GPR + grp);
   const int64_t slab_bytes = (int64_t)(a.bs + a.bs / 16) * D;  // one (block, head) slab
 
-  auto locate = [&](int64_t xx) { return locate_unit(a, s_pref, s_len, xx); };
+  auto locate = [&](int64_t xx) { return locate_unit(a, s_pref, s_len, xx, seg_units); };
   // byte offsets of the element rows / exponent rows of each 4-row load of a tile
   auto tile_offsets = [&](const Cursor &cu, int64_t (&eo)[NOFF], int64_t (&xo)[NOFF]) {
     const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
@@ -118,13 +123,13 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_kernel(
     for (int w = 0; w < RW; ++w) expand4(raw[w], out[2 * w], out[2 * w + 1]);
   };
 
-  Cursor cur = locate(x);
+  Cursor cur = locate_unit(a, s_pref, s_len, x_lo, seg_units, &x);
   int64_t eo[NOFF], xo[NOFF];
   uint32_t kraw[16][RW], kex[16], q[G][DW];
   tile_offsets(cur, eo, xo);
   load_tile(a.k, eo, xo, kraw, kex);
   load_q(cur, q);
-  publish_segment_row(a, s_pref, total, n_eff);
+  publish_segment_row(a, s_pref, total, n_eff, seg_units);
 
   float m[G], l[G], acc[G][1][EPL];
 #pragma unroll
@@ -266,9 +271,11 @@ __global__ __launch_bounds__(256, 2) void paged_decode_bfp8_kernel(
     cur = nxt;
 #pragma unroll
     for (int i = 0; i < NOFF; ++i) eo[i] = neo[i], xo[i] = nxo[i];
-    ++x;
+    x += same_seg ? 1 : 1 + seg_units;
   };
-  while (x + 1 < x_hi) process_tile(std::true_type{});
+  // the unit of the tile behind the current one: the next, or behind the next segment's leading units
+  auto next_tile_unit = [&]() { return x + (cur.tiles_left > 1 ? 1 : 1 + seg_units); };
+  while (next_tile_unit() < x_hi) process_tile(std::true_type{});
   process_tile(std::false_type{});
 }
 

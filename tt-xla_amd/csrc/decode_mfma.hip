@@ -72,20 +72,25 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
   __shared__ int s_wsum[kWavesPerBlock];
   extern __shared__ __attribute__((aligned(16))) uint16_t tiles[];
 
-  build_prefix(a, cur_pos, s_pref, s_len, s_wsum);
+  const int seg_units = a.seg_units;
+  build_prefix(a, cur_pos, s_pref, s_len, s_wsum, seg_units);
 
   const int lane = threadIdx.x & 63;
   const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int wave = blockIdx.x * kWavesPerBlock + wib;
-  const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
-  const int64_t total = (int64_t)total_tiles * a.hkv;
-  const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);
+  // The flat list in units: per segment `seg_units` units that stand for the cost of opening it,
+  // then its tiles.  A range of more than seg_units units holds at least one tile.
+  const int total_units = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
+  const int64_t total = (int64_t)total_units * a.hkv;
+  const int64_t max_ranges = total / (seg_units + 1);
+  const int n_eff = (int)(max_ranges < a.n_waves ? max_ranges : a.n_waves);  // wavefronts that get work
   if (total == 0 || wave >= n_eff) {
-    publish_segment_row(a, s_pref, total, n_eff);
+    publish_segment_row(a, s_pref, total, n_eff, seg_units);
     return;
   }
-  int64_t x = (int64_t)wave * total / n_eff;
+  const int64_t x_lo = (int64_t)wave * total / n_eff;
+  int64_t x = x_lo;  // set below to the unit of the first tile at or behind x_lo
   const int64_t x_hi = (int64_t)(wave + 1) * total / n_eff;
   uint16_t *ks = tiles + wib * (kTile * (KS + VS));
   uint16_t *vs = ks + kTile * KS;
@@ -101,7 +106,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
   const uint32_t exp_shift = (uint32_t)(8 * ((sr * GPR + sc) & 3));
   const int64_t slab = BFP8 ? (int64_t)(a.bs + a.bs / 16) * D : (int64_t)a.bs * D * 2;  // bytes
 
-  auto locate = [&](int64_t xx) { return locate_unit(a, s_pref, s_len, xx); };
+  auto locate = [&](int64_t xx) { return locate_unit(a, s_pref, s_len, xx, seg_units); };
   auto tile_offsets = [&](const Cursor &cu, int64_t (&eo)[NOFF], int64_t (&xo)[NOFF]) {
     const int32_t *pt_row = page_table + (int64_t)cu.u * a.pt_rs;
     const int tok0 = cu.t * kTile;
@@ -204,7 +209,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
     }
   };
 
-  Cursor cur = locate(x);
+  Cursor cur = locate_unit(a, s_pref, s_len, x_lo, seg_units, &x);
   int64_t eo[NOFF], xo[NOFF];
   u32x4 kraw[NL], vraw[NL];
   uint32_t kex[NL], vex[NL];
@@ -213,7 +218,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
   fetch(a.k, eo, xo, kraw, kex);
   fetch(a.v, eo, xo, vraw, vex);
   load_q(cur, qf);
-  publish_segment_row(a, s_pref, total, n_eff);
+  publish_segment_row(a, s_pref, total, n_eff, seg_units);
 
   floatx16 acc[DBLK];
 #pragma unroll
@@ -403,9 +408,11 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
       if constexpr (has_next) load_q(nxt, qf);
     }
     cur = nxt;
-    ++x;
+    x += same_seg ? 1 : 1 + seg_units;
   };
-  while (x + 1 < x_hi) process_tile(std::true_type{});
+  // the unit of the tile behind the current one: the next, or behind the next segment's leading units
+  auto next_tile_unit = [&]() { return x + (cur.tiles_left > 1 ? 1 : 1 + seg_units); };
+  while (next_tile_unit() < x_hi) process_tile(std::true_type{});
   process_tile(std::false_type{});
 }
 
