@@ -16,8 +16,8 @@ Other workloads (same JSON contract):
   config3  causal prefill, 4 x 2048 tokens: K fill + V fill + MFMA attention; value is
            useful TFLOP/s
 
-Prints ONE JSON line.  `roofline` is the dominant kernel alone, bracketed by HIP events
-inside the library; `cpu_baseline` is the CPU oracle timed on this box's host cores on a
+Prints ONE JSON line.  `roofline` is the dominant kernel alone, timed by a HIP event
+pair that its launch carries inside the library; `cpu_baseline` is the CPU oracle timed on this box's host cores on a
 bounded sample of the same workload.
 """
 
@@ -50,11 +50,11 @@ MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
     # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
     # the rotating workload copies; the summaries under profiles/ hold the runs)
-    "config2": ("paged_decode_mfma16_kernel", "bcd1c63630416cb6", 311092057),
-    "config5": ("paged_decode_mfma16_kernel", "bcd1c63630416cb6", 168806756),
-    "config4": ("paged_decode_mfma16_kernel", "bcd1c63630416cb6", 3444655083),
-    "config3": ("prefill_kernel", "6e6361ba6cb9745e", 234146442),
-    "latent": ("paged_decode_latent16_kernel", "489772a6bf7e481f", 654098077),
+    "config2": ("paged_decode_mfma16_kernel", "eecd11f58c0c0deb", 311093154),
+    "config5": ("paged_decode_mfma16_kernel", "eecd11f58c0c0deb", 168806152),
+    "config4": ("paged_decode_mfma16_kernel", "eecd11f58c0c0deb", 3444653863),
+    "config3": ("prefill_kernel", "caf4dfdc8092f655", 234149651),
+    "latent": ("paged_decode_latent16_kernel", "33cba915f8ae781e", 654097757),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}
@@ -278,7 +278,7 @@ def time_dominant_kernel(fns, iters):
 def time_decode_kernel_direct(copies, iters):
     """The decode kernel alone (the one the step runs: cache update inside), driven through the
     C ABI with preallocated output and workspace: the host enqueues far faster than the GPU executes, so the stream never runs
-    dry and the armed event pair brackets the kernel the way a kernel trace does.  Returns
+    dry and the armed event pair, which the kernel's launch carries, reads what a kernel trace reads.  Returns
     [(milliseconds, copy index)]."""
     import torch
 

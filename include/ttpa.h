@@ -265,10 +265,12 @@ int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t out_head_s
 
 /*
  * Measurement hook, no reference counterpart: the NEXT attention call made by this host
- * thread (decode or prefill) records `before` and `after` (hipEvent_t, as void*) on its
- * stream immediately around its dominant kernel (the split-K main kernel for decode, the
- * MFMA kernel for prefill), then forgets them.  Pass NULLs to clear.  Used by bench.py to
- * time that kernel alone, the way a profiler's kernel trace does.
+ * thread (decode or prefill) attaches `before` and `after` (hipEvent_t, as void*) to the
+ * launch of its dominant kernel (the split-K main kernel for decode, the MFMA kernel for
+ * prefill), so that they hold the dispatch's own begin and end timestamps, then forgets
+ * them (the VALU, 32x32 and workgroup-shared latent kernels record them on the stream in
+ * front of and behind the launch instead).  Pass NULLs to clear.  Used by bench.py to time
+ * that kernel alone, the way a profiler's kernel trace does.
  */
 int ttpa_profile_next_attention(void *before, void *after);
 

@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include <atomic>
@@ -18,8 +19,22 @@ int check_launch(const char *what);
 int device_cus();
 
 // Events armed by ttpa_profile_next_attention(); take_profile_events() hands them to the
-// launcher that brackets its dominant kernel and disarms them.
+// launcher that times its dominant kernel and disarms them.
 void take_profile_events(hipEvent_t &before, hipEvent_t &after);
+
+// Launches a call's dominant kernel.  Armed events ride on the dispatch itself, so they read the
+// kernel's own begin and end timestamps (what a profiler reports for the dispatch) and not the
+// gaps in front of and behind it, which events recorded around a launch include.
+template <typename... Params, typename... Args>
+inline void launch_dominant(void (*kernel)(Params...), dim3 grid, dim3 block, size_t lds, hipStream_t st,
+                            Args... args) {
+  hipEvent_t before, after;
+  take_profile_events(before, after);
+  if (before)
+    hipExtLaunchKernelGGL(kernel, grid, block, static_cast<uint32_t>(lds), st, before, after, 0u, args...);
+  else
+    kernel<<<grid, block, lds, st>>>(args...);
+}
 
 // Raises the dynamic-LDS limit of `kernel` to `bytes` on the current device, once per device:
 // `done_devices` is the call site's own record (one bit per device ordinal; ordinals from 64

@@ -504,8 +504,10 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
       return rc;
     }
   }
-  hipEvent_t ev0, ev1;
-  take_profile_events(ev0, ev1);
+  // armed profile events: the 16x16 kernel's launch carries them itself; the other kernels are
+  // bracketed here
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  if (!use_mfma16) take_profile_events(ev0, ev1);
   if (ev0) (void)hipEventRecord(ev0, st);
   int rc = TTPA_OK;
   if (use_mfma16) {
@@ -522,6 +524,7 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
     }
   }
   if (ev1) (void)hipEventRecord(ev1, st);
+  if (use_mfma16) take_profile_events(ev0, ev1);  // still armed only if the launch did not happen
   if (rc) return rc;
   decode_combine_kernel<<<dim3(users * kv_heads, combine_pieces(g, head_size)), dim3(256), 0, st>>>(a, g, head_size);
   return check_launch("paged_sdpa_decode");

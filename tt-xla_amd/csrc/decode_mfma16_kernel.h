@@ -585,7 +585,7 @@ bool launch(const DecodeArgs &a, hipStream_t st) {
   if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_mfma16_kernel<D, BFP8, RUNS, FUSED>), lds,
                           lds_ready))
     return false;
-  paged_decode_mfma16_kernel<D, BFP8, RUNS, FUSED><<<dim3(blocks), dim3(256), lds, st>>>(a, a.pt, a.cur);
+  launch_dominant(&paged_decode_mfma16_kernel<D, BFP8, RUNS, FUSED>, dim3(blocks), dim3(256), lds, st, a, a.pt, a.cur);
   return true;
 }
 

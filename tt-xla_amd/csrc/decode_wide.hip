@@ -593,7 +593,7 @@ bool launch_latent16(const DecodeArgs &a, const WideArgs &w, hipStream_t st) {
   static std::atomic<uint64_t> lds_ready{0};
   if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_latent16_kernel<DQK, DV>), lds, lds_ready))
     return false;
-  paged_decode_latent16_kernel<DQK, DV><<<dim3(a.n_waves / kWavesPerBlock), dim3(256), lds, st>>>(a, w, a.pt, a.cur);
+  launch_dominant(&paged_decode_latent16_kernel<DQK, DV>, dim3(a.n_waves / kWavesPerBlock), dim3(256), lds, st, a, w, a.pt, a.cur);
   return true;
 }
 
@@ -704,9 +704,9 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
   w.nkv = kv_heads, w.nhb = nhb, w.gseg = gseg, w.dv = head_dim_v, w.n_slices = head_dim_v / dvw;
 
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipEvent_t ev0, ev1;
-  take_profile_events(ev0, ev1);
-  if (ev0) (void)hipEventRecord(ev0, st);
+  // armed profile events: the 16-head kernel's launch carries them itself; the workgroup-shared
+  // kernel is bracketed below
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
   bool ok = false, built = true;
   const bool shared = v_cache == nullptr;
   // The 16-head form: V taken from K, one head block of up to 16 heads, tiles inside one block.
@@ -735,8 +735,8 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
     else if (head_size == 128 && head_dim_v == 128) ok = launch_latent16<128, 128>(a, w, st);
     else have = false;
     if (have) {
+      take_profile_events(ev0, ev1);  // still armed only if the launch did not happen
       if (!ok) return fail(TTPA_ERR_LAUNCH, "latent decode: cannot configure the kernel");
-      if (ev1) (void)hipEventRecord(ev1, st);
       if (int rc = check_launch("paged_mla_decode")) return rc;
       if (a.partial_bf16)
         decode_combine_bf16_kernel<<<dim3(users * kv_heads, combine_pieces(gseg, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
@@ -749,6 +749,8 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
     a.partial_bf16 = 0;
     a.slot_floats = slot_floats_for(gseg, head_dim_v);
   }
+  take_profile_events(ev0, ev1);
+  if (ev0) (void)hipEventRecord(ev0, st);
 #define TTPA_WIDE_CASE(DQK, DVW)                                                                   \
   if (head_size == DQK && dvw == DVW)                                                              \
     ok = shared ? launch<DQK, DVW, true>(a, w, st) : launch<DQK, DVW, false>(a, w, st);            \

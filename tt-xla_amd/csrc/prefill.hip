@@ -993,9 +993,6 @@ int launch_mode(const PrefillArgs &a, hipStream_t st) {
   static std::atomic<uint64_t> lds_ready{0};
   if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&prefill_kernel<D, HPW, MODE, RH>), lds, lds_ready))
     return fail(TTPA_ERR_LAUNCH, "prefill: cannot reserve %zu bytes of LDS", lds);
-  hipEvent_t ev0, ev1;
-  take_profile_events(ev0, ev1);
-  if (ev0) (void)hipEventRecord(ev0, st);
   const int ny8 = (a.batch * (a.hq / HPW) + 7) / 8;
   int grid = nqt * ny8 * 8;
   PrefillArgs b = a;
@@ -1012,8 +1009,7 @@ int launch_mode(const PrefillArgs &a, hipStream_t st) {
     // slots past the last real one exit at once (the kernel's range check)
     grid = ag >= fg ? grid + 8 * fg : 16 * fg;
   }
-  prefill_kernel<D, HPW, MODE, RH><<<dim3(grid), dim3(256), lds, st>>>(b);
-  if (ev1) (void)hipEventRecord(ev1, st);
+  launch_dominant(&prefill_kernel<D, HPW, MODE, RH>, dim3(grid), dim3(256), lds, st, b);
   return check_launch("sdpa_prefill");
 }
 
