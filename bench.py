@@ -50,11 +50,11 @@ MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
     # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
     # the rotating workload copies; the summaries under profiles/ hold the runs)
-    "config2": ("paged_decode_mfma16_kernel", "eecd11f58c0c0deb", 311093154),
-    "config5": ("paged_decode_mfma16_kernel", "eecd11f58c0c0deb", 168806152),
-    "config4": ("paged_decode_mfma16_kernel", "eecd11f58c0c0deb", 3444653863),
+    "config2": ("paged_decode_mfma16_kernel", "44709186f461ba13", 311091953),
+    "config5": ("paged_decode_mfma16_kernel", "44709186f461ba13", 168806899),
+    "config4": ("paged_decode_mfma16_kernel", "44709186f461ba13", 3444653748),
     "config3": ("prefill_kernel", "caf4dfdc8092f655", 234149651),
-    "latent": ("paged_decode_latent16_kernel", "33cba915f8ae781e", 654097757),
+    "latent": ("paged_decode_latent16_kernel", "33cba915f8ae781e", 654097655),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}

@@ -31,8 +31,11 @@ namespace ttpa {
 namespace decode {
 
 // BIG = block_size is a multiple of 64: a tile lies inside one physical block.
+// The grid is one workgroup per CU, so a second resident workgroup is asked of the register
+// allocator only where it costs nothing: from five query heads per KV head at head size 128, and
+// at head size 256, 256 registers spill (4 ... 864 of them) where 512 hold everything.
 template <int D, int G, bool BIG>
-__global__ __launch_bounds__(256, 2) void paged_decode_kernel(
+__global__ __launch_bounds__(256, (D <= 128 && G <= 4) ? 2 : 1) void paged_decode_kernel(
     DecodeArgs a, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
   // page_table / cur_pos are separate restrict parameters so that their wavefront-uniform
   // reads become scalar loads: a vector load + readfirstlane would have to wait for every
