@@ -25,6 +25,7 @@
 // when fragments are read.
 #include "common.h"
 #include "prefill_acc_regs.h"
+#include "build/prefill_stream_asm.h"
 
 #include <cstdlib>
 
@@ -71,6 +72,7 @@ struct PrefillArgs {
   int window;  // > 0 (causal only): row i attends keys offset + i - window < j <= offset + i
   float scale_log2e;
   int kv_bfp8;  // paged form: the caches are block-float-8 (mode 4)
+  int stream;   // run whole unmasked tiles through the hand-scheduled loop (stream_tiles)
 };
 
 // key / block_size without a division instruction sequence (about 30 instructions each, and the
@@ -433,6 +435,34 @@ __device__ __forceinline__ void rows64_loop(const PrefillArgs &a,
       }
     }
   });
+}
+
+// ---------------------------------------------------------------------------------------------
+// The hand-scheduled loop over whole unmasked tiles (head size 128, 32 rows per wavefront): one
+// block of assembly, written by gen_prefill_stream.py, which documents the schedule and the
+// state on entry and exit.  Everything the block touches is bound to the registers its text
+// names; the compiler moves values in and out around it and keeps its own out of the clobbered
+// ones.  Entered with K(0), V(0), K(1) requested and K(0) published; handles tiles 0 .. n - 1.
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+
+struct StreamState {
+  floatx16 acc[4];
+  float mc, lrun;  // reference of the probabilities (exponent domain), row sum
+};
+
+__device__ __forceinline__ void stream_tiles(StreamState &st, const u32x16 &q_lo, const u32x16 &q_hi,
+                                             const u32x8 &koff, const u32x4 &voff, const u32x4 &ldk,
+                                             const u32x4 &ldv, uint64_t kbase, uint64_t vbase,
+                                             uint32_t tile_stride, float c, int ntiles, int k_requests,
+                                             uint32_t m0_base) {
+  asm volatile(TTPA_STREAM_LOOP_TEXT
+               : "+{v[0:15]}"(st.acc[0]), "+{v[16:31]}"(st.acc[1]), "+{v[32:47]}"(st.acc[2]),
+                 "+{v[48:63]}"(st.acc[3]), "+{v196}"(st.mc), "+{v197}"(st.lrun), "+{s[64:65]}"(kbase),
+                 "+{s[66:67]}"(vbase), "+{s70}"(ntiles), "+{s71}"(k_requests)
+               : "{v[64:79]}"(q_lo), "{v[80:95]}"(q_hi), "{v[176:183]}"(koff), "{v[184:187]}"(voff),
+                 "{v[188:191]}"(ldk), "{v[192:195]}"(ldv), "{s68}"(tile_stride), "{s69}"(c), "{s72}"(m0_base)
+               : "memory", "vcc", "scc", "m0", TTPA_STREAM_LOOP_CLOBBERS);
 }
 
 // MODE 0: dense K/V; 1: paged, block_size a multiple of 64 (a tile lies in one block);
@@ -803,14 +833,61 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
         });
     return;
   }
+  // ---- whole unmasked tiles through the hand-scheduled loop -------------------------------
+  int kt_begin = first_tile;
+  if constexpr (D == 128 && HPW == 4 && RH == 1 && MODE == 0) {
+    // tiles every row of the wavefront sees in full
+    const int n_full = min(a.causal ? (offset + row0 + 1) / kKeysPerTile : ntiles, a.skv / kKeysPerTile);
+    // the loop requests tiles up to min(n + 1, last_tile) with whole-tile loads: a ragged last
+    // tile has to stay out of its reach
+    const bool last_is_whole = (last_tile + 1) * kKeysPerTile <= a.skv;
+    const int n = min(n_full, last_is_whole ? last_tile : last_tile - 2);
+    if (a.stream && wave_active && first_tile == 0 && n >= 1) {
+      StreamState ss;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ss.acc[i] = acc[0][i];
+      ss.mc = -INFINITY, ss.lrun = 0.f;
+      u32x16 q_lo, q_hi;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const u32x4 lo = __builtin_bit_cast(u32x4, qf[0][s]), hi = __builtin_bit_cast(u32x4, qf[0][s + 4]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) q_lo[4 * s + e] = lo[e], q_hi[4 * s + e] = hi[e];
+      }
+      const uint32_t lds0 = lds_address(smem);
+      u32x8 ko;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) ko[s] = koff[s] + lds0;
+      u32x4 vo, lk, lv;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        vo[j] = voff[j] + lds0;
+        // the loop's own split of a tile's 16 segments: wavefront w requests segments 4 w + j
+        const int r = (4 * wave + j) * T::RPI + lane / T::CPR, cp = lane % T::CPR;
+        const uint32_t row_bytes = 2u * (uint32_t)a.kv_ts;
+        lk[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_k(r)) + 3072u - 1024u * j;
+        lv[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_v(r)) + 3072u - 1024u * j;
+      }
+      const int64_t head = b * a.kv_bs + hk * a.kv_hs;
+      const uint64_t kb = reinterpret_cast<uint64_t>(a.k + head + (int64_t)2 * kKeysPerTile * a.kv_ts) - 3072u;
+      const uint64_t vb = reinterpret_cast<uint64_t>(a.v + head + (int64_t)kKeysPerTile * a.kv_ts) - 3072u;
+      stream_tiles(ss, q_lo, q_hi, ko, vo, lk, lv, kb, vb, (uint32_t)(2 * kKeysPerTile * a.kv_ts),
+                   a.scale_log2e, n, max(last_tile - 1, 0), lds0 + 4096u * (uint32_t)wave);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[0][i] = ss.acc[i];
+      m_run[0] = ss.mc / a.scale_log2e;
+      l_run[0] = ss.lrun;
+      kt_begin = n;
+    }
+  }
   // The first K fragments of a tile are read one tile ahead (K(t+1) has landed at the barrier
   // of tile t), so the score product starts without waiting for LDS.
   bf16x8 ring[KPRE];
   if (wave_active) {
 #pragma unroll
-    for (int i = 0; i < KPRE; ++i) ring[i] = read_k(smem + (first_tile & 1) * T::STAGE_BYTES, i);
+    for (int i = 0; i < KPRE; ++i) ring[i] = read_k(smem + (kt_begin & 1) * T::STAGE_BYTES, i);
   }
-  for (int kt = first_tile; kt < ntiles; ++kt) {
+  for (int kt = kt_begin; kt < ntiles; ++kt) {
     const unsigned char *cur = smem + (kt & 1) * T::STAGE_BYTES;
     const int key0 = kt * kKeysPerTile;
     // wavefront-uniform; with a window, tiles wholly below this wavefront's rows are skipped
@@ -1134,6 +1211,10 @@ static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_st
     TTPA_REQUIRE(page_table != nullptr, "prefill: a block-float-8 K / V is a paged cache");
     if (block_size % 16)
       return fail(TTPA_ERR_UNSUPPORTED, "prefill: a block-float-8 cache needs block_size %% 16 == 0");
+  }
+  {
+    const char *e = getenv("TTPA_PREFILL_STREAM");
+    a.stream = e ? atoi(e) : 0;
   }
   a.bs_magic = block_size >= 2 ? (uint32_t)((1ull << 32) / (uint32_t)block_size) + 1u : 0u;
   a.fill_kc = a.fill_vc = nullptr;
