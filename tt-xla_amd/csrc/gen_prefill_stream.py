@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
-"""Writes the hand-scheduled inner loop of the prefill kernel (head size 128, four query heads of
+"""Writes the hand-scheduled tile loop of the prefill kernel (head size 128, four query heads of
 one KV head per workgroup, 32 query rows per wavefront, two workgroups per CU) as one block of
-gfx950 assembly: build/prefill_stream_asm.h, included by prefill.hip.
+gfx950 assembly per K / V source: build/prefill_stream_asm.h, included by prefill.hip.
 
 Why assembly: the loop wants the matrix pipe and the vector ALU of a SIMD busy at the same time
 from one instruction stream, with every register chosen by hand (256 per wavefront at two
@@ -23,20 +23,31 @@ the plain loop.  The block then takes the slow path at the end of the iteration:
 new reference, accumulators and row sum rescaled, probabilities of the block recomputed.  The first
 block of a row always does (the reference starts at -inf).
 
+Masks: a lane holds the keys key0 + 4 h + {0..3, 8..11, 16..19, 24..27} of a block (h = lane / 32)
+for query row lane % 32, and may see keys up to its limit (causal diagonal, end of K / V).  Blocks
+from key `mask_from` on are masked in place, at the start of their iteration, before anything reads
+the scores: 16 compares of the key constants against limit - 4 h - key0 and 16 selects of -inf.
+Blocks in front of it skip that with one scalar branch.
+
 Tiles: K(t) and V(t) live in stage t & 1 of LDS (a stage = K tile, then V tile, 16 KiB each).
 The barrier of tile t sits at the start of iteration 2 t + 1: K(t + 1) and V(t), requested one
 barrier earlier, have landed for everyone; K(t) and V(t - 1) are not read any more, and K(t + 2),
-V(t + 1) are requested into their places (LDS-DMA loads, four per tensor, wavefront and tile).
+V(t + 1) are requested into their places (LDS-DMA loads, four per tensor, wavefront and tile),
+as long as such tiles exist.  Dense K / V: a tile is `stride` bytes behind the one before.  Paged
+(block size a multiple of 64): a tile lies in one block; the block-table entry of tile t + 3 is
+requested (a vector load, like the tiles, so one counter covers both) behind the tile requests
+of barrier t and read behind barrier t + 1, where K(t + 2) needs it; V(t + 2) uses the same
+offset one barrier later.  Entries outside [0, num_blocks) read block 0.
 
-The block is entered with K(0), V(0), K(1) requested and K(0) visible, and handles n tiles
-0 .. n - 1, all of them unmasked.  It leaves with the state the plain loop expects at the top of
-its iteration for tile n: accumulators, row sums and reference through tile n - 1; K(n) visible;
-K(n + 1) and V(n) requested.
+The block is entered with K(0), V(0), K(1) requested and K(0) visible (paged: and the entry of
+tile 2 requested), and handles tiles 0 .. n - 1.  It leaves with the state the plain loop expects
+at the top of its iteration for tile n: accumulators, row sums and reference through tile n - 1;
+K(n) visible; K(n + 1) and V(n) requested where they exist.
 
 Matrix-to-vector hazards the hardware does not interlock are kept by construction: the vector
 instructions that read a score bank start two matrix instructions after the last one that wrote
-it; a bank of probabilities is rewritten three matrix instructions after the last one that read
-it; the slow path and the exit wait out the matrix pipe with s_nop.
+it (the mask waits explicitly); a bank of probabilities is rewritten three matrix instructions
+after the last one that read it; the slow path and the exit wait out the matrix pipe with s_nop.
 """
 
 import os
@@ -55,22 +66,38 @@ KOFF = 176                     # LDS byte address of the lane's K fragment, k-st
 VOFF = 184                     # ... of the lane's V^T fragment, output block db (inputs)
 LDK = 188                      # per-lane global byte offsets of the 4 K loads of a tile (inputs)
 LDV = 192                      # ... of the 4 V loads
-MC, LRUN, LSUM, ALPHA = 196, 197, 198, 199
+MC, LRUN, LSUM, ALPHA = 196, 197, 198, 199   # MC, LRUN: inputs / outputs
 T = [200, 201, 202, 203]
 ORV, MLOC, MB, MCN = 204, 205, 206, 207
-PTREQ = 208                    # mode 1: the requested page-table entry
+PTREQ = 208                    # paged: the requested block-table entry (input)
+LIMIT = 212                    # last visible key of the lane's row, minus 4 h (input)
+LIMREL, NEGINF, VZERO = 213, 214, 215
+CLOBBERED = list(range(S[0], RING + 4 * NSLOT)) + list(range(LSUM, MCN + 1)) + [209, 210, 211, LIMREL, NEGINF, VZERO]
 
 # ---- scalar registers ---------------------------------------------------------------------------
-S_KBASE = "s[64:65]"           # next K tile to request (minus 3072, see dma)
+S_KBASE = "s[64:65]"           # dense: next K tile to request; paged: the K cache (both minus 3072, see dma)
 S_VBASE = "s[66:67]"
-S_STRIDE = "s68"               # mode 0: bytes from one tile to the next
+S_STRIDE = "s68"               # dense: bytes from one tile to the next; paged: bytes of one (block, head) slab
 S_C = "s69"                    # softmax scale times log2(e)
 S_NT = "s70"                   # tiles left
 S_KLEFT = "s71"                # K tiles left to request
 S_M0B = "s72"                  # LDS address of this wavefront's first 1 KiB segment in stage 0's K tile
+S_VLEFT = "s73"                # V tiles left to request
+S_MASKFROM = "s74"             # blocks whose first key is >= this are masked
+S_KEY0 = "s75"                 # first key of the block whose softmax comes next
+# paged only
+S_HKV, S_HK, S_NB, S_TPB = "s76", "s77", "s78", "s79"   # kv heads, this kv head, blocks in the cache, tiles per block
+S_CIN = "s80"                  # tile-in-block index of the next K tile to request
+S_RIN = "s81"                  # ... of the next tile whose entry is requested
+S_RPTR = "s[82:83]"            # address of that entry
+S_VOFF = "s[84:85]"            # byte offset in the cache of the next V tile to request
+S_RLEFT = "s86"                # entries left to request
+# temporaries s[87:95]
+SCALAR_CLOBBERS = [f"s{r}" for r in range(87, 96)]
 
 STAGE = 32768
 VTILE = 16384
+KEY_CONST = [8 * (r // 4) + r % 4 for r in range(16)]
 
 
 class Out:
@@ -86,7 +113,7 @@ class Out:
             return
         if PROBE['NOVALU'] and s.startswith('s_cbranch_vccnz'):
             return
-        if PROBE['NOBAR'] and (s.startswith('s_barrier') or s.startswith('s_waitcnt vmcnt') or s.startswith('global_load_lds')):
+        if PROBE['NOBAR'] and (s.startswith('s_barrier') or s.startswith('s_waitcnt vmcnt') or s.startswith('global_load')):
             return
         self.lines.append(s)
 
@@ -122,7 +149,7 @@ def mfma(m, slot):
     return f"v_mfma_f32_32x32x16_bf16 {d}, {a}, {vr(P[bank] + 4 * k4p, 4)}, {d}"
 
 
-def softmax_ops(q):
+def softmax_ops(q, test=True):
     """Vector instructions of sm(i) on bank q, in an order that keeps one instruction between a
     transcendental and its first use."""
     s, p = S[q], P[q]
@@ -138,21 +165,18 @@ def softmax_ops(q):
         if j < 7:
             ops += [B(2 * j + 2), B(2 * j + 3)]
         ops.append(D(j))
-    ops += [f"v_or3_b32 v{ORV}, v{p}, v{p + 1}, v{p + 2}",
-            f"v_or3_b32 v{ORV}, v{ORV}, v{p + 3}, v{p + 4}",
-            f"v_or3_b32 v{ORV}, v{ORV}, v{p + 5}, v{p + 6}",
-            f"v_or_b32 v{ORV}, v{ORV}, v{p + 7}",
-            f"v_and_b32 v{ORV}, 0x40004000, v{ORV}",
-            f"v_cmp_ne_u32 vcc, 0, v{ORV}"]
-    return ops
-
-
-def check_trans_distance(ops):
-    for i, op in enumerate(ops[:-1]):
+    if test:
+        ops += [f"v_or3_b32 v{ORV}, v{p}, v{p + 1}, v{p + 2}",
+                f"v_or3_b32 v{ORV}, v{ORV}, v{p + 3}, v{p + 4}",
+                f"v_or3_b32 v{ORV}, v{ORV}, v{p + 5}, v{p + 6}",
+                f"v_or_b32 v{ORV}, v{ORV}, v{p + 7}",
+                f"v_and_b32 v{ORV}, 0x40004000, v{ORV}",
+                f"v_cmp_ne_u32 vcc, 0, v{ORV}"]
+    for i, op in enumerate(ops[:-1]):  # a transcendental's result is not read by the next instruction
         if op.startswith("v_exp_f32"):
             dst = op.split()[1].rstrip(",")
-            nxt = ops[i + 1]
-            assert dst not in [t.rstrip(",") for t in nxt.split()[2:]], (op, nxt)
+            assert dst not in [t.rstrip(",") for t in ops[i + 1].split()[2:]], (op, ops[i + 1])
+    return ops
 
 
 def spread(ops, nslots, first=0):
@@ -202,9 +226,29 @@ def iteration_pairs(q, kstage, kb, vstage, vk4, has_pv=True):
     return pairs
 
 
+def mask_block(o, q, tag):
+    """Start of the iteration whose softmax reads bank q: masks the block in place if it needs it."""
+    s = S[q]
+    o.e(f"s_cmp_lt_i32 {S_KEY0}, {S_MASKFROM}")
+    o.e(f"s_cbranch_scc1 L_nomask_{tag}%=")
+    o.e("s_nop 15")  # the last matrix instruction into this bank has written
+    o.e(f"v_subrev_u32 v{LIMREL}, {S_KEY0}, v{LIMIT}")  # limit - 4 h - key0
+    o.e(f"v_mov_b32 v{NEGINF}, 0xff800000")
+    sel = lambda r: f"v_cndmask_b32_e64 v{s + r}, v{s + r}, v{NEGINF}, s[{88 + 2 * (r % 4)}:{89 + 2 * (r % 4)}]"
+    for r in range(16):
+        o.e(f"v_cmp_gt_i32_e64 s[{88 + 2 * (r % 4)}:{89 + 2 * (r % 4)}], {KEY_CONST[r]}, v{LIMREL}")
+        if r >= 3:  # a select reads its mask three instructions after the compare that wrote it
+            o.e(sel(r - 3))
+    o.e("s_nop 1")
+    for r in range(13, 16):
+        o.e(sel(r))
+    o.label(f"L_nomask_{tag}")
+    o.e(f"s_add_u32 {S_KEY0}, {S_KEY0}, 32")
+
+
 def slow_path(o, q, name, join):
     """Bank q: true row maximum, new reference, rescale, probabilities again."""
-    s, p = S[q], P[q]
+    s = S[q]
     o.label(name)
     o.e("s_nop 15")
     o.e("s_nop 15")
@@ -230,8 +274,7 @@ def slow_path(o, q, name, join):
     o.e(f"v_mul_f32 v{LRUN}, v{LRUN}, v{ALPHA}")
     for r in range(64):
         o.e(f"v_mul_f32 v{r}, v{ALPHA}, v{r}")
-    ops = softmax_ops(q)[:-6]  # without the test
-    for x in ops:
+    for x in softmax_ops(q, test=False):
         o.e(x)
     o.e("s_nop 4")
     o.e(f"s_branch {join}%=")
@@ -241,49 +284,93 @@ def stamp(o):
     """probe builds: wall clock (100 MHz) to the workgroup's stamp list; only where no LDS read is in flight"""
     if not PROBE['STAMPS']:
         return
-    o.e("s_memrealtime s[76:77]")
+    o.e("s_memrealtime s[92:93]")
     o.e("s_waitcnt lgkmcnt(0)")
-    o.e("v_mov_b32 v210, s76")
-    o.e("v_mov_b32 v211, s77")
-    o.e("v_mov_b32 v209, s78")
+    o.e("v_mov_b32 v210, s92")
+    o.e("v_mov_b32 v211, s93")
+    o.e("v_mov_b32 v209, s87")
     o.e("s_nop 1")
-    o.e("global_store_dwordx2 v209, v[210:211], s[74:75]")
-    o.e("s_add_u32 s78, s78, 8")
+    o.e("global_store_dwordx2 v209, v[210:211], s[96:97]")
+    o.e("s_add_u32 s87, s87, 8")
 
 
-def dma_block(o, tp, tag):
-    """Requests K(t + 2) into K stage tp (if there is one) and V(t + 1) into V stage 1 - tp.
+def four_loads(o, lane_regs, base):
+    for j in range(4):
+        o.e(f"global_load_lds_dwordx4 v{lane_regs + j}, {base} offset:{1024 * j}")
+
+
+def dma_block(o, tp, tag, paged):
+    """Requests K(t + 2) into K stage tp and V(t + 1) into V stage 1 - tp where those tiles exist.
     The instruction offset moves the LDS address as well as the global one: load j lands 1024 j
     bytes behind M0 and reads base + lane offset + 1024 j, so the lane offsets carry
     3072 - 1024 j and the bases - 3072."""
     o.e(f"s_cmp_eq_u32 {S_KLEFT}, 0")
     o.e(f"s_cbranch_scc1 L_nok_{tag}%=")
+    if paged:
+        o.e(f"v_readfirstlane_b32 s88, v{PTREQ}")
+        o.e(f"s_cmp_lt_u32 s88, {S_NB}")
+        o.e("s_cselect_b32 s88, s88, 0")
+        o.e(f"s_mul_i32 s88, s88, {S_HKV}")
+        o.e(f"s_add_u32 s90, s88, {S_HK}")            # block * kv_heads + kv_head
+        o.e(f"s_mul_hi_u32 s89, s90, {S_STRIDE}")
+        o.e(f"s_mul_i32 s88, s90, {S_STRIDE}")
+        o.e(f"s_lshl_b32 s90, {S_CIN}, 14")           # 64 tokens of 256 bytes per tile inside the block
+        o.e("s_add_u32 s88, s88, s90")
+        o.e("s_addc_u32 s89, s89, 0")                 # s[88:89]: byte offset of tile t + 2 in a cache
+        o.e("s_add_u32 s90, s64, s88")
+        o.e("s_addc_u32 s91, s65, s89")
+        o.e(f"s_add_u32 {S_CIN}, {S_CIN}, 1")
+        o.e(f"s_cmp_eq_u32 {S_CIN}, {S_TPB}")
+        o.e(f"s_cselect_b32 {S_CIN}, 0, {S_CIN}")
     o.e(f"s_add_u32 m0, {S_M0B}, {tp * STAGE}")
     o.e("s_nop 0")
-    for j in range(4):
-        o.e(f"global_load_lds_dwordx4 v{LDK + j}, {S_KBASE} offset:{1024 * j}")
-    o.e(f"s_add_u32 s64, s64, {S_STRIDE}")
-    o.e("s_addc_u32 s65, s65, 0")
+    four_loads(o, LDK, "s[90:91]" if paged else S_KBASE)
+    if not paged:
+        o.e(f"s_add_u32 s64, s64, {S_STRIDE}")
+        o.e("s_addc_u32 s65, s65, 0")
     o.e(f"s_sub_u32 {S_KLEFT}, {S_KLEFT}, 1")
     o.label(f"L_nok_{tag}")
+    o.e(f"s_cmp_eq_u32 {S_VLEFT}, 0")
+    o.e(f"s_cbranch_scc1 L_nov_{tag}%=")
+    if paged:
+        o.e("s_add_u32 s90, s66, s84")
+        o.e("s_addc_u32 s91, s67, s85")
     o.e(f"s_add_u32 m0, {S_M0B}, {(1 - tp) * STAGE + VTILE}")
     o.e("s_nop 0")
-    for j in range(4):
-        o.e(f"global_load_lds_dwordx4 v{LDV + j}, {S_VBASE} offset:{1024 * j}")
-    o.e(f"s_add_u32 s66, s66, {S_STRIDE}")
-    o.e("s_addc_u32 s67, s67, 0")
+    four_loads(o, LDV, "s[90:91]" if paged else S_VBASE)
+    if not paged:
+        o.e(f"s_add_u32 s66, s66, {S_STRIDE}")
+        o.e("s_addc_u32 s67, s67, 0")
+    o.e(f"s_sub_u32 {S_VLEFT}, {S_VLEFT}, 1")
+    o.label(f"L_nov_{tag}")
+    if paged:
+        # the offset of tile t + 2 serves V one barrier later (stale only when no such V is requested)
+        o.e("s_mov_b64 s[84:85], s[88:89]")
+        o.e(f"s_cmp_eq_u32 {S_RLEFT}, 0")
+        o.e(f"s_cbranch_scc1 L_noreq_{tag}%=")
+        o.e(f"global_load_dword v{PTREQ}, v{VZERO}, {S_RPTR}")
+        o.e(f"s_sub_u32 {S_RLEFT}, {S_RLEFT}, 1")
+        o.e(f"s_add_u32 {S_RIN}, {S_RIN}, 1")
+        o.e(f"s_cmp_lg_u32 {S_RIN}, {S_TPB}")
+        o.e(f"s_cbranch_scc1 L_noreq_{tag}%=")
+        o.e(f"s_mov_b32 {S_RIN}, 0")
+        o.e("s_add_u32 s82, s82, 4")
+        o.e("s_addc_u32 s83, s83, 0")
+        o.label(f"L_noreq_{tag}")
 
 
-def generate():
+def generate(paged):
     o = Out()
+    if PROBE['STAMPS']:
+        o.e("s_mov_b32 s87, 0")
     stamp(o)
+    o.e(f"v_mov_b32 v{VZERO}, 0")
     # ---- S(0), then iteration 0 (no PV yet): tile 0 is in stage 0 -----------------------------
     pairs = [(("S", 0, x), ("K", 0, 0, x)) for x in range(8)] + iteration_pairs(0, 0, 1, 0, 0, has_pv=False)
-    ops = softmax_ops(0)
-    check_trans_distance(ops)
-    chunks = spread(ops, 16, first=10)
-    chunks[9] = ["s_nop 15", "s_nop 7"]  # S(0) has been written
-    stream(o, pairs, chunks)
+    chunks = spread(softmax_ops(0), 16, first=10)
+    # the mask of block 0 sits behind the second matrix instruction after S(0); it waits itself
+    nop_then_mask = lambda: (o.e("s_nop 15"), mask_block(o, 0, "i0"))
+    stream(o, pairs, chunks, mid={10: nop_then_mask})
     o.e("s_cbranch_vccnz L_slow_i0%=")
     o.label("L_join_i0")
     o.e(f"v_add_f32 v{LRUN}, v{LRUN}, v{LSUM}")
@@ -293,6 +380,7 @@ def generate():
         o.label(f"L_period{tp}")
         # odd iteration 2 t + 1: barrier of tile t, PV(2 t) from V(t) key steps 0, 1, S(2 t + 2) from K(t + 1) block 0
         # even iteration 2 t + 2: PV(2 t + 1) from V(t) key steps 2, 3, S(2 t + 3) from K(t + 1) block 1
+        mask_block(o, 1, f"o{tp}")
         stamp(o)
         o.e("s_waitcnt vmcnt(0)")
         stamp(o)
@@ -308,10 +396,11 @@ def generate():
             o.e(f"s_sub_u32 {S_NT}, {S_NT}, 1")
             o.e(f"s_cmp_eq_u32 {S_NT}, 0")
             o.e(f"s_cbranch_scc1 L_exit{tp}%=")
+            mask_block(o, 0, f"e{tp}")
 
         # the requests go out behind the first fragment reads; stream() emits those first, so
         # the DMA block is hooked in front of pair 0
-        stream(o, pairs, chunks, mid={0: (lambda tp=tp: dma_block(o, tp, f"p{tp}")), 16: between})
+        stream(o, pairs, chunks, mid={0: (lambda tp=tp: dma_block(o, tp, f"p{tp}", paged)), 16: between})
         o.e(f"s_cbranch_vccnz L_slow_e{tp}%=")
         o.label(f"L_join_e{tp}")
         o.e(f"v_add_f32 v{LRUN}, v{LRUN}, v{LSUM}")
@@ -345,21 +434,17 @@ def generate():
     return o.lines
 
 
-def clobbers():
-    used = list(range(S[0], RING + 4 * NSLOT)) + list(range(LSUM, PTREQ + 1))
-    return ", ".join(f'"v{r}"' for r in used)
-
-
 def main():
-    lines = generate()
     out = sys.argv[1] if len(sys.argv) > 1 else "/dev/stdout"
     with open(out, "w") as f:
         f.write("// Generated by gen_prefill_stream.py; do not edit.\n#pragma once\n")
-        f.write("#define TTPA_STREAM_LOOP_TEXT \\\n")
-        for ln in lines:
-            f.write(f'  "{ln}\\n\\t" \\\n')
-        f.write('  ""\n')
-        f.write(f"#define TTPA_STREAM_LOOP_CLOBBERS {clobbers()}\n")
+        for name, paged in (("DENSE", False), ("PAGED", True)):
+            f.write(f"#define TTPA_STREAM_LOOP_TEXT_{name} \\\n")
+            for ln in generate(paged):
+                f.write(f'  "{ln}\\n\\t" \\\n')
+            f.write('  ""\n')
+        regs = ", ".join([f'"v{r}"' for r in CLOBBERED] + [f'"{r}"' for r in SCALAR_CLOBBERS])
+        f.write(f"#define TTPA_STREAM_LOOP_CLOBBERS {regs}\n")
 
 
 if __name__ == "__main__":

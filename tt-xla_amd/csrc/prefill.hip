@@ -451,17 +451,51 @@ struct StreamState {
   float mc, lrun;  // reference of the probabilities (exponent domain), row sum
 };
 
-__device__ __forceinline__ void stream_tiles(StreamState &st, const u32x16 &q_lo, const u32x16 &q_hi,
-                                             const u32x8 &koff, const u32x4 &voff, const u32x4 &ldk,
-                                             const u32x4 &ldv, uint64_t kbase, uint64_t vbase,
-                                             uint32_t tile_stride, float c, int ntiles, int k_requests,
-                                             uint32_t m0_base) {
-  asm volatile(TTPA_STREAM_LOOP_TEXT
-               : "+{v[0:15]}"(st.acc[0]), "+{v[16:31]}"(st.acc[1]), "+{v[32:47]}"(st.acc[2]),
-                 "+{v[48:63]}"(st.acc[3]), "+{v196}"(st.mc), "+{v197}"(st.lrun), "+{s[64:65]}"(kbase),
-                 "+{s[66:67]}"(vbase), "+{s70}"(ntiles), "+{s71}"(k_requests)
-               : "{v[64:79]}"(q_lo), "{v[80:95]}"(q_hi), "{v[176:183]}"(koff), "{v[184:187]}"(voff),
-                 "{v[188:191]}"(ldk), "{v[192:195]}"(ldv), "{s68}"(tile_stride), "{s69}"(c), "{s72}"(m0_base)
+// What both forms of the block share: q_lo / q_hi the eight Q fragments, koff / voff the lane's
+// LDS addresses of its K and V^T fragments, ldk / ldv the lane's byte offsets of the block's own
+// four loads per tile and tensor, limit the last key the lane's row may see minus 4 (lane / 32),
+// mask_from the first key from which blocks need their mask, k_requests / v_requests the K tiles
+// from tile 2 on and the V tiles from tile 1 on that exist.
+#define TTPA_STREAM_COMMON_OUT                                                                          \
+  "+{v[0:15]}"(st.acc[0]), "+{v[16:31]}"(st.acc[1]), "+{v[32:47]}"(st.acc[2]), "+{v[48:63]}"(st.acc[3]), \
+      "+{v196}"(st.mc), "+{v197}"(st.lrun), "+{s[64:65]}"(kbase), "+{s[66:67]}"(vbase), "+{s70}"(ntiles), \
+      "+{s71}"(k_requests), "+{s73}"(v_requests), "+{s75}"(key0)
+#define TTPA_STREAM_COMMON_IN                                                                       \
+  "{v[64:79]}"(q_lo), "{v[80:95]}"(q_hi), "{v[176:183]}"(koff), "{v[184:187]}"(voff),               \
+      "{v[188:191]}"(ldk), "{v[192:195]}"(ldv), "{v212}"(limit), "{s68}"(stride), "{s69}"(c), "{s72}"(m0_base), \
+      "{s74}"(mask_from)
+
+// Dense K / V: kbase / vbase point at tile 2 of K and tile 1 of V (minus 3072 bytes), a tile is
+// `stride` bytes behind the one before.
+__device__ __forceinline__ void stream_tiles_dense(StreamState &st, const u32x16 &q_lo, const u32x16 &q_hi,
+                                                   const u32x8 &koff, const u32x4 &voff, const u32x4 &ldk,
+                                                   const u32x4 &ldv, int limit, uint64_t kbase, uint64_t vbase,
+                                                   uint32_t stride, float c, int ntiles, int k_requests,
+                                                   int v_requests, int mask_from, uint32_t m0_base) {
+  int key0 = 0;
+  asm volatile(TTPA_STREAM_LOOP_TEXT_DENSE
+               : TTPA_STREAM_COMMON_OUT
+               : TTPA_STREAM_COMMON_IN
+               : "memory", "vcc", "scc", "m0", "v208", TTPA_STREAM_LOOP_CLOBBERS);
+}
+
+// Paged K / V (block_size = 64 tiles_per_block): kbase / vbase are the caches (minus 3072 bytes),
+// stride the bytes of one (block, head) slab; entry the block-table entry of tile 2 (requested by
+// the caller), entry_ptr the address of tile 3's, v_offset the byte offset of tile 1 in a cache.
+__device__ __forceinline__ void stream_tiles_paged(StreamState &st, const u32x16 &q_lo, const u32x16 &q_hi,
+                                                   const u32x8 &koff, const u32x4 &voff, const u32x4 &ldk,
+                                                   const u32x4 &ldv, int limit, uint64_t kbase, uint64_t vbase,
+                                                   uint32_t stride, float c, int ntiles, int k_requests,
+                                                   int v_requests, int mask_from, uint32_t m0_base, int kv_heads,
+                                                   int kv_head, int num_blocks, int tiles_per_block, int entry,
+                                                   uint64_t entry_ptr, uint64_t v_offset, int entry_requests) {
+  int key0 = 0;
+  int k_in_block = 2 % tiles_per_block, e_in_block = 3 % tiles_per_block;
+  asm volatile(TTPA_STREAM_LOOP_TEXT_PAGED
+               : TTPA_STREAM_COMMON_OUT, "+{s80}"(k_in_block), "+{s81}"(e_in_block), "+{s[82:83]}"(entry_ptr),
+                 "+{s[84:85]}"(v_offset), "+{s86}"(entry_requests), "+{v208}"(entry)
+               : TTPA_STREAM_COMMON_IN, "{s76}"(kv_heads), "{s77}"(kv_head), "{s78}"(num_blocks),
+                 "{s79}"(tiles_per_block)
                : "memory", "vcc", "scc", "m0", TTPA_STREAM_LOOP_CLOBBERS);
 }
 
@@ -522,6 +556,7 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
+  const int n_lane = n;
   // Workgroups are dealt to the 8 XCDs round-robin by linear id, and each XCD has its own
   // L2: all query tiles of one (batch, KV-head group) run on the same XCD, one after the
   // other, so that K/V of a group is fetched from HBM by one L2 only and stays resident there
@@ -833,16 +868,14 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
         });
     return;
   }
-  // ---- whole unmasked tiles through the hand-scheduled loop -------------------------------
+  // ---- whole tiles through the hand-scheduled loop --------------------------------------------
   int kt_begin = first_tile;
-  if constexpr (D == 128 && HPW == 4 && RH == 1 && MODE == 0) {
-    // tiles every row of the wavefront sees in full
-    const int n_full = min(a.causal ? (offset + row0 + 1) / kKeysPerTile : ntiles, a.skv / kKeysPerTile);
-    // the loop requests tiles up to min(n + 1, last_tile) with whole-tile loads: a ragged last
-    // tile has to stay out of its reach
+  if constexpr (D == 128 && HPW == 4 && RH == 1 && (MODE == 0 || MODE == 1)) {
+    // Dense K / V ending inside its last tile: the loop requests whole tiles, up to tile
+    // min(n + 1, last_tile), so it stops two tiles early and the plain loop finishes.
     const bool last_is_whole = (last_tile + 1) * kKeysPerTile <= a.skv;
-    const int n = min(n_full, last_is_whole ? last_tile : last_tile - 2);
-    if (a.stream && wave_active && first_tile == 0 && n >= 1) {
+    const int n = last_is_whole ? ntiles : last_tile - 2;
+    if (a.stream && a.window == 0 && a.mask == nullptr && wave_active && n >= 1) {
       StreamState ss;
 #pragma unroll
       for (int i = 0; i < 4; ++i) ss.acc[i] = acc[0][i];
@@ -859,20 +892,38 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
 #pragma unroll
       for (int s = 0; s < 8; ++s) ko[s] = koff[s] + lds0;
       u32x4 vo, lk, lv;
+      const uint32_t row_bytes = MODE == 0 ? 2u * (uint32_t)a.kv_ts : (uint32_t)T::RB;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         vo[j] = voff[j] + lds0;
         // the loop's own split of a tile's 16 segments: wavefront w requests segments 4 w + j
         const int r = (4 * wave + j) * T::RPI + lane / T::CPR, cp = lane % T::CPR;
-        const uint32_t row_bytes = 2u * (uint32_t)a.kv_ts;
         lk[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_k(r)) + 3072u - 1024u * j;
         lv[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_v(r)) + 3072u - 1024u * j;
       }
-      const int64_t head = b * a.kv_bs + hk * a.kv_hs;
-      const uint64_t kb = reinterpret_cast<uint64_t>(a.k + head + (int64_t)2 * kKeysPerTile * a.kv_ts) - 3072u;
-      const uint64_t vb = reinterpret_cast<uint64_t>(a.v + head + (int64_t)kKeysPerTile * a.kv_ts) - 3072u;
-      stream_tiles(ss, q_lo, q_hi, ko, vo, lk, lv, kb, vb, (uint32_t)(2 * kKeysPerTile * a.kv_ts),
-                   a.scale_log2e, n, max(last_tile - 1, 0), lds0 + 4096u * (uint32_t)wave);
+      // last key a row may see; rows past the end of q repeat the last one
+      const int row_limit = a.causal ? min(offset + min(row0 + n_lane, a.sq - 1), a.skv - 1) : a.skv - 1;
+      const int first_limit = a.causal ? min(offset + row0, a.skv - 1) : a.skv - 1;
+      const int k_requests = max(min(n + 1, last_tile) - 1, 0), v_requests = min(n, last_tile);
+      const uint32_t m0_base = lds0 + 4096u * (uint32_t)wave;
+      if constexpr (MODE == 0) {
+        const int64_t head = b * a.kv_bs + hk * a.kv_hs;
+        const uint64_t kb = reinterpret_cast<uint64_t>(a.k + head + (int64_t)2 * kKeysPerTile * a.kv_ts) - 3072u;
+        const uint64_t vb = reinterpret_cast<uint64_t>(a.v + head + (int64_t)kKeysPerTile * a.kv_ts) - 3072u;
+        stream_tiles_dense(ss, q_lo, q_hi, ko, vo, lk, lv, row_limit - 4 * h, kb, vb,
+                           (uint32_t)(2 * kKeysPerTile * a.kv_ts), a.scale_log2e, n, k_requests, v_requests,
+                           first_limit - 30, m0_base);
+      } else {
+        const int tpb = a.bs / kKeysPerTile;
+        const uint32_t slab = (uint32_t)a.bs * (uint32_t)T::RB;
+        // tile 1: its block is blk_v's, tile (1 % tpb) inside it
+        const uint64_t v_off = (uint64_t)((int64_t)blk_v.phys[0] * a.hkv + hk) * slab + (uint64_t)(1 % tpb) * T::TILE_BYTES;
+        const uint64_t e_ptr = reinterpret_cast<uint64_t>(a.pt + (int64_t)b * a.pt_rs + 3 / tpb);
+        stream_tiles_paged(ss, q_lo, q_hi, ko, vo, lk, lv, row_limit - 4 * h,
+                           reinterpret_cast<uint64_t>(a.k) - 3072u, reinterpret_cast<uint64_t>(a.v) - 3072u, slab,
+                           a.scale_log2e, n, k_requests, v_requests, first_limit - 30, m0_base, a.hkv, hk, a.nb,
+                           tpb, req.raw[0], e_ptr, v_off, max(last_tile - 2, 0));
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[0][i] = ss.acc[i];
       m_run[0] = ss.mc / a.scale_log2e;
@@ -883,7 +934,7 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
   // The first K fragments of a tile are read one tile ahead (K(t+1) has landed at the barrier
   // of tile t), so the score product starts without waiting for LDS.
   bf16x8 ring[KPRE];
-  if (wave_active) {
+  if (wave_active && kt_begin < ntiles) {
 #pragma unroll
     for (int i = 0; i < KPRE; ++i) ring[i] = read_k(smem + (kt_begin & 1) * T::STAGE_BYTES, i);
   }
