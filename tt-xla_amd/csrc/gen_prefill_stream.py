@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
-"""Writes the hand-scheduled tile loop of the prefill kernel (head size 128, four query heads of
-one KV head per workgroup, 32 query rows per wavefront, two workgroups per CU) as one block of
-gfx950 assembly per K / V source: build/prefill_stream_asm.h, included by prefill.hip.
+"""Writes the hand-scheduled loop of the prefill kernel (head size 128, four query heads of one KV
+head per workgroup, 32 query rows per wavefront, two workgroups per CU) as one block of gfx950
+assembly per K / V source: build/prefill_stream_asm.h, included by prefill.hip.
 
 Why assembly: the loop wants the matrix pipe and the vector ALU of a SIMD busy at the same time
 from one instruction stream, with every register chosen by hand (256 per wavefront at two
@@ -12,8 +12,9 @@ wavefronts per SIMD) and every wait counted.  The unit of work is a BLOCK of 32 
   PV(i)  8 matrix instructions   O^T += V^T . P^T of block i       (V^T fragments from LDS)
 
 Iteration i issues S(i + 1) and PV(i - 1) alternately, one slice of sm(i) and the LDS read of a
-fragment 8 matrix instructions ahead behind each.  Scores and probabilities alternate between two
-register banks by the parity of i, so nothing is copied.
+fragment 8 matrix instructions ahead behind each; the fragment reads run on across iterations.
+Scores and probabilities alternate between two register banks by the parity of i, so nothing is
+copied.
 
 The running maximum is not tracked per block.  Probabilities are taken relative to a reference
 m (kept as mc = m c + 7 in the exponent domain) that only moves when some probability of the
@@ -29,20 +30,22 @@ from key `mask_from` on are masked in place, at the start of their iteration, be
 the scores: 16 compares of the key constants against limit - 4 h - key0 and 16 selects of -inf.
 Blocks in front of it skip that with one scalar branch.
 
-Tiles: K(t) and V(t) live in stage t & 1 of LDS (a stage = K tile, then V tile, 16 KiB each).
-The barrier of tile t sits at the start of iteration 2 t + 1: K(t + 1) and V(t), requested one
-barrier earlier, have landed for everyone; K(t) and V(t - 1) are not read any more, and K(t + 2),
-V(t + 1) are requested into their places (LDS-DMA loads, four per tensor, wavefront and tile),
-as long as such tiles exist.  Dense K / V: a tile is `stride` bytes behind the one before.  Paged
-(block size a multiple of 64): a tile lies in one block; the block-table entry of tile t + 3 is
-requested (a vector load, like the tiles, so one counter covers both) behind the tile requests
-of barrier t and read behind barrier t + 1, where K(t + 2) needs it; V(t + 2) uses the same
-offset one barrier later.  Entries outside [0, num_blocks) read block 0.
+LDS: a ring of NS slots of 8 KiB (32 rows) for K blocks and one for V blocks; block j lives in
+slot j % NS.  Iteration i reads K block i + 1 and V block i - 1 and, through the running fragment
+reads, the first fragments of K block i + 2 and V block i.  Its barrier, at its start, says that
+nobody reads K block i and V block i - 2 any more; K block i + NS and V block i + NS - 2 are
+requested into their slots (LDS-DMA loads, two per tensor and wavefront).  A request has to have
+landed NS - 2 barriers later: the wait in front of a barrier lets the requests of the last two
+barriers stay in flight (vmcnt(8)), so a tile has three iterations to arrive with NS = 5, where
+two stages of whole tiles gave it two.  Once requests have been skipped (no such block) the wait
+is for everything.  Dense K / V: a block is `stride` bytes behind the one before.  Paged (block
+size a multiple of 64): two blocks are a tile, a tile lies in one cache block; the table entry of
+the tile K enters two iterations from now is requested in front of the tile requests of every
+odd iteration (so the same wait covers it) and read at the next odd one.  Entries outside
+[0, num_blocks) read cache block 0.
 
-The block is entered with K(0), V(0), K(1) requested and K(0) visible (paged: and the entry of
-tile 2 requested), and handles tiles 0 .. n - 1.  It leaves with the state the plain loop expects
-at the top of its iteration for tile n: accumulators, row sums and reference through tile n - 1;
-K(n) visible; K(n + 1) and V(n) requested where they exist.
+The block does everything between the Q fragments and the final normalisation: its own first
+requests (K blocks 0..NS-1, V blocks 0..NS-3), all `nblk` blocks, the last PV.
 
 Matrix-to-vector hazards the hardware does not interlock are kept by construction: the vector
 instructions that read a score bank start two matrix instructions after the last one that wrote
@@ -62,10 +65,10 @@ S = [96, 112]                  # score banks
 P = [128, 136]                 # probability banks (8 packed pairs each)
 RING = 144                     # 8 fragment slots of 4 registers
 NSLOT = 8
-KOFF = 176                     # LDS byte address of the lane's K fragment, k-step ks (inputs)
-VOFF = 184                     # ... of the lane's V^T fragment, output block db (inputs)
-LDK = 188                      # per-lane global byte offsets of the 4 K loads of a tile (inputs)
-LDV = 192                      # ... of the 4 V loads
+KOFF = 176                     # LDS byte address of the lane's K fragment in K slot 0, k-step ks (inputs)
+VOFF = 184                     # ... of the lane's V^T fragment in V slot 0, output block db (inputs)
+LDK = 188                      # per-lane global byte offsets of the 2 K loads of a block (inputs)
+LDV = 190                      # ... of the 2 V loads
 MC, LRUN, LSUM, ALPHA = 196, 197, 198, 199   # MC, LRUN: inputs / outputs
 T = [200, 201, 202, 203]
 ORV, MLOC, MB, MCN = 204, 205, 206, 207
@@ -75,28 +78,32 @@ LIMREL, NEGINF, VZERO = 213, 214, 215
 CLOBBERED = list(range(S[0], RING + 4 * NSLOT)) + list(range(LSUM, MCN + 1)) + [209, 210, 211, LIMREL, NEGINF, VZERO]
 
 # ---- scalar registers ---------------------------------------------------------------------------
-S_KBASE = "s[64:65]"           # dense: next K tile to request; paged: the K cache (both minus 3072, see dma)
+S_KBASE = "s[64:65]"           # dense: next K block to request; paged: the K cache (both minus 1024, see dma)
 S_VBASE = "s[66:67]"
-S_STRIDE = "s68"               # dense: bytes from one tile to the next; paged: bytes of one (block, head) slab
+S_STRIDE = "s68"               # dense: bytes from one block to the next; paged: bytes of one (cache block, head) slab
 S_C = "s69"                    # softmax scale times log2(e)
-S_NT = "s70"                   # tiles left
-S_KLEFT = "s71"                # K tiles left to request
-S_M0B = "s72"                  # LDS address of this wavefront's first 1 KiB segment in stage 0's K tile
-S_VLEFT = "s73"                # V tiles left to request
+S_NB = "s70"                   # blocks left
+S_KLEFT = "s71"                # K blocks left to request
+S_M0B = "s72"                  # LDS address of this wavefront's first 1 KiB segment in K slot 0
+S_VLEFT = "s73"                # V blocks left to request
 S_MASKFROM = "s74"             # blocks whose first key is >= this are masked
 S_KEY0 = "s75"                 # first key of the block whose softmax comes next
 # paged only
-S_HKV, S_HK, S_NB, S_TPB = "s76", "s77", "s78", "s79"   # kv heads, this kv head, blocks in the cache, tiles per block
-S_CIN = "s80"                  # tile-in-block index of the next K tile to request
-S_RIN = "s81"                  # ... of the next tile whose entry is requested
+S_HKV, S_HK, S_NCB, S_TPB = "s76", "s77", "s78", "s79"  # kv heads, this kv head, cache blocks, tiles per cache block
+S_CIN = "s80"                  # tile-in-cache-block index of the tile whose entry is read next
+S_RIN = "s81"                  # ... of the tile whose entry is requested next
 S_RPTR = "s[82:83]"            # address of that entry
-S_VOFF = "s[84:85]"            # byte offset in the cache of the next V tile to request
-S_RLEFT = "s86"                # entries left to request
-# temporaries s[87:95]
-SCALAR_CLOBBERS = [f"s{r}" for r in range(87, 96)]
+S_OFFV = "s[84:85]"            # byte offset in a cache of the tile V requests from (on entry: tile 1)
+S_OFFK = "s[86:87]"            # ... K requests from (on entry: tile 2)
+S_RLEFT = "s96"                # entries left to request
+S_OFF0 = "s[98:99]"            # byte offset of tile 0
+# temporaries s[88:95]
+SCALAR_CLOBBERS = [f"s{r}" for r in range(88, 96)]
 
-STAGE = 32768
-VTILE = 16384
+NS = 5                         # slots per ring
+UNROLL = 10                    # lcm(2, NS): score bank and slots repeat
+SLOT = 8192
+VRING = NS * SLOT              # LDS offset of the V ring; VOFF carries it
 KEY_CONST = [8 * (r // 4) + r % 4 for r in range(16)]
 
 
@@ -126,14 +133,14 @@ def vr(a, n=1):
 
 
 def frag_reads(frag, slot):
-    """LDS read instructions of a fragment into ring slot `slot`."""
+    """LDS read instructions of a fragment into ring slot `slot`.
+    ("K", LDS slot, k-step) or ("V", LDS slot, key step 0 / 1, output block)."""
     base = RING + 4 * slot
-    kind = frag[0]
-    if kind == "K":
-        _, stage, kb, ks = frag
-        return [f"ds_read_b128 {vr(base, 4)}, v{KOFF + ks} offset:{stage * STAGE + kb * 8192}"]
-    _, stage, k4, db = frag
-    off = stage * STAGE + VTILE + k4 * 4096
+    if frag[0] == "K":
+        _, ls, ks = frag
+        return [f"ds_read_b128 {vr(base, 4)}, v{KOFF + ks} offset:{ls * SLOT}"]
+    _, ls, k4, db = frag
+    off = ls * SLOT + k4 * 4096
     return [f"ds_read_b64_tr_b16 {vr(base, 2)}, v{VOFF + db} offset:{off}",
             f"ds_read_b64_tr_b16 {vr(base + 2, 2)}, v{VOFF + db} offset:{off + 2048}"]
 
@@ -188,41 +195,39 @@ def spread(ops, nslots, first=0):
     return out
 
 
-def stream(o, pairs, valu_chunks, mid=None):
-    """pairs: [(matrix instruction, fragment)].  Emits the initial fragment reads (NSLOT ahead),
-    then per pair: wait for its fragment, the matrix instruction, the read of the fragment NSLOT
-    pairs on, the vector chunk.  `mid`: {index: callable} emitted in front of pair `index`."""
+def stream(o, pairs, valu_chunks, in_flight, tail):
+    """pairs: [(matrix instruction, fragment)].  Per pair: wait for its fragment, the matrix
+    instruction, the read of the fragment NSLOT pairs on, the vector chunk.  in_flight: the first
+    NSLOT fragments have been requested by the code in front (else they are requested here);
+    tail: the fragments requested behind the last NSLOT pairs (the next iteration's first ones)."""
+    frags = [f for _, f in pairs] + list(tail)
     n = len(pairs)
-    issued = []  # (fragment index, instructions) in program order
-    for f in range(min(NSLOT, n)):
-        r = frag_reads(pairs[f][1], f % NSLOT)
-        for x in r:
-            o.e(x)
-        issued.append((f, len(r)))
+    count = lambda f: len(frag_reads(frags[f], 0))
+    if not in_flight:
+        for f in range(min(NSLOT, len(frags))):
+            for x in frag_reads(frags[f], f % NSLOT):
+                o.e(x)
     for j in range(n):
-        if mid and j in mid:
-            mid[j]()
-        after = sum(c for f, c in issued if f > j)
+        after = sum(count(f) for f in range(j + 1, min(j + NSLOT, len(frags))))
         assert after <= 15
         o.e(f"s_waitcnt lgkmcnt({after})")
         o.e(mfma(pairs[j][0], j % NSLOT))
-        if j + NSLOT < n:
-            r = frag_reads(pairs[j + NSLOT][1], j % NSLOT)
-            for x in r:
+        if j + NSLOT < len(frags):
+            for x in frag_reads(frags[j + NSLOT], j % NSLOT):
                 o.e(x)
-            issued.append((j + NSLOT, len(r)))
         for x in valu_chunks[j]:
             o.e(x)
 
 
-def iteration_pairs(q, kstage, kb, vstage, vk4, has_pv=True):
-    """Iteration of parity q: S(i + 1) into bank 1 - q from K (kstage, key block kb), PV(i - 1)
-    from bank 1 - q of the probabilities and V (vstage, key steps vk4, vk4 + 1)."""
+def iteration_pairs(p, has_pv=True):
+    """Iteration i = p (mod UNROLL): S(i + 1) into bank 1 - q from K block i + 1, PV(i - 1) from
+    bank 1 - q of the probabilities and V block i - 1."""
+    q = p % 2
     pairs = []
     for x in range(8):
-        pairs.append((("S", 1 - q, x), ("K", kstage, kb, x)))
+        pairs.append((("S", 1 - q, x), ("K", (p + 1) % NS, x)))
         if has_pv:
-            pairs.append((("PV", x % 4, 1 - q, x // 4), ("V", vstage, vk4 + x // 4, x % 4)))
+            pairs.append((("PV", x % 4, 1 - q, x // 4), ("V", (p - 1) % NS, x // 4, x % 4)))
     return pairs
 
 
@@ -280,155 +285,204 @@ def slow_path(o, q, name, join):
     o.e(f"s_branch {join}%=")
 
 
-def stamp(o):
-    """probe builds: wall clock (100 MHz) to the workgroup's stamp list; only where no LDS read is in flight"""
-    if not PROBE['STAMPS']:
-        return
-    o.e("s_memrealtime s[92:93]")
-    o.e("s_waitcnt lgkmcnt(0)")
-    o.e("v_mov_b32 v210, s92")
-    o.e("v_mov_b32 v211, s93")
-    o.e("v_mov_b32 v209, s87")
-    o.e("s_nop 1")
-    o.e("global_store_dwordx2 v209, v[210:211], s[96:97]")
-    o.e("s_add_u32 s87, s87, 8")
-
-
-def four_loads(o, lane_regs, base):
-    for j in range(4):
+def two_loads(o, lane_regs, base):
+    """The instruction offset moves the LDS address as well as the global one: load j lands 1024 j
+    bytes behind M0 and reads base + lane offset + 1024 j, so the lane offsets carry
+    1024 - 1024 j and the bases - 1024."""
+    for j in range(2):
         o.e(f"global_load_lds_dwordx4 v{lane_regs + j}, {base} offset:{1024 * j}")
 
 
-def dma_block(o, tp, tag, paged):
-    """Requests K(t + 2) into K stage tp and V(t + 1) into V stage 1 - tp where those tiles exist.
-    The instruction offset moves the LDS address as well as the global one: load j lands 1024 j
-    bytes behind M0 and reads base + lane offset + 1024 j, so the lane offsets carry
-    3072 - 1024 j and the bases - 3072."""
+def request_block(o, which, slot, tag, paged, half):
+    """One K or V block into LDS slot `slot` of its ring, if there is one left to request.
+    paged: the block is half `half` of the tile at S_OFFK / S_OFFV."""
+    left, lane, base, ring = (S_KLEFT, LDK, S_KBASE, 0) if which == "K" else (S_VLEFT, LDV, S_VBASE, VRING)
+    o.e(f"s_cmp_eq_u32 {left}, 0")
+    o.e(f"s_cbranch_scc1 L_no{which}_{tag}%=")
+    if paged:
+        lo, hi = (86, 87) if which == "K" else (84, 85)
+        b0 = int(base[2:4])
+        o.e(f"s_add_u32 s90, s{b0}, s{lo}")
+        o.e(f"s_addc_u32 s91, s{b0 + 1}, s{hi}")
+        if half:
+            o.e(f"s_add_u32 s90, s90, {SLOT}")
+            o.e("s_addc_u32 s91, s91, 0")
+    o.e(f"s_add_u32 m0, {S_M0B}, {ring + slot * SLOT}")
+    o.e("s_nop 0")
+    two_loads(o, lane, "s[90:91]" if paged else base)
+    if not paged:
+        b0 = int(base[2:4])
+        o.e(f"s_add_u32 s{b0}, s{b0}, {S_STRIDE}")
+        o.e(f"s_addc_u32 s{b0 + 1}, s{b0 + 1}, 0")
+    o.e(f"s_sub_u32 {left}, {left}, 1")
+    o.label(f"L_no{which}_{tag}")
+
+
+def next_tile(o, tag):
+    """paged, odd iterations: V moves on to the tile K was in, K to the tile whose entry has
+    arrived; the entry after that is requested."""
+    o.e("s_mov_b64 s[84:85], s[86:87]")
+    o.e(f"v_readfirstlane_b32 s88, v{PTREQ}")
+    o.e(f"s_cmp_lt_u32 s88, {S_NCB}")
+    o.e("s_cselect_b32 s88, s88, 0")
+    o.e(f"s_mul_i32 s88, s88, {S_HKV}")
+    o.e(f"s_add_u32 s90, s88, {S_HK}")            # cache block * kv_heads + kv_head
+    o.e(f"s_mul_hi_u32 s87, s90, {S_STRIDE}")
+    o.e(f"s_mul_i32 s86, s90, {S_STRIDE}")
+    o.e(f"s_lshl_b32 s90, {S_CIN}, 14")           # 64 tokens of 256 bytes per tile inside the cache block
+    o.e("s_add_u32 s86, s86, s90")
+    o.e("s_addc_u32 s87, s87, 0")
+    o.e(f"s_add_u32 {S_CIN}, {S_CIN}, 1")
+    o.e(f"s_cmp_eq_u32 {S_CIN}, {S_TPB}")
+    o.e(f"s_cselect_b32 {S_CIN}, 0, {S_CIN}")
+    o.e(f"s_cmp_eq_u32 {S_RLEFT}, 0")
+    o.e(f"s_cbranch_scc1 L_noreq_{tag}%=")
+    o.e(f"global_load_dword v{PTREQ}, v{VZERO}, {S_RPTR}")
+    o.e(f"s_sub_u32 {S_RLEFT}, {S_RLEFT}, 1")
+    o.e(f"s_add_u32 {S_RIN}, {S_RIN}, 1")
+    o.e(f"s_cmp_lg_u32 {S_RIN}, {S_TPB}")
+    o.e(f"s_cbranch_scc1 L_noreq_{tag}%=")
+    o.e(f"s_mov_b32 {S_RIN}, 0")
+    o.e("s_add_u32 s82, s82, 4")
+    o.e("s_addc_u32 s83, s83, 0")
+    o.label(f"L_noreq_{tag}")
+
+
+def iteration_head(o, p, tag, paged):
+    """Mask, barrier and requests of iteration i = p (mod UNROLL)."""
+    mask_block(o, p % 2, tag)
+    # requests of the last two barriers may stay in flight, unless some were skipped
+    if PROBE['STAMPS']:
+        o.e("s_memrealtime s[92:93]")
     o.e(f"s_cmp_eq_u32 {S_KLEFT}, 0")
-    o.e(f"s_cbranch_scc1 L_nok_{tag}%=")
-    if paged:
-        o.e(f"v_readfirstlane_b32 s88, v{PTREQ}")
-        o.e(f"s_cmp_lt_u32 s88, {S_NB}")
-        o.e("s_cselect_b32 s88, s88, 0")
-        o.e(f"s_mul_i32 s88, s88, {S_HKV}")
-        o.e(f"s_add_u32 s90, s88, {S_HK}")            # block * kv_heads + kv_head
-        o.e(f"s_mul_hi_u32 s89, s90, {S_STRIDE}")
-        o.e(f"s_mul_i32 s88, s90, {S_STRIDE}")
-        o.e(f"s_lshl_b32 s90, {S_CIN}, 14")           # 64 tokens of 256 bytes per tile inside the block
-        o.e("s_add_u32 s88, s88, s90")
-        o.e("s_addc_u32 s89, s89, 0")                 # s[88:89]: byte offset of tile t + 2 in a cache
-        o.e("s_add_u32 s90, s64, s88")
-        o.e("s_addc_u32 s91, s65, s89")
-        o.e(f"s_add_u32 {S_CIN}, {S_CIN}, 1")
-        o.e(f"s_cmp_eq_u32 {S_CIN}, {S_TPB}")
-        o.e(f"s_cselect_b32 {S_CIN}, 0, {S_CIN}")
-    o.e(f"s_add_u32 m0, {S_M0B}, {tp * STAGE}")
-    o.e("s_nop 0")
-    four_loads(o, LDK, "s[90:91]" if paged else S_KBASE)
-    if not paged:
-        o.e(f"s_add_u32 s64, s64, {S_STRIDE}")
-        o.e("s_addc_u32 s65, s65, 0")
-    o.e(f"s_sub_u32 {S_KLEFT}, {S_KLEFT}, 1")
-    o.label(f"L_nok_{tag}")
-    o.e(f"s_cmp_eq_u32 {S_VLEFT}, 0")
-    o.e(f"s_cbranch_scc1 L_nov_{tag}%=")
-    if paged:
-        o.e("s_add_u32 s90, s66, s84")
-        o.e("s_addc_u32 s91, s67, s85")
-    o.e(f"s_add_u32 m0, {S_M0B}, {(1 - tp) * STAGE + VTILE}")
-    o.e("s_nop 0")
-    four_loads(o, LDV, "s[90:91]" if paged else S_VBASE)
-    if not paged:
-        o.e(f"s_add_u32 s66, s66, {S_STRIDE}")
-        o.e("s_addc_u32 s67, s67, 0")
-    o.e(f"s_sub_u32 {S_VLEFT}, {S_VLEFT}, 1")
-    o.label(f"L_nov_{tag}")
-    if paged:
-        # the offset of tile t + 2 serves V one barrier later (stale only when no such V is requested)
-        o.e("s_mov_b64 s[84:85], s[88:89]")
-        o.e(f"s_cmp_eq_u32 {S_RLEFT}, 0")
-        o.e(f"s_cbranch_scc1 L_noreq_{tag}%=")
-        o.e(f"global_load_dword v{PTREQ}, v{VZERO}, {S_RPTR}")
-        o.e(f"s_sub_u32 {S_RLEFT}, {S_RLEFT}, 1")
-        o.e(f"s_add_u32 {S_RIN}, {S_RIN}, 1")
-        o.e(f"s_cmp_lg_u32 {S_RIN}, {S_TPB}")
-        o.e(f"s_cbranch_scc1 L_noreq_{tag}%=")
-        o.e(f"s_mov_b32 {S_RIN}, 0")
-        o.e("s_add_u32 s82, s82, 4")
-        o.e("s_addc_u32 s83, s83, 0")
-        o.label(f"L_noreq_{tag}")
+    o.e(f"s_cbranch_scc1 L_all_{tag}%=")
+    o.e("s_waitcnt vmcnt(8)")
+    o.e(f"s_branch L_bar_{tag}%=")
+    o.label(f"L_all_{tag}")
+    o.e("s_waitcnt vmcnt(0)")
+    o.label(f"L_bar_{tag}")
+    if PROBE['STAMPS']:
+        o.e("s_memrealtime s[94:95]")
+    o.e("s_barrier")
+    if PROBE['STAMPS']:  # (wall clock before / after the wait for the requests, per iteration)
+        o.e("s_waitcnt lgkmcnt(0)")
+        for k in range(4):
+            o.e(f"v_mov_b32 v{216 + k}, s{92 + k}")
+        o.e("v_mov_b32 v209, s97")
+        o.e("s_nop 1")
+        o.e("global_store_dwordx4 v209, v[216:219], s[100:101]")
+        o.e("s_add_u32 s97, s97, 16")
+    if paged and p % 2 == 1:
+        next_tile(o, tag)
+    # K block i + NS is half (i + NS) % 2 of its tile, V block i + NS - 2 the same half of its own
+    request_block(o, "K", p % NS, tag, paged, (p + NS) % 2)
+    request_block(o, "V", (p + NS - 2) % NS, tag, paged, (p + NS) % 2)
+
+
+def iteration_tail(o, tag, exit_label):
+    o.e(f"s_cbranch_vccnz L_slow_{tag}%=")
+    o.label(f"L_join_{tag}")
+    o.e(f"v_add_f32 v{LRUN}, v{LRUN}, v{LSUM}")
+    o.e(f"s_sub_u32 {S_NB}, {S_NB}, 1")
+    o.e(f"s_cmp_eq_u32 {S_NB}, 0")
+    o.e(f"s_cbranch_scc1 {exit_label}%=")
+
+
+def first_frags(p):
+    """The first NSLOT fragments of iteration p (mod UNROLL)."""
+    return [f for _, f in iteration_pairs(p % UNROLL)[:NSLOT]]
+
+
+def generate_first(paged):
+    """The first requests: K blocks 0 .. NS - 1, V blocks 0 .. NS - 3 (a block of its own, so that
+    the caller can put its Q loads behind them)."""
+    o = Out()
+    for j in range(NS):
+        if paged:  # tiles 0, 1, 2 at S_OFF0, S_OFFV, S_OFFK
+            src = ("s[98:99]", S_OFFV, S_OFFK)[j // 2]
+            lo = int(src[2:4])
+            o.e(f"s_cmp_eq_u32 {S_KLEFT}, 0")
+            o.e(f"s_cbranch_scc1 L_noK_pro{j}%=")
+            o.e(f"s_add_u32 s90, s64, s{lo}")
+            o.e(f"s_addc_u32 s91, s65, s{lo + 1}")
+            if j % 2:
+                o.e(f"s_add_u32 s90, s90, {SLOT}")
+                o.e("s_addc_u32 s91, s91, 0")
+            o.e(f"s_add_u32 m0, {S_M0B}, {j * SLOT}")
+            o.e("s_nop 0")
+            two_loads(o, LDK, "s[90:91]")
+            o.e(f"s_sub_u32 {S_KLEFT}, {S_KLEFT}, 1")
+            o.label(f"L_noK_pro{j}")
+        else:
+            request_block(o, "K", j, f"pro{j}", False, 0)
+    for j in range(NS - 2):
+        if paged:
+            src = ("s[98:99]", S_OFFV)[j // 2]
+            lo = int(src[2:4])
+            o.e(f"s_cmp_eq_u32 {S_VLEFT}, 0")
+            o.e(f"s_cbranch_scc1 L_noV_pro{j}%=")
+            o.e(f"s_add_u32 s90, s66, s{lo}")
+            o.e(f"s_addc_u32 s91, s67, s{lo + 1}")
+            if j % 2:
+                o.e(f"s_add_u32 s90, s90, {SLOT}")
+                o.e("s_addc_u32 s91, s91, 0")
+            o.e(f"s_add_u32 m0, {S_M0B}, {VRING + j * SLOT}")
+            o.e("s_nop 0")
+            two_loads(o, LDV, "s[90:91]")
+            o.e(f"s_sub_u32 {S_VLEFT}, {S_VLEFT}, 1")
+            o.label(f"L_noV_pro{j}")
+        else:
+            request_block(o, "V", j, f"pro{j}", False, 0)
+    return o.lines
 
 
 def generate(paged):
     o = Out()
+    assert NS == 5 and UNROLL == 10
     if PROBE['STAMPS']:
-        o.e("s_mov_b32 s87, 0")
-    stamp(o)
+        o.e("s_mov_b32 s97, 0")
     o.e(f"v_mov_b32 v{VZERO}, 0")
-    # ---- S(0), then iteration 0 (no PV yet): tile 0 is in stage 0 -----------------------------
-    pairs = [(("S", 0, x), ("K", 0, 0, x)) for x in range(8)] + iteration_pairs(0, 0, 1, 0, 0, has_pv=False)
-    chunks = spread(softmax_ops(0), 16, first=10)
-    # the mask of block 0 sits behind the second matrix instruction after S(0); it waits itself
-    nop_then_mask = lambda: (o.e("s_nop 15"), mask_block(o, 0, "i0"))
-    stream(o, pairs, chunks, mid={10: nop_then_mask})
-    o.e("s_cbranch_vccnz L_slow_i0%=")
-    o.label("L_join_i0")
-    o.e(f"v_add_f32 v{LRUN}, v{LRUN}, v{LSUM}")
+    o.e("s_waitcnt vmcnt(0)")
+    o.e("s_barrier")
+    # ---- S(0) from K block 0; behind it the fragments of iteration 0 (K block 1) ------------------
+    pairs = [(("S", 0, x), ("K", 0, x)) for x in range(8)]
+    it0 = iteration_pairs(0, has_pv=False)
+    stream(o, pairs, [[] for _ in pairs], False, [f for _, f in it0])
+    # ---- iteration 0: S(1), sm(0) ---------------------------------------------------------------
+    o.e("s_nop 7")
+    iteration_head(o, 0, "i0", paged)
+    stream(o, it0, spread(softmax_ops(0), 8), True, first_frags(1))
+    iteration_tail(o, "i0", "L_exit0")
+    # ---- iterations 1 .. : ten in a row, then round again -------------------------------------------
+    for k in range(UNROLL):
+        p = (k + 1) % UNROLL
+        o.label(f"L_it{p}")
+        iteration_head(o, p, f"p{p}", paged)
+        stream(o, iteration_pairs(p), spread(softmax_ops(p % 2), 16), True, first_frags(p + 1))
+        iteration_tail(o, f"p{p}", f"L_exit{p}")
+    o.e("s_branch L_it1%=")
 
-    # ---- two tile periods: t even (tp = 0), t odd (tp = 1) ---------------------------------------
-    for tp in (0, 1):
-        o.label(f"L_period{tp}")
-        # odd iteration 2 t + 1: barrier of tile t, PV(2 t) from V(t) key steps 0, 1, S(2 t + 2) from K(t + 1) block 0
-        # even iteration 2 t + 2: PV(2 t + 1) from V(t) key steps 2, 3, S(2 t + 3) from K(t + 1) block 1
-        mask_block(o, 1, f"o{tp}")
-        stamp(o)
-        o.e("s_waitcnt vmcnt(0)")
-        stamp(o)
-        o.e("s_barrier")
-        stamp(o)
-        pairs = iteration_pairs(1, 1 - tp, 0, tp, 0) + iteration_pairs(0, 1 - tp, 1, tp, 2)
-        chunks = spread(softmax_ops(1), 16) + spread(softmax_ops(0), 16)
-
-        def between(tp=tp):
-            o.e(f"s_cbranch_vccnz L_slow_o{tp}%=")
-            o.label(f"L_join_o{tp}")
-            o.e(f"v_add_f32 v{LRUN}, v{LRUN}, v{LSUM}")
-            o.e(f"s_sub_u32 {S_NT}, {S_NT}, 1")
-            o.e(f"s_cmp_eq_u32 {S_NT}, 0")
-            o.e(f"s_cbranch_scc1 L_exit{tp}%=")
-            mask_block(o, 0, f"e{tp}")
-
-        # the requests go out behind the first fragment reads; stream() emits those first, so
-        # the DMA block is hooked in front of pair 0
-        stream(o, pairs, chunks, mid={0: (lambda tp=tp: dma_block(o, tp, f"p{tp}", paged)), 16: between})
-        o.e(f"s_cbranch_vccnz L_slow_e{tp}%=")
-        o.label(f"L_join_e{tp}")
-        o.e(f"v_add_f32 v{LRUN}, v{LRUN}, v{LSUM}")
-        if tp == 1:
-            o.e("s_branch L_period0%=")
-
-    # ---- exits: PV of the last block (bank 1, V(t) key steps 2 and 3) ------------------------------
-    # The ring holds the first eight fragments of the even iteration: slots 1, 3, 5, 7 are
-    # V(t) key step 2, blocks 0..3; slots 0, 2, 4, 6 (K fragments nobody needs) take key step 3.
-    for tp in (0, 1):
-        o.label(f"L_exit{tp}")
+    # ---- exits: PV of the last block i = p (mod UNROLL) -----------------------------------------------
+    # The ring holds the first eight fragments of the iteration that is not coming: slots 1, 3, 5, 7
+    # are V block i, key step 0, output blocks 0..3; slots 0, 2, 4, 6 (K fragments nobody needs) take
+    # key step 1.
+    for p in range(UNROLL):
+        o.label(f"L_exit{p}")
         o.e("s_waitcnt lgkmcnt(0)")
         for db in range(4):
-            for x in frag_reads(("V", tp, 3, db), 2 * db):
+            for x in frag_reads(("V", p % NS, 1, db), 2 * db):
                 o.e(x)
         for db in range(4):
-            o.e(mfma(("PV", db, 1, 0), 2 * db + 1))
+            o.e(mfma(("PV", db, p % 2, 0), 2 * db + 1))
         o.e("s_waitcnt lgkmcnt(0)")
         for db in range(4):
-            o.e(mfma(("PV", db, 1, 1), 2 * db))
+            o.e(mfma(("PV", db, p % 2, 1), 2 * db))
         o.e("s_branch L_end%=")
 
     slow_path(o, 0, "L_slow_i0", "L_join_i0")
-    for tp in (0, 1):
-        slow_path(o, 1, f"L_slow_o{tp}", f"L_join_o{tp}")
-        slow_path(o, 0, f"L_slow_e{tp}", f"L_join_e{tp}")
+    for p in range(UNROLL):
+        slow_path(o, p % 2, f"L_slow_p{p}", f"L_join_p{p}")
     o.label("L_end")
-    stamp(o)
     o.e("s_nop 15")
     o.e("s_nop 15")
     return o.lines
@@ -439,12 +493,15 @@ def main():
     with open(out, "w") as f:
         f.write("// Generated by gen_prefill_stream.py; do not edit.\n#pragma once\n")
         for name, paged in (("DENSE", False), ("PAGED", True)):
-            f.write(f"#define TTPA_STREAM_LOOP_TEXT_{name} \\\n")
-            for ln in generate(paged):
-                f.write(f'  "{ln}\\n\\t" \\\n')
-            f.write('  ""\n')
+            for macro, lines in ((f"TTPA_STREAM_FIRST_TEXT_{name}", generate_first(paged)),
+                                 (f"TTPA_STREAM_LOOP_TEXT_{name}", generate(paged))):
+                f.write(f"#define {macro} \\\n")
+                for ln in lines:
+                    f.write(f'  "{ln}\\n\\t" \\\n')
+                f.write('  ""\n')
         regs = ", ".join([f'"v{r}"' for r in CLOBBERED] + [f'"{r}"' for r in SCALAR_CLOBBERS])
         f.write(f"#define TTPA_STREAM_LOOP_CLOBBERS {regs}\n")
+        f.write(f"#define TTPA_STREAM_LDS_BYTES {2 * NS * SLOT}\n#define TTPA_STREAM_V_RING {VRING}\n")
 
 
 if __name__ == "__main__":

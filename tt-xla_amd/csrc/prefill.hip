@@ -451,27 +451,48 @@ struct StreamState {
   float mc, lrun;  // reference of the probabilities (exponent domain), row sum
 };
 
-// What both forms of the block share: q_lo / q_hi the eight Q fragments, koff / voff the lane's
-// LDS addresses of its K and V^T fragments, ldk / ldv the lane's byte offsets of the block's own
-// four loads per tile and tensor, limit the last key the lane's row may see minus 4 (lane / 32),
-// mask_from the first key from which blocks need their mask, k_requests / v_requests the K tiles
-// from tile 2 on and the V tiles from tile 1 on that exist.
+// The requests of a workgroup's first blocks are a block of assembly of their own, issued in front
+// of the Q loads so that the two round trips to memory overlap.
+struct StreamRequests {
+  uint64_t kbase, vbase;       // dense: block 0 of K / V; paged: the caches (both minus 1024 bytes)
+  uint32_t stride;             // dense: bytes from a 32-key block to the next; paged: bytes of a (cache block, head) slab
+  uint32_t m0_base;            // LDS address of the wavefront's first segment in K slot 0
+  int k_requests, v_requests;  // blocks not requested yet
+  u32x2 ldk, ldv;              // the lane's byte offsets of its two loads per block
+  uint64_t off0, off1, off2;   // paged: byte offsets of tiles 0, 1, 2 in a cache
+};
+
+__device__ __forceinline__ void stream_first_dense(StreamRequests &r) {
+  asm volatile(TTPA_STREAM_FIRST_TEXT_DENSE
+               : "+{s[64:65]}"(r.kbase), "+{s[66:67]}"(r.vbase), "+{s71}"(r.k_requests), "+{s73}"(r.v_requests)
+               : "{v[188:189]}"(r.ldk), "{v[190:191]}"(r.ldv), "{s68}"(r.stride), "{s72}"(r.m0_base)
+               : "memory", "scc", "m0");
+}
+
+__device__ __forceinline__ void stream_first_paged(StreamRequests &r) {
+  asm volatile(TTPA_STREAM_FIRST_TEXT_PAGED
+               : "+{s71}"(r.k_requests), "+{s73}"(r.v_requests)
+               : "{v[188:189]}"(r.ldk), "{v[190:191]}"(r.ldv), "{s[64:65]}"(r.kbase), "{s[66:67]}"(r.vbase),
+                 "{s72}"(r.m0_base), "{s[84:85]}"(r.off1), "{s[86:87]}"(r.off2), "{s[98:99]}"(r.off0)
+               : "memory", "scc", "m0", "s90", "s91");
+}
+
 #define TTPA_STREAM_COMMON_OUT                                                                          \
   "+{v[0:15]}"(st.acc[0]), "+{v[16:31]}"(st.acc[1]), "+{v[32:47]}"(st.acc[2]), "+{v[48:63]}"(st.acc[3]), \
-      "+{v196}"(st.mc), "+{v197}"(st.lrun), "+{s[64:65]}"(kbase), "+{s[66:67]}"(vbase), "+{s70}"(ntiles), \
-      "+{s71}"(k_requests), "+{s73}"(v_requests), "+{s75}"(key0)
+      "+{v196}"(st.mc), "+{v197}"(st.lrun), "+{s[64:65]}"(r.kbase), "+{s[66:67]}"(r.vbase), "+{s70}"(nblk),  \
+      "+{s71}"(r.k_requests), "+{s73}"(r.v_requests), "+{s75}"(key0)
 #define TTPA_STREAM_COMMON_IN                                                                       \
   "{v[64:79]}"(q_lo), "{v[80:95]}"(q_hi), "{v[176:183]}"(koff), "{v[184:187]}"(voff),               \
-      "{v[188:191]}"(ldk), "{v[192:195]}"(ldv), "{v212}"(limit), "{s68}"(stride), "{s69}"(c), "{s72}"(m0_base), \
-      "{s74}"(mask_from)
+      "{v[188:189]}"(r.ldk), "{v[190:191]}"(r.ldv), "{v212}"(limit), "{s68}"(r.stride), "{s69}"(c),  \
+      "{s72}"(r.m0_base), "{s74}"(mask_from)
 
-// Dense K / V: kbase / vbase point at tile 2 of K and tile 1 of V (minus 3072 bytes), a tile is
-// `stride` bytes behind the one before.
-__device__ __forceinline__ void stream_tiles_dense(StreamState &st, const u32x16 &q_lo, const u32x16 &q_hi,
-                                                   const u32x8 &koff, const u32x4 &voff, const u32x4 &ldk,
-                                                   const u32x4 &ldv, int limit, uint64_t kbase, uint64_t vbase,
-                                                   uint32_t stride, float c, int ntiles, int k_requests,
-                                                   int v_requests, int mask_from, uint32_t m0_base) {
+// Everything behind the first requests.  q_lo / q_hi: the eight Q fragments; koff / voff: the lane's
+// LDS addresses of its K and V^T fragments in slot 0 of the K and V rings; limit: the last key the
+// lane's row may see minus 4 (lane / 32); mask_from: the first key from which blocks need their mask;
+// nblk: the 32-key blocks.
+__device__ __forceinline__ void stream_blocks_dense(StreamState &st, StreamRequests &r, const u32x16 &q_lo,
+                                                    const u32x16 &q_hi, const u32x8 &koff, const u32x4 &voff,
+                                                    int limit, float c, int nblk, int mask_from) {
   int key0 = 0;
   asm volatile(TTPA_STREAM_LOOP_TEXT_DENSE
                : TTPA_STREAM_COMMON_OUT
@@ -479,23 +500,21 @@ __device__ __forceinline__ void stream_tiles_dense(StreamState &st, const u32x16
                : "memory", "vcc", "scc", "m0", "v208", TTPA_STREAM_LOOP_CLOBBERS);
 }
 
-// Paged K / V (block_size = 64 tiles_per_block): kbase / vbase are the caches (minus 3072 bytes),
-// stride the bytes of one (block, head) slab; entry the block-table entry of tile 2 (requested by
-// the caller), entry_ptr the address of tile 3's, v_offset the byte offset of tile 1 in a cache.
-__device__ __forceinline__ void stream_tiles_paged(StreamState &st, const u32x16 &q_lo, const u32x16 &q_hi,
-                                                   const u32x8 &koff, const u32x4 &voff, const u32x4 &ldk,
-                                                   const u32x4 &ldv, int limit, uint64_t kbase, uint64_t vbase,
-                                                   uint32_t stride, float c, int ntiles, int k_requests,
-                                                   int v_requests, int mask_from, uint32_t m0_base, int kv_heads,
-                                                   int kv_head, int num_blocks, int tiles_per_block, int entry,
-                                                   uint64_t entry_ptr, uint64_t v_offset, int entry_requests) {
+// Paged: entry is the raw table entry of tile 3, entry_ptr the address of tile 4's.
+__device__ __forceinline__ void stream_blocks_paged(StreamState &st, StreamRequests &r, const u32x16 &q_lo,
+                                                    const u32x16 &q_hi, const u32x8 &koff, const u32x4 &voff,
+                                                    int limit, float c, int nblk, int mask_from, int kv_heads,
+                                                    int kv_head, int num_blocks, int tiles_per_block, int entry,
+                                                    uint64_t entry_ptr) {
   int key0 = 0;
-  int k_in_block = 2 % tiles_per_block, e_in_block = 3 % tiles_per_block;
+  int read_in_block = 3 % tiles_per_block, request_in_block = 4 % tiles_per_block;
+  int entry_requests = max((nblk - 1) / 2 - 3, 0);
   asm volatile(TTPA_STREAM_LOOP_TEXT_PAGED
-               : TTPA_STREAM_COMMON_OUT, "+{s80}"(k_in_block), "+{s81}"(e_in_block), "+{s[82:83]}"(entry_ptr),
-                 "+{s[84:85]}"(v_offset), "+{s86}"(entry_requests), "+{v208}"(entry)
+               : TTPA_STREAM_COMMON_OUT, "+{s80}"(read_in_block), "+{s81}"(request_in_block),
+                 "+{s[82:83]}"(entry_ptr), "+{s[84:85]}"(r.off1), "+{s[86:87]}"(r.off2), "+{s96}"(entry_requests),
+                 "+{v208}"(entry)
                : TTPA_STREAM_COMMON_IN, "{s76}"(kv_heads), "{s77}"(kv_head), "{s78}"(num_blocks),
-                 "{s79}"(tiles_per_block)
+                 "{s79}"(tiles_per_block), "{s[98:99]}"(r.off0)
                : "memory", "vcc", "scc", "m0", TTPA_STREAM_LOOP_CLOBBERS);
 }
 
@@ -586,6 +605,54 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
   const int wg_first_key = a.window > 0 ? max(0, offset + qt * ROWS * RPW - a.window + 1) : 0;
   const int wave_first_key = a.window > 0 ? max(0, offset + row0 - a.window + 1) : 0;
   const int first_tile = wg_first_key / kKeysPerTile;
+
+  // ---- the hand-scheduled loop takes workgroups of whole 32-key blocks; its first requests go out now ----
+  // (a dense K / V that ends inside a 64-key tile goes through the plain loop)
+  bool streamed = false;
+  StreamRequests sreq;
+  int stream_entry = 0;
+  if constexpr (D == 128 && HPW == 4 && RH == 1 && (MODE == 0 || MODE == 1)) {
+    streamed = a.stream && a.window == 0 && a.mask == nullptr && wave_active && (MODE == 1 || a.skv % kKeysPerTile == 0);
+    if (streamed) {
+      const uint32_t lds0 = lds_address(smem);
+      const uint32_t row_bytes = MODE == 0 ? 2u * (uint32_t)a.kv_ts : (uint32_t)T::RB;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        // a block is 8 segments of 1 KiB; wavefront w requests segments 2 w and 2 w + 1
+        const int r = (2 * wave + j) * T::RPI + lane / T::CPR, cp = lane % T::CPR;
+        sreq.ldk[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_k(r)) + 1024u - 1024u * j;
+        sreq.ldv[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_v(r)) + 1024u - 1024u * j;
+      }
+      sreq.m0_base = lds0 + 2048u * (uint32_t)wave;
+      sreq.k_requests = sreq.v_requests = (kv_end_wg + 31) / 32;
+      sreq.off0 = sreq.off1 = sreq.off2 = 0;
+      if constexpr (MODE == 0) {
+        const int64_t head = b * a.kv_bs + hk * a.kv_hs;
+        sreq.kbase = reinterpret_cast<uint64_t>(a.k + head) - 1024u;
+        sreq.vbase = reinterpret_cast<uint64_t>(a.v + head) - 1024u;
+        sreq.stride = (uint32_t)(64 * a.kv_ts);
+        stream_first_dense(sreq);
+      } else {
+        const int tpb = a.bs / kKeysPerTile, last = ntiles - 1;
+        sreq.kbase = reinterpret_cast<uint64_t>(a.k) - 1024u;
+        sreq.vbase = reinterpret_cast<uint64_t>(a.v) - 1024u;
+        sreq.stride = (uint32_t)a.bs * (uint32_t)T::RB;
+        int raw[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) raw[t] = a.pt[(int64_t)b * a.pt_rs + min(t, last) / tpb];
+        uint64_t off[3];
+#pragma unroll
+        for (int t = 0; t < 3; ++t) {
+          int phys = __builtin_amdgcn_readfirstlane(raw[t]);
+          if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+          off[t] = (uint64_t)((int64_t)phys * a.hkv + hk) * sreq.stride + (uint64_t)(min(t, last) % tpb) * T::TILE_BYTES;
+        }
+        sreq.off0 = off[0], sreq.off1 = off[1], sreq.off2 = off[2];
+        stream_entry = raw[3];
+        stream_first_paged(sreq);
+      }
+    }
+  }
 
   // ---- Q fragments (B operand: lane n = query row, 8 head-dim elements per k-step) -----
   // RH = 2: straight into accumulation registers (the matrix instructions read them from there),
@@ -836,6 +903,46 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
   };
   auto kbuf = [&](int t) { return RH == 1 ? (t & 1) : t % KST; };
   auto vbuf = [&](int t) { return RH == 1 ? (t & 1) : t % VST; };
+  int kt_begin = first_tile;
+  // ---- all blocks through the hand-scheduled loop ------------------------------------------------
+  if constexpr (D == 128 && HPW == 4 && RH == 1 && (MODE == 0 || MODE == 1)) {
+    if (streamed) {
+      StreamState ss;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ss.acc[i] = acc[0][i];
+      ss.mc = -INFINITY, ss.lrun = 0.f;
+      u32x16 q_lo, q_hi;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const u32x4 lo = __builtin_bit_cast(u32x4, qf[0][s]), hi = __builtin_bit_cast(u32x4, qf[0][s + 4]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) q_lo[4 * s + e] = lo[e], q_hi[4 * s + e] = hi[e];
+      }
+      const uint32_t lds0 = lds_address(smem);
+      u32x8 ko;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) ko[s] = koff[s] + lds0;
+      u32x4 vo;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) vo[j] = voff[j] + lds0 + TTPA_STREAM_V_RING;
+      // last key a row may see; rows past the end of q repeat the last one
+      const int row_limit = a.causal ? min(offset + min(row0 + n, a.sq - 1), a.skv - 1) : a.skv - 1;
+      const int first_limit = a.causal ? min(offset + row0, a.skv - 1) : a.skv - 1;
+      const int nblk = (kv_end_wg + 31) / 32;
+      if constexpr (MODE == 0) {
+        stream_blocks_dense(ss, sreq, q_lo, q_hi, ko, vo, row_limit - 4 * h, a.scale_log2e, nblk, first_limit - 30);
+      } else {
+        const int tpb = a.bs / kKeysPerTile;
+        stream_blocks_paged(ss, sreq, q_lo, q_hi, ko, vo, row_limit - 4 * h, a.scale_log2e, nblk, first_limit - 30,
+                            a.hkv, hk, a.nb, tpb, stream_entry,
+                            reinterpret_cast<uint64_t>(a.pt + (int64_t)b * a.pt_rs + 4 / tpb));
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[0][i] = ss.acc[i];
+      l_run[0] = ss.lrun;
+    }
+  }
+  if (streamed) kt_begin = ntiles;  // nothing is left for the plain loop; its first requests are skipped too
   Blocks blk_v = resolve(request(first_tile));     // blocks of the tile whose V is loaded next
   Blocks blk_k = resolve(request(first_tile + 1));  // ... whose K is loaded next
   Requested req = request(first_tile + 2);
@@ -844,7 +951,7 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
     commit_bfp8(fetch_bfp8(a.v, first_tile, blk_v), true, first_tile & 1);
     if (last_tile >= first_tile + 1)
       commit_bfp8(fetch_bfp8(a.k, first_tile + 1, blk_k), false, (first_tile + 1) & 1);
-  } else {
+  } else if (!streamed) {
     issue(a.k, ld_k, false, first_tile, kbuf(first_tile), blk_v);
     issue(a.v, ld_v, true, first_tile, vbuf(first_tile), blk_v);
     if (last_tile >= first_tile + 1) issue(a.k, ld_k, false, first_tile + 1, kbuf(first_tile + 1), blk_k);
@@ -867,69 +974,6 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
           req = request(tile + 3);
         });
     return;
-  }
-  // ---- whole tiles through the hand-scheduled loop --------------------------------------------
-  int kt_begin = first_tile;
-  if constexpr (D == 128 && HPW == 4 && RH == 1 && (MODE == 0 || MODE == 1)) {
-    // Dense K / V ending inside its last tile: the loop requests whole tiles, up to tile
-    // min(n + 1, last_tile), so it stops two tiles early and the plain loop finishes.
-    const bool last_is_whole = (last_tile + 1) * kKeysPerTile <= a.skv;
-    const int n = last_is_whole ? ntiles : last_tile - 2;
-    if (a.stream && a.window == 0 && a.mask == nullptr && wave_active && n >= 1) {
-      StreamState ss;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) ss.acc[i] = acc[0][i];
-      ss.mc = -INFINITY, ss.lrun = 0.f;
-      u32x16 q_lo, q_hi;
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const u32x4 lo = __builtin_bit_cast(u32x4, qf[0][s]), hi = __builtin_bit_cast(u32x4, qf[0][s + 4]);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) q_lo[4 * s + e] = lo[e], q_hi[4 * s + e] = hi[e];
-      }
-      const uint32_t lds0 = lds_address(smem);
-      u32x8 ko;
-#pragma unroll
-      for (int s = 0; s < 8; ++s) ko[s] = koff[s] + lds0;
-      u32x4 vo, lk, lv;
-      const uint32_t row_bytes = MODE == 0 ? 2u * (uint32_t)a.kv_ts : (uint32_t)T::RB;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        vo[j] = voff[j] + lds0;
-        // the loop's own split of a tile's 16 segments: wavefront w requests segments 4 w + j
-        const int r = (4 * wave + j) * T::RPI + lane / T::CPR, cp = lane % T::CPR;
-        lk[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_k(r)) + 3072u - 1024u * j;
-        lv[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_v(r)) + 3072u - 1024u * j;
-      }
-      // last key a row may see; rows past the end of q repeat the last one
-      const int row_limit = a.causal ? min(offset + min(row0 + n_lane, a.sq - 1), a.skv - 1) : a.skv - 1;
-      const int first_limit = a.causal ? min(offset + row0, a.skv - 1) : a.skv - 1;
-      const int k_requests = max(min(n + 1, last_tile) - 1, 0), v_requests = min(n, last_tile);
-      const uint32_t m0_base = lds0 + 4096u * (uint32_t)wave;
-      if constexpr (MODE == 0) {
-        const int64_t head = b * a.kv_bs + hk * a.kv_hs;
-        const uint64_t kb = reinterpret_cast<uint64_t>(a.k + head + (int64_t)2 * kKeysPerTile * a.kv_ts) - 3072u;
-        const uint64_t vb = reinterpret_cast<uint64_t>(a.v + head + (int64_t)kKeysPerTile * a.kv_ts) - 3072u;
-        stream_tiles_dense(ss, q_lo, q_hi, ko, vo, lk, lv, row_limit - 4 * h, kb, vb,
-                           (uint32_t)(2 * kKeysPerTile * a.kv_ts), a.scale_log2e, n, k_requests, v_requests,
-                           first_limit - 30, m0_base);
-      } else {
-        const int tpb = a.bs / kKeysPerTile;
-        const uint32_t slab = (uint32_t)a.bs * (uint32_t)T::RB;
-        // tile 1: its block is blk_v's, tile (1 % tpb) inside it
-        const uint64_t v_off = (uint64_t)((int64_t)blk_v.phys[0] * a.hkv + hk) * slab + (uint64_t)(1 % tpb) * T::TILE_BYTES;
-        const uint64_t e_ptr = reinterpret_cast<uint64_t>(a.pt + (int64_t)b * a.pt_rs + 3 / tpb);
-        stream_tiles_paged(ss, q_lo, q_hi, ko, vo, lk, lv, row_limit - 4 * h,
-                           reinterpret_cast<uint64_t>(a.k) - 3072u, reinterpret_cast<uint64_t>(a.v) - 3072u, slab,
-                           a.scale_log2e, n, k_requests, v_requests, first_limit - 30, m0_base, a.hkv, hk, a.nb,
-                           tpb, req.raw[0], e_ptr, v_off, max(last_tile - 2, 0));
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[0][i] = ss.acc[i];
-      m_run[0] = ss.mc / a.scale_log2e;
-      l_run[0] = ss.lrun;
-      kt_begin = n;
-    }
   }
   // The first K fragments of a tile are read one tile ahead (K(t+1) has landed at the barrier
   // of tile t), so the score product starts without waiting for LDS.
@@ -1117,7 +1161,9 @@ int launch_mode(const PrefillArgs &a, hipStream_t st) {
   constexpr int ROWS = kRowsPerWave * RH;
   const int nqt = (a.sq + ROWS * RPW - 1) / (ROWS * RPW);
   // two stages of a K and a V tile; with two row blocks three K tiles and two V tiles
-  const size_t lds = RH == 2 ? 5 * Tile<D>::TILE_BYTES : 2 * Tile<D>::STAGE_BYTES;
+  // (the hand-scheduled loop keeps two rings of five 8 KiB blocks)
+  constexpr bool kStreams = D == 128 && HPW == 4 && RH == 1 && (MODE == 0 || MODE == 1);
+  const size_t lds = RH == 2 ? 5 * Tile<D>::TILE_BYTES : (kStreams ? (size_t)TTPA_STREAM_LDS_BYTES : 2 * Tile<D>::STAGE_BYTES);
   static std::atomic<uint64_t> lds_ready{0};
   if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&prefill_kernel<D, HPW, MODE, RH>), lds, lds_ready))
     return fail(TTPA_ERR_LAUNCH, "prefill: cannot reserve %zu bytes of LDS", lds);
@@ -1264,8 +1310,9 @@ static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_st
       return fail(TTPA_ERR_UNSUPPORTED, "prefill: a block-float-8 cache needs block_size %% 16 == 0");
   }
   {
+    // (TTPA_PREFILL_STREAM=0, read on every call, sends every shape through the plain loop)
     const char *e = getenv("TTPA_PREFILL_STREAM");
-    a.stream = e ? atoi(e) : 0;
+    a.stream = e ? atoi(e) : 1;
   }
   a.bs_magic = block_size >= 2 ? (uint32_t)((1ull << 32) / (uint32_t)block_size) + 1u : 0u;
   a.fill_kc = a.fill_vc = nullptr;
