@@ -183,6 +183,27 @@ int ttpa_paged_sdpa_decode_windowed(void *out, int64_t out_user_stride, int64_t 
                                     size_t workspace_bytes, void *stream);
 
 /*
+ * Decode with an explicit additive mask in place of the causal rule: the `is_causal=False` form
+ * of tt::paged_scaled_dot_product_attention_decode (python_package/tt_torch/custom_ops.py:1296-1311,
+ * attn_weight += attn_mask) and of tt::scaled_dot_product_attention_decode on a static cache
+ * (custom_ops.py:817-842, where the mask differs between heads:
+ * tests/torch/ops/test_custom_ops.py:126-130).  mask is bfloat16, added to the scaled scores;
+ * the element for (user, query head, position) is mask[user * mask_user_stride +
+ * head * mask_head_stride + position] (a head stride of 0 shares one row between the heads).
+ * cur_pos[u] is the last position that is attended at all (the caller passes
+ * table_width * block_size - 1 to attend every position of the table).  bfloat16 caches, up to
+ * 8 query heads per KV head; the rest as ttpa_paged_sdpa_decode.
+ */
+int ttpa_paged_sdpa_decode_masked(void *out, int64_t out_user_stride, int64_t out_head_stride,
+                                  const void *q, int64_t q_user_stride, int64_t q_head_stride,
+                                  const void *k_cache, const void *v_cache, const int32_t *page_table,
+                                  int64_t page_table_row_stride, const void *cur_pos, int cur_pos_is_i64,
+                                  int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
+                                  int32_t block_size, int32_t table_width, int32_t num_blocks, float scale,
+                                  const void *mask, int64_t mask_user_stride, int64_t mask_head_stride,
+                                  void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * The decode step of the attention backend in one call: the cache update
  * (ttpa_paged_update_cache_kv with update_indices = cur_pos: the new token of user u goes to
  * position cur_pos[u]) followed by ttpa_paged_sdpa_decode_windowed on the updated caches
@@ -262,6 +283,23 @@ int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t out_head_s
                           int32_t head_dim_v, int32_t block_size, int32_t table_width,
                           int32_t num_blocks, float scale, const float *attention_sink,
                           void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * The same with an explicit additive mask (tt::paged_flash_mla_decode with is_causal=False,
+ * custom_ops.py:590-608: additive_mask = attn_mask; tt::flash_mla_prefill with attn_mask,
+ * custom_ops.py:343-357, served with query row i as user i).  mask as in
+ * ttpa_paged_sdpa_decode_masked; scale must not be 0.  Runs on the workgroup-shared kernel for
+ * every shape.
+ */
+int ttpa_paged_mla_decode_masked(void *out, int64_t out_user_stride, int64_t out_head_stride,
+                                 const void *q, int64_t q_user_stride, int64_t q_head_stride,
+                                 const void *k_cache, const void *v_cache, const int32_t *page_table,
+                                 int64_t page_table_row_stride, const void *cur_pos, int cur_pos_is_i64,
+                                 int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
+                                 int32_t head_dim_v, int32_t block_size, int32_t table_width,
+                                 int32_t num_blocks, float scale, const void *mask, int64_t mask_user_stride,
+                                 int64_t mask_head_stride, void *workspace, size_t workspace_bytes,
+                                 void *stream);
 
 /*
  * Measurement hook, no reference counterpart: the NEXT attention call made by this host

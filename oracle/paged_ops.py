@@ -474,15 +474,20 @@ def fill_cache(cache, fill_value, batch_offset=None):
     return out
 
 
-def sdpa_decode_static(query, key, value, cur_pos_tensor, scale=None):
-    """custom_ops.py:817-842 with attn_mask=None: additive mask of -inf to the right of each
-    user's position, then the library SDPA with grouped heads, in the query's dtype."""
+def sdpa_decode_static(query, key, value, cur_pos_tensor, scale=None, attn_mask=None):
+    """custom_ops.py:817-842: with attn_mask=None an additive mask of -inf to the right of each
+    user's position; with one (is_causal=False), the mask itself, one row per query head
+    ([batch, 1, heads, max_seq] reshaped to [batch, heads, 1, max_seq], custom_ops.py:820-821).
+    Then the library SDPA with grouped heads, in the query's dtype."""
     batch, heads, d = query.shape[1], query.shape[2], query.shape[3]
     max_seq = key.shape[-2]
     q = query.reshape(batch, heads, 1, d)
-    mask = torch.zeros(batch, heads, 1, max_seq, dtype=q.dtype)
-    for b in range(batch):
-        mask[b, ..., int(cur_pos_tensor[b]) + 1 :] = float("-inf")
+    if attn_mask is not None:
+        mask = attn_mask.reshape(batch, heads, 1, max_seq)
+    else:
+        mask = torch.zeros(batch, heads, 1, max_seq, dtype=q.dtype)
+        for b in range(batch):
+            mask[b, ..., int(cur_pos_tensor[b]) + 1 :] = float("-inf")
     out = F.scaled_dot_product_attention(q, key, value, mask, is_causal=False, scale=scale, enable_gqa=True)
     return out.reshape(1, batch, heads, d)
 
@@ -498,9 +503,11 @@ def flash_mla_prefill(query, key, head_dim_v, value=None, attn_mask=None, is_cau
                                           scale=scale, enable_gqa=True)
 
 
-def paged_flash_mla_decode(query, key, head_dim_v, page_table, value=None, cur_pos_tensor=None, scale=None):
-    """custom_ops.py:551-610, causal form: gather each user's blocks, additive mask to the right
-    of cur_pos, library SDPA with grouped heads, in the query's dtype."""
+def paged_flash_mla_decode(query, key, head_dim_v, page_table, value=None, cur_pos_tensor=None, scale=None,
+                           attn_mask=None):
+    """custom_ops.py:551-610: gather each user's blocks; additive mask to the right of cur_pos
+    (causal form) or attn_mask itself (is_causal=False, custom_ops.py:590-592); library SDPA
+    with grouped heads, in the query's dtype."""
     block_size, nkv, dh = key.shape[-2], key.shape[-3], key.shape[-1]
     users, hq = query.shape[1], query.shape[2]
     max_seq = page_table.shape[1] * block_size
@@ -511,9 +518,12 @@ def paged_flash_mla_decode(query, key, head_dim_v, page_table, value=None, cur_p
     else:
         gv = gk[..., :head_dim_v]
     q = query.reshape(users, hq, 1, dh)
-    mask = torch.zeros(users, 1, 1, max_seq, dtype=query.dtype)
-    for i in range(users):
-        mask[i, :, :, int(cur_pos_tensor[i]) + 1 :] = float("-inf")
+    if attn_mask is not None:
+        mask = attn_mask
+    else:
+        mask = torch.zeros(users, 1, 1, max_seq, dtype=query.dtype)
+        for i in range(users):
+            mask[i, :, :, int(cur_pos_tensor[i]) + 1 :] = float("-inf")
     scale_val = 1.0 / (dh**0.5) if scale is None else scale
     out = F.scaled_dot_product_attention(q, gk, gv, mask, is_causal=False, scale=scale_val, enable_gqa=True)
     return out.reshape(1, users, hq, head_dim_v)

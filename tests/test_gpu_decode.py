@@ -313,7 +313,29 @@ def test_decode_with_explicit_mask(hq, hkv, d, bs, bfp8):
     want_b = O.paged_sdpa_decode(q.float(), key.float(), value.float(), table, False,
                                  torch.zeros(users, 1, 1, span).masked_fill(~keep, float("-inf")), cur, None, 0.11)
     torch.testing.assert_close(got_b.float(), want_b, atol=ATOL, rtol=RTOL)
-    with pytest.raises(NotImplementedError):  # a mask per head
-        torch.ops.tt.paged_scaled_dot_product_attention_decode(
-            q.cuda(), kd, vd, table.cuda(), is_causal=False, attn_mask=mask.expand(users, hq, 1, span).cuda(),
-            cur_pos_tensor=cur.cuda())
+    # a mask per head: on the decode kernel for bfloat16 caches, refused on the gathered form
+    mask_h = (mask + 0.5 * torch.randn(users, hq, 1, span, generator=g).to(torch.bfloat16)).to(torch.bfloat16)
+    if bfp8:
+        with pytest.raises(NotImplementedError):
+            torch.ops.tt.paged_scaled_dot_product_attention_decode(
+                q.cuda(), kd, vd, table.cuda(), is_causal=False, attn_mask=mask_h.cuda(), cur_pos_tensor=cur.cuda())
+    else:
+        got_h = torch.ops.tt.paged_scaled_dot_product_attention_decode(
+            q.cuda(), kd, vd, table.cuda(), is_causal=False, attn_mask=mask_h.cuda(), cur_pos_tensor=cur.cuda(),
+            scale=0.11).cpu()
+        want_h = O.paged_sdpa_decode(q.float(), key.float(), value.float(), table, False, mask_h.float(), cur, None, 0.11)
+        err = (got_h.float() - want_h).abs().max().item()
+        print(f"{name}, one mask row per head: max-abs error {err:.3e}", flush=True)
+        torch.testing.assert_close(got_h.float(), want_h, atol=ATOL, rtol=RTOL)
+    # table entries outside the cache (padding -1, ids past the last block) read block 0, as the
+    # kernels promise; with -inf on their positions the result is that of the valid part
+    bad = table.clone()
+    bad[0, w - 1], bad[1, w - 2] = -1, nb + 7
+    mask_b = mask.clone()
+    mask_b[0, :, :, (w - 1) * bs:] = float("-inf")
+    mask_b[1, :, :, (w - 2) * bs:(w - 1) * bs] = float("-inf")
+    got_x = torch.ops.tt.paged_scaled_dot_product_attention_decode(
+        q.cuda(), kd, vd, bad.cuda(), is_causal=False, attn_mask=mask_b.cuda(), cur_pos_tensor=cur.cuda(),
+        scale=0.11).cpu()
+    want_x = O.paged_sdpa_decode(q.float(), key.float(), value.float(), table, False, mask_b.float(), cur, None, 0.11)
+    torch.testing.assert_close(got_x.float(), want_x, atol=ATOL, rtol=RTOL)

@@ -109,10 +109,6 @@ def test_mla_decode_padded_row_sink_and_errors():
         lse = torch.logsumexp((q[0, u].float() @ kk.T) / math.sqrt(dh), dim=-1)  # [hq]
         want = base[0, u] * torch.sigmoid(lse - sink).unsqueeze(-1)
         torch.testing.assert_close(got[0, u].float(), want, atol=ATOL, rtol=RTOL)
-    with pytest.raises(NotImplementedError):
-        torch.ops.tt.paged_flash_mla_decode(q.cuda(), key.cuda(), dv, table.cuda(), None, False,
-                                            torch.zeros(users, 1, 1, width * bs, dtype=torch.bfloat16).cuda(),
-                                            pos.cuda(), None, None)
     with pytest.raises(AssertionError):
         torch.ops.tt.paged_flash_mla_decode(q.cuda(), key.cuda(), 600, table.cuda(), None, True, None,
                                             pos.cuda(), None, None)
@@ -140,8 +136,65 @@ def test_flash_mla_prefill(b, hq, s, dh, nkv, dv, has_value):
     assert got.shape == (b, hq, s, dv)
     want = O.flash_mla_prefill(q.float(), k.float(), dv, None if v is None else v.float(), None, True, 1.0)
     _check(f"mla prefill b{b} h{hq} s{s} dh{dh} dv{dv}", got, want)
-    with pytest.raises(NotImplementedError):
-        torch.ops.tt.flash_mla_prefill(q.cuda(), k.cuda(), dv, None, torch.zeros(b, 1, s, s, dtype=torch.bfloat16).cuda(), False, 1.0)
+
+
+MASKED_PREFILL = [
+    # batch, heads, seq, head_size, kv_heads, head_dim_v, has_value: the is_causal=False rows of the
+    # reference grid (tests/torch/ops/test_custom_ops.py:236-248), one mask [b, 1, s, s] for all heads
+    (1, 16, 64, 192, 1, 128, False),
+    (2, 16, 128, 192, 1, 128, False),
+    (1, 32, 64, 128, 1, 128, False),
+    (2, 16, 128, 128, 1, 64, True),
+    (1, 16, 96, 576, 1, 512, False),   # latent serving shape
+]
+
+
+@pytest.mark.parametrize("per_head", [False, True])
+@pytest.mark.parametrize("b,hq,s,dh,nkv,dv,has_value", MASKED_PREFILL)
+def test_flash_mla_prefill_with_mask(b, hq, s, dh, nkv, dv, has_value, per_head):
+    print(f"case: masked mla prefill b{b} h{hq} s{s} dh{dh} kv{nkv} dv{dv} value={has_value} per_head={per_head}", flush=True)
+    g = torch.Generator().manual_seed(s + dh + hq + 1)
+    q = (_bf(g, b, hq, s, dh).float() * 0.15).to(torch.bfloat16)
+    k = _bf(g, b, nkv, s, dh)
+    v = _bf(g, b, nkv, s, dv) if has_value else None
+    mask = _bf(g, b, hq if per_head else 1, s, s)
+    keep = torch.rand(b, 1, s, s, generator=g) > 0.3
+    keep[..., 0] = True
+    mask = mask.masked_fill(~keep, float("-inf"))
+    got = torch.ops.tt.flash_mla_prefill(q.cuda(), k.cuda(), dv, v.cuda() if has_value else None, mask.cuda(), False, 1.0).cpu()
+    assert got.shape == (b, hq, s, dv)
+    want = O.flash_mla_prefill(q.float(), k.float(), dv, None if v is None else v.float(), mask.float(), False, 1.0)
+    _check(f"masked mla prefill b{b} h{hq} s{s} dh{dh} dv{dv}", got, want)
+
+
+@pytest.mark.parametrize("users,hq,nkv,dh,dv,has_value,bs,width,scale", [
+    (8, 16, 1, 192, 128, False, 32, 16, 1.0), (8, 32, 1, 128, 128, False, 32, 16, 1.0),
+    (8, 16, 1, 128, 64, True, 32, 16, 1.0), (8, 16, 4, 192, 128, False, 32, 16, 1.0),
+    (4, 16, 1, 576, 512, False, 32, 24, None), (3, 128, 1, 576, 512, False, 64, 12, None),
+])
+def test_paged_flash_mla_decode_with_mask(users, hq, nkv, dh, dv, has_value, bs, width, scale):
+    """is_causal=False (reference custom_ops.py:590-592): every position of the table, weighted by
+    attn_mask; one row for all heads and one row per head."""
+    g = torch.Generator().manual_seed(users * dh + hq + bs + 5)
+    nb = width * users
+    q = (_bf(g, 1, users, hq, dh).float() * (0.15 if scale == 1.0 else 1.0)).to(torch.bfloat16)
+    key = _bf(g, nb, nkv, bs, dh)
+    value = _bf(g, nb, nkv, bs, dv) if has_value else None
+    table = torch.randperm(nb, generator=g).view(users, width).to(torch.int32)
+    span = width * bs
+    for per_head in (False, True):
+        print(f"case: masked mla decode u{users} h{hq}x{nkv} dh{dh} dv{dv} bs{bs} w{width} per_head={per_head}", flush=True)
+        mask = _bf(g, users, hq if per_head else 1, 1, span)
+        keep = torch.rand(users, 1, 1, span, generator=g) > 0.4
+        keep[..., 0] = True
+        mask = mask.masked_fill(~keep, float("-inf"))
+        got = torch.ops.tt.paged_flash_mla_decode(
+            q.cuda(), key.cuda(), dv, table.cuda(), value.cuda() if has_value else None, False, mask.cuda(),
+            None, None, scale).cpu()
+        assert got.shape == (1, users, hq, dv)
+        want = O.paged_flash_mla_decode(q.float(), key.float(), dv, table, None if value is None else value.float(),
+                                        None, scale, mask.float())
+        _check(f"masked mla decode u{users} h{hq}x{nkv} dh{dh} dv{dv} per_head={per_head}", got, want)
 
 
 def test_mla_backend_prefill_then_decode():

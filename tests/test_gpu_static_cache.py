@@ -84,6 +84,36 @@ def test_static_decode(b, hq, hkv, s, d, pos):
     torch.testing.assert_close(got.float(), want, atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("b,hq,d,hkv,s", [
+    # the is_causal=False rows of the reference grid (tests/torch/ops/test_custom_ops.py:99-110)
+    (1, 12, 128, 12, 32), (1, 12, 128, 12, 128), (8, 12, 128, 12, 128),
+    (1, 12, 128, 4, 32), (1, 12, 128, 4, 128), (8, 12, 128, 4, 128),
+    (3, 16, 64, 2, 96),   # eight heads per KV head
+])
+def test_static_decode_with_mask(b, hq, d, hkv, s):
+    """attn_mask [B, 1, heads, S] with is_causal=False (reference custom_ops.py:817-842): every
+    position, one mask row per query head, against the oracle and against an fp32 loop."""
+    g = torch.Generator().manual_seed(s + d + hq + b)
+    key, value = _bf(g, b, hkv, s, d), _bf(g, b, hkv, s, d)
+    q = (_bf(g, 1, b, hq, d).float() * 0.3).to(torch.bfloat16)
+    cur = torch.arange(b, dtype=torch.int32)
+    mask = _bf(g, b, 1, hq, s)
+    keep = torch.rand(b, 1, hq, s, generator=g) > 0.3
+    keep[..., 0] = True
+    mask = mask.masked_fill(~keep, float("-inf"))
+    got = torch.ops.tt.scaled_dot_product_attention_decode(q.cuda(), key.cuda(), value.cuda(), cur.cuda(),
+                                                           mask.cuda(), None, False, 1.0).cpu()
+    want = O.sdpa_decode_static(q, key, value, cur, 1.0, mask)
+    err = (got.float() - want.float()).abs().max().item()
+    print(f"masked static decode b{b} h{hq}x{hkv} s{s} d{d}: max-abs error {err:.3e}", flush=True)
+    torch.testing.assert_close(got.float(), want.float(), atol=2e-2, rtol=2e-2)
+    grp = hq // hkv
+    for u in range(b):
+        for h in range(hq):
+            w = torch.softmax(q[0, u, h].float() @ key[u, h // grp].float().T + mask[u, 0, h].float(), dim=-1)
+            torch.testing.assert_close(got[0, u, h].float(), w @ value[u, h // grp].float(), atol=2e-2, rtol=2e-2)
+
+
 def test_copy_kv_blocks_round_trip():
     """Block swap (reference model_runner.py:5433-5474): d2h then h2d into other block ids
     reproduces the blocks bit for bit, other blocks stay untouched, and the no-op rules hold."""

@@ -41,3 +41,21 @@ def test_static_decode_is_the_paged_decode_on_an_identity_table_and_the_fp32_loo
     torch.testing.assert_close(got, want, atol=1e-5, rtol=1e-5)
     paged = O.paged_sdpa_decode(q, key, value, table, True, None, pos, None, None)
     torch.testing.assert_close(got, paged.float(), atol=1e-5, rtol=1e-5)
+
+
+def test_static_decode_with_a_mask_per_head_against_an_fp32_loop():
+    """attn_mask [B, 1, heads, S] (reference custom_ops.py:817-842 with is_causal=False): all positions,
+    score + the head's mask row; cur_pos plays no part."""
+    g = torch.Generator().manual_seed(4)
+    b, hq, hkv, s, d = 3, 6, 2, 20, 16
+    key, value = torch.randn(b, hkv, s, d, generator=g), torch.randn(b, hkv, s, d, generator=g)
+    q = torch.randn(1, b, hq, d, generator=g)
+    mask = torch.randn(b, 1, hq, s, generator=g)
+    mask[..., 2::5] = float("-inf")
+    got = O.sdpa_decode_static(q, key, value, torch.zeros(b, dtype=torch.int32), 0.25, mask)
+    other = O.sdpa_decode_static(q, key, value, torch.full((b,), s - 1, dtype=torch.int32), 0.25, mask)
+    assert torch.equal(got, other)
+    for u in range(b):
+        for h in range(hq):
+            p = torch.softmax((key[u, h // 3] @ q[0, u, h]) * 0.25 + mask[u, 0, h], dim=0)
+            torch.testing.assert_close(got[0, u, h], p @ value[u, h // 3], atol=1e-5, rtol=1e-5)

@@ -200,6 +200,9 @@ __global__ __launch_bounds__(256, (D <= 128 && G <= 4) ? 2 : 1) void paged_decod
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       float sv = valid ? s[g] * a.scale_log2e : -INFINITY;
+      if (a.mask != nullptr && valid)
+        sv += bf16_lo(a.mask[cur.u * a.mask_us + (int64_t)(cur.h * G + g) * a.mask_hs + cur.t * kTile + 4 * my_step + r]) *
+              1.4426950408889634f;
       float mx = fmaxf(m[g], row16_max(sv));
       float msafe = (mx == -INFINITY) ? 0.f : mx;
       float alpha = __builtin_amdgcn_exp2f(m[g] - msafe);
@@ -379,7 +382,8 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
                        int32_t kv_format, int32_t sliding_window, const float *attention_sink,
                        void *workspace, size_t workspace_bytes, void *stream,
                        const void *k_new = nullptr, const void *v_new = nullptr,
-                       int64_t new_user_stride = 0, int64_t new_head_stride = 0) {
+                       int64_t new_user_stride = 0, int64_t new_head_stride = 0,
+                       const void *mask = nullptr, int64_t mask_user_stride = 0, int64_t mask_head_stride = 0) {
   TTPA_REQUIRE(sliding_window >= 0, "decode: sliding_window %d is negative", sliding_window);
   TTPA_REQUIRE(out && q && k_cache && v_cache && page_table && cur_pos, "null pointer argument");
   TTPA_REQUIRE(users > 0 && q_heads > 0 && kv_heads > 0 && head_size > 0 && block_size > 0 &&
@@ -430,6 +434,11 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   a.sink = attention_sink;
   a.k_new = a.v_new = nullptr;
   a.new_us = a.new_hs = 0;
+  a.mask = static_cast<const uint16_t *>(mask);
+  a.mask_us = mask_user_stride, a.mask_hs = mask_head_stride;
+  if (mask && (g > 8 || kv_format != TTPA_KV_BF16))
+    return fail(TTPA_ERR_UNSUPPORTED,
+                "masked decode: built for bfloat16 caches and up to 8 query heads per KV head (got %d)", g);
 
   hipStream_t st = static_cast<hipStream_t>(stream);
   // Kernel choice.  The VALU kernel spends per-head work on every tile; the matrix-core kernels
@@ -464,6 +473,7 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   if (forced == 1 && g <= 8 && !(kv_format == TTPA_KV_BFP8 && head_size == 256)) use_mfma = use_mfma16 = false;
   if (forced == 2 && mfma_ok) use_mfma = true, use_mfma16 = false;
   if (forced == 3 && mfma16_ok) use_mfma16 = true, use_mfma = false;
+  if (mask) use_mfma = use_mfma16 = false;  // only the dot-product kernel applies a mask
   // The matrix-core kernels get at most one workgroup per CU whatever the cache format: the 32x32
   // kernel fills the CU's LDS with one, and the 16x16 kernel streams as fast with one as with the
   // two that would fit, while twice the partials cost the merge kernel more.  On a bfloat16 cache
@@ -560,6 +570,22 @@ extern "C" int ttpa_paged_sdpa_decode_windowed(
                      v_cache, page_table, page_table_row_stride, cur_pos, cur_pos_is_i64, users,
                      q_heads, kv_heads, head_size, block_size, table_width, num_blocks, scale,
                      kv_format, sliding_window, attention_sink, workspace, workspace_bytes, stream);
+}
+
+extern "C" int ttpa_paged_sdpa_decode_masked(
+    void *out, int64_t out_user_stride, int64_t out_head_stride, const void *q,
+    int64_t q_user_stride, int64_t q_head_stride, const void *k_cache, const void *v_cache,
+    const int32_t *page_table, int64_t page_table_row_stride, const void *cur_pos,
+    int cur_pos_is_i64, int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
+    int32_t block_size, int32_t table_width, int32_t num_blocks, float scale, const void *mask,
+    int64_t mask_user_stride, int64_t mask_head_stride, void *workspace, size_t workspace_bytes,
+    void *stream) {
+  TTPA_REQUIRE(mask != nullptr, "masked decode: null mask");
+  return decode_impl(out, out_user_stride, out_head_stride, q, q_user_stride, q_head_stride, k_cache,
+                     v_cache, page_table, page_table_row_stride, cur_pos, cur_pos_is_i64, users,
+                     q_heads, kv_heads, head_size, block_size, table_width, num_blocks, scale,
+                     TTPA_KV_BF16, 0, nullptr, workspace, workspace_bytes, stream, nullptr, nullptr, 0, 0,
+                     mask, mask_user_stride, mask_head_stride);
 }
 
 // ---- the entry point that allocates nothing ------------------------------------------------

@@ -45,6 +45,12 @@ struct DecodeArgs {
   // k_new / v_new [users][>= hkv heads][head_size] instead of the cache, and written to it.
   const uint16_t *k_new, *v_new;
   int64_t new_us, new_hs;
+  // Additive mask on the scaled scores (bfloat16, natural-log units), or null: the element for
+  // (user, query head, position) is mask[user * mask_us + head * mask_hs + position].  Applied by the
+  // dot-product kernel (decode.hip) and by the workgroup-shared latent kernel (decode_wide.hip); the
+  // entry points that take a mask launch only those.
+  const uint16_t *mask = nullptr;
+  int64_t mask_us = 0, mask_hs = 0;
 };
 
 // First attended position of a user whose attended range ends at `len` (exclusive).

@@ -200,6 +200,18 @@ __global__ __launch_bounds__(256, 1) void paged_decode_wide_kernel(
           if (key >= nvalid || key < nbelow) st[kb][r] = -INFINITY;
         }
     }
+    if (a.mask != nullptr) {  // additive mask, brought to the units of the raw scores
+      const float unit = 1.4426950408889634f / a.scale_log2e;
+      const uint16_t *mrow = a.mask + cur.u * a.mask_us + (int64_t)(cur.h * G + min(n, G - 1)) * a.mask_hs +
+                             cur.t * kTile + 4 * h;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = 32 * kb + 8 * (r >> 2) + (r & 3);
+          if (key + 4 * h < nvalid) st[kb][r] += bf16_lo(mrow[key]) * unit;
+        }
+    }
     const float scale = a.scale_log2e;
     float mloc = -INFINITY;  // the maximum is tracked on scaled scores (the scale may be negative)
 #pragma unroll
@@ -643,15 +655,16 @@ extern "C" size_t ttpa_paged_mla_decode_workspace_bytes(int32_t users, int32_t q
   return header_bytes(users, kv_heads * nhb) + ((size_t)cus * kWavesPerBlockHost + segs) * slot;
 }
 
-extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t out_head_stride,
-                                     const void *q, int64_t q_user_stride, int64_t q_head_stride,
-                                     const void *k_cache, const void *v_cache, const int32_t *page_table,
-                                     int64_t page_table_row_stride, const void *cur_pos,
-                                     int cur_pos_is_i64, int32_t users, int32_t q_heads,
-                                     int32_t kv_heads, int32_t head_size, int32_t head_dim_v,
-                                     int32_t block_size, int32_t table_width, int32_t num_blocks,
-                                     float scale, const float *attention_sink, void *workspace,
-                                     size_t workspace_bytes, void *stream) {
+static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stride,
+                           const void *q, int64_t q_user_stride, int64_t q_head_stride,
+                           const void *k_cache, const void *v_cache, const int32_t *page_table,
+                           int64_t page_table_row_stride, const void *cur_pos,
+                           int cur_pos_is_i64, int32_t users, int32_t q_heads,
+                           int32_t kv_heads, int32_t head_size, int32_t head_dim_v,
+                           int32_t block_size, int32_t table_width, int32_t num_blocks,
+                           float scale, const float *attention_sink, void *workspace,
+                           size_t workspace_bytes, void *stream, const void *mask,
+                           int64_t mask_user_stride, int64_t mask_head_stride) {
   TTPA_REQUIRE(out && q && k_cache && page_table && cur_pos, "null pointer argument");
   TTPA_REQUIRE(users > 0 && q_heads > 0 && kv_heads > 0 && head_size > 0 && head_dim_v > 0 &&
                    block_size > 0 && table_width > 0 && num_blocks > 0,
@@ -700,6 +713,9 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
   a.kv_format = TTPA_KV_BF16;
   a.window = 0;
   a.sink = attention_sink;
+  a.mask = static_cast<const uint16_t *>(mask);
+  a.mask_us = mask_user_stride, a.mask_hs = mask_head_stride;
+  if (mask) TTPA_REQUIRE(scale != 0.f, "masked latent decode: scale must not be 0");
   WideArgs w;
   w.nkv = kv_heads, w.nhb = nhb, w.gseg = gseg, w.dv = head_dim_v, w.n_slices = head_dim_v / dvw;
 
@@ -712,7 +728,8 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
   // The 16-head form: V taken from K, one head block of up to 16 heads, tiles inside one block.
   // TTPA_LATENT_KERNEL=wide (read on every call) keeps such shapes on the workgroup-shared form.
   const char *force = getenv("TTPA_LATENT_KERNEL");
-  const bool want16 = shared && nhb == 1 && gseg <= 16 && block_size % 16 == 0 && !(force && force[0] == 'w');
+  // (only the workgroup-shared form applies a mask)
+  const bool want16 = !mask && shared && nhb == 1 && gseg <= 16 && block_size % 16 == 0 && !(force && force[0] == 'w');
   if (want16) {
     // three wavefront ranges per CU: 131 us per step on the 128-user workload against 134 at four
     // (fewer partials of 32 KiB each), 139 at 2.5 and 159 at two; TTPA_DECODE_WAVES_PER_CU overrides,
@@ -771,4 +788,36 @@ extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t
   if (int rc = check_launch("paged_mla_decode")) return rc;
   decode_combine_kernel<<<dim3(users * kv_heads * nhb, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
   return check_launch("paged_mla_decode");
+}
+
+extern "C" int ttpa_paged_mla_decode(void *out, int64_t out_user_stride, int64_t out_head_stride,
+                                     const void *q, int64_t q_user_stride, int64_t q_head_stride,
+                                     const void *k_cache, const void *v_cache, const int32_t *page_table,
+                                     int64_t page_table_row_stride, const void *cur_pos,
+                                     int cur_pos_is_i64, int32_t users, int32_t q_heads,
+                                     int32_t kv_heads, int32_t head_size, int32_t head_dim_v,
+                                     int32_t block_size, int32_t table_width, int32_t num_blocks,
+                                     float scale, const float *attention_sink, void *workspace,
+                                     size_t workspace_bytes, void *stream) {
+  return mla_decode_impl(out, out_user_stride, out_head_stride, q, q_user_stride, q_head_stride, k_cache, v_cache,
+                         page_table, page_table_row_stride, cur_pos, cur_pos_is_i64, users, q_heads, kv_heads,
+                         head_size, head_dim_v, block_size, table_width, num_blocks, scale, attention_sink,
+                         workspace, workspace_bytes, stream, nullptr, 0, 0);
+}
+
+extern "C" int ttpa_paged_mla_decode_masked(void *out, int64_t out_user_stride, int64_t out_head_stride,
+                                            const void *q, int64_t q_user_stride, int64_t q_head_stride,
+                                            const void *k_cache, const void *v_cache, const int32_t *page_table,
+                                            int64_t page_table_row_stride, const void *cur_pos,
+                                            int cur_pos_is_i64, int32_t users, int32_t q_heads,
+                                            int32_t kv_heads, int32_t head_size, int32_t head_dim_v,
+                                            int32_t block_size, int32_t table_width, int32_t num_blocks,
+                                            float scale, const void *mask, int64_t mask_user_stride,
+                                            int64_t mask_head_stride, void *workspace, size_t workspace_bytes,
+                                            void *stream) {
+  TTPA_REQUIRE(mask != nullptr, "masked latent decode: null mask");
+  return mla_decode_impl(out, out_user_stride, out_head_stride, q, q_user_stride, q_head_stride, k_cache, v_cache,
+                         page_table, page_table_row_stride, cur_pos, cur_pos_is_i64, users, q_heads, kv_heads,
+                         head_size, head_dim_v, block_size, table_width, num_blocks, scale, nullptr, workspace,
+                         workspace_bytes, stream, mask, mask_user_stride, mask_head_stride);
 }

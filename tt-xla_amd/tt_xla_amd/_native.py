@@ -56,6 +56,11 @@ SIGNATURES = {
         [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _i64, _p, _int, _i32, _i32, _i32, _i32, _i32,
          _i32, _i32, _f32, _i32, _i32, _p, _p, _sz, _p],
     ),
+    "ttpa_paged_sdpa_decode_masked": (
+        _int,
+        [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _i64, _p, _int, _i32, _i32, _i32, _i32, _i32,
+         _i32, _i32, _f32, _p, _i64, _i64, _p, _sz, _p],
+    ),
     "ttpa_paged_update_decode": (
         _int,
         [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _int, _i32, _i32,
@@ -73,6 +78,11 @@ SIGNATURES = {
         _int,
         [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _i64, _p, _int, _i32, _i32, _i32, _i32, _i32,
          _i32, _i32, _i32, _f32, _p, _p, _sz, _p],
+    ),
+    "ttpa_paged_mla_decode_masked": (
+        _int,
+        [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _i64, _p, _int, _i32, _i32, _i32, _i32, _i32,
+         _i32, _i32, _i32, _f32, _p, _i64, _i64, _p, _sz, _p],
     ),
     "ttpa_sdpa_prefill": (
         _int,

@@ -383,7 +383,7 @@ def _decode(query, key, value, page_table, is_causal, attn_mask, cur_pos_tensor,
     else:
         _check_out(out, (1, users, hq, d), "decode")
     ws_bytes = N.lib().ttpa_paged_decode_workspace_bytes(users, hq, hkv, d)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=query.device)
+    ws = _workspace(ws_bytes, query.device)
     sink = None
     if attention_sink is not None:
         if attention_sink.numel() != hq:
@@ -419,13 +419,45 @@ def _decode(query, key, value, page_table, is_causal, attn_mask, cur_pos_tensor,
     return out
 
 
+_WORKSPACES = {}
+
+
+def _workspace(nbytes: int, device) -> torch.Tensor:
+    """A per-device scratch tensor for the split-K partials of a decode launch, grown on demand and
+    reused by later calls: launches of one stream run in order, so one buffer serves them all, and
+    an eager serving loop pays no allocator round trip per layer and step.  Under graph capture the
+    allocation has to belong to the graph's pool, and a call on another stream must not share the
+    buffer, so both get a fresh tensor."""
+    if torch.cuda.is_current_stream_capturing() or torch.cuda.current_stream(device) != torch.cuda.default_stream(device):
+        return torch.empty(nbytes, dtype=torch.uint8, device=device)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _WORKSPACES[key] = ws
+    return ws
+
+
+def _decode_mask_rows(attn_mask, users, hq, skv):
+    """The additive mask of a one-token pass as (bfloat16 tensor, user stride, head stride): anything
+    that broadcasts to [users, heads, 1, skv]; a head stride of 0 shares one row between the heads."""
+    m = _additive_mask(attn_mask)
+    if m.dim() != 4 or m.shape[2] != 1 or m.shape[3] != skv or m.shape[0] not in (1, users) or m.shape[1] not in (1, hq):
+        raise ValueError(f"attn_mask must broadcast to [{users}, {hq}, 1, {skv}], got {tuple(attn_mask.shape)}")
+    if m.stride(-1) != 1:
+        m = m.contiguous()
+    return m, (m.stride(0) if m.shape[0] == users and users > 1 else 0), (m.stride(1) if m.shape[1] == hq and hq > 1 else 0)
+
+
 def _decode_masked(query, key, value, page_table, attn_mask, attention_sink, scale, sliding_window_size, out):
     """Decode with ``is_causal=False``: every position of the user's table is attended, weighted by
-    the additive ``attn_mask`` [users, 1, 1, table_width * block_size] (reference CPU branch
-    custom_ops.py:1296-1311; the one-token pass of a pooling / encoder model, never the
-    generative serving path).  Runs on the prefill kernel's masked dense form: the user's blocks
-    are gathered in table order (block-float-8 ones dequantised on the way) and the query token
-    is the first row of a 32-row tile.  A mask that differs between heads is not built."""
+    the additive ``attn_mask`` (anything that broadcasts to [users, heads, 1, table_width * block_size];
+    reference CPU branch custom_ops.py:1296-1311; the one-token pass of a pooling / encoder model,
+    never the generative serving path).  bfloat16 caches with up to 8 query heads per KV head run on
+    the decode kernel with the mask as an operand.  The rest (block-float-8 caches, wider groups)
+    goes through the prefill kernel's masked dense form, with one mask row for all heads: the user's
+    blocks are gathered in table order (ids outside the cache read block 0, as in the kernels) and
+    the query token is the first row of a 32-row tile."""
     if attn_mask is None:
         raise ValueError("attn_mask must be provided when is_causal is False")
     if attention_sink is not None or sliding_window_size is not None:
@@ -438,13 +470,36 @@ def _decode_masked(query, key, value, page_table, attn_mask, attention_sink, sca
         raise ValueError(f"query {tuple(query.shape)} {query.dtype} does not match the cache geometry")
     width = page_table.shape[1]
     skv = width * bs
-    if attn_mask.dim() != 4 or attn_mask.shape[0] != users or attn_mask.shape[2] != 1 or attn_mask.shape[3] != skv:
-        raise ValueError(f"attn_mask must be [users, 1, 1, {skv}], got {tuple(attn_mask.shape)}")
-    if attn_mask.shape[1] != 1:
-        raise NotImplementedError("a decode attn_mask that differs between heads is not built")
+    mask, mask_us, mask_hs = _decode_mask_rows(attn_mask, users, hq, skv)
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    if fmt == N.KV_BF16 and hq // hkv <= 8 and bs % 4 == 0:
+        q = _rows_contiguous(query)
+        pt = _table(page_table)
+        if out is None:
+            out = torch.empty((1, users, hq, d), dtype=query.dtype, device=query.device)
+        else:
+            _check_out(out, (1, users, hq, d), "decode")
+        last = torch.full((users,), skv - 1, dtype=torch.int32, device=query.device)
+        ws_bytes = N.lib().ttpa_paged_decode_workspace_bytes(users, hq, hkv, d)
+        ws = _workspace(ws_bytes, query.device)
+        N.call(
+            "ttpa_paged_sdpa_decode_masked",
+            out.data_ptr(), out.stride(1), out.stride(2), q.data_ptr(), q.stride(1), q.stride(2),
+            key.data_ptr(), value.data_ptr(), pt.data_ptr(), pt.stride(0), last.data_ptr(), 0,
+            users, hq, hkv, d, bs, width, nb, float(scale), mask.data_ptr(), mask_us, mask_hs,
+            ws.data_ptr(), ws_bytes, _stream(),
+        )
+        return out
+    if mask_hs != 0:
+        raise NotImplementedError(
+            "a decode attn_mask that differs between heads is built for bfloat16 caches with up to 8 query heads per KV head")
+
+    ids = page_table.reshape(-1).to(torch.int64)
+    ids = torch.where((ids >= 0) & (ids < nb), ids, torch.zeros_like(ids))
 
     def dense(cache):
-        g = torch.index_select(cache, 0, page_table.reshape(-1).to(torch.int64))
+        g = torch.index_select(cache, 0, ids)
         if fmt == N.KV_BFP8:
             g = bfp8_unpack_cache(g)
         return g.view(users, width, hkv, bs, d).permute(0, 2, 1, 3, 4).reshape(users, hkv, skv, d)
@@ -452,7 +507,7 @@ def _decode_masked(query, key, value, page_table, attn_mask, attention_sink, sca
     rows = 32  # the prefill kernel's query tile
     q = torch.zeros((users, hq, rows, d), dtype=torch.bfloat16, device=query.device)
     q[:, :, 0] = query[0]
-    mask = _additive_mask(attn_mask).expand(users, 1, rows, skv).contiguous()
+    mask = mask.expand(users, 1, 1, skv).expand(users, 1, rows, skv).contiguous()
     res = _prefill(q, dense(key), dense(value), None, None, mask, False, scale)[:, :, 0]  # [users, hq, d]
     if out is None:
         return res.unsqueeze(0).contiguous()
@@ -780,8 +835,9 @@ def paged_fill_kv_prefill_out_(
 _MLA_MAX_USERS = 1024  # users per launch of the latent decode kernel
 
 
-def _mla_decode_launch(out, q, key, value, page_table, cur, head_dim_v, scale, sink):
-    """out [users, heads, dv] / q [users, heads, dh] by strides; caches in the paged layout."""
+def _mla_decode_launch(out, q, key, value, page_table, cur, head_dim_v, scale, sink, mask=None):
+    """out [users, heads, dv] / q [users, heads, dh] by strides; caches in the paged layout.
+    mask: (bfloat16 tensor [users or 1, heads or 1, 1, positions], user stride, head stride) or None."""
     nb, nkv, bs, dh = key.shape
     users, hq = q.shape[0], q.shape[1]
     for u0 in range(0, users, _MLA_MAX_USERS):
@@ -792,8 +848,18 @@ def _mla_decode_launch(out, q, key, value, page_table, cur, head_dim_v, scale, s
                 f"latent attention with {hq} query heads over {nkv} KV heads is not built "
                 "(heads per KV head: up to 32 or a multiple of 32)"
             )
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+        ws = _workspace(ws_bytes, q.device)
         qs, os_, pts, curs = q[u0 : u0 + n], out[u0 : u0 + n], page_table[u0 : u0 + n], cur[u0 : u0 + n]
+        if mask is not None:
+            m, m_us, m_hs = mask
+            N.call(
+                "ttpa_paged_mla_decode_masked",
+                os_.data_ptr(), os_.stride(0), os_.stride(1), qs.data_ptr(), qs.stride(0), qs.stride(1),
+                key.data_ptr(), _ptr(value), pts.data_ptr(), pts.stride(0), curs.data_ptr(),
+                int(curs.dtype == torch.int64), n, hq, nkv, dh, head_dim_v, bs, pts.shape[1], nb,
+                float(scale), m.data_ptr() + 2 * u0 * m_us, m_us, m_hs, ws.data_ptr(), ws_bytes, _stream(),
+            )
+            continue
         N.call(
             "ttpa_paged_mla_decode",
             os_.data_ptr(), os_.stride(0), os_.stride(1), qs.data_ptr(), qs.stride(0), qs.stride(1),
@@ -842,10 +908,9 @@ def paged_flash_mla_decode(
         assert not is_causal, "attn_mask requires is_causal to be False."
     else:
         assert is_causal, "is_causal must be True when attn_mask is not provided"
-    if not is_causal:
-        raise NotImplementedError("latent decode with an explicit attn_mask is not built")
-    assert len(cur_pos_tensor.shape) == 1, "cur_pos_tensor must be a 1D tensor: [num_users]."
-    assert cur_pos_tensor.shape[0] == query.shape[1], "cur_pos_tensor number of users must match query number of users."
+    if is_causal:
+        assert len(cur_pos_tensor.shape) == 1, "cur_pos_tensor must be a 1D tensor: [num_users]."
+        assert cur_pos_tensor.shape[0] == query.shape[1], "cur_pos_tensor number of users must match query number of users."
     if query.dtype != torch.bfloat16 or key.dtype != torch.bfloat16 or not key.is_contiguous():
         raise ValueError("query and the key cache must be bfloat16, the cache contiguous")
     if value is not None and (value.dtype != torch.bfloat16 or not value.is_contiguous()):
@@ -860,8 +925,17 @@ def paged_flash_mla_decode(
         if attention_sink.numel() != hq:
             raise ValueError(f"attention_sink must hold one logit per query head ({hq})")
         sink = attention_sink.reshape(hq).to(device=query.device, dtype=torch.float32).contiguous()
-    _mla_decode_launch(out[0], q, key, value, _table(page_table), _index_tensor(cur_pos_tensor),
-                       head_dim_v, scale, sink)
+    if is_causal:
+        _mla_decode_launch(out[0], q, key, value, _table(page_table), _index_tensor(cur_pos_tensor),
+                           head_dim_v, scale, sink)
+        return out
+    # is_causal=False (reference custom_ops.py:590-592): every position of the table, weighted by the mask
+    if sink is not None:
+        raise NotImplementedError("attention_sink with an explicit attn_mask is not built")
+    skv = page_table.shape[1] * key.shape[2]
+    last = torch.full((users,), skv - 1, dtype=torch.int32, device=query.device)
+    _mla_decode_launch(out[0], q, key, value, _table(page_table), last, head_dim_v, scale, None,
+                       _decode_mask_rows(attn_mask, users, hq, skv))
     return out
 
 
@@ -906,8 +980,8 @@ def flash_mla_prefill(
     if attn_mask is not None:
         assert is_causal == False, "is_causal cannot be True when attn_mask is provided."  # noqa: E712
         assert attn_mask.shape[0] == query.shape[0], "attention mask batch size must match query batch size."
-        raise NotImplementedError("latent prefill with an explicit attn_mask is not built")
-    assert is_causal == True, "is_causal must be True if attn_mask is not provided"  # noqa: E712
+    else:
+        assert is_causal == True, "is_causal must be True if attn_mask is not provided"  # noqa: E712
     if query.dtype != torch.bfloat16 or key.dtype != torch.bfloat16:
         raise ValueError("query and key must be bfloat16")
     b, hq, s, dh = query.shape
@@ -918,11 +992,25 @@ def flash_mla_prefill(
     v = value.contiguous() if value is not None else None
     out = torch.empty((b, hq, s, head_dim_v), dtype=query.dtype, device=query.device)
     table = torch.zeros((s, 1), dtype=torch.int32, device=query.device)
-    cur = torch.arange(s, dtype=torch.int32, device=query.device)
+    mask = None
+    if attn_mask is None:
+        cur = torch.arange(s, dtype=torch.int32, device=query.device)
+    else:
+        # every key, weighted by the mask row of the query token (reference custom_ops.py:349-357):
+        # anything that broadcasts to [b, heads, s, s]; row i of a sequence is user i
+        cur = torch.full((s,), s - 1, dtype=torch.int32, device=query.device)
+        mask = _additive_mask(attn_mask)
+        if mask.dim() != 4 or mask.shape[1] not in (1, hq) or mask.shape[2] != s or mask.shape[3] != s:
+            raise ValueError(f"attn_mask must broadcast to [{b}, {hq}, {s}, {s}], got {tuple(attn_mask.shape)}")
+        if mask.stride(-1) != 1:
+            mask = mask.contiguous()
     for i in range(b):
         # [s, heads, d] views: token-major "users", the sequence as a single block of s tokens
+        rows = None
+        if mask is not None:
+            rows = (mask[i], mask.stride(2), mask.stride(1) if mask.shape[1] == hq and hq > 1 else 0)
         _mla_decode_launch(out[i].transpose(0, 1), q[i].transpose(0, 1), k[i : i + 1],
-                           None if v is None else v[i : i + 1], table, cur, head_dim_v, scale, None)
+                           None if v is None else v[i : i + 1], table, cur, head_dim_v, scale, None, rows)
     return out
 
 
@@ -1065,11 +1153,23 @@ def scaled_dot_product_attention_decode(
     assert query.shape[1] == key.shape[0], "query and key must have the same batch size."
     if is_causal:
         assert attn_mask is None, "attn_mask must be None when is_causal is True."
-    if attn_mask is not None:
-        raise NotImplementedError("static-cache decode with an explicit attn_mask is not built")
     _static_geometry(key), _static_geometry(value)
     if key.shape[2] % 4:
         raise NotImplementedError("static-cache decode needs max_seq_len to be a multiple of 4")
+    if attn_mask is not None:
+        # is_causal=False: all max_seq_len positions, weighted by the mask, one row per query head
+        # ([B, 1, heads, S] reshaped to [B, heads, 1, S], reference custom_ops.py:820-821)
+        assert not is_causal, "attn_mask requires is_causal to be False."
+        b, heads, seq = key.shape[0], query.shape[2], key.shape[2]
+        if attn_mask.numel() != b * heads * seq:
+            raise ValueError(f"attn_mask must hold batch x heads x max_seq_len = {b} x {heads} x {seq} values")
+        if attention_sink is not None:
+            raise NotImplementedError("attention_sink with an explicit attn_mask is not built")
+        return paged_scaled_dot_product_attention_decode(
+            query, key, value, _identity_table(b, key.device), is_causal=False,
+            attn_mask=attn_mask.reshape(b, heads, 1, seq), scale=scale,
+        )
+    assert is_causal, "is_causal must be True when attn_mask is not provided"
     # the cache tensor already has the paged layout [blocks = B, kv_heads, block_size = S, D]
     return paged_scaled_dot_product_attention_decode(
         query, key, value, _identity_table(key.shape[0], key.device), is_causal=True,
