@@ -44,7 +44,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 KERNEL_SOURCES = {
     "paged_decode_mfma16_kernel": ["decode_mfma16_kernel.h", "decode_common.h", "common.h", "decode.hip"],  # the grid rule is in decode.hip
     "paged_decode_latent16_kernel": ["decode_wide.hip", "decode_common.h", "common.h"],
-    "prefill_kernel": ["prefill.hip", "prefill_acc_regs.h", "common.h"],
+    "prefill_kernel": ["prefill.hip", "gen_prefill_stream.py", "common.h"],
 }
 MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
@@ -244,17 +244,30 @@ class StepRunner:
             self._graph(rem).replay()
 
 
-def time_steps(runner, steps, warmup):
+TIMED_BLOCKS = 7  # the block of `steps` steps is timed this many times; the median is reported
+
+
+def time_steps_spread(runner, steps, warmup, blocks=TIMED_BLOCKS):
+    """(median, min, max) milliseconds per step over `blocks` timed blocks of exactly `steps` steps,
+    each bracketed by a device synchronisation on both sides."""
     import torch
 
     runner.prepare(steps)
     runner.prepare(warmup)
     runner.run(warmup)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    runner.run(steps)
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) * 1e3 / steps
+    per_step = []
+    for _ in range(blocks):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        runner.run(steps)
+        torch.cuda.synchronize()
+        per_step.append((time.perf_counter() - t0) * 1e3 / steps)
+    per_step.sort()
+    return per_step[len(per_step) // 2], per_step[0], per_step[-1]
+
+
+def time_steps(runner, steps, warmup):
+    return time_steps_spread(runner, steps, warmup)[0]
 
 
 def time_dominant_kernel(fns, iters):
@@ -428,7 +441,7 @@ def run_decode(args):
     step_bytes = [b + c.update_bytes() for b, c in zip(dec_bytes, copies)]
     fns = [(lambda c=c: decode_step(c)) for c in copies]
     runner = StepRunner(fns, args.launch == "graph", args.steps_per_graph)
-    ms = time_steps(runner, args.steps, args.warmup)
+    ms, ms_min, ms_max = time_steps_spread(runner, args.steps, args.warmup)
     n = len(copies)
     avg_step_bytes = sum(step_bytes[i] for i in runner.sequence(args.steps)) / args.steps
     durs = time_decode_kernel_direct(copies, min(args.steps, 100))
@@ -440,6 +453,7 @@ def run_decode(args):
         "value": avg_step_bytes / (ms * 1e-3) / 1e9,
         "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "ms_per_step_min": ms_min, "ms_per_step_max": ms_max, "timed_blocks": TIMED_BLOCKS,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "synthetic",
         "config": {
@@ -501,7 +515,7 @@ def run_latent(args):
     nbytes = [c[4] * dh * 2 + users * hq * (dh + dv) * 2 + users * (c[2].shape[1] * 4 + 4) for c in copies]
     runner = StepRunner(fns, args.launch == "graph", args.steps_per_graph)
     steps = min(args.steps, 100)
-    ms = time_steps(runner, steps, min(args.warmup, 10))
+    ms, ms_min, ms_max = time_steps_spread(runner, steps, min(args.warmup, 10))
     avg_bytes = sum(nbytes[i] for i in runner.sequence(steps)) / steps
     durs = time_dominant_kernel(fns, min(steps, 50))
     kern_ms = sum(d for d, _ in durs) / len(durs)
@@ -512,6 +526,7 @@ def run_latent(args):
         "metric": "paged_decode_attention_hbm_throughput",
         "value": avg_bytes / (ms * 1e-3) / 1e9, "unit": "GB/s",
         "n_gpus": 1, "steps": steps, "warmup": min(args.warmup, 10), "ms_per_step": ms,
+        "ms_per_step_min": ms_min, "ms_per_step_max": ms_max, "timed_blocks": TIMED_BLOCKS,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {
@@ -545,7 +560,7 @@ def run_prefill(args):
     fns = [(lambda i=i: prefill_step(impls[i], copies[i], outs[i])) for i in range(len(copies))]
     runner = StepRunner(fns, args.launch == "graph", args.steps_per_graph)
     steps = min(args.steps, 100)
-    ms = time_steps(runner, steps, min(args.warmup, 10))
+    ms, ms_min, ms_max = time_steps_spread(runner, steps, min(args.warmup, 10))
     w = copies[0]
     flops = w.useful_flops()
     durs = time_dominant_kernel(fns, min(steps, 50))
@@ -556,6 +571,7 @@ def run_prefill(args):
         "value": flops / (ms * 1e-3) / 1e12,
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": steps, "warmup": min(args.warmup, 10), "ms_per_step": ms,
+        "ms_per_step_min": ms_min, "ms_per_step_max": ms_max, "timed_blocks": TIMED_BLOCKS,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {
@@ -583,22 +599,26 @@ def run_prefill(args):
 
 
 def secondary_runs(args):
-    """Short runs of the prefill workload (config3) and of the block-float-8 decode workload
-    (config5) in the headline's process, so that their figures come under the same clock: the
-    same functions as `--workload config3|config5`, fewer steps, only the key figures."""
+    """Short runs of the other workloads (config3 prefill, config5 block-float-8 decode, config4
+    large decode with its chunked-prefill pass, latent decode) in the headline's process, so that
+    their figures come under the same clock: the same functions as `--workload ...`, fewer steps,
+    only the key figures."""
     import copy
     import gc
 
     import torch
 
     out = {}
-    for wl, steps, warmup in (("config3", 30, 5), ("config5", 96, 12)):
+    for wl, steps, warmup in (("config3", 30, 5), ("config5", 96, 12), ("config4", 20, 4), ("latent", 40, 8)):
         gc.collect()
         torch.cuda.empty_cache()
         sub = copy.copy(args)
         sub.workload, sub.steps, sub.warmup = wl, steps, warmup
-        r = run_prefill(sub) if wl == "config3" else run_decode(sub)
-        keep = {k: r[k] for k in ("metric", "value", "unit", "steps", "warmup", "ms_per_step", "dtype", "roofline")}
+        if wl == "config4":
+            sub.rotate = 1  # one copy of the 128-user pool is already far beyond the caches
+        r = run_prefill(sub) if wl == "config3" else (run_latent(sub) if wl == "latent" else run_decode(sub))
+        keep = {k: r[k] for k in ("metric", "value", "unit", "steps", "warmup", "ms_per_step", "ms_per_step_min",
+                                  "ms_per_step_max", "dtype", "roofline")}
         keep["workload"] = r["config"]["workload"]
         for extra in ("pct_of_hbm_peak", "chunk_pass"):
             if extra in r:

@@ -90,3 +90,17 @@ def test_latent_decode_entry_validates_on_the_host():
                                        512, 32, 1, 1, 1.0, None, None, 0, None)
     assert rc == N.ERR_INVALID_ARGUMENT
     assert b"null" in N.lib().ttpa_last_error()
+
+
+def test_latent_decode_refuses_more_segments_than_the_grid_has_threads(native, monkeypatch):
+    """The 16-head latent kernel publishes one segment row per thread of its grid: a grid made
+    small by TTPA_DECODE_WAVES_PER_CU must be refused on the host when users x kv_heads does not
+    fit, before any launch (the merge would read rows nobody wrote)."""
+    lib = native.lib()
+    monkeypatch.setenv("TTPA_DECODE_WAVES_PER_CU", "0.01")
+    users, hq, hkv, d = 1024, 64, 8, 128
+    need = lib.ttpa_paged_mla_decode_workspace_bytes(users, hq, hkv, d)
+    assert need > 0
+    rc = lib.ttpa_paged_mla_decode(256, 8 * d, d, 256, 8 * d, d, 256, None, 256, 1, 256, 0, users, hq, hkv, d, d,
+                                   32, 1, 4, 1.0, None, 256, need, None)
+    assert rc == native.ERR_UNSUPPORTED and b"segments" in lib.ttpa_last_error()

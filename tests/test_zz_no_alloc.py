@@ -91,3 +91,42 @@ def test_shape_beyond_the_static_array_is_refused():
                                              hkv, d, 64, 8, 16, 1.0, 0, 0, None, None)
     assert rc == _native.ERR_WORKSPACE
     assert b"static scratch" in lib.ttpa_last_error()
+
+
+def test_calls_allocate_no_device_memory_and_replay_from_a_graph():
+    """What the entry point exists for: after ttpa_static_scratch_init() and a warm-up call, further
+    calls leave the device's free memory unchanged, and a call captured into a graph (where an
+    allocation would fail the capture) replays to the eager result."""
+    from tt_xla_amd import _native, workloads
+
+    lib = _native.lib()
+    assert lib.ttpa_static_scratch_init() == 0
+    wl = workloads.decode_ragged("static scratch, no allocation", 13, 5, 32, 8, 128, 64, 64,
+                                 [900, 64, 200, 1, 1300])
+    dev = wl.to("cuda")
+    k, v, out = dev.k_cache.clone(), dev.v_cache.clone(), torch.empty_like(dev.q)
+    stream = torch.cuda.current_stream().cuda_stream
+    _native.call("ttpa_paged_update_decode_static", *_step_args(dev, out, k, v), stream)  # warm-up
+    torch.cuda.synchronize()
+    eager = out.clone()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(5):
+        _native.call("ttpa_paged_update_decode_static", *_step_args(dev, out, k, v), stream)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, f"device memory moved by {free_before - free_after} bytes over five calls"
+    assert torch.equal(out.view(torch.int16), eager.view(torch.int16))
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            _native.call("ttpa_paged_update_decode_static", *_step_args(dev, out, k, v), side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(3):  # every replay, with eager work in between, against the eager result
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), "a replay differs from the eager call"

@@ -22,6 +22,7 @@
 //   multiplies its V elements.
 //   The G query heads of a group share every K/V load: each element is read once
 //   per KV head.
+#include <algorithm>
 #include "decode_common.h"
 
 #include <cstdlib>
@@ -314,7 +315,8 @@ int waves_for_device(double default_per_cu) {
   int cus = device_cus();
   if (cus <= 0) cus = 256;
   const int waves = (int)(cus * per_cu + 0.5);
-  return (waves + kWavesPerBlock - 1) / kWavesPerBlock * kWavesPerBlock;
+  // (whole workgroups, at least one)
+  return std::max(kWavesPerBlock, (waves + kWavesPerBlock - 1) / kWavesPerBlock * kWavesPerBlock);
 }
 
 template <int D, int G>

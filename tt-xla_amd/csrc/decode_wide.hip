@@ -735,6 +735,10 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
     // (fewer partials of 32 KiB each), 139 at 2.5 and 159 at two; TTPA_DECODE_WAVES_PER_CU overrides,
     // up to the four per CU that the workspace is sized for
     a.n_waves = std::min(cus * kWavesPerBlockHost, waves_for_device(3.0));
+    // one thread of the grid per segment publishes the segment's partial slots
+    if ((int64_t)users * kv_heads > (int64_t)a.n_waves * kWave)
+      return fail(TTPA_ERR_UNSUPPORTED, "latent decode: %d x %d segments need a grid of more than %d wavefronts",
+                  users, kv_heads, a.n_waves);
     // three units in front of every segment of the flat list (a partial here is 32 KiB, a tile
     // 18 KiB): 130 us per step against 131-134 with none
     a.seg_units = segment_units(3);

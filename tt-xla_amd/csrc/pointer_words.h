@@ -8,7 +8,7 @@ namespace ttpa {
 
 // Each word goes through uint32_t before it is widened: widened as a signed int, a low word with
 // bit 31 set would smear ones over the high word and turn a valid address into a wild one.
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 __host__ __device__
 #endif
 inline uint64_t address_from_words(int low_word, int high_word) {

@@ -24,7 +24,6 @@
 // position inside a row, applied on the global side (which chunk a lane fetches) and again
 // when fragments are read.
 #include "common.h"
-#include "prefill_acc_regs.h"
 #include "build/prefill_stream_asm.h"
 
 #include <cstdlib>
@@ -157,287 +156,6 @@ __device__ __forceinline__ void fill_workgroup(const PrefillArgs &a, int f) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// The loop of a wavefront that owns 64 query rows (two blocks of 32: "halves"), one wavefront
-// per SIMD.  The unit of work is a BLOCK of 32 keys (half a K / V tile) over both halves:
-//   S(i):  16 x 32 x D scores of block i        KSTEPS K fragments, each feeding both halves
-//   sm(i): online softmax of block i            one row per lane and half: 32 scores per lane
-//   PV(i): O^T += V^T P^T of block i            2 DBLK V^T fragments, each feeding both halves
-// software-pipelined so that the matrix pipe and the vector ALU of the SIMD work at the same
-// time on different blocks: iteration i issues the matrix instructions of PV(i-1) and S(i+1)
-// and, one slice behind every one of them, the vector work of sm(i), which needs about as many
-// cycles.  The matrix instructions are written in assembly to say where their operands live:
-// the output accumulators and Q stay in accumulation registers for the whole kernel
-// (prefill_acc_regs.h), which leaves the 256 architectural registers to scores, probabilities
-// and fragments.  The compiler does not see the hazards of such instructions: the waits it would
-// have placed between a matrix result and its first vector read are written out.
-// Order inside an iteration is pinned with scheduling fences, slice by slice.
-template <int B, int E, class F>
-__device__ __forceinline__ void static_for(F &&f) {
-  if constexpr (B < E) {
-    f(std::integral_constant<int, B>{});
-    static_for<B + 1, E>(f);
-  }
-}
-#define TTPA_FENCE() __builtin_amdgcn_sched_barrier(0)
-
-template <int D, class KS, class VS, class BAR>
-__device__ __forceinline__ void rows64_loop(const PrefillArgs &a,
-                                            const uint32_t (&koff)[D / 16], const uint32_t (&voff)[D / 32],
-                                            int first_tile, int nblk, int row0, int offset, int b, int hq,
-                                            int n, int h, KS kstage, VS vstage, BAR tile_barrier) {
-  constexpr int KSTEPS = D / 16, DBLK = D / 32;
-  using T = Tile<D>;
-  constexpr int NFV = 2 * DBLK;  // V^T fragments of a block (2 key steps x DBLK output blocks)
-  constexpr int NFK = KSTEPS;    // K fragments of a block
-  constexpr int PRE = NFV < 8 ? NFV : 8;  // fragments in flight (an LDS read takes a few hundred cycles to come back)
-  constexpr int NITEMS = 6 + 32; // slices of sm(i)
-
-  auto read_kf = [&](int tile, int kb, int s) -> u32x4 {
-    const uint4 t = *reinterpret_cast<const uint4 *>(kstage(tile) + koff[s] + 32 * kb * T::RB);
-    return u32x4{t.x, t.y, t.z, t.w};
-  };
-  auto read_vf = [&](int tile, int k4, int db) -> u32x4 {
-    typedef __attribute__((address_space(3))) shortx4 *lds_v4;
-    const unsigned char *vk = vstage(tile) + voff[db] + 16 * k4 * T::RB;
-    const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk));
-    const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(vk + 8 * T::RB));
-    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-    return u32x4{l2.x, l2.y, h2.x, h2.y};
-  };
-
-  accregs::clear_outputs<0, 2 * DBLK>();
-  float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
-  float alpha_c[2] = {1.f, 1.f};  // what sm of the newest block wants the accumulators scaled by
-  floatx16 st[2][2];              // [block parity][half]
-  u32x4 pf[2][2][2];              // [block parity][half][key step]
-  u32x4 ring[PRE];
-
-  // Applies alpha_c to the accumulators (rare: lazy rescaling), once PV of the previous block is done.
-  auto rescale = [&]() {
-    if (__builtin_amdgcn_ballot_w64(alpha_c[0] != 1.0f || alpha_c[1] != 1.0f) != 0) {
-      static_for<0, 2 * DBLK>([&](auto k) { accregs::scale_output<decltype(k)::value>(alpha_c[decltype(k)::value / DBLK]); });
-    }
-  };
-  // Masks block i of both halves (diagonal, ragged end, window edge, explicit mask).
-  auto apply_mask = [&](int i, floatx16 (&sc)[2]) {
-#pragma unroll
-    for (int x = 0; x < 2; ++x) {
-      const int qrow = row0 + 32 * x + n;
-      const int limit = a.causal ? min(offset + qrow, a.skv - 1) : a.skv - 1;
-      const int lowest = a.window > 0 ? offset + qrow - a.window + 1 : 0;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
-        float v = sc[x][r];
-        if (a.mask) {
-          const int kc = min(key, a.skv - 1), qc = min(qrow, a.sq - 1);
-          v += bf16_lo(a.mask[b * a.mask_bs + (int64_t)qc * a.mask_rs + kc]) * (1.4426950408889634f / a.scale_log2e);
-        }
-        sc[x][r] = (key > limit || key < lowest) ? -INFINITY : v;
-      }
-    }
-  };
-
-  // One iteration: block i of parity PAR.  HAS_PV: block i - 1 exists (its PV is issued here);
-  // HAS_S: block i + 1 exists (its scores are issued here).  On entry the ring holds the first
-  // PRE V^T fragments of PV(i - 1) (HAS_PV); on exit those of PV(i).
-  auto iteration = [&](auto par_tag, auto pv_tag, auto s_tag, int i) {
-    constexpr int PAR = decltype(par_tag)::value;
-    constexpr bool HAS_PV = decltype(pv_tag)::value, HAS_S = decltype(s_tag)::value;
-    constexpr int NF = (HAS_PV ? NFV : 0) + (HAS_S ? NFK : 0);  // this iteration's own fragments
-    constexpr int M = 2 * NF;                                   // matrix instructions
-    const int tile = i >> 1;
-    floatx16(&sc)[2] = st[PAR];
-    // fragment f of this iteration (own, then the first of PV(i))
-    auto fetch_fragment = [&](auto f_tag) -> u32x4 {
-      constexpr int f = decltype(f_tag)::value;
-      if constexpr (HAS_PV && f < NFV) return read_vf((i - 1) >> 1, 2 * (1 - PAR) + f / DBLK, f % DBLK);
-      else if constexpr (f < NF) return read_kf((i + 1) >> 1, 1 - PAR, f - (HAS_PV ? NFV : 0));
-      else return read_vf(tile, 2 * PAR + (f - NF) / DBLK, (f - NF) % DBLK);
-    };
-    asm volatile("s_nop 15\n\ts_nop 7" : "+v"(sc[0]), "+v"(sc[1]));  // the scores have been written
-    const bool need_mask = (a.causal && 32 * i + 31 > offset + row0) || 32 * i + 32 > a.skv || a.mask != nullptr ||
-                           (a.window > 0 && 32 * i <= offset + row0 + 63 - a.window);
-    if (need_mask) apply_mask(i, sc);
-    if constexpr (HAS_PV) rescale();
-    if constexpr (PAR == 0 && !HAS_PV) tile_barrier(tile);
-    if constexpr (!HAS_PV && HAS_S) {
-      static_for<0, PRE>([&](auto f) { ring[decltype(f)::value] = fetch_fragment(f); });
-    }
-
-    float mloc[2], mc[2], lsum[2] = {0.f, 0.f}, p_even = 0.f;
-    u32x4 hold = ring[0];
-    // slice w of sm(i)
-    auto item = [&](auto w_tag) {
-      constexpr int w = decltype(w_tag)::value;
-      if constexpr (w < 6) {
-        constexpr int x = w / 3, part = w % 3;
-        if constexpr (part == 0) {
-          mloc[x] = fmaxf(sc[x][0], sc[x][1]);
-          mloc[x] = max3(mloc[x], sc[x][2], sc[x][3]);
-          mloc[x] = max3(mloc[x], sc[x][4], sc[x][5]);
-          mloc[x] = max3(mloc[x], sc[x][6], sc[x][7]);
-          asm volatile("" : "+v"(mloc[x]));
-        } else if constexpr (part == 1) {
-          mloc[x] = max3(mloc[x], sc[x][8], sc[x][9]);
-          mloc[x] = max3(mloc[x], sc[x][10], sc[x][11]);
-          mloc[x] = max3(mloc[x], sc[x][12], sc[x][13]);
-          mloc[x] = max3(mloc[x], sc[x][14], sc[x][15]);
-          float ma = mloc[x], mb = mloc[x];
-          asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(ma), "+v"(mb));
-          mloc[x] = max3(ma, mb, mb);
-          asm volatile("" : "+v"(mloc[x]));
-        } else {
-          const float kLazy = 8.0f;
-          const bool move = !((mloc[x] - m_run[x]) * a.scale_log2e <= kLazy);  // also true from -inf
-          const float m_new = move ? mloc[x] : m_run[x];
-          const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-          alpha_c[x] = move ? __builtin_amdgcn_exp2f((m_run[x] - m_safe) * a.scale_log2e) : 1.0f;
-          mc[x] = m_safe * a.scale_log2e;
-          m_run[x] = m_new;
-          asm volatile("" : "+v"(mc[x]), "+v"(alpha_c[x]), "+v"(m_run[x]));
-        }
-      } else {
-        constexpr int e = w - 6, x = e / 16, r = e % 16;
-        const float pr = __builtin_amdgcn_exp2f(fmaf(sc[x][r], a.scale_log2e, -mc[x]));
-        // (the empty statements pin each slice where it is written: without them the compiler
-        // sinks this arithmetic towards its use, a whole iteration later)
-        if constexpr (r % 2 == 0) {
-          p_even = pr;
-          asm volatile("" : "+v"(p_even));
-        } else {
-          const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
-          const bf16x2 pp = {(__bf16)p_even, (__bf16)pr};
-          uint32_t packed = __builtin_bit_cast(uint32_t, pp);
-          lsum[x] = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, lsum[x], false);
-          asm volatile("" : "+v"(packed), "+v"(lsum[x]));
-          pf[PAR][x][r / 8][(r % 8) / 2] = packed;
-        }
-      }
-    };
-    if constexpr (M == 0) {
-      static_for<0, NITEMS>(item);
-    } else {
-      static_for<0, M>([&](auto j_tag) {
-        constexpr int j = decltype(j_tag)::value, f = j / 2, x = j % 2;
-        if constexpr (PAR == 0 && HAS_PV && j == 2 * NFV) {  // between the two products
-          TTPA_FENCE();
-          tile_barrier(tile);
-          TTPA_FENCE();
-        }
-        const u32x4 frag = ring[f % PRE];
-        if constexpr (HAS_PV && f < NFV) {
-          accregs::mfma_output<x * DBLK + f % DBLK>(frag, pf[1 - PAR][x][f / DBLK]);
-        } else {
-          constexpr int s = f - (HAS_PV ? NFV : 0);
-          accregs::mfma_scores<x * KSTEPS + s, (s > 0)>(st[1 - PAR][x], frag);
-        }
-        TTPA_FENCE();
-        static_for<(j * NITEMS) / M, ((j + 1) * NITEMS) / M>(item);
-        if constexpr (x == 1 && (HAS_S || f + PRE < NF) && f + PRE < NF + NFV) ring[f % PRE] = fetch_fragment(std::integral_constant<int, f + PRE>{});
-        // A matrix instruction issued behind another one reads its operands when it starts, up
-        // to a whole instruction later, and nothing stops a later write to those registers from
-        // overtaking it (measured: the second instruction of a pair saw the address arithmetic
-        // that followed it).  So an operand's registers stay allocated for two more fragments.
-        if constexpr (x == 1) {
-          asm volatile("" : : "v"(hold));
-          hold = frag;
-        }
-        TTPA_FENCE();
-      });
-    }
-#pragma unroll
-    for (int x = 0; x < 2; ++x) l_run[x] = l_run[x] * alpha_c[x] + lsum[x];
-    if constexpr (M > 0) {
-      // (as above, for the last fragment and for the probabilities PV(i - 1) has consumed)
-      asm volatile("" : : "v"(hold));
-      if constexpr (HAS_PV)
-        asm volatile("" : : "v"(pf[1 - PAR][0][0]), "v"(pf[1 - PAR][0][1]), "v"(pf[1 - PAR][1][0]), "v"(pf[1 - PAR][1][1]));
-    }
-    if constexpr (!HAS_S) {
-      // the last block: the fragments of its PV are fetched behind the barrier that publishes its V tile
-      if constexpr (PAR == 0 && HAS_PV) {
-        TTPA_FENCE();
-        tile_barrier(tile);
-      }
-      static_for<0, PRE>([&](auto f) { ring[decltype(f)::value] = fetch_fragment(std::integral_constant<int, NF + decltype(f)::value>{}); });
-    }
-  };
-  // PV of the last block, with nothing left to overlap it
-  auto last_output = [&](auto par_tag, int i) {
-    constexpr int PAR = decltype(par_tag)::value;
-    rescale();
-    u32x4 hold = ring[0];
-    static_for<0, 2 * NFV>([&](auto j_tag) {
-      constexpr int j = decltype(j_tag)::value, f = j / 2, x = j % 2;
-      const u32x4 frag = ring[f % PRE];
-      accregs::mfma_output<x * DBLK + f % DBLK>(frag, pf[PAR][x][f / DBLK]);
-      TTPA_FENCE();
-      if constexpr (x == 1 && f + PRE < NFV) ring[f % PRE] = read_vf(i >> 1, 2 * PAR + (f + PRE) / DBLK, (f + PRE) % DBLK);
-      if constexpr (x == 1) {
-        asm volatile("" : : "v"(hold));
-        hold = frag;
-      }
-      TTPA_FENCE();
-    });
-    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" : : "v"(hold), "v"(pf[PAR][0][0]), "v"(pf[PAR][0][1]), "v"(pf[PAR][1][0]), "v"(pf[PAR][1][1]));
-  };
-
-  using Even = std::integral_constant<int, 0>;
-  using Odd = std::integral_constant<int, 1>;
-  using Yes = std::true_type;
-  using No = std::false_type;
-  // scores of the first block
-  const int i0 = 2 * first_tile;
-  static_for<0, KSTEPS>([&](auto s_tag) {
-    constexpr int s = decltype(s_tag)::value;
-    const u32x4 kf = read_kf(first_tile, 0, s);
-    accregs::mfma_scores<s, (s > 0)>(st[0][0], kf);
-    accregs::mfma_scores<KSTEPS + s, (s > 0)>(st[0][1], kf);
-    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" : : "v"(kf));
-  });
-  int i = i0;
-  if (nblk - i0 == 1) {
-    iteration(Even{}, No{}, No{}, i);
-    last_output(Even{}, i);
-  } else {
-    iteration(Even{}, No{}, Yes{}, i);
-    ++i;
-    while (i + 2 < nblk) {
-      iteration(Odd{}, Yes{}, Yes{}, i);
-      iteration(Even{}, Yes{}, Yes{}, i + 1);
-      i += 2;
-    }
-    if (i + 1 < nblk) {
-      iteration(Odd{}, Yes{}, Yes{}, i);
-      iteration(Even{}, Yes{}, No{}, i + 1);
-      last_output(Even{}, i + 1);
-    } else {
-      iteration(Odd{}, Yes{}, No{}, i);
-      last_output(Odd{}, i);
-    }
-  }
-
-  // ---- normalise and store: lane (n, h) holds head-dim elements 32 db + 8 j + 4 h + i ----
-  static_for<0, 2 * DBLK>([&](auto k_tag) {
-    constexpr int k = decltype(k_tag)::value, x = k / DBLK, db = k % DBLK;
-    const float l_tot = l_run[x] + __shfl_xor(l_run[x], 32);
-    const float inv = 1.0f / l_tot;
-    const int qrow = row0 + 32 * x + n;
-    uint16_t *op = a.out + b * a.out_bs + hq * a.out_hs + (int64_t)qrow * a.out_ts + 4 * h;
-    const floatx16 t = accregs::read_output<k>();
-    if (qrow < a.sq) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        uint32_t lo = f32_to_bf16_bits(t[4 * j] * inv) | (f32_to_bf16_bits(t[4 * j + 1] * inv) << 16);
-        uint32_t hi = f32_to_bf16_bits(t[4 * j + 2] * inv) | (f32_to_bf16_bits(t[4 * j + 3] * inv) << 16);
-        *reinterpret_cast<uint2 *>(op + 32 * db + 8 * j) = make_uint2(lo, hi);
-      }
-    }
-  });
-}
-
-// ---------------------------------------------------------------------------------------------
 // The hand-scheduled loop over whole unmasked tiles (head size 128, 32 rows per wavefront): one
 // block of assembly, written by gen_prefill_stream.py, which documents the schedule and the
 // state on entry and exit.  Everything the block touches is bound to the registers its text
@@ -536,12 +254,9 @@ __device__ __forceinline__ void stream_blocks_paged(StreamState &st, StreamReque
 // barrier too.  LDS operand reads run a few fragments ahead of the matrix instructions that
 // consume them.
 //
-// RH = 2: a wavefront owns TWO blocks of 32 query rows (64 consecutive rows of its head) and the
-// workgroup has the CU to itself (one wavefront per SIMD, up to 512 registers).  Every K and V
-// fragment read from LDS then feeds two matrix instructions, which halves the LDS operand
-// traffic per flop (at 32 rows the four wavefronts of a workgroup read 128 KiB per tile, as much
-// as the LDS delivers in the time the matrix pipes need for that tile), and half as many
-// workgroups pay the start-up and the store.
+// RH: blocks of 32 query rows per wavefront; only 1 is built (a form with two, one workgroup per
+// CU and every K / V fragment feeding two matrix instructions, measured slower: with one wavefront
+// per SIMD nobody fills the waits for fragments and barriers).
 template <int RH>
 constexpr int prefill_wgs_per_cu(int d, int mode) { return RH == 1 && d <= 128 ? 2 : 1; }
 
@@ -655,24 +370,13 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
   }
 
   // ---- Q fragments (B operand: lane n = query row, 8 head-dim elements per k-step) -----
-  // RH = 2: straight into accumulation registers (the matrix instructions read them from there),
-  // by a load the compiler does not track: the wait for the first K / V tiles (vmcnt(0), below)
-  // covers it.
+  static_assert(RH == 1, "one block of 32 query rows per wavefront");
   bf16x8 qf[RH][KSTEPS];
-  if constexpr (RH == 2) {
-    accregs::reserve_accumulation_registers();
-    static_for<0, 2 * KSTEPS>([&](auto k_tag) {
-      constexpr int k = decltype(k_tag)::value, x = k / KSTEPS, s = k % KSTEPS;
-      const int qrow = min(row0 + 32 * x + n, a.sq - 1);
-      accregs::load_q_fragment<k>(a.q + b * a.q_bs + hq * a.q_hs + (int64_t)qrow * a.q_ts + 8 * h + 16 * s);
-    });
-  } else {
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-      const int qrow = min(row0 + n, a.sq - 1);
-      const uint16_t *qp = a.q + b * a.q_bs + hq * a.q_hs + (int64_t)qrow * a.q_ts + 8 * h;
-      qf[0][s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 16 * s));
-    }
+  for (int s = 0; s < KSTEPS; ++s) {
+    const int qrow = min(row0 + n, a.sq - 1);
+    const uint16_t *qp = a.q + b * a.q_bs + hq * a.q_hs + (int64_t)qrow * a.q_ts + 8 * h;
+    qf[0][s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 16 * s));
   }
 
   floatx16 acc[RH][DBLK];
@@ -720,13 +424,8 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
     // hold the last key again (readable, and masked like any key past the end)
     return key0 + min((4 * j + wave) * T::RPI, (a.skv - 1 - key0) / T::RPI * T::RPI);
   };
-  // LDS byte offset of a tile: stages of a K and a V tile each (RH = 1), or KST K tiles followed
-  // by VST V tiles (RH = 2, where K runs further ahead of its use than V)
-  constexpr int KST = 3, VST = 2;
-  auto tile_offset = [&](bool is_v, int buf) {
-    if constexpr (RH == 1) return (uint32_t)(buf * T::STAGE_BYTES + (is_v ? T::TILE_BYTES : 0));
-    else return (uint32_t)((is_v ? KST + buf : buf) * T::TILE_BYTES);
-  };
+  // LDS byte offset of a tile: stages of a K and a V tile each
+  auto tile_offset = [&](bool is_v, int buf) { return (uint32_t)(buf * T::STAGE_BYTES + (is_v ? T::TILE_BYTES : 0)); };
   auto issue = [&](const uint16_t *src, const uint32_t (&ld)[T::NI], bool is_v, int kt, int buf,
                    const Blocks &blk) {
     const int key0 = kt * kKeysPerTile;
@@ -901,8 +600,8 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
     }
     return blk;
   };
-  auto kbuf = [&](int t) { return RH == 1 ? (t & 1) : t % KST; };
-  auto vbuf = [&](int t) { return RH == 1 ? (t & 1) : t % VST; };
+  auto kbuf = [&](int t) { return t & 1; };
+  auto vbuf = [&](int t) { return t & 1; };
   int kt_begin = first_tile;
   // ---- all blocks through the hand-scheduled loop ------------------------------------------------
   if constexpr (D == 128 && HPW == 4 && RH == 1 && (MODE == 0 || MODE == 1)) {
@@ -958,23 +657,6 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
   }
   blk_v = blk_k;
   wait_loads_and_sync();
-  if constexpr (RH == 2) {
-    // key blocks (of 32) any row of the workgroup can see
-    const int nblk = min(2 * ntiles, (kv_end_wg + 31) / 32);
-    rows64_loop<D>(
-        a, koff, voff, first_tile, nblk, row0, offset, b, hq, n, h,
-        [&](int t) { return smem + kbuf(t) * T::TILE_BYTES; },
-        [&](int t) { return smem + (KST + vbuf(t)) * T::TILE_BYTES; },
-        [&](int tile) {  // the barrier of tile `tile`: K(tile + 1) and V(tile) become visible
-          wait_loads_and_sync();
-          blk_k = resolve(req);
-          if (tile + 2 <= last_tile) issue(a.k, ld_k, false, tile + 2, kbuf(tile + 2), blk_k);
-          if (tile + 1 <= last_tile) issue(a.v, ld_v, true, tile + 1, vbuf(tile + 1), blk_v);
-          blk_v = blk_k;
-          req = request(tile + 3);
-        });
-    return;
-  }
   // The first K fragments of a tile are read one tile ahead (K(t+1) has landed at the barrier
   // of tile t), so the score product starts without waiting for LDS.
   bf16x8 ring[KPRE];
@@ -1160,10 +842,10 @@ int launch_mode(const PrefillArgs &a, hipStream_t st) {
   constexpr int RPW = 4 / HPW;
   constexpr int ROWS = kRowsPerWave * RH;
   const int nqt = (a.sq + ROWS * RPW - 1) / (ROWS * RPW);
-  // two stages of a K and a V tile; with two row blocks three K tiles and two V tiles
+  // two stages of a K and a V tile
   // (the hand-scheduled loop keeps two rings of five 8 KiB blocks)
   constexpr bool kStreams = D == 128 && HPW == 4 && RH == 1 && (MODE == 0 || MODE == 1);
-  const size_t lds = RH == 2 ? 5 * Tile<D>::TILE_BYTES : (kStreams ? (size_t)TTPA_STREAM_LDS_BYTES : 2 * Tile<D>::STAGE_BYTES);
+  const size_t lds = kStreams ? (size_t)TTPA_STREAM_LDS_BYTES : 2 * Tile<D>::STAGE_BYTES;
   static std::atomic<uint64_t> lds_ready{0};
   if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&prefill_kernel<D, HPW, MODE, RH>), lds, lds_ready))
     return fail(TTPA_ERR_LAUNCH, "prefill: cannot reserve %zu bytes of LDS", lds);
@@ -1187,21 +869,6 @@ int launch_mode(const PrefillArgs &a, hipStream_t st) {
   return check_launch("sdpa_prefill");
 }
 
-// Row blocks per wavefront.  Two (one workgroup per CU, 64 rows per wavefront, the software-
-// pipelined loop above) is built for head sizes up to 128, bfloat16 K / V and four query heads
-// per KV head and workgroup; it is chosen only on request (TTPA_PREFILL_ROW_BLOCKS=2, read on
-// every call): on the 4 x 2048-token causal workload it measures 240 us against 213 us for two
-// 32-row workgroups per CU.  A matrix instruction keeps the SIMD's vector ALU port for 16 of
-// its 32 cycles (measured: one 32x32x16 instruction plus n independent v_fma_f32 take
-// 32 + 4.4 (n - 4) cycles), the softmax needs about as many vector cycles as the products need
-// matrix cycles, and a wavefront alone on its SIMD has nobody to fill its waits for LDS
-// fragments and for the barrier of a tile.
-inline int row_blocks_for(const PrefillArgs &a, int d, int hpw) {
-  if (d > 128 || a.kv_bfp8 || hpw != 4) return 1;
-  const char *e = getenv("TTPA_PREFILL_ROW_BLOCKS");
-  return e && atoi(e) == 2 ? 2 : 1;
-}
-
 template <int D, int HPW, int RH>
 int launch_rh(const PrefillArgs &a, hipStream_t st) {
   if (!a.pt) return launch_mode<D, HPW, 0, RH>(a, st);
@@ -1213,9 +880,6 @@ int launch_rh(const PrefillArgs &a, hipStream_t st) {
 template <int D, int HPW>
 int launch(const PrefillArgs &a, hipStream_t st) {
   if (a.pt && a.kv_bfp8) return launch_mode<D, HPW, 4, 1>(a, st);
-  if constexpr (D <= 128 && HPW == 4) {
-    if (row_blocks_for(a, D, HPW) == 2) return launch_rh<D, HPW, 2>(a, st);
-  }
   return launch_rh<D, HPW, 1>(a, st);
 }
 

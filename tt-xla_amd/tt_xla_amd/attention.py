@@ -455,7 +455,11 @@ class TTAttentionBackendImpl(_ImplBase):
         """[NB, Hkv, bs, D] -> [users, Hkv, num_tokens, D] in page-table order (a block-float-8
         cache comes out as the bfloat16 values it encodes)."""
         users, width = page_table.shape
-        g = torch.index_select(cache, 0, page_table.reshape(-1))
+        # ids outside the cache (padding -1, stale entries) read block 0, as in the kernels; left
+        # alone they would trip a device-side index assert
+        ids = page_table.reshape(-1).to(torch.int64)
+        ids = torch.where((ids >= 0) & (ids < cache.shape[0]), ids, torch.zeros_like(ids))
+        g = torch.index_select(cache, 0, ids)
         if cache.dtype == torch.uint8:
             g = custom_ops.bfp8_unpack_cache(g)
         _, hkv, bs, d = g.shape
