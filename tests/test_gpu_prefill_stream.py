@@ -1,12 +1,13 @@
-"""GPU parity for the prefill kernel's 64-rows-per-wavefront form (one workgroup per CU, software-
-pipelined loop, output accumulators and Q in fixed accumulation registers), which the library
-uses only on request: TTPA_PREFILL_ROW_BLOCKS=2, read on every call.  It serves head sizes up to
-128 with a multiple of four query heads per KV head; every other shape takes the 32-row form
-whatever the variable says.  Same oracle, inputs and bar (atol = rtol = 2e-2) as
-tests/test_gpu_prefill.py, on the shapes of that file and of tests/test_gpu_window_sink.py that
-the form serves, plus shapes chosen for its own corners: an odd number of 32-key blocks, a
-single block, query lengths that are not multiples of 64 (the operator asks for multiples of
-32), an additive mask, the ragged end of K / V inside a block."""
+"""GPU parity for the two inner loops of the prefill kernel.  Shapes with head size 128 and a multiple
+of four query heads per KV head, causal or unmasked, dense or paged bfloat16, run the hand-scheduled
+loop (32-key blocks in LDS rings, written as one assembly block by csrc/gen_prefill_stream.py);
+TTPA_PREFILL_STREAM=0, read on every call, sends them through the compiler-scheduled loop that serves
+every other shape, and TTPA_PREFILL_WGS_PER_GROUP=n makes a workgroup of the hand-scheduled loop walk
+several blocks of query rows in turn instead of one.  Every case runs under each setting.  Same
+oracle, inputs and bar (atol = rtol = 2e-2) as tests/test_gpu_prefill.py, on the shapes of that file
+and of tests/test_gpu_window_sink.py, plus shapes chosen for the loops' corners: an odd number of
+32-key blocks, a single block, fewer blocks than the rings hold, query lengths that are not multiples
+of 64, an additive mask, the ragged end of K / V inside a block, paged blocks smaller than a tile."""
 
 import pytest
 import torch
@@ -17,9 +18,13 @@ from oracle import paged_ops as O
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True)
-def _two_row_blocks(monkeypatch):
-    monkeypatch.setenv("TTPA_PREFILL_ROW_BLOCKS", "2")
+@pytest.fixture(autouse=True, params=["plain", "stream", "stream-2", "stream-3"])
+def _loop(request, monkeypatch):
+    monkeypatch.setenv("TTPA_PREFILL_STREAM", "0" if request.param == "plain" else "1")
+    if "-" in request.param:
+        monkeypatch.setenv("TTPA_PREFILL_WGS_PER_GROUP", request.param.split("-")[1])
+    else:
+        monkeypatch.delenv("TTPA_PREFILL_WGS_PER_GROUP", raising=False)
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -29,7 +34,7 @@ def _pkg():
 
 
 def _served(hq, hkv, d):
-    return (hq // hkv) % 4 == 0 and d <= 128
+    return (hq // hkv) % 4 == 0 and d == 128
 
 
 DENSE = [c for c in P.DENSE if _served(c[1], c[4], c[3])] + [
@@ -41,6 +46,9 @@ DENSE = [c for c in P.DENSE if _served(c[1], c[4], c[3])] + [
     (1, 8, 128, 128, 2, 77, False),    # additive mask, K / V ending inside a block
     (2, 16, 64, 128, 4, 300, False),   # more keys than rows
     (4, 32, 256, 128, 8, 256, True),
+    (1, 8, 416, 128, 2, 416, True),    # thirteen row blocks: uneven shares when a workgroup takes several
+    (1, 4, 64, 128, 1, 1024, False),   # long unmasked rows: the rings wrap several times
+    (2, 8, 96, 128, 2, 192, False),
 ]
 
 
@@ -98,12 +106,13 @@ def test_scores_that_force_a_rescale():
     P._check("rescale", got.cpu(), want)
 
 
-def test_same_result_as_the_32_row_form(monkeypatch):
+def test_loops_agree(monkeypatch):
     g = torch.Generator().manual_seed(9)
     q, k, v = P._bf(g, 2, 32, 320, 128), P._bf(g, 2, 8, 320, 128), P._bf(g, 2, 8, 320, 128)
-    two = torch.ops.tt.scaled_dot_product_attention(q.cuda(), k.cuda(), v.cuda(), is_causal=True)
-    monkeypatch.setenv("TTPA_PREFILL_ROW_BLOCKS", "1")
-    one = torch.ops.tt.scaled_dot_product_attention(q.cuda(), k.cuda(), v.cuda(), is_causal=True)
-    # the two forms split a tile differently (32 keys at a time against 64), so the running
-    # maxima and the bfloat16 roundings of the probabilities differ slightly
-    torch.testing.assert_close(two.float(), one.float(), atol=1e-2, rtol=1e-2)
+    monkeypatch.setenv("TTPA_PREFILL_STREAM", "1")
+    stream = torch.ops.tt.scaled_dot_product_attention(q.cuda(), k.cuda(), v.cuda(), is_causal=True)
+    monkeypatch.setenv("TTPA_PREFILL_STREAM", "0")
+    plain = torch.ops.tt.scaled_dot_product_attention(q.cuda(), k.cuda(), v.cuda(), is_causal=True)
+    # the loops split a tile differently (32 keys at a time against 64), so the running maxima and the
+    # bfloat16 roundings of the probabilities differ slightly
+    torch.testing.assert_close(stream.float(), plain.float(), atol=1e-2, rtol=1e-2)

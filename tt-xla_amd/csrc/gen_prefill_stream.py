@@ -44,8 +44,16 @@ the tile K enters two iterations from now is requested in front of the tile requ
 odd iteration (so the same wait covers it) and read at the next odd one.  Entries outside
 [0, num_blocks) read cache block 0.
 
-The block does everything between the Q fragments and the final normalisation: its own first
-requests (K blocks 0..NS-1, V blocks 0..NS-3), all `nblk` blocks, the last PV.
+A workgroup takes several ITEMS (blocks of 32 query rows of its four heads) one after the other:
+item k of the workgroup in slot j of `spg` slots is row block nqt - 1 - d with
+d = k spg + (k even ? j : spg - 1 - j), as long as d < nqt.  Row blocks are dealt heavy first and in
+alternating direction, so that with causal masking every workgroup gets about the same number of
+key blocks, and a launch is one round of workgroups: no workgroup waits for a free slot, and the
+start of a workgroup is paid once for several row blocks.  Per item the block does everything
+between the Q fragments and the stored output rows: its first requests (K blocks 0..NS-1, V blocks
+0..NS-3; for the first item they are a block of assembly of their own, so that the caller's Q loads
+overlap them), all blocks, the last PV, normalisation and store; then the next item's Q fragments
+and first requests go out in front of the store of the finished one.
 
 Matrix-to-vector hazards the hardware does not interlock are kept by construction: the vector
 instructions that read a score bank start two matrix instructions after the last one that wrote
@@ -56,7 +64,7 @@ after the last one that read it; the slow path and the exit wait out the matrix 
 import os
 import sys
 
-PROBE = {k: bool(int(os.environ.get('PROBE_' + k, '0'))) for k in ('NOVALU', 'NOBAR', 'NODS', 'NOMFMA', 'STAMPS')}
+PROBE = {k: bool(int(os.environ.get('PROBE_' + k, '0'))) for k in ('NOVALU', 'NOBAR', 'NODS', 'NOMFMA', 'STAMPS', 'ITEMSTAMPS')}
 
 # ---- register map (vector registers) ---------------------------------------------------------
 ACC = [0, 16, 32, 48]          # output accumulators, head-dim blocks 0..3 (inputs / outputs)
@@ -75,7 +83,11 @@ ORV, MLOC, MB, MCN = 204, 205, 206, 207
 PTREQ = 208                    # paged: the requested block-table entry (input)
 LIMIT = 212                    # last visible key of the lane's row, minus 4 h (input)
 LIMREL, NEGINF, VZERO = 213, 214, 215
-CLOBBERED = list(range(S[0], RING + 4 * NSLOT)) + list(range(LSUM, MCN + 1)) + [209, 210, 211, LIMREL, NEGINF, VZERO]
+QBASE, OUTBASE = 216, 218      # per lane, 64-bit: q / out of row 0 of the lane's head, at the lane's 8 h / 4 h elements (inputs)
+VN, V4H = 220, 221             # lane % 32 and 4 (lane / 32) (inputs)
+OUTP, PTMP, VT0, VROW = 222, 224, 226, 227
+CLOBBERED = (list(range(0, QF)) + list(range(S[0], RING + 4 * NSLOT)) + list(range(MC, MCN + 1)) + [209, 210, 211, LIMIT, LIMREL, NEGINF, VZERO]
+             + list(range(OUTP, VROW + 1)))
 
 # ---- scalar registers ---------------------------------------------------------------------------
 S_KBASE = "s[64:65]"           # dense: next K block to request; paged: the K cache (both minus 1024, see dma)
@@ -97,8 +109,16 @@ S_OFFV = "s[84:85]"            # byte offset in a cache of the tile V requests f
 S_OFFK = "s[86:87]"            # ... K requests from (on entry: tile 2)
 S_RLEFT = "s96"                # entries left to request
 S_OFF0 = "s[98:99]"            # byte offset of tile 0
-# temporaries s[88:95]
-SCALAR_CLOBBERS = [f"s{r}" for r in range(88, 96)]
+# items
+S_K, S_J, S_SPG, S_NQT = "s40", "s41", "s42", "s43"      # item counter, slot of the workgroup, slots, row blocks
+S_SQ, S_SKV, S_OFFSET, S_CAUSAL = "s44", "s45", "s46", "s47"
+S_QTS, S_OTS = "s48", "s49"    # bytes from a query / output row to the next
+# dense: s[50:51], s[52:53] K / V block 0 (minus 1024); paged: tile 1 and 2 offsets, s54 entry of tile 3,
+# s55 / s56 tile-in-cache-block of tiles 3 / 4, s[58:59] address of tile 4's entry
+S_ROW0 = "s57"                 # first query row of the item
+S_STOREMASK = "s[60:61]"
+# temporaries s[88:95], s[62:63]
+SCALAR_CLOBBERS = [f"s{r}" for r in list(range(88, 96)) + [60, 61, 62, 63, 74, 75]]
 
 NS = 5                         # slots per ring
 UNROLL = 10                    # lcm(2, NS): score bank and slots repeat
@@ -393,7 +413,149 @@ def first_frags(p):
     return [f for _, f in iteration_pairs(p % UNROLL)[:NSLOT]]
 
 
-def generate_first(paged):
+def item_setup(o, tag):
+    """Per-item state from S_ROW0: output pointers, the rows' key limits, the mask threshold, cleared
+    accumulators and softmax state."""
+    o.e(f"v_add_u32 v{VROW}, {S_ROW0}, v{VN}")                                   # the lane's query row
+    o.e(f"v_mad_u64_u32 v[{OUTP}:{OUTP + 1}], s[92:93], v{VROW}, {S_OTS}, v[{OUTBASE}:{OUTBASE + 1}]")
+    o.e(f"v_cmp_gt_i32_e64 {S_STOREMASK}, {S_SQ}, v{VROW}")                      # rows that exist are stored
+    o.e(f"s_sub_u32 s88, {S_SQ}, 1")
+    o.e(f"v_min_i32 v{VT0}, s88, v{VROW}")                                       # rows past the end repeat the last one
+    o.e(f"v_add_u32 v{VT0}, {S_OFFSET}, v{VT0}")
+    o.e(f"s_sub_u32 s89, {S_SKV}, 1")
+    o.e(f"v_min_i32 v{VT0}, s89, v{VT0}")                                        # causal: min(offset + row, skv - 1)
+    o.e(f"s_add_u32 s88, {S_OFFSET}, {S_ROW0}")
+    o.e("s_min_i32 s88, s88, s89")
+    o.e(f"s_cmp_eq_u32 {S_CAUSAL}, 0")
+    o.e("s_cselect_b32 s88, s89, s88")                                           # the first row's limit
+    o.e(f"s_cbranch_scc0 L_causal_{tag}%=")
+    o.e(f"v_mov_b32 v{VT0}, s89")                                                # not causal: skv - 1 for every row
+    o.label(f"L_causal_{tag}")
+    o.e(f"v_sub_u32 v{LIMIT}, v{VT0}, v{V4H}")
+    o.e(f"s_sub_u32 {S_MASKFROM}, s88, 30")
+    o.e(f"s_mov_b32 {S_KEY0}, 0")
+    o.e(f"v_mov_b32 v{MC}, 0xff800000")
+    o.e(f"v_mov_b32 v{LRUN}, 0")
+    for r in range(64):
+        o.e(f"v_mov_b32 v{r}, 0")
+
+
+def item_blocks(o):
+    """S_NB / requests left from S_ROW0: the 32-key blocks any row of the item can see."""
+    o.e(f"s_add_u32 s88, {S_ROW0}, 32")
+    o.e(f"s_min_i32 s88, s88, {S_SQ}")
+    o.e(f"s_add_u32 s88, s88, {S_OFFSET}")
+    o.e(f"s_min_i32 s88, s88, {S_SKV}")
+    o.e(f"s_cmp_eq_u32 {S_CAUSAL}, 0")
+    o.e(f"s_cselect_b32 s88, {S_SKV}, s88")
+    o.e("s_add_u32 s88, s88, 31")
+    o.e(f"s_lshr_b32 {S_NB}, s88, 5")
+    o.e(f"s_mov_b32 {S_KLEFT}, {S_NB}")
+    o.e(f"s_mov_b32 {S_VLEFT}, {S_NB}")
+
+
+def epilogue(o):
+    """Normalises the item's accumulators and stores its rows: lane (n, h) holds, in accumulator
+    register 16 db + 4 j + i, head-dim element 32 db + 8 j + 4 h + i of query row n.  The output pointer
+    of lane (n, h) is row n's plus 16 h bytes."""
+    o.e(f"v_mov_b32 v{MB}, v{LRUN}")
+    o.e("s_nop 1")
+    o.e(f"v_permlane32_swap_b32 v{LRUN}, v{MB}")
+    o.e("s_nop 1")
+    o.e(f"v_add_f32 v{ALPHA}, v{LRUN}, v{MB}")          # the row's sum: both halves of its keys
+    o.e(f"v_rcp_f32 v{ALPHA}, v{ALPHA}")
+    o.e("s_nop 1")
+    for r in range(64):
+        o.e(f"v_mul_f32 v{r}, v{ALPHA}, v{r}")
+    for i in range(32):
+        o.e(f"v_cvt_pk_bf16_f32 v{S[0] + i}, v{2 * i}, v{2 * i + 1}")
+    o.e("s_nop 1")
+    # The two lanes of a row trade halves, so that each stores 16 consecutive bytes (a row's 32 bytes per
+    # instruction): lane (n, 0) keeps its block j and takes (n, 1)'s, lane (n, 1) ends with both blocks j + 1.
+    for db in range(4):
+        for jp in range(2):
+            x = S[0] + 8 * db + 4 * jp
+            o.e(f"v_permlane32_swap_b32 v{x}, v{x + 2}")
+            o.e(f"v_permlane32_swap_b32 v{x + 1}, v{x + 3}")
+    o.e("s_nop 3")
+    o.e(f"s_and_saveexec_b64 s[62:63], {S_STOREMASK}")
+    o.e("s_nop 1")
+    for db in range(4):
+        for jp in range(2):
+            src = S[0] + 8 * db + 4 * jp
+            o.e(f"global_store_dwordx4 v[{OUTP}:{OUTP + 1}], v[{src}:{src + 3}], off offset:{64 * db + 32 * jp}")
+    o.e("s_mov_b64 exec, s[62:63]")
+    o.e("s_nop 1")
+
+
+def tstamp(o, reg):
+    """probe builds: low word of the wall clock (10 ns units) into a vector register"""
+    if PROBE['ITEMSTAMPS']:
+        o.e("s_memrealtime s[94:95]")
+        o.e("s_waitcnt lgkmcnt(0)")
+        o.e(f"v_mov_b32 v{reg}, s94")
+
+
+def next_item(o, paged):
+    """Behind the last PV of an item: is there another one?  Its Q fragments and first requests go
+    out first, then the finished item is stored, then the state of the new one is set up."""
+    o.e(f"s_add_u32 {S_K}, {S_K}, 1")
+    o.e(f"s_mul_i32 s88, {S_K}, {S_SPG}")
+    o.e(f"s_sub_u32 s89, {S_SPG}, 1")
+    o.e(f"s_sub_u32 s89, s89, {S_J}")
+    o.e(f"s_bitcmp1_b32 {S_K}, 0")
+    o.e(f"s_cselect_b32 s89, s89, {S_J}")               # odd items are dealt in the other direction
+    o.e("s_add_u32 s88, s88, s89")                      # d: the item's rank among the row blocks, heavy first
+    o.e(f"s_cmp_ge_u32 s88, {S_NQT}")
+    o.e("s_cbranch_scc1 L_last_item%=")
+    o.e(f"s_sub_u32 s88, {S_NQT}, s88")
+    o.e("s_sub_u32 s88, s88, 1")
+    o.e(f"s_lshl_b32 {S_ROW0}, s88, 5")                 # (the finished item's pointers and store mask stay in registers)
+    tstamp(o, 232)
+    o.e("s_barrier")                                    # everybody has left the rings
+    tstamp(o, 233)
+    o.e(f"v_add_u32 v{VROW}, {S_ROW0}, v{VN}")
+    o.e(f"s_sub_u32 s88, {S_SQ}, 1")
+    o.e(f"v_min_i32 v{VROW}, s88, v{VROW}")
+    o.e(f"v_mad_u64_u32 v[{PTMP}:{PTMP + 1}], s[92:93], v{VROW}, {S_QTS}, v[{QBASE}:{QBASE + 1}]")
+    for ks in range(8):
+        o.e(f"global_load_dwordx4 {vr(QF + 4 * ks, 4)}, v[{PTMP}:{PTMP + 1}], off offset:{32 * ks}")
+    tstamp(o, 234)
+    item_blocks(o)
+    if paged:
+        o.e("s_mov_b64 s[84:85], s[50:51]")
+        o.e("s_mov_b64 s[86:87], s[52:53]")
+        o.e(f"v_mov_b32 v{PTREQ}, s54")
+        o.e(f"s_mov_b32 {S_CIN}, s55")
+        o.e(f"s_mov_b32 {S_RIN}, s56")
+        o.e("s_mov_b64 s[82:83], s[58:59]")
+        o.e(f"s_sub_u32 s88, {S_NB}, 1")
+        o.e("s_lshr_b32 s88, s88, 1")
+        o.e("s_sub_u32 s88, s88, 3")
+        o.e("s_max_i32 s88, s88, 0")
+        o.e(f"s_mov_b32 {S_RLEFT}, s88")
+    else:
+        o.e("s_mov_b64 s[64:65], s[50:51]")
+        o.e("s_mov_b64 s[66:67], s[52:53]")
+    for ln in generate_first(paged, "nx"):
+        o.lines.append(ln)
+    tstamp(o, 235)
+    epilogue(o)
+    tstamp(o, 236)
+    item_setup(o, "nx")
+    tstamp(o, 237)
+    if PROBE['ITEMSTAMPS']:
+        o.e("v_mov_b32 v209, s97")
+        o.e("s_nop 1")
+        o.e("global_store_dwordx4 v209, v[232:235], s[100:101]")
+        o.e("global_store_dwordx4 v209, v[236:239], s[100:101] offset:16")
+        o.e("s_add_u32 s97, s97, 32")
+    o.e("s_branch L_item_top%=")
+    o.label("L_last_item")
+    epilogue(o)
+
+
+def generate_first(paged, suffix=""):
     """The first requests: K blocks 0 .. NS - 1, V blocks 0 .. NS - 3 (a block of its own, so that
     the caller can put its Q loads behind them)."""
     o = Out()
@@ -402,7 +564,7 @@ def generate_first(paged):
             src = ("s[98:99]", S_OFFV, S_OFFK)[j // 2]
             lo = int(src[2:4])
             o.e(f"s_cmp_eq_u32 {S_KLEFT}, 0")
-            o.e(f"s_cbranch_scc1 L_noK_pro{j}%=")
+            o.e(f"s_cbranch_scc1 L_noK_pro{j}{suffix}%=")
             o.e(f"s_add_u32 s90, s64, s{lo}")
             o.e(f"s_addc_u32 s91, s65, s{lo + 1}")
             if j % 2:
@@ -412,15 +574,15 @@ def generate_first(paged):
             o.e("s_nop 0")
             two_loads(o, LDK, "s[90:91]")
             o.e(f"s_sub_u32 {S_KLEFT}, {S_KLEFT}, 1")
-            o.label(f"L_noK_pro{j}")
+            o.label(f"L_noK_pro{j}{suffix}")
         else:
-            request_block(o, "K", j, f"pro{j}", False, 0)
+            request_block(o, "K", j, f"pro{j}{suffix}", False, 0)
     for j in range(NS - 2):
         if paged:
             src = ("s[98:99]", S_OFFV)[j // 2]
             lo = int(src[2:4])
             o.e(f"s_cmp_eq_u32 {S_VLEFT}, 0")
-            o.e(f"s_cbranch_scc1 L_noV_pro{j}%=")
+            o.e(f"s_cbranch_scc1 L_noV_pro{j}{suffix}%=")
             o.e(f"s_add_u32 s90, s66, s{lo}")
             o.e(f"s_addc_u32 s91, s67, s{lo + 1}")
             if j % 2:
@@ -430,18 +592,28 @@ def generate_first(paged):
             o.e("s_nop 0")
             two_loads(o, LDV, "s[90:91]")
             o.e(f"s_sub_u32 {S_VLEFT}, {S_VLEFT}, 1")
-            o.label(f"L_noV_pro{j}")
+            o.label(f"L_noV_pro{j}{suffix}")
         else:
-            request_block(o, "V", j, f"pro{j}", False, 0)
+            request_block(o, "V", j, f"pro{j}{suffix}", False, 0)
     return o.lines
 
 
 def generate(paged):
     o = Out()
     assert NS == 5 and UNROLL == 10
-    if PROBE['STAMPS']:
+    if PROBE['STAMPS'] or PROBE['ITEMSTAMPS']:
         o.e("s_mov_b32 s97, 0")
+    if PROBE['ITEMSTAMPS']:  # QBASE / OUTBASE are borrowed for the stamps: copies
+        for k in range(4):
+            o.e(f"v_mov_b32 v{228 + k}, v{216 + k}")
     o.e(f"v_mov_b32 v{VZERO}, 0")
+    item_setup(o, "first")
+    o.label("L_item_top")
+    if PROBE['ITEMSTAMPS']:
+        o.e("s_memrealtime s[92:93]")
+        o.e("s_waitcnt lgkmcnt(0)")
+        o.e("v_mov_b32 v216, s92")
+        o.e("v_mov_b32 v217, s93")
     o.e("s_waitcnt vmcnt(0)")
     o.e("s_barrier")
     # ---- S(0) from K block 0; behind it the fragments of iteration 0 (K block 1) ------------------
@@ -485,6 +657,21 @@ def generate(paged):
     o.label("L_end")
     o.e("s_nop 15")
     o.e("s_nop 15")
+    if PROBE['ITEMSTAMPS']:  # (start and end of the item, wall clock; QBASE is borrowed, so only one item is correct... the probe build keeps it in v[228:229])
+        o.e("s_memrealtime s[94:95]")
+        o.e("s_waitcnt lgkmcnt(0)")
+        o.e("v_mov_b32 v218, s94")
+        o.e("v_mov_b32 v219, s95")
+        o.e("v_mov_b32 v209, s97")
+        o.e("s_nop 1")
+        o.e("global_store_dwordx4 v209, v[216:219], s[100:101]")
+        o.e("s_add_u32 s97, s97, 16")
+        o.e("s_waitcnt vmcnt(0)")
+        o.e("v_mov_b32 v216, v228")
+        o.e("v_mov_b32 v217, v229")
+        o.e("v_mov_b32 v218, v230")
+        o.e("v_mov_b32 v219, v231")
+    next_item(o, paged)
     return o.lines
 
 

@@ -26,6 +26,7 @@
 #include "common.h"
 #include "build/prefill_stream_asm.h"
 
+#include <algorithm>
 #include <cstdlib>
 
 namespace ttpa {
@@ -71,7 +72,9 @@ struct PrefillArgs {
   int window;  // > 0 (causal only): row i attends keys offset + i - window < j <= offset + i
   float scale_log2e;
   int kv_bfp8;  // paged form: the caches are block-float-8 (mode 4)
-  int stream;   // run whole unmasked tiles through the hand-scheduled loop (stream_tiles)
+  int stream;   // the hand-scheduled loop serves this launch (head size 128, 4 heads per workgroup, whole blocks)
+  int spg;      // ... with this many workgroups per (batch entry, head group), each taking several row blocks
+  int spg_even; // > 0: when the row blocks weigh about the same, only this many of them work (equal shares)
 };
 
 // key / block_size without a division instruction sequence (about 30 instructions each, and the
@@ -164,75 +167,90 @@ __device__ __forceinline__ void fill_workgroup(const PrefillArgs &a, int f) {
 typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
 
-struct StreamState {
-  floatx16 acc[4];
-  float mc, lrun;  // reference of the probabilities (exponent domain), row sum
-};
-
 // The requests of a workgroup's first blocks are a block of assembly of their own, issued in front
-// of the Q loads so that the two round trips to memory overlap.
+// of the Q loads so that the two round trips to memory overlap.  (Scalars only: with the per-lane
+// offsets in the same struct the compiler keeps the whole of it in vector registers.)
 struct StreamRequests {
   uint64_t kbase, vbase;       // dense: block 0 of K / V; paged: the caches (both minus 1024 bytes)
   uint32_t stride;             // dense: bytes from a 32-key block to the next; paged: bytes of a (cache block, head) slab
   uint32_t m0_base;            // LDS address of the wavefront's first segment in K slot 0
   int k_requests, v_requests;  // blocks not requested yet
-  u32x2 ldk, ldv;              // the lane's byte offsets of its two loads per block
   uint64_t off0, off1, off2;   // paged: byte offsets of tiles 0, 1, 2 in a cache
 };
 
-__device__ __forceinline__ void stream_first_dense(StreamRequests &r) {
+__device__ __forceinline__ void stream_first_dense(StreamRequests &r, const u32x2 &ldk, const u32x2 &ldv) {
   asm volatile(TTPA_STREAM_FIRST_TEXT_DENSE
                : "+{s[64:65]}"(r.kbase), "+{s[66:67]}"(r.vbase), "+{s71}"(r.k_requests), "+{s73}"(r.v_requests)
-               : "{v[188:189]}"(r.ldk), "{v[190:191]}"(r.ldv), "{s68}"(r.stride), "{s72}"(r.m0_base)
+               : "{v[188:189]}"(ldk), "{v[190:191]}"(ldv), "{s68}"(r.stride), "{s72}"(r.m0_base)
                : "memory", "scc", "m0");
 }
 
-__device__ __forceinline__ void stream_first_paged(StreamRequests &r) {
+__device__ __forceinline__ void stream_first_paged(StreamRequests &r, const u32x2 &ldk, const u32x2 &ldv) {
   asm volatile(TTPA_STREAM_FIRST_TEXT_PAGED
                : "+{s71}"(r.k_requests), "+{s73}"(r.v_requests)
-               : "{v[188:189]}"(r.ldk), "{v[190:191]}"(r.ldv), "{s[64:65]}"(r.kbase), "{s[66:67]}"(r.vbase),
+               : "{v[188:189]}"(ldk), "{v[190:191]}"(ldv), "{s[64:65]}"(r.kbase), "{s[66:67]}"(r.vbase),
                  "{s72}"(r.m0_base), "{s[84:85]}"(r.off1), "{s[86:87]}"(r.off2), "{s[98:99]}"(r.off0)
                : "memory", "scc", "m0", "s90", "s91");
 }
 
-#define TTPA_STREAM_COMMON_OUT                                                                          \
-  "+{v[0:15]}"(st.acc[0]), "+{v[16:31]}"(st.acc[1]), "+{v[32:47]}"(st.acc[2]), "+{v[48:63]}"(st.acc[3]), \
-      "+{v196}"(st.mc), "+{v197}"(st.lrun), "+{s[64:65]}"(r.kbase), "+{s[66:67]}"(r.vbase), "+{s70}"(nblk),  \
-      "+{s71}"(r.k_requests), "+{s73}"(r.v_requests), "+{s75}"(key0)
-#define TTPA_STREAM_COMMON_IN                                                                       \
-  "{v[64:79]}"(q_lo), "{v[80:95]}"(q_hi), "{v[176:183]}"(koff), "{v[184:187]}"(voff),               \
-      "{v[188:189]}"(r.ldk), "{v[190:191]}"(r.ldv), "{v212}"(limit), "{s68}"(r.stride), "{s69}"(c),  \
-      "{s72}"(r.m0_base), "{s74}"(mask_from)
+// The items of a workgroup (see gen_prefill_stream.py): which row blocks, and what the block needs
+// to set one up.
+// Values the compiler may hold in vector registers although they are the same in every lane: the
+// block binds them to scalar registers.
+__device__ __forceinline__ int uni(int x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ uint32_t uni(uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); }
+__device__ __forceinline__ uint64_t uni(uint64_t x) {
+  return address_from_words(__builtin_amdgcn_readfirstlane((int)(uint32_t)x), __builtin_amdgcn_readfirstlane((int)(uint32_t)(x >> 32)));
+}
 
-// Everything behind the first requests.  q_lo / q_hi: the eight Q fragments; koff / voff: the lane's
-// LDS addresses of its K and V^T fragments in slot 0 of the K and V rings; limit: the last key the
-// lane's row may see minus 4 (lane / 32); mask_from: the first key from which blocks need their mask;
-// nblk: the 32-key blocks.
-__device__ __forceinline__ void stream_blocks_dense(StreamState &st, StreamRequests &r, const u32x16 &q_lo,
-                                                    const u32x16 &q_hi, const u32x8 &koff, const u32x4 &voff,
-                                                    int limit, float c, int nblk, int mask_from) {
-  int key0 = 0;
+struct StreamItems {
+  int k, j, spg, nqt;          // item counter (starts at 0), the workgroup's slot, slots, row blocks
+  int sq, skv, offset, causal;
+  uint32_t q_row_bytes, out_row_bytes;
+  int row0;                    // first query row of item 0
+};
+
+#define TTPA_STREAM_COMMON_OUT                                                                        \
+  "+{v[64:79]}"(q_lo), "+{v[80:95]}"(q_hi), "+{s[64:65]}"(r.kbase), "+{s[66:67]}"(r.vbase), "+{s70}"(nblk), \
+      "+{s71}"(r.k_requests), "+{s73}"(r.v_requests), "+{s40}"(it.k), "+{s57}"(it.row0)
+#define TTPA_STREAM_COMMON_IN                                                                       \
+  "{v[176:183]}"(koff), "{v[184:187]}"(voff), "{v[188:189]}"(ldk), "{v[190:191]}"(ldv),         \
+      "{v[216:217]}"(q_base), "{v[218:219]}"(out_base), "{v220}"(lane_n), "{v221}"(lane_h4),       \
+      "{s68}"(r.stride), "{s69}"(c), "{s72}"(r.m0_base), "{s41}"(it.j), "{s42}"(it.spg), "{s43}"(it.nqt), \
+      "{s44}"(it.sq), "{s45}"(it.skv), "{s46}"(it.offset), "{s47}"(it.causal), "{s48}"(it.q_row_bytes),  \
+      "{s49}"(it.out_row_bytes)
+
+// Everything behind the first requests of item 0, through the stored output rows of the last item.
+// q_lo / q_hi: the eight Q fragments of item 0; koff / voff: the lane's LDS addresses of its K and
+// V^T fragments in slot 0 of the K and V rings; nblk: the 32-key blocks of item 0; kbase0 / vbase0:
+// block 0 of K / V again, for the items that follow.
+__device__ __forceinline__ void stream_items_dense(StreamRequests &r, StreamItems &it, u32x16 q_lo, u32x16 q_hi,
+                                                   const u32x8 &koff, const u32x4 &voff, const u32x2 &ldk,
+                                                   const u32x2 &ldv, uint64_t q_base, uint64_t out_base, int lane_n,
+                                                   int lane_h4, float c, int nblk, uint64_t kbase0, uint64_t vbase0) {
   asm volatile(TTPA_STREAM_LOOP_TEXT_DENSE
                : TTPA_STREAM_COMMON_OUT
-               : TTPA_STREAM_COMMON_IN
+               : TTPA_STREAM_COMMON_IN, "{s[50:51]}"(kbase0), "{s[52:53]}"(vbase0)
                : "memory", "vcc", "scc", "m0", "v208", TTPA_STREAM_LOOP_CLOBBERS);
 }
 
 // Paged: entry is the raw table entry of tile 3, entry_ptr the address of tile 4's.
-__device__ __forceinline__ void stream_blocks_paged(StreamState &st, StreamRequests &r, const u32x16 &q_lo,
-                                                    const u32x16 &q_hi, const u32x8 &koff, const u32x4 &voff,
-                                                    int limit, float c, int nblk, int mask_from, int kv_heads,
-                                                    int kv_head, int num_blocks, int tiles_per_block, int entry,
-                                                    uint64_t entry_ptr) {
-  int key0 = 0;
+__device__ __forceinline__ void stream_items_paged(StreamRequests &r, StreamItems &it, u32x16 q_lo, u32x16 q_hi,
+                                                   const u32x8 &koff, const u32x4 &voff, const u32x2 &ldk,
+                                                   const u32x2 &ldv, uint64_t q_base, uint64_t out_base, int lane_n,
+                                                   int lane_h4, float c, int nblk, int kv_heads, int kv_head, int num_blocks, int tiles_per_block,
+                                                   int entry, uint64_t entry_ptr) {
   int read_in_block = 3 % tiles_per_block, request_in_block = 4 % tiles_per_block;
+  const int read_in_block0 = read_in_block, request_in_block0 = request_in_block, entry0 = entry;
+  const uint64_t entry_ptr0 = entry_ptr, off1 = r.off1, off2 = r.off2;
   int entry_requests = max((nblk - 1) / 2 - 3, 0);
   asm volatile(TTPA_STREAM_LOOP_TEXT_PAGED
                : TTPA_STREAM_COMMON_OUT, "+{s80}"(read_in_block), "+{s81}"(request_in_block),
                  "+{s[82:83]}"(entry_ptr), "+{s[84:85]}"(r.off1), "+{s[86:87]}"(r.off2), "+{s96}"(entry_requests),
                  "+{v208}"(entry)
                : TTPA_STREAM_COMMON_IN, "{s76}"(kv_heads), "{s77}"(kv_head), "{s78}"(num_blocks),
-                 "{s79}"(tiles_per_block), "{s[98:99]}"(r.off0)
+                 "{s79}"(tiles_per_block), "{s[98:99]}"(r.off0), "{s[50:51]}"(off1), "{s[52:53]}"(off2),
+                 "{s54}"(entry0), "{s55}"(read_in_block0), "{s56}"(request_in_block0), "{s[58:59]}"(entry_ptr0)
                : "memory", "vcc", "scc", "m0", TTPA_STREAM_LOOP_CLOBBERS);
 }
 
@@ -297,11 +315,15 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
   // while its query tiles stream through.
   const int nqt = (a.sq + ROWS * RPW - 1) / (ROWS * RPW);
   const int groups = a.hq / HPW;
+  // (the hand-scheduled loop: a.spg workgroups per group, each taking several row blocks, heavy first)
+  constexpr bool kStreams = D == 128 && HPW == 4 && RH == 1 && (MODE == 0 || MODE == 1);
+  const bool streamed = kStreams && a.stream != 0;
+  const int per_group = streamed ? a.spg : nqt;
   const int xcd = wg & 7, slot = wg >> 3;
-  const int yl = slot / nqt;
+  const int yl = slot / per_group;
   const int y = yl * 8 + xcd;
   if (y >= a.batch * groups) return;  // grid is padded to a multiple of 8 groups
-  const int qt = nqt - 1 - (slot - yl * nqt);  // heavy (late) tiles are scheduled first
+  const int qt = nqt - 1 - (slot - yl * per_group);  // heavy (late) tiles are scheduled first
   const int b = y / groups;
   const int hq0 = (y - b * groups) * HPW;
   const int g = a.hq / a.hkv;
@@ -321,34 +343,41 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
   const int wave_first_key = a.window > 0 ? max(0, offset + row0 - a.window + 1) : 0;
   const int first_tile = wg_first_key / kKeysPerTile;
 
-  // ---- the hand-scheduled loop takes workgroups of whole 32-key blocks; its first requests go out now ----
-  // (a dense K / V that ends inside a 64-key tile goes through the plain loop)
-  bool streamed = false;
+  // ---- the hand-scheduled loop: its first requests go out now, in front of the Q loads ----------
   StreamRequests sreq;
+  u32x2 stream_ldk = {0, 0}, stream_ldv = {0, 0};
   int stream_entry = 0;
-  if constexpr (D == 128 && HPW == 4 && RH == 1 && (MODE == 0 || MODE == 1)) {
-    streamed = a.stream && a.window == 0 && a.mask == nullptr && wave_active && (MODE == 1 || a.skv % kKeysPerTile == 0);
+  if constexpr (kStreams) {
     if (streamed) {
+      int spg = a.spg;
+      if (a.spg_even > 0) {
+        const int lightest = a.causal ? min(offset + ROWS, a.skv) : a.skv;
+        const int heaviest = a.causal ? min(offset + a.sq, a.skv) : a.skv;
+        if (4 * lightest >= 3 * heaviest) {
+          spg = a.spg_even;
+          if (slot - yl * per_group >= spg) return;
+        }
+      }
       const uint32_t lds0 = lds_address(smem);
       const uint32_t row_bytes = MODE == 0 ? 2u * (uint32_t)a.kv_ts : (uint32_t)T::RB;
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         // a block is 8 segments of 1 KiB; wavefront w requests segments 2 w and 2 w + 1
         const int r = (2 * wave + j) * T::RPI + lane / T::CPR, cp = lane % T::CPR;
-        sreq.ldk[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_k(r)) + 1024u - 1024u * j;
-        sreq.ldv[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_v(r)) + 1024u - 1024u * j;
+        stream_ldk[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_k(r)) + 1024u - 1024u * j;
+        stream_ldv[j] = (uint32_t)r * row_bytes + 16u * (uint32_t)(cp ^ T::swz_v(r)) + 1024u - 1024u * j;
       }
-      sreq.m0_base = lds0 + 2048u * (uint32_t)wave;
-      sreq.k_requests = sreq.v_requests = (kv_end_wg + 31) / 32;
+      sreq.m0_base = uni(lds0 + 2048u * (uint32_t)wave);
+      sreq.k_requests = sreq.v_requests = __builtin_amdgcn_readfirstlane((kv_end_wg + 31) / 32);
       sreq.off0 = sreq.off1 = sreq.off2 = 0;
       if constexpr (MODE == 0) {
         const int64_t head = b * a.kv_bs + hk * a.kv_hs;
-        sreq.kbase = reinterpret_cast<uint64_t>(a.k + head) - 1024u;
-        sreq.vbase = reinterpret_cast<uint64_t>(a.v + head) - 1024u;
+        sreq.kbase = uni(reinterpret_cast<uint64_t>(a.k + head) - 1024u);
+        sreq.vbase = uni(reinterpret_cast<uint64_t>(a.v + head) - 1024u);
         sreq.stride = (uint32_t)(64 * a.kv_ts);
-        stream_first_dense(sreq);
+        stream_first_dense(sreq, stream_ldk, stream_ldv);
       } else {
-        const int tpb = a.bs / kKeysPerTile, last = ntiles - 1;
+        const int tpb = a.bs / kKeysPerTile, last = a.w * tpb - 1;  // (entries exist for every tile of the table)
         sreq.kbase = reinterpret_cast<uint64_t>(a.k) - 1024u;
         sreq.vbase = reinterpret_cast<uint64_t>(a.v) - 1024u;
         sreq.stride = (uint32_t)a.bs * (uint32_t)T::RB;
@@ -362,10 +391,55 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
           if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
           off[t] = (uint64_t)((int64_t)phys * a.hkv + hk) * sreq.stride + (uint64_t)(min(t, last) % tpb) * T::TILE_BYTES;
         }
-        sreq.off0 = off[0], sreq.off1 = off[1], sreq.off2 = off[2];
+        sreq.off0 = uni(off[0]), sreq.off1 = uni(off[1]), sreq.off2 = uni(off[2]);
         stream_entry = raw[3];
-        stream_first_paged(sreq);
+        stream_first_paged(sreq, stream_ldk, stream_ldv);
       }
+      // Q fragments behind the requests (B operand: lane n = query row, 8 head-dim elements per k-step)
+      u32x16 q_lo, q_hi;
+      {
+        const int qrow = min(row0 + n, a.sq - 1);
+        const uint16_t *qp = a.q + b * a.q_bs + hq * a.q_hs + (int64_t)qrow * a.q_ts + 8 * h;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const uint4 lo = *reinterpret_cast<const uint4 *>(qp + 16 * s), hi = *reinterpret_cast<const uint4 *>(qp + 16 * (s + 4));
+          q_lo[4 * s] = lo.x, q_lo[4 * s + 1] = lo.y, q_lo[4 * s + 2] = lo.z, q_lo[4 * s + 3] = lo.w;
+          q_hi[4 * s] = hi.x, q_hi[4 * s + 1] = hi.y, q_hi[4 * s + 2] = hi.z, q_hi[4 * s + 3] = hi.w;
+        }
+      }
+      // LDS operand addresses of the lane inside slot 0 of the K ring and of the V ring (the formulas
+      // of the plain loop below: K fragment of k-step s, V^T fragment of output block db)
+      u32x8 ko;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) ko[s] = lds0 + (uint32_t)(n * T::RB + 16 * ((2 * s + h) ^ T::swz_k(n)));
+      u32x4 vo;
+      {
+        const int grp = lane >> 4, a16 = lane & 15, vr = 4 * (grp >> 1) + (a16 >> 2);
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          const int c = 4 * db + 2 * (grp & 1) + ((a16 & 3) >> 1);
+          vo[db] = lds0 + TTPA_STREAM_V_RING + (uint32_t)(vr * T::RB + 16 * (c ^ T::swz_v(vr)) + 8 * (a16 & 1));
+        }
+      }
+      StreamItems it;
+      it.k = 0, it.j = uni(slot - yl * per_group), it.spg = uni(spg), it.nqt = uni(nqt);
+      it.sq = uni(a.sq), it.skv = uni(a.skv), it.offset = uni(offset), it.causal = uni(a.causal);
+      it.q_row_bytes = uni(2u * (uint32_t)a.q_ts), it.out_row_bytes = uni(2u * (uint32_t)a.out_ts);
+      it.row0 = __builtin_amdgcn_readfirstlane(row0);
+      // per lane: row 0 of the lane's head, at the lane's 8 (lane / 32) / 4 (lane / 32) elements
+      const uint64_t q_base = reinterpret_cast<uint64_t>(a.q + b * a.q_bs + hq * a.q_hs + 8 * h);
+      const uint64_t out_base = reinterpret_cast<uint64_t>(a.out + b * a.out_bs + hq * a.out_hs + 8 * h);
+      const int nblk = __builtin_amdgcn_readfirstlane((kv_end_wg + 31) / 32);
+      if constexpr (MODE == 0) {
+        const int64_t head = b * a.kv_bs + hk * a.kv_hs;
+        stream_items_dense(sreq, it, q_lo, q_hi, ko, vo, stream_ldk, stream_ldv, q_base, out_base, n, 4 * h, a.scale_log2e, nblk,
+                           uni(reinterpret_cast<uint64_t>(a.k + head) - 1024u), uni(reinterpret_cast<uint64_t>(a.v + head) - 1024u));
+      } else {
+        const int tpb = a.bs / kKeysPerTile;
+        stream_items_paged(sreq, it, q_lo, q_hi, ko, vo, stream_ldk, stream_ldv, q_base, out_base, n, 4 * h, a.scale_log2e, nblk, uni(a.hkv), uni(hk), uni(a.nb), uni(tpb), stream_entry,
+                           uni(reinterpret_cast<uint64_t>(a.pt + (int64_t)b * a.pt_rs + 4 / tpb)));
+      }
+      return;
     }
   }
 
@@ -603,45 +677,6 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
   auto kbuf = [&](int t) { return t & 1; };
   auto vbuf = [&](int t) { return t & 1; };
   int kt_begin = first_tile;
-  // ---- all blocks through the hand-scheduled loop ------------------------------------------------
-  if constexpr (D == 128 && HPW == 4 && RH == 1 && (MODE == 0 || MODE == 1)) {
-    if (streamed) {
-      StreamState ss;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) ss.acc[i] = acc[0][i];
-      ss.mc = -INFINITY, ss.lrun = 0.f;
-      u32x16 q_lo, q_hi;
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const u32x4 lo = __builtin_bit_cast(u32x4, qf[0][s]), hi = __builtin_bit_cast(u32x4, qf[0][s + 4]);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) q_lo[4 * s + e] = lo[e], q_hi[4 * s + e] = hi[e];
-      }
-      const uint32_t lds0 = lds_address(smem);
-      u32x8 ko;
-#pragma unroll
-      for (int s = 0; s < 8; ++s) ko[s] = koff[s] + lds0;
-      u32x4 vo;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) vo[j] = voff[j] + lds0 + TTPA_STREAM_V_RING;
-      // last key a row may see; rows past the end of q repeat the last one
-      const int row_limit = a.causal ? min(offset + min(row0 + n, a.sq - 1), a.skv - 1) : a.skv - 1;
-      const int first_limit = a.causal ? min(offset + row0, a.skv - 1) : a.skv - 1;
-      const int nblk = (kv_end_wg + 31) / 32;
-      if constexpr (MODE == 0) {
-        stream_blocks_dense(ss, sreq, q_lo, q_hi, ko, vo, row_limit - 4 * h, a.scale_log2e, nblk, first_limit - 30);
-      } else {
-        const int tpb = a.bs / kKeysPerTile;
-        stream_blocks_paged(ss, sreq, q_lo, q_hi, ko, vo, row_limit - 4 * h, a.scale_log2e, nblk, first_limit - 30,
-                            a.hkv, hk, a.nb, tpb, stream_entry,
-                            reinterpret_cast<uint64_t>(a.pt + (int64_t)b * a.pt_rs + 4 / tpb));
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[0][i] = ss.acc[i];
-      l_run[0] = ss.lrun;
-    }
-  }
-  if (streamed) kt_begin = ntiles;  // nothing is left for the plain loop; its first requests are skipped too
   Blocks blk_v = resolve(request(first_tile));     // blocks of the tile whose V is loaded next
   Blocks blk_k = resolve(request(first_tile + 1));  // ... whose K is loaded next
   Requested req = request(first_tile + 2);
@@ -650,7 +685,7 @@ __global__ __launch_bounds__(256, prefill_wgs_per_cu<RH>(D, MODE)) void prefill_
     commit_bfp8(fetch_bfp8(a.v, first_tile, blk_v), true, first_tile & 1);
     if (last_tile >= first_tile + 1)
       commit_bfp8(fetch_bfp8(a.k, first_tile + 1, blk_k), false, (first_tile + 1) & 1);
-  } else if (!streamed) {
+  } else {
     issue(a.k, ld_k, false, first_tile, kbuf(first_tile), blk_v);
     issue(a.v, ld_v, true, first_tile, vbuf(first_tile), blk_v);
     if (last_tile >= first_tile + 1) issue(a.k, ld_k, false, first_tile + 1, kbuf(first_tile + 1), blk_k);
@@ -850,8 +885,33 @@ int launch_mode(const PrefillArgs &a, hipStream_t st) {
   if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&prefill_kernel<D, HPW, MODE, RH>), lds, lds_ready))
     return fail(TTPA_ERR_LAUNCH, "prefill: cannot reserve %zu bytes of LDS", lds);
   const int ny8 = (a.batch * (a.hq / HPW) + 7) / 8;
-  int grid = nqt * ny8 * 8;
   PrefillArgs b = a;
+  // The hand-scheduled loop takes launches of whole 32-key blocks without a window or an explicit mask
+  // (a dense K / V that ends inside a 64-key tile goes through the plain loop).  One workgroup per
+  // block of 32 query rows and head group, heavy blocks first, and the dispatcher deals them to the CUs
+  // as slots free up: the loop can also give a workgroup several row blocks (spg workgroups per group,
+  // TTPA_PREFILL_WGS_PER_GROUP), but one round of two workgroups per CU measured 204 us against 150 on
+  // the 4 x 2048-token causal workload (a change of row block costs a workgroup about 4 us in which
+  // nothing of its own overlaps, and a static deal cannot make up for workgroups that start late).
+  b.stream = kStreams && a.stream && a.window == 0 && a.mask == nullptr && (MODE == 1 || a.skv % kKeysPerTile == 0);
+  b.spg = b.spg_even = 0;
+  int per_group = nqt;
+  if (b.stream) {
+    b.spg = nqt;
+    // Row blocks of nearly one weight (a chunk far into its sequence, or no causal mask) that fill the
+    // chip more than once: one round of workgroups with equal shares instead, which saves the later
+    // rounds' start-up (267 -> 261 us on 4 x 512-token chunks behind 4096 tokens, 64 heads).  The
+    // chunk's start is in device memory, so the kernel decides: the workgroups past the round exit.
+    int cus = device_cus();
+    if (cus <= 0) cus = 256;
+    const int one_round = (2 * cus + ny8 * 8 - 1) / (ny8 * 8);
+    b.spg_even = one_round < nqt && nqt % one_round == 0 ? one_round : 0;
+    if (const char *e = getenv("TTPA_PREFILL_WGS_PER_GROUP")) {  // (read on every call) an experiment's override
+      if (atoi(e) > 0) b.spg = std::min(nqt, atoi(e)), b.spg_even = 0;
+    }
+    per_group = b.spg;
+  }
+  int grid = per_group * ny8 * 8;
   if (MODE == 0 && a.fill_kc) {
     // The fill workgroups are spread over the launch in groups of 8, one group behind every
     // attn_per_fill groups of attention workgroups, so that their memory traffic runs while the
