@@ -609,7 +609,7 @@ def secondary_runs(args):
     import torch
 
     out = {}
-    for wl, steps, warmup in (("config3", 30, 5), ("config5", 96, 12), ("config4", 20, 4), ("latent", 40, 8)):
+    for wl, steps, warmup in (("config3", 96, 8), ("config5", 96, 12), ("config4", 32, 4), ("latent", 96, 8)):
         gc.collect()
         torch.cuda.empty_cache()
         sub = copy.copy(args)

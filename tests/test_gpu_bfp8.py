@@ -259,6 +259,11 @@ def test_config5_full_size():
     (1, 16, 4, 128, 64, 6, 200, 128),    # a prefix that ends inside a block
     (2, 8, 2, 256, 32, 6, 64, 64),       # head size 256
     (3, 12, 4, 128, 48, 4, 100, 32),     # a block size that is no power of two
+    # shapes the expansion pass serves (head size 128, four query heads per workgroup, blocks of 64 n tokens)
+    (2, 32, 8, 128, 64, 6, 192, 128),
+    (3, 16, 4, 128, 128, 3, 130, 200),   # a prefix that ends inside a block, rows past the last full tile
+    (1, 8, 2, 128, 64, 9, 0, 300),       # first chunk: columns behind the chunk are skipped
+    (2, 64, 8, 128, 64, 5, 288, 32),     # one block of rows at the end of the table
 ])
 def test_chunked_prefill_over_a_bfp8_cache(users, hq, hkv, d, bs, nbpu, start, lc):
     """tt::chunked_scaled_dot_product_attention on block-float-8 caches (the reference's one test
@@ -284,6 +289,55 @@ def test_chunked_prefill_over_a_bfp8_cache(users, hq, hkv, d, bs, nbpu, start, l
     err = (got.float() - want).abs().max().item()
     print(f"{name}: max-abs error {err:.3e}", flush=True)
     torch.testing.assert_close(got.float(), want, atol=2e-2, rtol=2e-2)
+
+
+def test_expansion_pass_matches_tile_by_tile_expansion():
+    """ttpa_sdpa_prefill_expanded with scratch (bfloat16 copies of the blocks first, then the bfloat16
+    kernel) against the same entry point without (every tile expanded on its way into LDS), through
+    the C ABI: the decode is exact either way, the loops round the probabilities differently.  A
+    scratch one byte short is no error and takes the second route; table entries out of range read
+    block 0 on both."""
+    from tt_xla_amd import _native as N
+    from tt_xla_amd import custom_ops as ops
+
+    users, hq, hkv, d, bs, nbpu, start, lc = 3, 32, 8, 128, 64, 7, 256, 160
+    g = torch.Generator().manual_seed(77)
+    nb = users * nbpu + 1
+    key = torch.randn(nb, hkv, bs, d, generator=g).to(torch.bfloat16)
+    value = torch.randn(nb, hkv, bs, d, generator=g).to(torch.bfloat16)
+    table = (torch.randperm(nb - 1, generator=g) + 1).view(users, nbpu).to(torch.int32)
+    table[1, 2] = -1
+    table[2, 0] = nb + 5
+    q = (torch.randn(users, hq, lc, d, generator=g) * 0.5).to(torch.bfloat16).cuda()
+    cs = torch.tensor([start], dtype=torch.int32).cuda()
+    kp, vp = ops.bfp8_pack_cache(key.cuda()), ops.bfp8_pack_cache(value.cuda())
+    tb = table.cuda()
+    need = int(N.lib().ttpa_sdpa_prefill_workspace_bytes(users, hkv, d, bs, nbpu, N.KV_BFP8))
+    assert need == 2 * users * nbpu * hkv * bs * d * 2 + 256
+    assert N.lib().ttpa_sdpa_prefill_workspace_bytes(users, hkv, d, bs, nbpu, N.KV_BF16) == 0
+    ws = torch.full((need,), 0xAB, dtype=torch.uint8, device="cuda")
+
+    def run(ws_ptr, ws_bytes):
+        out = torch.empty_like(q)
+        N.call("ttpa_sdpa_prefill_expanded", out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
+               q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), kp.data_ptr(), vp.data_ptr(), 0, 0, 0,
+               tb.data_ptr(), tb.stride(0), cs.data_ptr(), 0, 0, 0, users, hq, hkv, lc, nbpu * bs, d, bs, nbpu, nb, 1,
+               d ** -0.5, 0, N.KV_BFP8, ws_ptr, ws_bytes, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        return out
+
+    expanded = run(ws.data_ptr(), need)
+    tiles = run(0, 0)
+    short = run(ws.data_ptr(), need - 1)
+    assert torch.equal(short, tiles)
+    torch.testing.assert_close(expanded.float(), tiles.float(), atol=1e-2, rtol=1e-2)
+    # the scratch holds what the pass read: the blocks of the first (start + lc) tokens of user 0, exact
+    cols = (start + lc + bs - 1) // bs
+    k_rt = C.unpack_cache(kp.cpu(), bs).to(torch.bfloat16)
+    copies = ws[: users * nbpu * hkv * bs * d * 2].view(torch.bfloat16).view(users, nbpu, hkv, bs, d).cpu()
+    for c in range(cols):
+        assert torch.equal(copies[0, c], k_rt[int(table[0, c])]), f"expanded copy of column {c} differs from the codec's decode"
+    assert torch.equal(copies[1, 2], k_rt[0]), "an entry out of range reads block 0"
 
 
 def test_backend_flow_on_a_bfp8_cache():

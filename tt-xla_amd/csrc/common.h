@@ -21,6 +21,8 @@ int device_cus();
 // Events armed by ttpa_profile_next_attention(); take_profile_events() hands them to the
 // launcher that times its dominant kernel and disarms them.
 void take_profile_events(hipEvent_t &before, hipEvent_t &after);
+// Arms events again from inside the library (a call of two launches hands `after` on to its second one).
+void arm_profile_events(void *before, void *after);
 
 // Launches a call's dominant kernel.  Armed events ride on the dispatch itself, so they read the
 // kernel's own begin and end timestamps (what a profiler reports for the dispatch) and not the
@@ -30,7 +32,7 @@ inline void launch_dominant(void (*kernel)(Params...), dim3 grid, dim3 block, si
                             Args... args) {
   hipEvent_t before, after;
   take_profile_events(before, after);
-  if (before)
+  if (before || after)
     hipExtLaunchKernelGGL(kernel, grid, block, static_cast<uint32_t>(lds), st, before, after, 0u, args...);
   else
     kernel<<<grid, block, lds, st>>>(args...);

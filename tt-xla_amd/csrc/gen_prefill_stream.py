@@ -483,7 +483,7 @@ def epilogue(o):
     for db in range(4):
         for jp in range(2):
             src = S[0] + 8 * db + 4 * jp
-            o.e(f"global_store_dwordx4 v[{OUTP}:{OUTP + 1}], v[{src}:{src + 3}], off offset:{64 * db + 32 * jp}")
+            o.e(f"global_store_dwordx4 v[{OUTP}:{OUTP + 1}], v[{src}:{src + 3}], off offset:{64 * db + 32 * jp} nt")   # written once, read by a later kernel
     o.e("s_mov_b64 exec, s[62:63]")
     o.e("s_nop 1")
 

@@ -71,7 +71,8 @@ struct PrefillArgs {
   int fill_groups, attn_per_fill, n_fill;
   int window;  // > 0 (causal only): row i attends keys offset + i - window < j <= offset + i
   float scale_log2e;
-  int kv_bfp8;  // paged form: the caches are block-float-8 (mode 4)
+  int kv_bfp8;  // paged form: the caches are block-float-8 (mode 4, or expanded into `expand` first)
+  void *expand; // scratch for bfloat16 copies of the block-float-8 blocks of this pass, or null
   int stream;   // the hand-scheduled loop serves this launch (head size 128, 4 heads per workgroup, whole blocks)
   int spg;      // ... with this many workgroups per (batch entry, head group), each taking several row blocks
   int spg_even; // > 0: when the row blocks weigh about the same, only this many of them work (equal shares)
@@ -154,7 +155,59 @@ __device__ __forceinline__ void fill_workgroup(const PrefillArgs &a, int f) {
     const int off = t - div_block(a, t) * a.bs;
     // (no early exit from the loop: the arrays must stay in registers)
     if (t < a.skv && (unsigned)phys[p] < (unsigned)a.nb)
-      *reinterpret_cast<u32x4 *>(cache + (((int64_t)phys[p] * a.hkv + h) * a.bs + off) * D + 8 * c) = val[p];
+      __builtin_nontemporal_store(val[p], reinterpret_cast<u32x4 *>(cache + (((int64_t)phys[p] * a.hkv + h) * a.bs + off) * D + 8 * c));
+  }
+}
+
+// Expansion of the block-float-8 blocks a chunk pass reads into bfloat16 copies, so that the
+// hand-scheduled loop (which wants bfloat16 blocks it can request straight into LDS) serves a
+// block-float-8 cache too: workgroup (x, y) expands the slab of table entry x = batch entry * width
+// + column and of (KV head, K or V) y into block x of a scratch cache, and writes entry x of the
+// identity table that goes with it.  Columns behind the last key of the pass are skipped.  Memory
+// work (1 byte in, 2 out per element) of about a tenth of the attention's time.
+struct ExpandArgs {
+  const uint8_t *kc, *vc;  // the block-float-8 caches
+  uint16_t *k, *v;         // scratch caches [batch * width][KV heads][block size][D]
+  int32_t *table;          // [batch][width]
+  const int32_t *pt;
+  int64_t pt_rs;
+  const int32_t *chunk_start;
+  int w, hkv, bs, nb, sq, causal;
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void bfp8_expand_kernel(ExpandArgs e) {
+  const int x = blockIdx.x, b = x / e.w, j = x - b * e.w;
+  const int h = blockIdx.y >> 1;
+  const bool is_v = blockIdx.y & 1;
+  if (blockIdx.y == 0 && threadIdx.x == 0) e.table[x] = x;
+  const int skv = e.w * e.bs;
+  const int kv_end = e.causal ? min(skv, (e.chunk_start ? e.chunk_start[0] : 0) + e.sq) : skv;
+  if (j * e.bs >= kv_end) return;
+  int phys = e.pt[(int64_t)b * e.pt_rs + j];
+  if ((unsigned)phys >= (unsigned)e.nb) phys = 0;  // (as the attention kernels treat a bad entry)
+  const int64_t slab = (int64_t)(e.bs + e.bs / 16) * D;
+  const uint8_t *src = (is_v ? e.vc : e.kc) + ((int64_t)phys * e.hkv + h) * slab;
+  const uint8_t *exps = src + (int64_t)e.bs * D;
+  uint16_t *dst = (is_v ? e.v : e.k) + ((int64_t)x * e.hkv + h) * e.bs * D;
+  const int groups = e.bs * D / 16;
+  for (int g = threadIdx.x; g < groups; g += 256) {
+    const u32x4 bytes = *reinterpret_cast<const u32x4 *>(src + 16 * g);
+    const float sc = bfp8_group_scale(exps[g]), off = -128.f * sc;
+    u32x4 lo, hi;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const uint32_t v = bytes[w];
+      const float f0 = fmaf((float)(v & 0xffu), sc, off), f1 = fmaf((float)((v >> 8) & 0xffu), sc, off);
+      const float f2 = fmaf((float)((v >> 16) & 0xffu), sc, off), f3 = fmaf((float)(v >> 24), sc, off);
+      // the products are exact in bfloat16: their upper halves are the elements
+      const uint32_t p0 = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f1), __builtin_bit_cast(uint32_t, f0), 0x07060302u);
+      const uint32_t p1 = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f3), __builtin_bit_cast(uint32_t, f2), 0x07060302u);
+      if (w < 2) lo[2 * w] = p0, lo[2 * w + 1] = p1;
+      else hi[2 * (w - 2)] = p0, hi[2 * (w - 2) + 1] = p1;
+    }
+    *reinterpret_cast<u32x4 *>(dst + 16 * g) = lo;
+    *reinterpret_cast<u32x4 *>(dst + 16 * g + 8) = hi;
   }
 }
 
@@ -937,9 +990,45 @@ int launch_rh(const PrefillArgs &a, hipStream_t st) {
   return launch_mode<D, HPW, 2, RH>(a, st);
 }
 
+// Bytes of the scratch an expanded block-float-8 pass needs: K and V copies of batch * width blocks
+// and their table.
+inline int64_t expand_bytes(int batch, int width, int kv_heads, int block_size, int d) {
+  const int64_t blocks = (int64_t)batch * width;
+  return 2 * blocks * kv_heads * block_size * d * 2 + ((blocks * 4 + 255) & ~int64_t(255));
+}
+
 template <int D, int HPW>
 int launch(const PrefillArgs &a, hipStream_t st) {
-  if (a.pt && a.kv_bfp8) return launch_mode<D, HPW, 4, 1>(a, st);
+  if (a.pt && a.kv_bfp8) {
+    // With scratch from the caller, a pass that the hand-scheduled loop can serve reads bfloat16
+    // copies of its blocks (written by one launch in front of it) instead of expanding every
+    // tile once per workgroup on its way into LDS.
+    constexpr bool kStreams = D == 128 && HPW == 4;
+    if (kStreams && a.expand && a.stream && a.window == 0 && a.mask == nullptr && a.bs % kKeysPerTile == 0) {
+      const int64_t blocks = (int64_t)a.batch * a.w;
+      const int64_t cache_elems = blocks * a.hkv * a.bs * D;
+      ExpandArgs e;
+      e.kc = reinterpret_cast<const uint8_t *>(a.k), e.vc = reinterpret_cast<const uint8_t *>(a.v);
+      e.k = static_cast<uint16_t *>(a.expand), e.v = e.k + cache_elems;
+      e.table = reinterpret_cast<int32_t *>(e.v + cache_elems);
+      e.pt = a.pt, e.pt_rs = a.pt_rs, e.chunk_start = a.chunk_start;
+      e.w = a.w, e.hkv = a.hkv, e.bs = a.bs, e.nb = a.nb, e.sq = a.sq, e.causal = a.causal;
+      // armed events: the pair brackets both launches
+      hipEvent_t before, after;
+      take_profile_events(before, after);
+      const dim3 grid((unsigned)blocks, (unsigned)(2 * a.hkv));
+      if (before)
+        hipExtLaunchKernelGGL(bfp8_expand_kernel<D>, grid, dim3(256), 0u, st, before, nullptr, 0u, e);
+      else
+        bfp8_expand_kernel<D><<<grid, dim3(256), 0, st>>>(e);
+      if (const int rc = check_launch("sdpa_prefill (block-float-8 expansion)")) return rc;
+      if (after) arm_profile_events(nullptr, after);
+      PrefillArgs b = a;
+      b.k = e.k, b.v = e.v, b.pt = e.table, b.pt_rs = a.w, b.nb = (int)blocks, b.kv_bfp8 = 0, b.expand = nullptr;
+      return launch_mode<D, HPW, 1, 1>(b, st);
+    }
+    return launch_mode<D, HPW, 4, 1>(a, st);
+  }
   return launch_rh<D, HPW, 1>(a, st);
 }
 
@@ -976,7 +1065,8 @@ static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_st
                                  int32_t kv_heads, int32_t q_len, int32_t kv_len, int32_t head_size,
                                  int32_t block_size, int32_t table_width, int32_t num_blocks,
                                  int32_t causal, float scale, int32_t sliding_window, void *stream,
-                                 const FillSpec *fill = nullptr, int32_t kv_format = TTPA_KV_BF16) {
+                                 const FillSpec *fill = nullptr, int32_t kv_format = TTPA_KV_BF16,
+                                 void *workspace = nullptr, int64_t workspace_bytes = 0) {
   TTPA_REQUIRE(out && q && k && v, "null pointer argument");
   TTPA_REQUIRE(sliding_window >= 0, "prefill: sliding_window %d is negative", sliding_window);
   TTPA_REQUIRE(sliding_window == 0 || causal, "prefill: a sliding window needs causal masking");
@@ -1028,10 +1118,16 @@ static int prefill_impl(void *out, int64_t out_batch_stride, int64_t out_head_st
   if (kv_format != TTPA_KV_BF16 && kv_format != TTPA_KV_BFP8)
     return fail(TTPA_ERR_INVALID_ARGUMENT, "prefill: unknown kv_format %d", kv_format);
   a.kv_bfp8 = kv_format == TTPA_KV_BFP8;
+  a.expand = nullptr;
   if (a.kv_bfp8) {
     TTPA_REQUIRE(page_table != nullptr, "prefill: a block-float-8 K / V is a paged cache");
     if (block_size % 16)
       return fail(TTPA_ERR_UNSUPPORTED, "prefill: a block-float-8 cache needs block_size %% 16 == 0");
+    TTPA_REQUIRE(workspace_bytes >= 0 && (workspace != nullptr || workspace_bytes == 0),
+                 "prefill: workspace_bytes %lld with a null workspace", (long long)workspace_bytes);
+    if (workspace && aligned16(workspace) && (int64_t)batch * table_width < (1ll << 31) &&
+        workspace_bytes >= expand_bytes(batch, table_width, kv_heads, block_size, head_size))
+      a.expand = workspace;  // (a smaller one is not an error: the pass expands tile by tile instead)
   }
   {
     // (TTPA_PREFILL_STREAM=0, read on every call, sends every shape through the plain loop)
@@ -1082,6 +1178,18 @@ extern "C" int ttpa_sdpa_prefill_windowed(TTPA_PREFILL_PARAMS, int32_t sliding_w
 extern "C" int ttpa_sdpa_prefill_format(TTPA_PREFILL_PARAMS, int32_t sliding_window, int32_t kv_format,
                                         void *stream) {
   return prefill_impl(TTPA_PREFILL_ARGS, sliding_window, stream, nullptr, kv_format);
+}
+
+extern "C" int ttpa_sdpa_prefill_expanded(TTPA_PREFILL_PARAMS, int32_t sliding_window, int32_t kv_format,
+                                          void *workspace, int64_t workspace_bytes, void *stream) {
+  return prefill_impl(TTPA_PREFILL_ARGS, sliding_window, stream, nullptr, kv_format, workspace, workspace_bytes);
+}
+
+extern "C" int64_t ttpa_sdpa_prefill_workspace_bytes(int32_t batch, int32_t kv_heads, int32_t head_size,
+                                                     int32_t block_size, int32_t table_width, int32_t kv_format) {
+  if (kv_format != TTPA_KV_BFP8 || batch <= 0 || kv_heads <= 0 || head_size <= 0 || block_size <= 0 || table_width <= 0)
+    return 0;
+  return expand_bytes(batch, table_width, kv_heads, block_size, head_size);
 }
 
 extern "C" int ttpa_sdpa_prefill_fill(

@@ -99,6 +99,12 @@ SIGNATURES = {
         [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _i64, _p, _p,
          _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _p],
     ),
+    "ttpa_sdpa_prefill_expanded": (
+        _int,
+        [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _i64, _p, _p,
+         _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _p, _i64, _p],
+    ),
+    "ttpa_sdpa_prefill_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32, _i32, _i32]),
     "ttpa_sdpa_prefill_fill": (
         _int,
         [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64,

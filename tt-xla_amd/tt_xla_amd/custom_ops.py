@@ -422,6 +422,10 @@ def _decode(query, key, value, page_table, is_causal, attn_mask, cur_pos_tensor,
 _WORKSPACES = {}
 
 
+# Largest scratch a block-float-8 chunk pass may ask for (bfloat16 copies of its users' blocks).
+_EXPANSION_LIMIT = 8 << 30
+
+
 def _workspace(nbytes: int, device) -> torch.Tensor:
     """A per-device scratch tensor for the split-K partials of a decode launch, grown on demand and
     reused by later calls: launches of one stream run in order, so one buffer serves them all, and
@@ -633,13 +637,21 @@ def _prefill(query, key, value, page_table, chunk_start, attn_mask, is_causal, s
         if m.stride(-1) != 1:
             m = m.contiguous()
         mask_ptr, mask_bs, mask_rs = m.data_ptr(), m.stride(0), m.stride(2)
+    # block-float-8 caches: scratch for bfloat16 copies of the blocks the pass reads (the library uses
+    # it for the shapes its fastest loop serves and ignores it otherwise)
+    ws_ptr, ws_bytes = 0, 0
+    if fmt == N.KV_BFP8 and d == 128 and (hq // hkv) % 4 == 0 and bs % 64 == 0 and not window and attn_mask is None:
+        need = int(N.lib().ttpa_sdpa_prefill_workspace_bytes(b, hkv, d, bs, w, fmt))
+        if 0 < need <= _EXPANSION_LIMIT:
+            ws = _workspace(need, q.device)
+            ws_ptr, ws_bytes = ws.data_ptr(), need
     N.call(
-        "ttpa_sdpa_prefill_format",
+        "ttpa_sdpa_prefill_expanded",
         out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
         q.data_ptr(), q.stride(0), q.stride(1), q.stride(2),
         k.data_ptr(), v.data_ptr(), *kv_strides, pt_ptr, pt_rs, _ptr(chunk_start),
         mask_ptr, mask_bs, mask_rs, b, hq, hkv, s, skv, d, bs, w, nb, int(is_causal),
-        float(scale), int(window), fmt, _stream(),
+        float(scale), int(window), fmt, ws_ptr, ws_bytes, _stream(),
     )
     return out
 
