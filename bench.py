@@ -44,6 +44,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 KERNEL_SOURCES = {
     "paged_decode_mfma16_kernel": ["decode_mfma16_kernel.h", "decode_common.h", "common.h", "decode.hip"],  # the grid rule is in decode.hip
     "paged_decode_latent16_kernel": ["decode_wide.hip", "decode_common.h", "common.h"],
+    "paged_decode_latent128_kernel": ["decode_wide.hip", "decode_common.h", "common.h"],
+    "latent_prefill_kernel": ["decode_wide.hip", "decode_common.h", "common.h"],
     "prefill_kernel": ["prefill.hip", "gen_prefill_stream.py", "common.h"],
 }
 MEASURED_TRAFFIC = {
@@ -91,7 +93,7 @@ def parse():
                     help="consecutive steps captured in one graph: a decode forward replays one "
                          "attention step per layer inside one graph, and Llama-3-8B has 32 layers; "
                          "1 = one graph launch per step")
-    ap.add_argument("--workload", choices=["config2", "config3", "config4", "config5", "latent"], default="config2")
+    ap.add_argument("--workload", choices=["config2", "config3", "config4", "config5", "latent", "latent128", "latent-prefill"], default="config2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true",
                     help="config2 only: leave out the short config3 / config5 runs reported under 'secondary'")
@@ -490,15 +492,17 @@ def run_decode(args):
     return out
 
 
-def run_latent(args):
+def run_latent(args, hq=16):
     """Latent (MLA) decode at the shape one rank of a latent-attention model serves: 16 query heads
     over one latent KV head of 576 = 512 + 64 features, V = its 512 leading features; 128 users,
     contexts uniform in [512, 8192], block 64.  The step is tt::paged_flash_mla_decode (attention +
     merge of the split-K partials); the cache write of the step is the plain tt::paged_update_cache
-    on the latent cache and is not part of it."""
+    on the latent cache and is not part of it.  hq = 128 is the layer with all of its heads on one
+    GPU: 242 flop per byte of the cache, so the matrix pipes bound it and not the memory; the
+    figure stays in bytes per second so that the two shapes read on one scale."""
     import torch
 
-    users, hq, dh, dv, bs, lo, hi = 128, 16, 576, 512, 64, 512, 8192
+    users, dh, dv, bs, lo, hi = 128, 576, 512, 64, 512, 8192
     dev = "cuda:0"
     copies = []
     for i in range(max(1, min(args.rotate, 2))):
@@ -521,7 +525,8 @@ def run_latent(args):
     kern_ms = sum(d for d, _ in durs) / len(durs)
     kern_bytes = sum(nbytes[w] for _, w in durs) / len(durs)
     achieved = kern_bytes / (kern_ms * 1e-3) / 1e9
-    kernel = "paged_decode_latent16_kernel"
+    kernel = "paged_decode_latent16_kernel" if hq <= 16 else "paged_decode_latent128_kernel"
+    flops = 2.0 * kern_bytes / (dh * 2) * hq * (dh + dv)
     return {
         "metric": "paged_decode_attention_hbm_throughput",
         "value": avg_bytes / (ms * 1e-3) / 1e9, "unit": "GB/s",
@@ -540,10 +545,60 @@ def run_latent(args):
         "pct_of_hbm_peak": 100.0 * avg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "roofline": {
             "kernel": kernel, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic("latent", kernel),
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic("latent" if hq <= 16 else "latent128", kernel),
             "kernel_source_hash": kernel_source_hash(kernel),
             "kernel_us": kern_ms * 1e3, "kernel_us_min": min(d for d, _ in durs) * 1e3,
             "bytes_per_launch": kern_bytes, "timed_launches": len(durs),
+            "tflops": flops / (kern_ms * 1e-3) / 1e12,
+            "frac_of_bf16_mfma_peak": flops / (kern_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+        },
+    }
+
+
+def run_latent_prefill(args):
+    """tt::flash_mla_prefill at the latent serving shape: 4 prompts of 2048 tokens, 16 query heads
+    over one latent head of 576 features, V = its 512 leading ones, causal.  Useful flops:
+    2 (576 + 512) per (row, key <= row) pair."""
+    import torch
+
+    b, hq, s, dh, dv = 4, 16, 2048, 576, 512
+    dev = "cuda:0"
+    copies = []
+    for i in range(max(1, min(args.rotate, 2))):
+        g = torch.Generator().manual_seed(21 + i)
+        q = (torch.randn(b, hq, s, dh, generator=g) * 0.15).to(torch.bfloat16).to(dev)
+        k = torch.randn(b, 1, s, dh, generator=g).to(torch.bfloat16).to(dev)
+        copies.append((q, k))
+    fns = [(lambda c=c: torch.ops.tt.flash_mla_prefill(c[0], c[1], dv, None, None, True, dh ** -0.5)) for c in copies]
+    runner = StepRunner(fns, args.launch == "graph", args.steps_per_graph)
+    steps = min(args.steps, 100)
+    ms, ms_min, ms_max = time_steps_spread(runner, steps, min(args.warmup, 10))
+    flops = 2.0 * b * hq * (s * (s + 1) / 2) * (dh + dv)
+    durs = time_dominant_kernel(fns, min(steps, 50))
+    kern_ms = sum(d for d, _ in durs) / len(durs)
+    achieved = flops / (kern_ms * 1e-3) / 1e12
+    return {
+        "metric": "latent_prefill_attention_useful_tflops",
+        "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": steps, "warmup": min(args.warmup, 10), "ms_per_step": ms,
+        "ms_per_step_min": ms_min, "ms_per_step_max": ms_max, "timed_blocks": TIMED_BLOCKS,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "workload": f"latent-prefill-b{b}x{s}-h{hq}x1-d{dh}/{dv}",
+            "step": "causal latent prefill attention over freshly built latent K (V = its leading features), one launch",
+            "launch": args.launch, "steps_per_graph": runner.per_graph if args.launch == "graph" else None,
+            "rotating_copies": len(copies), "users": b, "tokens_per_user": s, "q_heads": hq, "kv_heads": 1,
+            "head_size": dh, "head_dim_v": dv,
+        },
+        "tokens_per_s": b * s / (ms * 1e-3),
+        "roofline": {
+            "kernel": "latent_prefill_kernel", "bound": "mfma", "achieved": achieved,
+            "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+            "traffic": measured_traffic("latent-prefill", "latent_prefill_kernel"),
+            "kernel_source_hash": kernel_source_hash("latent_prefill_kernel"),
+            "kernel_us": kern_ms * 1e3, "kernel_us_min": min(d for d, _ in durs) * 1e3,
+            "flops_per_launch": flops, "timed_launches": len(durs),
         },
     }
 
@@ -598,6 +653,18 @@ def run_prefill(args):
     }
 
 
+def run_workload(args):
+    if args.workload == "config3":
+        return run_prefill(args)
+    if args.workload == "latent":
+        return run_latent(args)
+    if args.workload == "latent128":
+        return run_latent(args, hq=128)
+    if args.workload == "latent-prefill":
+        return run_latent_prefill(args)
+    return run_decode(args)
+
+
 def secondary_runs(args):
     """Short runs of the other workloads (config3 prefill, config5 block-float-8 decode, config4
     large decode with its chunked-prefill pass, latent decode) in the headline's process, so that
@@ -609,14 +676,15 @@ def secondary_runs(args):
     import torch
 
     out = {}
-    for wl, steps, warmup in (("config3", 96, 8), ("config5", 96, 12), ("config4", 32, 4), ("latent", 96, 8)):
+    for wl, steps, warmup in (("config3", 96, 8), ("config5", 96, 12), ("config4", 32, 4), ("latent", 96, 8),
+                              ("latent128", 32, 4), ("latent-prefill", 32, 4)):
         gc.collect()
         torch.cuda.empty_cache()
         sub = copy.copy(args)
         sub.workload, sub.steps, sub.warmup = wl, steps, warmup
         if wl == "config4":
             sub.rotate = 1  # one copy of the 128-user pool is already far beyond the caches
-        r = run_prefill(sub) if wl == "config3" else (run_latent(sub) if wl == "latent" else run_decode(sub))
+        r = run_workload(sub)
         keep = {k: r[k] for k in ("metric", "value", "unit", "steps", "warmup", "ms_per_step", "ms_per_step_min",
                                   "ms_per_step_max", "dtype", "roofline")}
         keep["workload"] = r["config"]["workload"]
@@ -650,8 +718,8 @@ def main():
         out = run_prefill(args)
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_prefill_baseline(args)
-    elif args.workload == "latent":
-        out = run_latent(args)  # (no CPU leg: the headline workload carries it)
+    elif args.workload.startswith("latent"):
+        out = run_workload(args)  # (no CPU leg: the headline workload carries it)
     else:
         out = run_decode(args)
         if args.workload == "config2" and not args.no_secondary:

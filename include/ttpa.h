@@ -450,6 +450,28 @@ int ttpa_bfp8_quantize(const void *src_bf16, void *elem_u8, void *exps_u8, int64
 int ttpa_bfp8_dequantize(const void *elem_u8, const void *exps_u8, void *dst_bf16,
                          int64_t n_elems, void *stream);
 
+/*
+ * tt::flash_mla_prefill with V taken from K (reference python_package/tt_torch/custom_ops.py:223-378,
+ * the form the latent backend calls: integrations/vllm_plugin/vllm_tt/attention_impls/
+ * attention_mla.py:302-330): out[b, h, i, :] = softmax_j(scale * q[b, h, i] . k[b, h / G, j] + mask)
+ * . k[b, h / G, j, :head_dim_v] over the keys j <= i (causal) or over all keys with an additive
+ * bfloat16 mask [batch, 1 or q_heads, seq_len, seq_len] (mask_head_stride 0 shares one mask between
+ * the heads; causal and mask exclude each other, as in the reference's asserts).  q [batch, q_heads,
+ * seq_len, head_size], k [batch, kv_heads, seq_len, head_size], out [batch, q_heads, seq_len,
+ * head_dim_v], all bfloat16 with explicit element strides (innermost dimension contiguous).  One
+ * launch of a matrix-instruction kernel in which 128 (token, head) rows share every K tile; built
+ * for (head_size, head_dim_v) = (576, 512), (192, 128), (128, 128), anything else returns
+ * TTPA_ERR_UNSUPPORTED.
+ */
+int ttpa_latent_prefill(void *out, int64_t out_batch_stride, int64_t out_head_stride,
+                        int64_t out_token_stride, const void *q, int64_t q_batch_stride,
+                        int64_t q_head_stride, int64_t q_token_stride, const void *k,
+                        int64_t k_batch_stride, int64_t k_head_stride, int64_t k_token_stride,
+                        const void *mask, int64_t mask_batch_stride, int64_t mask_head_stride,
+                        int64_t mask_row_stride, int32_t batch, int32_t q_heads, int32_t kv_heads,
+                        int32_t seq_len, int32_t head_size, int32_t head_dim_v, int32_t causal,
+                        float scale, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -44,6 +44,10 @@ DECODE = [
     (3, 128, 1, 576, 512, False, 64, 12, None),   # all 128 heads: four head blocks per user
     (2, 64, 2, 192, 128, False, 16, 40, 0.11),
     (3, 16, 1, 576, 384, False, 32, 12, None),    # a value width that is not a power of two (merge kernel)
+    (2, 48, 1, 192, 128, False, 32, 6, 0.2),      # three of the eight wavefronts of the 128-head form have heads
+    (2, 40, 2, 128, 128, False, 16, 20, 0.2),     # 20 heads per KV head: a wavefront with four heads
+    (2, 256, 1, 576, 512, False, 64, 6, None),    # two segments of 128 heads per user
+    (6, 128, 1, 576, 384, False, 128, 5, None),   # blocks of two tiles
 ]
 
 
@@ -90,6 +94,37 @@ def test_mla_decode_16_heads_either_partial_format(monkeypatch, partials, dv):
     _check(f"mla decode partials={partials} dv{dv}", got, want)
 
 
+@pytest.mark.parametrize("kernel,partials", [("", "bf16"), ("", "f32"), ("wide", "f32")])
+def test_mla_decode_128_heads_every_form(monkeypatch, kernel, partials):
+    """All 128 heads of a latent layer on one GPU: the form in which eight wavefronts of a workgroup take
+    16 heads each on shared K tiles, with bfloat16 and with float partials, and the older form it
+    replaced (TTPA_LATENT_KERNEL=wide: blocks of 32 heads, every score computed four times), which still
+    serves masks and a separate V.  Contexts from one token to several tiles per workgroup range."""
+    monkeypatch.setenv("TTPA_LATENT_PARTIALS", partials)
+    if kernel:
+        monkeypatch.setenv("TTPA_LATENT_KERNEL", kernel)
+    else:
+        monkeypatch.delenv("TTPA_LATENT_KERNEL", raising=False)
+    users, hq, dh, dv, bs, width = 6, 128, 576, 512, 64, 400
+    print(f"case: mla decode 128 heads kernel={kernel or 'default'} partials={partials}", flush=True)
+    g = torch.Generator().manual_seed(4242)
+    pos = torch.tensor([0, 63, 64, 1000, 25599, 12345], dtype=torch.int32)
+    blocks = [int(p) // bs + 1 for p in pos]
+    nb = sum(blocks) + 1
+    q = _bf(g, 1, users, hq, dh)
+    key = _bf(g, nb, 1, bs, dh)
+    table = torch.zeros(users, width, dtype=torch.int32)
+    perm = (torch.randperm(nb - 1, generator=g) + 1).to(torch.int32)
+    at = 0
+    for u, nblk in enumerate(blocks):
+        table[u, :nblk] = perm[at : at + nblk]
+        at += nblk
+    got = torch.ops.tt.paged_flash_mla_decode(q.cuda(), key.cuda(), dv, table.cuda(), None, True, None,
+                                              pos.cuda(), None, None).cpu()
+    want = O.paged_flash_mla_decode(q, key, dv, table, None, pos, None)
+    _check(f"mla decode 128 heads kernel={kernel or 'default'} partials={partials}", got, want)
+
+
 def test_mla_decode_padded_row_sink_and_errors():
     g = torch.Generator().manual_seed(3)
     users, hq, dh, dv, bs, width = 3, 16, 576, 512, 32, 8
@@ -121,7 +156,12 @@ PREFILL = [
     (1, 32, 64, 128, 1, 128, False),
     (1, 16, 64, 128, 1, 64, True),
     (2, 16, 256, 576, 1, 512, False),  # latent serving shape
-    (1, 8, 1184, 192, 1, 128, False),  # more query rows than one launch takes
+    (1, 8, 1184, 192, 1, 128, False),  # more query rows than one launch of the decode kernels takes
+    (1, 16, 2048, 576, 1, 512, False), # a full prompt at the latent serving shape
+    (1, 128, 64, 576, 1, 512, False),  # the unsharded layer: 128 heads, a workgroup per token
+    (1, 12, 96, 192, 1, 128, False),   # 12 heads: a wavefront's 16 rows straddle two tokens
+    (2, 8, 160, 128, 2, 128, False),   # two KV heads, a last row block of 4 heads x 8 tokens short of 128 rows
+    (1, 4, 32, 576, 1, 512, False),    # 128 rows in all: one workgroup
 ]
 
 
@@ -146,6 +186,7 @@ MASKED_PREFILL = [
     (1, 32, 64, 128, 1, 128, False),
     (2, 16, 128, 128, 1, 64, True),
     (1, 16, 96, 576, 1, 512, False),   # latent serving shape
+    (1, 12, 160, 192, 1, 128, False),  # rows of two tokens in one wavefront, each with its own mask row
 ]
 
 

@@ -609,6 +609,493 @@ bool launch_latent16(const DecodeArgs &a, const WideArgs &w, hipStream_t st) {
   return true;
 }
 
+// ---------------------------------------------------------------------------------------------
+// More than 16 query heads per KV head with V taken from K (the latent layer with all of its 128
+// heads on one GPU): a segment is a block of up to 128 heads, a range of the flat list of 64-token
+// tiles belongs to a workgroup of eight wavefronts, and wavefront i computes heads 16 i .. 16 i + 15
+// exactly as the 16-head form does, on K tiles that the eight share in LDS (four 16-row pieces laid
+// out like that form's stages, one eighth of the requests per wavefront, two stages, one barrier per
+// tile).  Nothing is computed twice and a latent row is read from memory once per 128 heads; the
+// workgroup-shared form above re-reads it per block of 32 heads and computes every score four times.
+template <int DQK, int DV>
+__global__ __launch_bounds__(512) void paged_decode_latent128_kernel(
+    DecodeArgs a, WideArgs w, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
+  using L = Latent16<DQK, DV>;
+  typedef float floatx4 __attribute__((ext_vector_type(4)));
+  constexpr int SUB = L::TILE, NSUB = kTile / SUB, NWAVES = 8;
+  constexpr int KSTEPS = DQK / 32, VB = DV / 16;
+  constexpr int PER_WAVE = NSUB * L::NDMA / NWAVES;
+  static_assert(NSUB == 4 && 2 * PER_WAVE == L::NDMA, "two wavefronts request each 16-row piece");
+  constexpr int STAGE = NSUB * L::STAGE;
+
+  __shared__ int s_pref[kMaxUsersWide + 1];
+  __shared__ int s_len[kMaxUsersWide];
+  __shared__ int s_wsum[NWAVES];
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  build_prefix(a, cur_pos, s_pref, s_len, s_wsum);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n = lane & 15, quad = lane >> 4;
+  const int wg = blockIdx.x;
+  const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
+  const int64_t total = (int64_t)total_tiles * a.hkv;
+  const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);  // workgroups that get work
+  if (total == 0 || wg >= n_eff) {
+    publish_segment_row(a, s_pref, total, n_eff);
+    return;
+  }
+  int64_t x = (int64_t)wg * total / n_eff;
+  const int64_t x_hi = (int64_t)(wg + 1) * total / n_eff;
+  const int G = w.gseg;
+  const int hg = 16 * wave + n;  // this lane's head inside the segment
+
+  // ---- tile requests: wavefronts 2 i and 2 i + 1 fetch piece i (16 consecutive cache rows) -----
+  const int sub_w = wave >> 1;
+  uint32_t src_off[PER_WAVE];
+#pragma unroll
+  for (int j = 0; j < PER_WAVE; ++j) {
+    const int kk = (wave & 1) * PER_WAVE + j;
+    const int P = 64 * kk + lane, rr = P / L::CPR, p = P % L::CPR;
+    src_off[j] = (uint32_t)(rr * L::ROW + 16 * L::position(rr, p));
+  }
+  const uint32_t lds0 = lds_address(smem);
+  auto issue_tile = [&](const Cursor &cu, int buf) {
+    const int kvh = cu.h / w.nhb;
+    const int tok0 = cu.t * kTile + SUB * sub_w;
+    const int col = tok0 / a.bs;
+    int phys = (col < a.w) ? page_table[(int64_t)cu.u * a.pt_rs + col] : 0;
+    if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
+    const int64_t row0 = ((int64_t)phys * w.nkv + kvh) * a.bs + (tok0 - col * a.bs);
+    const uint64_t addr = reinterpret_cast<uint64_t>(a.k) + (uint64_t)row0 * L::ROW;
+    const char *src = reinterpret_cast<const char *>(address_from_words(
+        __builtin_amdgcn_readfirstlane((int)(uint32_t)addr), __builtin_amdgcn_readfirstlane((int)(uint32_t)(addr >> 32))));
+    const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(
+        (int)(lds0 + (uint32_t)(buf * STAGE + sub_w * L::STAGE + 1024 * (wave & 1) * PER_WAVE)));
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j) dma16_streaming(src, src_off[j], dst + 1024u * j);
+  };
+  // Rows past the attended length may be cache rows nobody ever wrote: their scores are masked,
+  // but as V rows they would turn 0 * Inf into NaN, so they are cleared in LDS.
+  auto clear_unattended_rows = [&](int buf, int nvalid) {
+    for (int r = nvalid + wave; r < kTile; r += NWAVES) {
+      uint4 *row = reinterpret_cast<uint4 *>(smem + buf * STAGE + (r / SUB) * L::STAGE + (r % SUB) * L::ROW);
+      for (int c = lane; c < L::ROW / 16; c += 64) row[c] = make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto load_q = [&](const Cursor &cu, bf16x8 (&qf)[KSTEPS]) {
+    const uint16_t *qp = a.q + cu.u * a.q_us + (int64_t)(cu.h * G + min(hg, G - 1)) * a.q_hs + 8 * quad;
+    const uint32_t qmask = hg < G ? 0xffffffffu : 0u;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      uint4 t = *reinterpret_cast<const uint4 *>(qp + 32 * s);
+      t.x &= qmask, t.y &= qmask, t.z &= qmask, t.w &= qmask;
+      qf[s] = __builtin_bit_cast(bf16x8, t);
+    }
+  };
+
+  // ---- fragment addresses inside a 16-row piece (as in the 16-head form) -----------------------
+  constexpr int GC = L::HALF_PERIOD ? 8 : 16;
+  constexpr int KB = GC / 4, VBASES = GC / 2;
+  uint32_t kfrag[KB], vfrag[VBASES];
+#pragma unroll
+  for (int i = 0; i < KB; ++i) kfrag[i] = (uint32_t)(n * L::ROW + 16 * L::position(n, 4 * i + quad));
+  {
+    const int rv = 4 * quad + (n >> 2), q4 = n & 3;
+#pragma unroll
+    for (int i = 0; i < VBASES; ++i)
+      vfrag[i] = (uint32_t)(rv * L::ROW + 16 * L::position(rv, 2 * i + (q4 >> 1)) + 8 * (q4 & 1));
+  }
+  auto read_k = [&](const unsigned char *piece, int s) {
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(piece + kfrag[s % KB] + 16 * GC * (s / KB)));
+  };
+  auto read_v = [&](const unsigned char *piece, int vb) {
+    typedef __attribute__((address_space(3))) shortx4 *lds_v4;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(piece + vfrag[vb % VBASES] + 16 * GC * (vb / VBASES)));
+  };
+  constexpr int KPRE = KSTEPS < 4 ? KSTEPS : 4;
+  constexpr int VPRE = VB < 6 ? VB : 6;
+
+  Cursor cur = locate_unit(a, s_pref, s_len, x);
+  bf16x8 qf[KSTEPS];
+  issue_tile(cur, 0);
+  load_q(cur, qf);
+  publish_segment_row(a, s_pref, total, n_eff);
+
+  floatx4 acc[VB];
+#pragma unroll
+  for (int i = 0; i < VB; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+  const float scale = a.scale_log2e;
+  const bool wave_active = 16 * wave < G;
+
+  for (int it = 0; x < x_hi; ++x, ++it) {
+    const int buf = it & 1;
+    const int nvalid = cur.len - cur.t * kTile;
+    const bool partial = nvalid < kTile;
+    const int nbelow = cur.lo - cur.t * kTile;  // sliding window: > 0 only in a segment's first tile
+    const bool has_next = x + 1 < x_hi;
+    const bool same_seg = has_next && cur.tiles_left > 1;
+
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's share of the tile has landed
+    __syncthreads();                     // the tile is complete; everybody has left the other stage
+    Cursor nxt = cur;
+    if (has_next) {
+      if (same_seg) {
+        nxt.t = cur.t + 1;
+        nxt.tiles_left = cur.tiles_left - 1;
+      } else {
+        nxt = locate_unit(a, s_pref, s_len, x + 1);
+      }
+      issue_tile(nxt, buf ^ 1);
+    }
+    if (partial) {
+      clear_unattended_rows(buf, max(nvalid, 0));
+      __syncthreads();
+    }
+    if (wave_active) {
+#pragma unroll 1
+      for (int sub = 0; sub < NSUB; ++sub) {
+        if (SUB * sub >= nvalid) break;
+        const unsigned char *piece = smem + buf * STAGE + sub * L::STAGE;
+        // ---- S^T = K . Q^T -------------------------------------------------------------------
+        floatx4 st = {0.f, 0.f, 0.f, 0.f};
+        {
+          bf16x8 ring[KPRE];
+#pragma unroll
+          for (int s = 0; s < KPRE; ++s) ring[s] = read_k(piece, s);
+#pragma unroll
+          for (int s = 0; s < KSTEPS; ++s) {
+            st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % KPRE], qf[s], st, 0, 0, 0);
+            if (s + KPRE < KSTEPS) ring[s % KPRE] = read_k(piece, s + KPRE);
+          }
+#pragma unroll
+          for (int s = 0; s < KSTEPS; ++s) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (s + KPRE < KSTEPS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+        }
+        // ---- online softmax: lane (head, quad) holds keys 16 sub + 4 quad + r ---------------------
+        float sc[4], mloc = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int key = SUB * sub + 4 * quad + r;
+          sc[r] = (key >= nvalid || key < nbelow) ? -INFINITY : st[r] * scale;
+          mloc = fmaxf(mloc, sc[r]);
+        }
+        mloc = max_over_quads(mloc);
+        const bool move = !(mloc - m_run <= 8.0f);  // (lazy: also true from -inf)
+        const float m_new = move ? mloc : m_run;
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = move ? __builtin_amdgcn_exp2f(m_run - m_safe) : 1.0f;
+        m_run = m_new;
+        float lsum = 0.f;
+        shortx4 pf;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float p = __builtin_amdgcn_exp2f(sc[r] - m_safe);
+          const __bf16 pb = (__bf16)p;
+          lsum += (float)pb;  // the normaliser sums the weights that multiply V
+          pf[r] = __builtin_bit_cast(short, pb);
+        }
+        l_run = l_run * alpha + lsum;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+          for (int i = 0; i < VB; ++i) acc[i] *= alpha;
+        }
+        // ---- O^T += V^T . P^T -------------------------------------------------------------------
+        {
+          shortx4 vring[VPRE];
+#pragma unroll
+          for (int vb = 0; vb < VPRE; ++vb) vring[vb] = read_v(piece, vb);
+#pragma unroll
+          for (int vb = 0; vb < VB; ++vb) {
+            acc[vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vring[vb % VPRE], pf, acc[vb], 0, 0, 0);
+            if (vb + VPRE < VB) vring[vb % VPRE] = read_v(piece, vb + VPRE);
+          }
+#pragma unroll
+          for (int vb = 0; vb < VB; ++vb) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (vb + VPRE < VB) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+        }
+      }
+    }
+    // ---- close the segment: every wavefront writes its heads' part of the partial -----------------
+    if (!same_seg) {
+      float *slot = a.ws_slots + ((int64_t)wg + (int64_t)cur.u * a.hkv + cur.h) * a.slot_floats;
+      const float l_tot = sum_over_quads(l_run);
+      if (hg < G) {
+        if (a.partial_bf16) {  // wavefront-uniform
+          uint32_t *dst = reinterpret_cast<uint32_t *>(slot) + (hg * DV + 4 * quad) / 2;
+#pragma unroll
+          for (int vb = 0; vb < VB; ++vb)
+            *reinterpret_cast<uint2 *>(dst + 8 * vb) =
+                make_uint2(pack_bf16x2(acc[vb][0], acc[vb][1]), pack_bf16x2(acc[vb][2], acc[vb][3]));
+          if (quad == 0) {
+            slot[G * DV / 2 + hg] = m_run;
+            slot[G * DV / 2 + G + hg] = l_tot;
+          }
+        } else {
+          float *dst = slot + hg * DV + 4 * quad;
+#pragma unroll
+          for (int vb = 0; vb < VB; ++vb)
+            *reinterpret_cast<float4 *>(dst + 16 * vb) = make_float4(acc[vb][0], acc[vb][1], acc[vb][2], acc[vb][3]);
+          if (quad == 0) {
+            slot[G * DV + hg] = m_run;
+            slot[G * DV + G + hg] = l_tot;
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < VB; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+      m_run = -INFINITY;
+      l_run = 0.f;
+      if (has_next) load_q(nxt, qf);
+    }
+    cur = nxt;
+  }
+}
+
+template <int DQK, int DV>
+bool launch_latent128(const DecodeArgs &a, const WideArgs &w, hipStream_t st) {
+  using L = Latent16<DQK, DV>;
+  const size_t lds = 2 * 4 * (size_t)L::STAGE;
+  static std::atomic<uint64_t> lds_ready{0};
+  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_latent128_kernel<DQK, DV>), lds, lds_ready))
+    return false;
+  launch_dominant(&paged_decode_latent128_kernel<DQK, DV>, dim3(a.n_waves), dim3(512), lds, st, a, w, a.pt, a.cur);
+  return true;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Prefill over freshly built latent K with V taken from K: the rows of a (batch entry, KV head) are
+// its (token, head) pairs, token-major, and a workgroup of eight wavefronts owns 128 consecutive ones
+// (eight tokens of a 16-head group, one token of a 128-head group), 16 per wavefront in the N
+// dimension of the products of the 16-head decode form above.  The eight wavefronts share every K
+// tile of 64 keys in LDS (four 16-row pieces, each laid out and swizzled like a stage of that form,
+// requested by LDS-DMA, one eighth per wavefront), so a K row is read from memory once per 128 rows
+// and not once per row; two stages, one barrier per tile.  Every lane keeps the causal limit of its
+// own row; a wavefront leaves out the 16-key pieces behind the limit of its last row.
+struct LatentPrefillArgs {
+  uint16_t *out;
+  int64_t out_bs, out_hs, out_ts;
+  const uint16_t *q;
+  int64_t q_bs, q_hs, q_ts;
+  const uint16_t *k;
+  int64_t k_bs, k_hs, k_ts;
+  const uint16_t *mask;  // additive, [batch, 1 or heads, s, s], or null
+  int64_t mask_bs, mask_hs, mask_rs;
+  int batch, heads, nkv, s, causal;
+  float scale_log2e;
+};
+
+template <int DQK, int DV>
+__global__ __launch_bounds__(512) void latent_prefill_kernel(LatentPrefillArgs a) {
+  using L = Latent16<DQK, DV>;
+  typedef float floatx4 __attribute__((ext_vector_type(4)));
+  constexpr int SUB = L::TILE, NSUB = 4, KEYS = SUB * NSUB, NWAVES = 8, ROWS = 16 * NWAVES;
+  constexpr int KSTEPS = DQK / 32, VB = DV / 16;
+  constexpr int PER_WAVE = NSUB * L::NDMA / NWAVES;
+  static_assert(NSUB * L::NDMA % NWAVES == 0, "a tile's requests must divide among the wavefronts");
+  constexpr int STAGE = NSUB * L::STAGE;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n = lane & 15, quad = lane >> 4;
+  const int G = a.heads / a.nkv;
+  const int rows_total = G * a.s;
+  const int nblk = (rows_total + ROWS - 1) / ROWS;
+  const int groups = a.batch * a.nkv;
+  // late (heavy) row blocks first; neighbouring workgroups take the same block of different groups
+  const int blk = nblk - 1 - (int)blockIdx.x / groups;
+  const int grp = (int)blockIdx.x % groups;
+  const int b = grp / a.nkv, kvh = grp - b * a.nkv;
+
+  const int r0 = blk * ROWS + wave * 16;
+  const bool wave_active = r0 < rows_total;
+  const int r = min(r0 + n, rows_total - 1);
+  const int t = r / G, head = kvh * G + (r - t * G);
+  const bool row_valid = r0 + n < rows_total;
+  const int limit = a.causal ? t : a.s - 1;
+  const int wave_limit = a.causal ? min(r0 + 15, rows_total - 1) / G : a.s - 1;
+  const int wg_limit = a.causal ? min(blk * ROWS + ROWS - 1, rows_total - 1) / G : a.s - 1;
+  const int ntiles = wg_limit / KEYS + 1;
+
+  // ---- tile requests: instruction k = wave * PER_WAVE + j of the tile's NSUB * NDMA -----------
+  const uint16_t *kbase_g = a.k + b * a.k_bs + kvh * a.k_hs;
+  const uint32_t row_bytes = 2u * (uint32_t)a.k_ts;
+  int req_row[PER_WAVE];
+  uint32_t req_chunk[PER_WAVE];
+#pragma unroll
+  for (int j = 0; j < PER_WAVE; ++j) {
+    const int k = wave * PER_WAVE + j, sub = k / L::NDMA, kk = k % L::NDMA;
+    const int P = 64 * kk + lane, rr = P / L::CPR, p = P % L::CPR;
+    req_row[j] = SUB * sub + rr;
+    req_chunk[j] = 16u * (uint32_t)L::position(rr, p);
+  }
+  const uint32_t lds0 = lds_address(smem);
+  auto request_tile = [&](int tile, int buf) {
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j) {
+      const int k = wave * PER_WAVE + j;
+      const int key = min(tile * KEYS + req_row[j], a.s - 1);  // rows past the end repeat the last one
+      dma16(kbase_g, (uint32_t)key * row_bytes + req_chunk[j],
+            (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)(buf * STAGE + 1024 * k))));
+    }
+  };
+
+  // ---- fragment addresses inside a 16-row piece (as in the 16-head decode form) ----------------
+  constexpr int GC = L::HALF_PERIOD ? 8 : 16;
+  constexpr int KB = GC / 4, VBASES = GC / 2;
+  uint32_t kfrag[KB], vfrag[VBASES];
+#pragma unroll
+  for (int i = 0; i < KB; ++i) kfrag[i] = (uint32_t)(n * L::ROW + 16 * L::position(n, 4 * i + quad));
+  {
+    const int rv = 4 * quad + (n >> 2), q4 = n & 3;
+#pragma unroll
+    for (int i = 0; i < VBASES; ++i)
+      vfrag[i] = (uint32_t)(rv * L::ROW + 16 * L::position(rv, 2 * i + (q4 >> 1)) + 8 * (q4 & 1));
+  }
+  auto read_k = [&](const unsigned char *piece, int s) {
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(piece + kfrag[s % KB] + 16 * GC * (s / KB)));
+  };
+  auto read_v = [&](const unsigned char *piece, int vb) {
+    typedef __attribute__((address_space(3))) shortx4 *lds_v4;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(piece + vfrag[vb % VBASES] + 16 * GC * (vb / VBASES)));
+  };
+  constexpr int KPRE = KSTEPS < 4 ? KSTEPS : 4;
+  constexpr int VPRE = VB < 6 ? VB : 6;
+
+  request_tile(0, 0);
+  // B operand of the score product: lane (row, quad) holds features 32 s + 8 quad .. + 7 of its row
+  bf16x8 qf[KSTEPS];
+  {
+    const uint16_t *qp = a.q + b * a.q_bs + head * a.q_hs + (int64_t)t * a.q_ts + 8 * quad;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) qf[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 32 * s));
+  }
+  const uint16_t *mrow = a.mask ? a.mask + b * a.mask_bs + head * a.mask_hs + (int64_t)t * a.mask_rs : nullptr;
+
+  floatx4 acc[VB];
+#pragma unroll
+  for (int i = 0; i < VB; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+  const float scale = a.scale_log2e;
+
+  for (int tile = 0; tile < ntiles; ++tile) {
+    const int buf = tile & 1;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's share of the tile has landed
+    __syncthreads();                      // ... everybody's has, and the other stage is free
+    if (tile + 1 < ntiles) request_tile(tile + 1, buf ^ 1);
+    if (!wave_active) continue;
+#pragma unroll 1
+    for (int sub = 0; sub < NSUB; ++sub) {
+      const int key0 = tile * KEYS + sub * SUB;
+      if (key0 > wave_limit) break;
+      const unsigned char *piece = smem + buf * STAGE + sub * L::STAGE;
+      // ---- S^T = K . Q^T ---------------------------------------------------------------------
+      floatx4 st = {0.f, 0.f, 0.f, 0.f};
+      {
+        // (two accumulation chains: a matrix instruction waits for the one it accumulates onto)
+        floatx4 st1 = {0.f, 0.f, 0.f, 0.f};
+        bf16x8 ring[KPRE];
+#pragma unroll
+        for (int s = 0; s < KPRE; ++s) ring[s] = read_k(piece, s);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+          if (s & 1) st1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % KPRE], qf[s], st1, 0, 0, 0);
+          else st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % KPRE], qf[s], st, 0, 0, 0);
+          if (s + KPRE < KSTEPS) ring[s % KPRE] = read_k(piece, s + KPRE);
+        }
+        st += st1;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (s + KPRE < KSTEPS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+      }
+      // ---- online softmax: lane (row, quad) holds keys key0 + 4 quad + r of its row ------------
+      float sc[4], mloc = -INFINITY;
+      float madd[4] = {0.f, 0.f, 0.f, 0.f};
+      if (mrow) {  // wavefront-uniform
+        const int kq = min(key0 + 4 * quad, a.s - 4);
+        const uint2 mw = *reinterpret_cast<const uint2 *>(mrow + kq);
+        madd[0] = bf16_lo(mw.x) * 1.4426950408889634f, madd[1] = bf16_hi(mw.x) * 1.4426950408889634f;
+        madd[2] = bf16_lo(mw.y) * 1.4426950408889634f, madd[3] = bf16_hi(mw.y) * 1.4426950408889634f;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = key0 + 4 * quad + i;
+        sc[i] = key > limit ? -INFINITY : st[i] * scale + madd[i];
+        mloc = fmaxf(mloc, sc[i]);
+      }
+      mloc = max_over_quads(mloc);
+      const bool move = !(mloc - m_run <= 8.0f);  // (lazy: also true from -inf)
+      const float m_new = move ? mloc : m_run;
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = move ? __builtin_amdgcn_exp2f(m_run - m_safe) : 1.0f;
+      m_run = m_new;
+      float lsum = 0.f;
+      shortx4 pf;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pr = __builtin_amdgcn_exp2f(sc[i] - m_safe);
+        const __bf16 pb = (__bf16)pr;
+        lsum += (float)pb;
+        pf[i] = __builtin_bit_cast(short, pb);
+      }
+      l_run = l_run * alpha + lsum;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+        for (int i = 0; i < VB; ++i) acc[i] *= alpha;
+      }
+      // ---- O^T += V^T . P^T ---------------------------------------------------------------------
+      {
+        shortx4 vring[VPRE];
+#pragma unroll
+        for (int vb = 0; vb < VPRE; ++vb) vring[vb] = read_v(piece, vb);
+#pragma unroll
+        for (int vb = 0; vb < VB; ++vb) {
+          acc[vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vring[vb % VPRE], pf, acc[vb], 0, 0, 0);
+          if (vb + VPRE < VB) vring[vb % VPRE] = read_v(piece, vb + VPRE);
+        }
+#pragma unroll
+        for (int vb = 0; vb < VB; ++vb) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (vb + VPRE < VB) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+      }
+    }
+  }
+  if (!wave_active) return;
+  // ---- normalise and store: lane (row, quad) holds values 16 vb + 4 quad .. + 3 of its row --------
+  const float l_tot = sum_over_quads(l_run);
+  const float inv = 1.0f / l_tot;
+  if (row_valid) {
+    uint16_t *op = a.out + b * a.out_bs + head * a.out_hs + (int64_t)t * a.out_ts + 4 * quad;
+#pragma unroll
+    for (int vb = 0; vb < VB; ++vb)
+      *reinterpret_cast<uint2 *>(op + 16 * vb) =
+          make_uint2(pack_bf16x2(acc[vb][0] * inv, acc[vb][1] * inv), pack_bf16x2(acc[vb][2] * inv, acc[vb][3] * inv));
+  }
+}
+
+template <int DQK, int DV>
+int launch_latent_prefill(const LatentPrefillArgs &a, hipStream_t st) {
+  using L = Latent16<DQK, DV>;
+  const size_t lds = 2 * 4 * (size_t)L::STAGE;
+  static std::atomic<uint64_t> lds_ready{0};
+  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&latent_prefill_kernel<DQK, DV>), lds, lds_ready))
+    return fail(TTPA_ERR_LAUNCH, "latent prefill: cannot reserve %zu bytes of LDS", lds);
+  const int64_t rows = (int64_t)(a.heads / a.nkv) * a.s;
+  const int64_t grid = (rows + 127) / 128 * a.batch * a.nkv;
+  launch_dominant(&latent_prefill_kernel<DQK, DV>, dim3((unsigned)grid), dim3(512), lds, st, a);
+  return check_launch("latent_prefill");
+}
+
 template <int DQK, int DVW, bool SHARED_V>
 bool launch(const DecodeArgs &a, const WideArgs &w, hipStream_t st) {
   using L = WideLds<DQK, DVW, SHARED_V>;
@@ -642,17 +1129,39 @@ static int wide_geometry(int32_t q_heads, int32_t kv_heads, int32_t &nhb, int32_
   return TTPA_OK;
 }
 
+// The 128-head form: more than 16 heads per KV head in segments of up to 128.
+static bool latent128_geometry(int32_t q_heads, int32_t kv_heads, int32_t &nhb, int32_t &gseg) {
+  const int g = q_heads / kv_heads;
+  if (g <= 16) return false;
+  if (g <= 128) {
+    nhb = 1, gseg = g;
+    return true;
+  }
+  if (g % 128) return false;
+  nhb = g / 128, gseg = 128;
+  return true;
+}
+
 extern "C" size_t ttpa_paged_mla_decode_workspace_bytes(int32_t users, int32_t q_heads, int32_t kv_heads,
                                                         int32_t head_dim_v) {
   if (users <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim_v <= 0 || q_heads % kv_heads) return 0;
-  int32_t nhb, gseg;
-  if (wide_geometry(q_heads, kv_heads, nhb, gseg) != TTPA_OK) return 0;
   int cus = device_cus();
   if (cus <= 0) cus = 256;
-  const size_t segs = (size_t)users * kv_heads * nhb;
-  const size_t slot = (size_t)slot_floats_for(gseg, head_dim_v) * sizeof(float);
-  // one slot per range of the largest grid (at most four wavefront ranges per CU in the 16-head form)
-  return header_bytes(users, kv_heads * nhb) + ((size_t)cus * kWavesPerBlockHost + segs) * slot;
+  size_t need = 0;
+  int32_t nhb, gseg;
+  // (error text of a geometry the workgroup-shared form refuses is not this function's business)
+  if (wide_geometry(q_heads, kv_heads, nhb, gseg) == TTPA_OK) {
+    const size_t segs = (size_t)users * kv_heads * nhb;
+    const size_t slot = (size_t)slot_floats_for(gseg, head_dim_v) * sizeof(float);
+    // one slot per range of the largest grid (at most four wavefront ranges per CU in the 16-head form)
+    need = header_bytes(users, kv_heads * nhb) + ((size_t)cus * kWavesPerBlockHost + segs) * slot;
+  }
+  if (latent128_geometry(q_heads, kv_heads, nhb, gseg)) {
+    const size_t segs = (size_t)users * kv_heads * nhb;
+    const size_t slot = (size_t)slot_floats_for(gseg, head_dim_v) * sizeof(float);
+    need = std::max(need, header_bytes(users, kv_heads * nhb) + ((size_t)cus + segs) * slot);  // one range per CU
+  }
+  return need;
 }
 
 static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stride,
@@ -675,7 +1184,15 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
   if (users > kMaxUsersWide)
     return fail(TTPA_ERR_UNSUPPORTED, "latent decode: %d users exceeds the limit of %d", users, kMaxUsersWide);
   int32_t nhb, gseg;
-  if (int rc = wide_geometry(q_heads, kv_heads, nhb, gseg)) return rc;
+  // The 128-head form: V taken from K, more than 16 heads per KV head, 16-row pieces inside one block,
+  // no mask.  TTPA_LATENT_KERNEL=wide (read on every call) keeps such shapes on the workgroup-shared form.
+  const char *force = getenv("TTPA_LATENT_KERNEL");
+  const bool built128 = (head_size == 576 && (head_dim_v == 512 || head_dim_v == 384)) ||
+                        (head_size == 192 && head_dim_v == 128) || (head_size == 128 && head_dim_v == 128);
+  const bool want128 = !mask && !v_cache && built128 && block_size % 16 == 0 && !(force && force[0] == 'w') &&
+                       latent128_geometry(q_heads, kv_heads, nhb, gseg);
+  if (!want128)
+    if (int rc = wide_geometry(q_heads, kv_heads, nhb, gseg)) return rc;
   TTPA_REQUIRE(aligned16(q) && aligned16(k_cache) && aligned16(out) && (!v_cache || aligned16(v_cache)),
                "latent decode: q / caches / out must be 16-byte aligned");
   TTPA_REQUIRE(q_user_stride % 8 == 0 && q_head_stride % 8 == 0,
@@ -725,9 +1242,28 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   bool ok = false, built = true;
   const bool shared = v_cache == nullptr;
+  if (want128) {
+    if ((int64_t)users * kv_heads * nhb > ((int64_t)a.n_waves + 1) * 256)
+      return fail(TTPA_ERR_UNSUPPORTED, "latent decode: %d x %d segments need a grid of more than %d workgroups",
+                  users, kv_heads * nhb, a.n_waves);
+    // partials as bfloat16, as in the 16-head form (TTPA_LATENT_PARTIALS=f32 keeps floats)
+    const char *pf = getenv("TTPA_LATENT_PARTIALS");
+    a.partial_bf16 = !(pf && pf[0] == 'f') && out_user_stride % 2 == 0 && out_head_stride % 2 == 0 &&
+                     reinterpret_cast<uintptr_t>(out) % 4 == 0;
+    if (a.partial_bf16) a.slot_floats = slot_floats_bf16_for(gseg, head_dim_v);
+    if (head_size == 576 && head_dim_v == 512) ok = launch_latent128<576, 512>(a, w, st);
+    else if (head_size == 576 && head_dim_v == 384) ok = launch_latent128<576, 384>(a, w, st);
+    else if (head_size == 192 && head_dim_v == 128) ok = launch_latent128<192, 128>(a, w, st);
+    else ok = launch_latent128<128, 128>(a, w, st);
+    if (!ok) return fail(TTPA_ERR_LAUNCH, "latent decode: cannot configure the kernel");
+    if (int rc = check_launch("paged_mla_decode")) return rc;
+    if (a.partial_bf16)
+      decode_combine_bf16_kernel<<<dim3(users * kv_heads * nhb, combine_pieces(gseg, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+    else
+      decode_combine_kernel<<<dim3(users * kv_heads * nhb, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+    return check_launch("paged_mla_decode");
+  }
   // The 16-head form: V taken from K, one head block of up to 16 heads, tiles inside one block.
-  // TTPA_LATENT_KERNEL=wide (read on every call) keeps such shapes on the workgroup-shared form.
-  const char *force = getenv("TTPA_LATENT_KERNEL");
   // (only the workgroup-shared form applies a mask)
   const bool want16 = !mask && shared && nhb == 1 && gseg <= 16 && block_size % 16 == 0 && !(force && force[0] == 'w');
   if (want16) {
@@ -824,4 +1360,56 @@ extern "C" int ttpa_paged_mla_decode_masked(void *out, int64_t out_user_stride, 
                          page_table, page_table_row_stride, cur_pos, cur_pos_is_i64, users, q_heads, kv_heads,
                          head_size, head_dim_v, block_size, table_width, num_blocks, scale, nullptr, workspace,
                          workspace_bytes, stream, mask, mask_user_stride, mask_head_stride);
+}
+
+extern "C" int ttpa_latent_prefill(void *out, int64_t out_batch_stride, int64_t out_head_stride,
+                                   int64_t out_token_stride, const void *q, int64_t q_batch_stride,
+                                   int64_t q_head_stride, int64_t q_token_stride, const void *k,
+                                   int64_t k_batch_stride, int64_t k_head_stride, int64_t k_token_stride,
+                                   const void *mask, int64_t mask_batch_stride, int64_t mask_head_stride,
+                                   int64_t mask_row_stride, int32_t batch, int32_t q_heads, int32_t kv_heads,
+                                   int32_t seq_len, int32_t head_size, int32_t head_dim_v, int32_t causal,
+                                   float scale, void *stream) {
+  TTPA_REQUIRE(out && q && k, "null pointer argument");
+  TTPA_REQUIRE(batch > 0 && q_heads > 0 && kv_heads > 0 && seq_len > 0 && head_size > 0 && head_dim_v > 0,
+               "non-positive dimension");
+  TTPA_REQUIRE(q_heads % kv_heads == 0, "q_heads %d not divisible by kv_heads %d", q_heads, kv_heads);
+  TTPA_REQUIRE(head_dim_v <= head_size, "head_dim_v %d exceeds head_size %d while V is taken from K", head_dim_v,
+               head_size);
+  TTPA_REQUIRE(!(mask && causal), "an additive mask excludes causal masking");
+  TTPA_REQUIRE(scale > 0.f, "latent prefill: scale %g must be positive", (double)scale);
+  TTPA_REQUIRE(aligned16(q) && aligned16(k) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0,
+               "latent prefill: q / k must be 16-byte aligned, out 8-byte aligned");
+  TTPA_REQUIRE(q_batch_stride % 8 == 0 && q_head_stride % 8 == 0 && q_token_stride % 8 == 0 && k_batch_stride % 8 == 0 &&
+                   k_head_stride % 8 == 0 && k_token_stride % 8 == 0,
+               "latent prefill: q / k strides must be multiples of 8 elements");
+  TTPA_REQUIRE(out_batch_stride % 4 == 0 && out_head_stride % 4 == 0 && out_token_stride % 4 == 0,
+               "latent prefill: out strides must be multiples of 4 elements");
+  TTPA_REQUIRE((int64_t)seq_len * k_token_stride * 2 < (1ll << 32), "latent prefill: a K head must stay below 4 GiB");
+  if (mask) {
+    TTPA_REQUIRE(seq_len % 4 == 0 && (reinterpret_cast<uintptr_t>(mask) & 7u) == 0 && mask_batch_stride % 4 == 0 &&
+                     mask_head_stride % 4 == 0 && mask_row_stride % 4 == 0,
+                 "latent prefill: a mask needs seq_len %% 4 == 0, 8-byte alignment and strides that are multiples of 4 elements");
+  }
+  const int64_t rows = (int64_t)(q_heads / kv_heads) * seq_len;
+  TTPA_REQUIRE(rows < (1ll << 31) && (rows + 127) / 128 * batch * kv_heads < (1ll << 31),
+               "latent prefill: too many rows for one launch");
+  LatentPrefillArgs a;
+  a.out = static_cast<uint16_t *>(out);
+  a.out_bs = out_batch_stride, a.out_hs = out_head_stride, a.out_ts = out_token_stride;
+  a.q = static_cast<const uint16_t *>(q);
+  a.q_bs = q_batch_stride, a.q_hs = q_head_stride, a.q_ts = q_token_stride;
+  a.k = static_cast<const uint16_t *>(k);
+  a.k_bs = k_batch_stride, a.k_hs = k_head_stride, a.k_ts = k_token_stride;
+  a.mask = static_cast<const uint16_t *>(mask);
+  a.mask_bs = mask_batch_stride, a.mask_hs = mask_head_stride, a.mask_rs = mask_row_stride;
+  a.batch = batch, a.heads = q_heads, a.nkv = kv_heads, a.s = seq_len, a.causal = causal ? 1 : 0;
+  a.scale_log2e = scale * 1.4426950408889634f;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (head_size == 576 && head_dim_v == 512) return launch_latent_prefill<576, 512>(a, st);
+  if (head_size == 192 && head_dim_v == 128) return launch_latent_prefill<192, 128>(a, st);
+  if (head_size == 128 && head_dim_v == 128) return launch_latent_prefill<128, 128>(a, st);
+  return fail(TTPA_ERR_UNSUPPORTED,
+              "latent prefill: (head_size, head_dim_v) = (%d, %d); built for (576, 512), (192, 128), (128, 128)",
+              head_size, head_dim_v);
 }

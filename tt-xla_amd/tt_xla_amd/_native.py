@@ -105,6 +105,11 @@ SIGNATURES = {
          _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _p, _i64, _p],
     ),
     "ttpa_sdpa_prefill_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32, _i32, _i32]),
+    "ttpa_latent_prefill": (
+        _int,
+        [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i64, _i64,
+         _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _p],
+    ),
     "ttpa_sdpa_prefill_fill": (
         _int,
         [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64,

@@ -958,6 +958,10 @@ def _(query, key, head_dim_v, page_table, value=None, is_causal=True, attn_mask=
                        dtype=query.dtype, device=query.device)
 
 
+# (head size, value width) pairs ttpa_latent_prefill is built for
+_LATENT_PREFILL_SHAPES = {(576, 512), (192, 128), (128, 128)}
+
+
 @torch.library.custom_op("tt::flash_mla_prefill", mutates_args=[], device_types=["cuda"])
 def flash_mla_prefill(
     query: torch.Tensor,
@@ -971,8 +975,8 @@ def flash_mla_prefill(
     """Causal prefill over freshly built latent K (reference custom_ops.py:223-378): query
     [b, nqh, s, dh_qk], key [b, nkv, s, dh_qk], optional value [b, nkv, s, head_dim_v].
 
-    Runs on the latent decode kernel: query row i of a sequence is a user at position i
-    whose cache is the sequence itself (one block of s tokens, a one-column page table)."""
+    With V taken from K and a head size the prefill kernel is built for, one launch of
+    ttpa_latent_prefill; otherwise the latent decode kernels, one launch per batch entry."""
     assert len(query.shape) == 4, "query must be a 4D tensor: [b, nqh, s, dh_qk]."
     assert len(key.shape) == 4, "key must be a 4D tensor: [b, nkv, s, dh_qk]."
     assert key.shape[-1] == query.shape[-1], "key and query must have the same head size (dh_qk)."
@@ -1003,6 +1007,27 @@ def flash_mla_prefill(
     k = key.contiguous()
     v = value.contiguous() if value is not None else None
     out = torch.empty((b, hq, s, head_dim_v), dtype=query.dtype, device=query.device)
+    if v is None and (dh, head_dim_v) in _LATENT_PREFILL_SHAPES:
+        # the prefill kernel: 128 (token, head) rows share every K tile
+        mask_ptr, mask_strides = 0, (0, 0, 0)
+        if attn_mask is not None:
+            m = _additive_mask(attn_mask)
+            if m.dim() != 4 or m.shape[0] != b or m.shape[1] not in (1, hq) or m.shape[2] != s or m.shape[3] != s:
+                raise ValueError(f"attn_mask must broadcast to [{b}, {hq}, {s}, {s}], got {tuple(attn_mask.shape)}")
+            if m.stride(-1) != 1 or any(st % 4 for st in m.stride()[:3]) or m.data_ptr() % 8:
+                m = m.contiguous()
+            mask_ptr = m.data_ptr()
+            mask_strides = (m.stride(0), m.stride(1) if m.shape[1] == hq and hq > 1 else 0, m.stride(2))
+        N.call(
+            "ttpa_latent_prefill",
+            out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
+            q.data_ptr(), q.stride(0), q.stride(1), q.stride(2),
+            k.data_ptr(), k.stride(0), k.stride(1), k.stride(2),
+            mask_ptr, *mask_strides, b, hq, key.shape[1], s, dh, head_dim_v, int(is_causal), float(scale), _stream(),
+        )
+        return out
+    # other shapes, and a separate V: the decode kernels, query row i of a sequence being a user at
+    # position i whose cache is the sequence itself (one block of s tokens, a one-column page table)
     table = torch.zeros((s, 1), dtype=torch.int32, device=query.device)
     mask = None
     if attn_mask is None:
