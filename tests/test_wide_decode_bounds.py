@@ -33,10 +33,23 @@ SHAPES = [
 # every case of the GPU test's own lists
 SHAPES += [(dh, dv, has_v, hq, nkv, bs, width, width * users, users)
            for users, hq, nkv, dh, dv, has_v, bs, width, _ in G.DECODE]
-# prefill runs on the decode kernel: query row i is a user, the sequence one block of s tokens,
-# at most 1024 users per launch
+# prefill with a separate V runs on the decode kernels: query row i is a user, the sequence one block
+# of s tokens, at most 1024 users per launch
 SHAPES += [(dh, dv, has_v, hq, nkv, s, 1, 1, min(s, 1024)) for _, hq, s, dh, nkv, dv, has_v in G.PREFILL]
 SHAPES = sorted(set(SHAPES))
+BUILT_16 = {(576, 512), (576, 384), (192, 128), (128, 128)}
+
+
+def _form_128(shape):
+    """Shapes the 128-head form takes from the workgroup-shared one: V from K, more than 16 heads per
+    KV head in segments of up to 128, 16-row pieces inside one block."""
+    dqk, dv, sep_v, hq, nkv, bs = shape[:6]
+    g = hq // nkv
+    return not sep_v and (dqk, dv) in BUILT_16 and bs % 16 == 0 and g > 16 and (g <= 128 or g % 128 == 0)
+
+
+SHAPES_128 = [s for s in SHAPES if _form_128(s)]
+SHAPES = [s for s in SHAPES if not _form_128(s)] + [(576, 512, False, 128, 1, 64, 12, 36, 3), (128, 128, False, 32, 1, 32, 16, 128, 8)]
 
 
 def _geometry(hq, nkv):
@@ -130,7 +143,6 @@ def test_every_address_stays_in_bounds(dqk, dv, sep_v, hq, nkv, bs, width, nb, u
 
 
 # ---- the 16-head form (every wavefront streams its own 16-token tiles) ---------------------------
-BUILT_16 = {(576, 512), (576, 384), (192, 128), (128, 128)}
 SHAPES_16 = [s for s in SHAPES
              if not s[2] and s[3] // s[4] <= 16 and s[5] % 16 == 0 and (s[0], s[1]) in BUILT_16]
 
@@ -203,3 +215,98 @@ def test_every_address_of_the_16_head_form_stays_in_bounds(dqk, dv, sep_v, hq, n
             assert g * dv + g + n < slot_floats
     segs, cus = users * nkv, 256
     assert (waves * cus - 1) + (segs - 1) < waves * cus + segs     # slot index = wavefront + segment
+
+
+# ---- the 128-head form and the prefill kernel: eight wavefronts on shared tiles of four 16-row pieces ----
+def _shared_tile_checks(dqk, dv):
+    """What both kernels share: the stage of four pieces laid out like the 16-head form's, every chunk
+    of a tile requested exactly once by the wavefronts' shares, destinations inside the stage."""
+    row_bytes, sub, nsub, waves = 2 * dqk, 16, 4, 8
+    cpr = row_bytes // 16
+    piece = sub * row_bytes
+    ndma = piece // 1024
+    stage = nsub * piece
+    assert piece % 1024 == 0 and (nsub * ndma) % waves == 0
+    per_wave = nsub * ndma // waves
+    assert STATIC_LDS + 2 * stage <= LDS_PER_CU
+    seen = set()
+    for wave in range(waves):
+        for j in range(per_wave):
+            k = wave * per_wave + j
+            piece_i, kk = k // ndma, k % ndma
+            for lane in range(64):
+                pos = 64 * kk + lane
+                rr, p = pos // cpr, pos % cpr
+                assert rr < sub
+                off = (sub * piece_i + rr, _position(row_bytes, rr, p))      # (row of the tile, chunk of the row)
+                assert off[1] < cpr
+                seen.add(off)
+            for buf in (0, 1):
+                dst = STATIC_LDS + buf * stage + 1024 * k
+                assert dst % 16 == 0 and dst + 1024 <= STATIC_LDS + (buf + 1) * stage <= LDS_PER_CU
+    assert len(seen) == nsub * sub * cpr, "every chunk of the tile is fetched exactly once"
+    return row_bytes, piece, stage, per_wave, ndma
+
+
+def test_the_128_head_form_is_exercised():
+    assert any(s[3] // s[4] == 128 for s in SHAPES_128) and any(s[3] // s[4] % 16 for s in SHAPES_128)
+    assert any(s[3] // s[4] > 128 for s in SHAPES_128)
+
+
+@pytest.mark.parametrize("dqk,dv,sep_v,hq,nkv,bs,width,nb,users", SHAPES_128)
+def test_every_address_of_the_128_head_form_stays_in_bounds(dqk, dv, sep_v, hq, nkv, bs, width, nb, users):
+    row_bytes, piece, stage, per_wave, ndma = _shared_tile_checks(dqk, dv)
+    assert 2 * per_wave == ndma, "wavefronts 2 i and 2 i + 1 fetch piece i"
+    g = hq // nkv
+    nhb, gseg = (1, g) if g <= 128 else (g // 128, 128)
+    assert nhb * gseg == g
+    cache_bytes = nb * nkv * bs * row_bytes
+    cap = width * bs
+    for t in {0, (cap - 1) // K_TILE}:
+        for wave in range(8):
+            tok0 = t * K_TILE + 16 * (wave >> 1)
+            col = tok0 // bs
+            assert tok0 - col * bs + 16 <= bs, "a piece lies inside one block"
+            for phys, kvh in itertools.product({0, nb - 1}, {0, nkv - 1}):
+                p = phys if col < width else 0
+                base = ((p * nkv + kvh) * bs + (tok0 - col * bs)) * row_bytes
+                assert base % 16 == 0 and base + piece <= cache_bytes
+    vb = dv // 16
+    slot_floats = (gseg * dv + 2 * gseg + 3) // 4 * 4
+    slot_floats_bf16 = (gseg * dv // 2 + 2 * gseg + 3) // 4 * 4
+    for wave, n, quad in itertools.product(range(8), (0, 15), (0, 3)):
+        hg = 16 * wave + n
+        if hg < gseg:
+            assert hg * dv + 4 * quad + 16 * (vb - 1) + 4 <= gseg * dv
+            assert gseg * dv + gseg + hg < slot_floats
+            assert gseg * dv // 2 + gseg + hg < slot_floats_bf16
+    for seg_h in (0, nkv * nhb - 1):
+        assert seg_h * gseg + gseg - 1 < hq and seg_h // nhb < nkv
+    segs, cus = users * nkv * nhb, 256
+    assert segs <= (cus + 1) * 256, "one thread of the grid publishes each segment's partial slots"
+
+
+PREFILL_SHAPES = [(dh, dv, hq, nkv, s, b) for b, hq, s, dh, nkv, dv, has_v in G.PREFILL + G.MASKED_PREFILL
+                  if not has_v and (dh, dv) in {(576, 512), (192, 128), (128, 128)}]
+
+
+@pytest.mark.parametrize("dqk,dv,hq,nkv,s,batch", sorted(set(PREFILL_SHAPES)))
+def test_every_address_of_the_prefill_kernel_stays_in_bounds(dqk, dv, hq, nkv, s, batch):
+    row_bytes, piece, stage, per_wave, ndma = _shared_tile_checks(dqk, dv)
+    g = hq // nkv
+    rows_total = g * s
+    nblk = (rows_total + 127) // 128
+    k_bytes = s * row_bytes                      # one (batch entry, KV head) of a contiguous K
+    for blk in {0, nblk - 1}:
+        last_row = min(blk * 128 + 127, rows_total - 1)
+        ntiles = (last_row // g) // K_TILE + 1
+        for tile in {0, ntiles - 1}:
+            for r in (0, 63):
+                key = min(tile * K_TILE + r, s - 1)
+                assert key * row_bytes + row_bytes <= k_bytes
+        for wave, n in itertools.product(range(8), range(16)):
+            r = min(blk * 128 + 16 * wave + n, rows_total - 1)
+            t, head = r // g, r % g
+            assert 0 <= t < s and head < g
+            assert 32 * (dqk // 32 - 1) + 8 * 3 + 8 <= dqk and 16 * (dv // 16 - 1) + 4 * 3 + 4 <= dv
+    assert batch * nkv * nblk < 2 ** 31
