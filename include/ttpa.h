@@ -191,8 +191,10 @@ int ttpa_paged_sdpa_decode_windowed(void *out, int64_t out_user_stride, int64_t 
  * the element for (user, query head, position) is mask[user * mask_user_stride +
  * head * mask_head_stride + position] (a head stride of 0 shares one row between the heads).
  * cur_pos[u] is the last position that is attended at all (the caller passes
- * table_width * block_size - 1 to attend every position of the table).  bfloat16 caches, up to
- * 8 query heads per KV head; the rest as ttpa_paged_sdpa_decode.
+ * table_width * block_size - 1 to attend every position of the table).  Built for up to 8 query
+ * heads per KV head on bfloat16 caches (dot-product kernel) and up to 16 on either cache format
+ * (kv_format as in ttpa_paged_sdpa_decode_windowed) where the 16x16x32 matrix-core kernel applies;
+ * other shapes return TTPA_ERR_UNSUPPORTED.  The rest as ttpa_paged_sdpa_decode.
  */
 int ttpa_paged_sdpa_decode_masked(void *out, int64_t out_user_stride, int64_t out_head_stride,
                                   const void *q, int64_t q_user_stride, int64_t q_head_stride,
@@ -200,8 +202,9 @@ int ttpa_paged_sdpa_decode_masked(void *out, int64_t out_user_stride, int64_t ou
                                   int64_t page_table_row_stride, const void *cur_pos, int cur_pos_is_i64,
                                   int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
                                   int32_t block_size, int32_t table_width, int32_t num_blocks, float scale,
-                                  const void *mask, int64_t mask_user_stride, int64_t mask_head_stride,
-                                  void *workspace, size_t workspace_bytes, void *stream);
+                                  int32_t kv_format, const void *mask, int64_t mask_user_stride,
+                                  int64_t mask_head_stride, void *workspace, size_t workspace_bytes,
+                                  void *stream);
 
 /*
  * The decode step of the attention backend in one call: the cache update

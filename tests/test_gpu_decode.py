@@ -271,14 +271,27 @@ def test_decode_more_than_1024_users_on_the_matrix_core_kernel(bfp8):
     _check(name, got[:, live], want[:, live])
 
 
-@pytest.mark.parametrize("hq,hkv,d,bs,bfp8", [(8, 8, 64, 32, False), (32, 8, 128, 64, False), (16, 4, 128, 32, True)])
-def test_decode_with_explicit_mask(hq, hkv, d, bs, bfp8):
+@pytest.mark.parametrize("hq,hkv,d,bs,bfp8,kernel", [
+    (8, 8, 64, 32, False, ""), (32, 8, 128, 64, False, ""), (16, 4, 128, 32, True, ""),
+    (32, 8, 128, 64, False, "valu"),     # the dot-product kernel where the matrix-core one is the default
+    (8, 8, 64, 32, False, "mfma16"),     # ... and the other way round
+    (48, 4, 128, 32, False, ""),         # 12 heads per group: the matrix-core kernel only
+    (16, 1, 256, 16, True, ""),          # 16 heads, head size 256, block-float-8
+    (24, 2, 64, 48, True, ""),           # a block size that is no power of two
+    (64, 2, 128, 32, False, ""),         # 32 heads per group: gathered through the dense kernel, one mask row for all heads
+])
+def test_decode_with_explicit_mask(monkeypatch, hq, hkv, d, bs, bfp8, kernel):
     """is_causal=False with an additive attn_mask [users, 1, 1, W*bs] (reference CPU branch
     custom_ops.py:1299-1311; the one-token pass of an encoder / pooling model) against the
     oracle's masked form: every position of the table is attended, weighted by the mask.  A
     boolean mask means "attend where True"."""
     from oracle import bfp8_codec as C
     from tt_xla_amd import custom_ops as ops
+
+    if kernel:
+        monkeypatch.setenv("TTPA_DECODE_KERNEL", kernel)
+    else:
+        monkeypatch.delenv("TTPA_DECODE_KERNEL", raising=False)
 
     g = torch.Generator().manual_seed(hq + d)
     users, w = 3, 5
@@ -293,7 +306,7 @@ def test_decode_with_explicit_mask(hq, hkv, d, bs, bfp8):
     keep = torch.rand(users, 1, 1, span, generator=g) > 0.4
     keep[:, :, :, 0] = True
     mask = mask.masked_fill(~keep, float("-inf"))
-    name = f"masked decode h{hq}x{hkv} d{d} bs{bs} bfp8={bfp8}"
+    name = f"masked decode h{hq}x{hkv} d{d} bs{bs} bfp8={bfp8} kernel={kernel or 'default'}"
     print(name, flush=True)
     if bfp8:
         kd, vd = ops.bfp8_pack_cache(key.cuda()), ops.bfp8_pack_cache(value.cuda())
@@ -313,9 +326,9 @@ def test_decode_with_explicit_mask(hq, hkv, d, bs, bfp8):
     want_b = O.paged_sdpa_decode(q.float(), key.float(), value.float(), table, False,
                                  torch.zeros(users, 1, 1, span).masked_fill(~keep, float("-inf")), cur, None, 0.11)
     torch.testing.assert_close(got_b.float(), want_b, atol=ATOL, rtol=RTOL)
-    # a mask per head: on the decode kernel for bfloat16 caches, refused on the gathered form
+    # a mask per head: on the decode kernels (up to 16 heads per group), refused on the gathered form
     mask_h = (mask + 0.5 * torch.randn(users, hq, 1, span, generator=g).to(torch.bfloat16)).to(torch.bfloat16)
-    if bfp8:
+    if hq // hkv > 16:
         with pytest.raises(NotImplementedError):
             torch.ops.tt.paged_scaled_dot_product_attention_decode(
                 q.cuda(), kd, vd, table.cuda(), is_causal=False, attn_mask=mask_h.cuda(), cur_pos_tensor=cur.cuda())

@@ -438,9 +438,6 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   a.new_us = a.new_hs = 0;
   a.mask = static_cast<const uint16_t *>(mask);
   a.mask_us = mask_user_stride, a.mask_hs = mask_head_stride;
-  if (mask && (g > 8 || kv_format != TTPA_KV_BF16))
-    return fail(TTPA_ERR_UNSUPPORTED,
-                "masked decode: built for bfloat16 caches and up to 8 query heads per KV head (got %d)", g);
 
   hipStream_t st = static_cast<hipStream_t>(stream);
   // Kernel choice.  The VALU kernel spends per-head work on every tile; the matrix-core kernels
@@ -475,7 +472,17 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   if (forced == 1 && g <= 8 && !(kv_format == TTPA_KV_BFP8 && head_size == 256)) use_mfma = use_mfma16 = false;
   if (forced == 2 && mfma_ok) use_mfma = true, use_mfma16 = false;
   if (forced == 3 && mfma16_ok) use_mfma16 = true, use_mfma = false;
-  if (mask) use_mfma = use_mfma16 = false;  // only the dot-product kernel applies a mask
+  if (mask) {
+    // A mask is applied by the dot-product kernel (bfloat16 caches, up to 8 heads per group) and by
+    // the 16x16x32 kernel (either format, up to 16); a forced choice holds where it is built.
+    const bool valu_ok = g <= 8 && kv_format == TTPA_KV_BF16;
+    if (!valu_ok && !mfma16_ok)
+      return fail(TTPA_ERR_UNSUPPORTED,
+                  "masked decode: %d query heads per KV head with this cache format and block size is not built "
+                  "(bfloat16 up to 8, or up to 16 on the matrix-core kernel's shapes)", g);
+    use_mfma = false;
+    use_mfma16 = mfma16_ok && (!valu_ok || forced == 3 || (forced != 1 && g >= 4));
+  }
   // The matrix-core kernels get at most one workgroup per CU whatever the cache format: the 32x32
   // kernel fills the CU's LDS with one, and the 16x16 kernel streams as fast with one as with the
   // two that would fit, while twice the partials cost the merge kernel more.  On a bfloat16 cache
@@ -579,14 +586,14 @@ extern "C" int ttpa_paged_sdpa_decode_masked(
     int64_t q_user_stride, int64_t q_head_stride, const void *k_cache, const void *v_cache,
     const int32_t *page_table, int64_t page_table_row_stride, const void *cur_pos,
     int cur_pos_is_i64, int32_t users, int32_t q_heads, int32_t kv_heads, int32_t head_size,
-    int32_t block_size, int32_t table_width, int32_t num_blocks, float scale, const void *mask,
-    int64_t mask_user_stride, int64_t mask_head_stride, void *workspace, size_t workspace_bytes,
-    void *stream) {
+    int32_t block_size, int32_t table_width, int32_t num_blocks, float scale, int32_t kv_format,
+    const void *mask, int64_t mask_user_stride, int64_t mask_head_stride, void *workspace,
+    size_t workspace_bytes, void *stream) {
   TTPA_REQUIRE(mask != nullptr, "masked decode: null mask");
   return decode_impl(out, out_user_stride, out_head_stride, q, q_user_stride, q_head_stride, k_cache,
                      v_cache, page_table, page_table_row_stride, cur_pos, cur_pos_is_i64, users,
                      q_heads, kv_heads, head_size, block_size, table_width, num_blocks, scale,
-                     TTPA_KV_BF16, 0, nullptr, workspace, workspace_bytes, stream, nullptr, nullptr, 0, 0,
+                     kv_format, 0, nullptr, workspace, workspace_bytes, stream, nullptr, nullptr, 0, 0,
                      mask, mask_user_stride, mask_head_stride);
 }
 

@@ -126,8 +126,9 @@ __device__ inline void write_negative_position(const DecodeArgs &a, const int32_
   }
 }
 
-// RUNS: 1, 2, 4, or 0 for one run per load.
-template <int D, bool BFP8, int RUNS, bool FUSED>
+// RUNS: 1, 2, 4, or 0 for one run per load.  MASKED: an additive mask row per (user, head) joins the
+// scores (a.mask; the form of a pass that is not causal, built with RUNS = 0 and without the update).
+template <int D, bool BFP8, int RUNS, bool FUSED, bool MASKED = false>
 __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     DecodeArgs a, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
   static_assert(D == 64 || D == 128 || D == 256, "shapes built");
@@ -464,6 +465,16 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
     }
     // the factors taken out of the K tile and out of Q come back in the scale
     const float scale = BFP8 ? __builtin_ldexpf(a.scale_log2e, eref_k + eq - 260) : a.scale_log2e;
+    if constexpr (MASKED) {  // the mask, brought to the units of the raw scores
+      const float unit = 1.4426950408889634f / scale;
+      const uint16_t *mrow = a.mask + cur.u * a.mask_us + (int64_t)(cur.h * G + min(n, G - 1)) * a.mask_hs +
+                             cur.t * TILE + 4 * quad;
+#pragma unroll
+      for (int b = 0; b < KBLK; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (16 * b + 4 * quad + r < nvalid) st[b][r] += bf16_lo(mrow[16 * b + r]) * unit;
+    }
     float mloc = -INFINITY;
     if (scale >= 0.f) {
 #pragma unroll
@@ -577,15 +588,15 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma16_kernel(
   process_tile(std::false_type{});
 }
 
-template <int D, bool BFP8, int RUNS, bool FUSED>
+template <int D, bool BFP8, int RUNS, bool FUSED, bool MASKED = false>
 bool launch(const DecodeArgs &a, hipStream_t st) {
   const int blocks = a.n_waves / kWavesPerBlock;
   const size_t lds = (size_t)kWavesPerBlock * tile_bytes<D, BFP8>();
   static std::atomic<uint64_t> lds_ready{0};
-  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_mfma16_kernel<D, BFP8, RUNS, FUSED>), lds,
+  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_mfma16_kernel<D, BFP8, RUNS, FUSED, MASKED>), lds,
                           lds_ready))
     return false;
-  launch_dominant(&paged_decode_mfma16_kernel<D, BFP8, RUNS, FUSED>, dim3(blocks), dim3(256), lds, st, a, a.pt, a.cur);
+  launch_dominant(&paged_decode_mfma16_kernel<D, BFP8, RUNS, FUSED, MASKED>, dim3(blocks), dim3(256), lds, st, a, a.pt, a.cur);
   return true;
 }
 
@@ -595,6 +606,7 @@ template <int D, bool BFP8>
 bool launch_for_block_size(const DecodeArgs &a, hipStream_t st) {
   constexpr int TILE = tile_bytes<D, BFP8>() / (2 * D);
   const bool fused = a.k_new != nullptr;
+  if (a.mask != nullptr) return !fused && launch<D, BFP8, 0, false, true>(a, st);
   if (a.bs % TILE == 0) return fused ? launch<D, BFP8, 1, true>(a, st) : launch<D, BFP8, 1, false>(a, st);
   if (a.bs % (TILE / 2) == 0) return fused ? launch<D, BFP8, 2, true>(a, st) : launch<D, BFP8, 2, false>(a, st);
   if (a.bs % (TILE / 4) == 0) return fused ? launch<D, BFP8, 4, true>(a, st) : launch<D, BFP8, 4, false>(a, st);

@@ -59,7 +59,7 @@ SIGNATURES = {
     "ttpa_paged_sdpa_decode_masked": (
         _int,
         [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _i64, _p, _int, _i32, _i32, _i32, _i32, _i32,
-         _i32, _i32, _f32, _p, _i64, _i64, _p, _sz, _p],
+         _i32, _i32, _f32, _i32, _p, _i64, _i64, _p, _sz, _p],
     ),
     "ttpa_paged_update_decode": (
         _int,

@@ -457,9 +457,9 @@ def _decode_masked(query, key, value, page_table, attn_mask, attention_sink, sca
     """Decode with ``is_causal=False``: every position of the user's table is attended, weighted by
     the additive ``attn_mask`` (anything that broadcasts to [users, heads, 1, table_width * block_size];
     reference CPU branch custom_ops.py:1296-1311; the one-token pass of a pooling / encoder model,
-    never the generative serving path).  bfloat16 caches with up to 8 query heads per KV head run on
-    the decode kernel with the mask as an operand.  The rest (block-float-8 caches, wider groups)
-    goes through the prefill kernel's masked dense form, with one mask row for all heads: the user's
+    never the generative serving path).  Up to 16 query heads per KV head (either cache format) run
+    on the decode kernels with the mask as an operand.  Wider groups go through the prefill
+    kernel's masked dense form, with one mask row for all heads: the user's
     blocks are gathered in table order (ids outside the cache read block 0, as in the kernels) and
     the query token is the first row of a 32-row tile."""
     if attn_mask is None:
@@ -477,7 +477,11 @@ def _decode_masked(query, key, value, page_table, attn_mask, attention_sink, sca
     mask, mask_us, mask_hs = _decode_mask_rows(attn_mask, users, hq, skv)
     if scale is None:
         scale = 1.0 / math.sqrt(d)
-    if fmt == N.KV_BF16 and hq // hkv <= 8 and bs % 4 == 0:
+    g = hq // hkv
+    rows_per_load = max(1, 1024 // (d * (1 if fmt == N.KV_BFP8 else 2)))
+    on_dot_kernel = fmt == N.KV_BF16 and g <= 8 and bs % 4 == 0
+    on_matrix_kernel = g <= 16 and d in (64, 128, 256) and bs % rows_per_load == 0 and users <= 2048
+    if on_dot_kernel or on_matrix_kernel:
         q = _rows_contiguous(query)
         pt = _table(page_table)
         if out is None:
@@ -491,13 +495,13 @@ def _decode_masked(query, key, value, page_table, attn_mask, attention_sink, sca
             "ttpa_paged_sdpa_decode_masked",
             out.data_ptr(), out.stride(1), out.stride(2), q.data_ptr(), q.stride(1), q.stride(2),
             key.data_ptr(), value.data_ptr(), pt.data_ptr(), pt.stride(0), last.data_ptr(), 0,
-            users, hq, hkv, d, bs, width, nb, float(scale), mask.data_ptr(), mask_us, mask_hs,
+            users, hq, hkv, d, bs, width, nb, float(scale), fmt, mask.data_ptr(), mask_us, mask_hs,
             ws.data_ptr(), ws_bytes, _stream(),
         )
         return out
     if mask_hs != 0:
         raise NotImplementedError(
-            "a decode attn_mask that differs between heads is built for bfloat16 caches with up to 8 query heads per KV head")
+            "a decode attn_mask that differs between heads is built for up to 16 query heads per KV head")
 
     ids = page_table.reshape(-1).to(torch.int64)
     ids = torch.where((ids >= 0) & (ids < nb), ids, torch.zeros_like(ids))
