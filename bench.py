@@ -52,11 +52,13 @@ MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
     # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
     # the rotating workload copies; the summaries under profiles/ hold the runs)
-    "config2": ("paged_decode_mfma16_kernel", "44709186f461ba13", 311091953),
-    "config5": ("paged_decode_mfma16_kernel", "44709186f461ba13", 168806899),
-    "config4": ("paged_decode_mfma16_kernel", "44709186f461ba13", 3444653748),
-    "config3": ("prefill_kernel", "caf4dfdc8092f655", 234149651),
-    "latent": ("paged_decode_latent16_kernel", "33cba915f8ae781e", 654097655),
+    "config2": ("paged_decode_mfma16_kernel", "be3a15e04ef564b8", 310439571),
+    "config5": ("paged_decode_mfma16_kernel", "be3a15e04ef564b8", 168447693),
+    "config4": ("paged_decode_mfma16_kernel", "be3a15e04ef564b8", 3415584888),
+    "config3": ("prefill_kernel", "335508424dd21a98", 244479198),
+    "latent": ("paged_decode_latent16_kernel", "0168059ef989a648", 654196617),
+    "latent128": ("paged_decode_latent128_kernel", "0168059ef989a648", 749333547),
+    "latent-prefill": ("latent_prefill_kernel", "0168059ef989a648", 333087947),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}
