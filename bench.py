@@ -55,7 +55,7 @@ MEASURED_TRAFFIC = {
     "config2": ("paged_decode_mfma16_kernel", "be3a15e04ef564b8", 310439571),
     "config5": ("paged_decode_mfma16_kernel", "be3a15e04ef564b8", 168447693),
     "config4": ("paged_decode_mfma16_kernel", "be3a15e04ef564b8", 3415584888),
-    "config3": ("prefill_kernel", "335508424dd21a98", 244479198),
+    "config3": ("prefill_kernel", "82cebe7e857b87ff", 244479198),
     "latent": ("paged_decode_latent16_kernel", "0168059ef989a648", 654196617),
     "latent128": ("paged_decode_latent128_kernel", "0168059ef989a648", 749333547),
     "latent-prefill": ("latent_prefill_kernel", "0168059ef989a648", 333087947),

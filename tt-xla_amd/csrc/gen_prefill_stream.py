@@ -44,12 +44,13 @@ the tile K enters two iterations from now is requested in front of the tile requ
 odd iteration (so the same wait covers it) and read at the next odd one.  Entries outside
 [0, num_blocks) read cache block 0.
 
-A workgroup takes several ITEMS (blocks of 32 query rows of its four heads) one after the other:
-item k of the workgroup in slot j of `spg` slots is row block nqt - 1 - d with
+A workgroup takes one or several ITEMS (blocks of 32 query rows of its four heads) one after the
+other: item k of the workgroup in slot j of `spg` slots is row block nqt - 1 - d with
 d = k spg + (k even ? j : spg - 1 - j), as long as d < nqt.  Row blocks are dealt heavy first and in
 alternating direction, so that with causal masking every workgroup gets about the same number of
-key blocks, and a launch is one round of workgroups: no workgroup waits for a free slot, and the
-start of a workgroup is paid once for several row blocks.  Per item the block does everything
+key blocks.  The launcher's default is one item per workgroup (spg = nqt: the hardware deals the
+workgroups as slots free up, which measured faster than one static round), several when the row
+blocks weigh the same and divide evenly over one round.  Per item the block does everything
 between the Q fragments and the stored output rows: its first requests (K blocks 0..NS-1, V blocks
 0..NS-3; for the first item they are a block of assembly of their own, so that the caller's Q loads
 overlap them), all blocks, the last PV, normalisation and store; then the next item's Q fragments
@@ -61,10 +62,8 @@ it (the mask waits explicitly); a bank of probabilities is rewritten three matri
 after the last one that read it; the slow path and the exit wait out the matrix pipe with s_nop.
 """
 
-import os
 import sys
 
-PROBE = {k: bool(int(os.environ.get('PROBE_' + k, '0'))) for k in ('NOVALU', 'NOBAR', 'NODS', 'NOMFMA', 'STAMPS', 'ITEMSTAMPS')}
 
 # ---- register map (vector registers) ---------------------------------------------------------
 ACC = [0, 16, 32, 48]          # output accumulators, head-dim blocks 0..3 (inputs / outputs)
@@ -132,16 +131,6 @@ class Out:
         self.lines = []
 
     def e(self, s):
-        if PROBE['NODS'] and (s.startswith('ds_read') or s.startswith('s_waitcnt lgkmcnt')):
-            return
-        if PROBE['NOMFMA'] and s.startswith('v_mfma'):
-            return
-        if PROBE['NOVALU'] and s.startswith('v_') and not s.startswith('v_mfma'):
-            return
-        if PROBE['NOVALU'] and s.startswith('s_cbranch_vccnz'):
-            return
-        if PROBE['NOBAR'] and (s.startswith('s_barrier') or s.startswith('s_waitcnt vmcnt') or s.startswith('global_load')):
-            return
         self.lines.append(s)
 
     def label(self, name):
@@ -372,8 +361,6 @@ def iteration_head(o, p, tag, paged):
     """Mask, barrier and requests of iteration i = p (mod UNROLL)."""
     mask_block(o, p % 2, tag)
     # requests of the last two barriers may stay in flight, unless some were skipped
-    if PROBE['STAMPS']:
-        o.e("s_memrealtime s[92:93]")
     o.e(f"s_cmp_eq_u32 {S_KLEFT}, 0")
     o.e(f"s_cbranch_scc1 L_all_{tag}%=")
     o.e("s_waitcnt vmcnt(8)")
@@ -381,17 +368,7 @@ def iteration_head(o, p, tag, paged):
     o.label(f"L_all_{tag}")
     o.e("s_waitcnt vmcnt(0)")
     o.label(f"L_bar_{tag}")
-    if PROBE['STAMPS']:
-        o.e("s_memrealtime s[94:95]")
     o.e("s_barrier")
-    if PROBE['STAMPS']:  # (wall clock before / after the wait for the requests, per iteration)
-        o.e("s_waitcnt lgkmcnt(0)")
-        for k in range(4):
-            o.e(f"v_mov_b32 v{216 + k}, s{92 + k}")
-        o.e("v_mov_b32 v209, s97")
-        o.e("s_nop 1")
-        o.e("global_store_dwordx4 v209, v[216:219], s[100:101]")
-        o.e("s_add_u32 s97, s97, 16")
     if paged and p % 2 == 1:
         next_tile(o, tag)
     # K block i + NS is half (i + NS) % 2 of its tile, V block i + NS - 2 the same half of its own
@@ -488,14 +465,6 @@ def epilogue(o):
     o.e("s_nop 1")
 
 
-def tstamp(o, reg):
-    """probe builds: low word of the wall clock (10 ns units) into a vector register"""
-    if PROBE['ITEMSTAMPS']:
-        o.e("s_memrealtime s[94:95]")
-        o.e("s_waitcnt lgkmcnt(0)")
-        o.e(f"v_mov_b32 v{reg}, s94")
-
-
 def next_item(o, paged):
     """Behind the last PV of an item: is there another one?  Its Q fragments and first requests go
     out first, then the finished item is stored, then the state of the new one is set up."""
@@ -511,16 +480,13 @@ def next_item(o, paged):
     o.e(f"s_sub_u32 s88, {S_NQT}, s88")
     o.e("s_sub_u32 s88, s88, 1")
     o.e(f"s_lshl_b32 {S_ROW0}, s88, 5")                 # (the finished item's pointers and store mask stay in registers)
-    tstamp(o, 232)
     o.e("s_barrier")                                    # everybody has left the rings
-    tstamp(o, 233)
     o.e(f"v_add_u32 v{VROW}, {S_ROW0}, v{VN}")
     o.e(f"s_sub_u32 s88, {S_SQ}, 1")
     o.e(f"v_min_i32 v{VROW}, s88, v{VROW}")
     o.e(f"v_mad_u64_u32 v[{PTMP}:{PTMP + 1}], s[92:93], v{VROW}, {S_QTS}, v[{QBASE}:{QBASE + 1}]")
     for ks in range(8):
         o.e(f"global_load_dwordx4 {vr(QF + 4 * ks, 4)}, v[{PTMP}:{PTMP + 1}], off offset:{32 * ks}")
-    tstamp(o, 234)
     item_blocks(o)
     if paged:
         o.e("s_mov_b64 s[84:85], s[50:51]")
@@ -539,17 +505,8 @@ def next_item(o, paged):
         o.e("s_mov_b64 s[66:67], s[52:53]")
     for ln in generate_first(paged, "nx"):
         o.lines.append(ln)
-    tstamp(o, 235)
     epilogue(o)
-    tstamp(o, 236)
     item_setup(o, "nx")
-    tstamp(o, 237)
-    if PROBE['ITEMSTAMPS']:
-        o.e("v_mov_b32 v209, s97")
-        o.e("s_nop 1")
-        o.e("global_store_dwordx4 v209, v[232:235], s[100:101]")
-        o.e("global_store_dwordx4 v209, v[236:239], s[100:101] offset:16")
-        o.e("s_add_u32 s97, s97, 32")
     o.e("s_branch L_item_top%=")
     o.label("L_last_item")
     epilogue(o)
@@ -601,19 +558,9 @@ def generate_first(paged, suffix=""):
 def generate(paged):
     o = Out()
     assert NS == 5 and UNROLL == 10
-    if PROBE['STAMPS'] or PROBE['ITEMSTAMPS']:
-        o.e("s_mov_b32 s97, 0")
-    if PROBE['ITEMSTAMPS']:  # QBASE / OUTBASE are borrowed for the stamps: copies
-        for k in range(4):
-            o.e(f"v_mov_b32 v{228 + k}, v{216 + k}")
     o.e(f"v_mov_b32 v{VZERO}, 0")
     item_setup(o, "first")
     o.label("L_item_top")
-    if PROBE['ITEMSTAMPS']:
-        o.e("s_memrealtime s[92:93]")
-        o.e("s_waitcnt lgkmcnt(0)")
-        o.e("v_mov_b32 v216, s92")
-        o.e("v_mov_b32 v217, s93")
     o.e("s_waitcnt vmcnt(0)")
     o.e("s_barrier")
     # ---- S(0) from K block 0; behind it the fragments of iteration 0 (K block 1) ------------------
@@ -657,20 +604,6 @@ def generate(paged):
     o.label("L_end")
     o.e("s_nop 15")
     o.e("s_nop 15")
-    if PROBE['ITEMSTAMPS']:  # (start and end of the item, wall clock; QBASE is borrowed, so only one item is correct... the probe build keeps it in v[228:229])
-        o.e("s_memrealtime s[94:95]")
-        o.e("s_waitcnt lgkmcnt(0)")
-        o.e("v_mov_b32 v218, s94")
-        o.e("v_mov_b32 v219, s95")
-        o.e("v_mov_b32 v209, s97")
-        o.e("s_nop 1")
-        o.e("global_store_dwordx4 v209, v[216:219], s[100:101]")
-        o.e("s_add_u32 s97, s97, 16")
-        o.e("s_waitcnt vmcnt(0)")
-        o.e("v_mov_b32 v216, v228")
-        o.e("v_mov_b32 v217, v229")
-        o.e("v_mov_b32 v218, v230")
-        o.e("v_mov_b32 v219, v231")
     next_item(o, paged)
     return o.lines
 
