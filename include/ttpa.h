@@ -192,9 +192,10 @@ int ttpa_paged_sdpa_decode_windowed(void *out, int64_t out_user_stride, int64_t 
  * head * mask_head_stride + position] (a head stride of 0 shares one row between the heads).
  * cur_pos[u] is the last position that is attended at all (the caller passes
  * table_width * block_size - 1 to attend every position of the table).  Built for up to 8 query
- * heads per KV head on bfloat16 caches (dot-product kernel) and up to 16 on either cache format
- * (kv_format as in ttpa_paged_sdpa_decode_windowed) where the 16x16x32 matrix-core kernel applies;
- * other shapes return TTPA_ERR_UNSUPPORTED.  The rest as ttpa_paged_sdpa_decode.
+ * heads per KV head on bfloat16 caches (dot-product kernel) and up to 32 on either cache format
+ * (kv_format as in ttpa_paged_sdpa_decode_windowed) where a matrix-core kernel applies (16x16x32 up
+ * to 16 heads, 32x32x16 up to 32 at head sizes 64 / 128); other shapes return TTPA_ERR_UNSUPPORTED.
+ * The rest as ttpa_paged_sdpa_decode.
  */
 int ttpa_paged_sdpa_decode_masked(void *out, int64_t out_user_stride, int64_t out_head_stride,
                                   const void *q, int64_t q_user_stride, int64_t q_head_stride,

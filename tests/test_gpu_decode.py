@@ -278,7 +278,10 @@ def test_decode_more_than_1024_users_on_the_matrix_core_kernel(bfp8):
     (48, 4, 128, 32, False, ""),         # 12 heads per group: the matrix-core kernel only
     (16, 1, 256, 16, True, ""),          # 16 heads, head size 256, block-float-8
     (24, 2, 64, 48, True, ""),           # a block size that is no power of two
-    (64, 2, 128, 32, False, ""),         # 32 heads per group: gathered through the dense kernel, one mask row for all heads
+    (64, 2, 128, 32, False, ""),         # 32 heads per group: the 32x32x16 kernel
+    (48, 2, 64, 32, True, ""),           # 24 heads per group, block-float-8, head size 64: the same
+    (16, 4, 128, 32, False, "mfma"),     # ... forced where the 16x16x32 kernel is the default
+    (80, 2, 128, 32, False, ""),         # 40 heads per group: gathered through the dense kernel, one mask row for all heads
 ])
 def test_decode_with_explicit_mask(monkeypatch, hq, hkv, d, bs, bfp8, kernel):
     """is_causal=False with an additive attn_mask [users, 1, 1, W*bs] (reference CPU branch
@@ -326,9 +329,9 @@ def test_decode_with_explicit_mask(monkeypatch, hq, hkv, d, bs, bfp8, kernel):
     want_b = O.paged_sdpa_decode(q.float(), key.float(), value.float(), table, False,
                                  torch.zeros(users, 1, 1, span).masked_fill(~keep, float("-inf")), cur, None, 0.11)
     torch.testing.assert_close(got_b.float(), want_b, atol=ATOL, rtol=RTOL)
-    # a mask per head: on the decode kernels (up to 16 heads per group), refused on the gathered form
+    # a mask per head: on the decode kernels (up to 32 heads per group), refused on the gathered form
     mask_h = (mask + 0.5 * torch.randn(users, hq, 1, span, generator=g).to(torch.bfloat16)).to(torch.bfloat16)
-    if hq // hkv > 16:
+    if hq // hkv > 32:
         with pytest.raises(NotImplementedError):
             torch.ops.tt.paged_scaled_dot_product_attention_decode(
                 q.cuda(), kd, vd, table.cuda(), is_causal=False, attn_mask=mask_h.cuda(), cur_pos_tensor=cur.cuda())

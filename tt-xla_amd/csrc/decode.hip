@@ -474,14 +474,20 @@ static int decode_impl(void *out, int64_t out_user_stride, int64_t out_head_stri
   if (forced == 3 && mfma16_ok) use_mfma16 = true, use_mfma = false;
   if (mask) {
     // A mask is applied by the dot-product kernel (bfloat16 caches, up to 8 heads per group) and by
-    // the 16x16x32 kernel (either format, up to 16); a forced choice holds where it is built.
+    // the matrix-core kernels (either format; 16x16x32 up to 16 heads, 32x32x16 up to 32); a forced
+    // choice holds where it is built.
     const bool valu_ok = g <= 8 && kv_format == TTPA_KV_BF16;
-    if (!valu_ok && !mfma16_ok)
+    if (!valu_ok && !mfma16_ok && !mfma_ok)
       return fail(TTPA_ERR_UNSUPPORTED,
-                  "masked decode: %d query heads per KV head with this cache format and block size is not built "
-                  "(bfloat16 up to 8, or up to 16 on the matrix-core kernel's shapes)", g);
-    use_mfma = false;
-    use_mfma16 = mfma16_ok && (!valu_ok || forced == 3 || (forced != 1 && g >= 4));
+                  "masked decode: %d query heads per KV head with this cache format, head size and block size is not "
+                  "built (bfloat16 up to 8, or up to 32 on the matrix-core kernels' shapes)", g);
+    if (forced == 2 && mfma_ok) use_mfma = true, use_mfma16 = false;
+    else if (forced == 3 && mfma16_ok) use_mfma = false, use_mfma16 = true;
+    else if (forced == 1 && valu_ok) use_mfma = use_mfma16 = false;
+    else {
+      use_mfma16 = mfma16_ok && (g >= 4 || !valu_ok);
+      use_mfma = !use_mfma16 && !valu_ok;
+    }
   }
   // The matrix-core kernels get at most one workgroup per CU whatever the cache format: the 32x32
   // kernel fills the CU's LDS with one, and the 16x16 kernel streams as fast with one as with the

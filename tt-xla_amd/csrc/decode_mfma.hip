@@ -292,13 +292,25 @@ __global__ __launch_bounds__(256, 1) void paged_decode_mfma_kernel(
           if (key >= nvalid || key < nbelow) st[kb][r] = -INFINITY;
         }
     }
+    // > 0 or < 0: the maximum is tracked on scaled scores.  Block-float-8: the factors taken
+    // out of the K tile and out of Q come back here.
+    const float scale = BFP8 ? __builtin_ldexpf(a.scale_log2e, eref_k + eq - 260) : a.scale_log2e;
+    if (a.mask != nullptr) {  // an additive mask row per (user, head), brought to the units of the raw scores
+      const float unit = 1.4426950408889634f / scale;
+      const uint16_t *mrow = a.mask + cur.u * a.mask_us + (int64_t)(cur.h * G + min(n, G - 1)) * a.mask_hs +
+                             cur.t * kTile + 4 * h;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = 32 * kb + 8 * (r >> 2) + (r & 3);
+          if (key + 4 * h < nvalid) st[kb][r] += bf16_lo(mrow[key]) * unit;
+        }
+    }
     float mloc = fmaxf(st[0][0], st[1][0]);
 #pragma unroll
     for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(st[0][r], st[1][r]));
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-    // > 0 or < 0: the maximum is tracked on scaled scores.  Block-float-8: the factors taken
-    // out of the K tile and out of Q come back here.
-    const float scale = BFP8 ? __builtin_ldexpf(a.scale_log2e, eref_k + eq - 260) : a.scale_log2e;
     mloc *= scale;
     // a negative scale would turn the max into a min; scores are scaled before comparing then
     if (scale < 0.f) {

@@ -457,11 +457,8 @@ def _decode_masked(query, key, value, page_table, attn_mask, attention_sink, sca
     """Decode with ``is_causal=False``: every position of the user's table is attended, weighted by
     the additive ``attn_mask`` (anything that broadcasts to [users, heads, 1, table_width * block_size];
     reference CPU branch custom_ops.py:1296-1311; the one-token pass of a pooling / encoder model,
-    never the generative serving path).  Up to 16 query heads per KV head (either cache format) run
-    on the decode kernels with the mask as an operand.  Wider groups go through the prefill
-    kernel's masked dense form, with one mask row for all heads: the user's
-    blocks are gathered in table order (ids outside the cache read block 0, as in the kernels) and
-    the query token is the first row of a 32-row tile."""
+    never the generative serving path).  Up to 32 query heads per KV head (either cache format) run
+    on the decode kernels with the mask as an operand; the rest is _decode_masked_gathered."""
     if attn_mask is None:
         raise ValueError("attn_mask must be provided when is_causal is False")
     if attention_sink is not None or sliding_window_size is not None:
@@ -480,7 +477,8 @@ def _decode_masked(query, key, value, page_table, attn_mask, attention_sink, sca
     g = hq // hkv
     rows_per_load = max(1, 1024 // (d * (1 if fmt == N.KV_BFP8 else 2)))
     on_dot_kernel = fmt == N.KV_BF16 and g <= 8 and bs % 4 == 0
-    on_matrix_kernel = g <= 16 and d in (64, 128, 256) and bs % rows_per_load == 0 and users <= 2048
+    on_matrix_kernel = bs % rows_per_load == 0 and ((g <= 16 and d in (64, 128, 256) and users <= 2048) or
+                                                    (g <= 32 and d in (64, 128) and users <= 1024))
     if on_dot_kernel or on_matrix_kernel:
         q = _rows_contiguous(query)
         pt = _table(page_table)
@@ -499,9 +497,21 @@ def _decode_masked(query, key, value, page_table, attn_mask, attention_sink, sca
             ws.data_ptr(), ws_bytes, _stream(),
         )
         return out
+    return _decode_masked_gathered(query, key, value, page_table, mask, mask_hs, scale, out)
+
+
+def _decode_masked_gathered(query, key, value, page_table, mask, mask_hs, scale, out):
+    """What no decode kernel takes with a mask (more than 32 query heads per KV head, head size 256 with
+    more than 16, block sizes that split a 1 KiB load with more than 8 or on a block-float-8 cache):
+    the user's blocks gathered in table order, then the prefill kernel's masked dense form on a query
+    padded to its 32-row tile.  One mask row for all heads."""
     if mask_hs != 0:
         raise NotImplementedError(
-            "a decode attn_mask that differs between heads is built for up to 16 query heads per KV head")
+            "a decode attn_mask that differs between heads is built for up to 32 query heads per KV head")
+    nb, hkv, bs, d, fmt = _attention_cache_geometry(key)
+    _, users, hq, _ = query.shape
+    width = page_table.shape[1]
+    skv = width * bs
 
     ids = page_table.reshape(-1).to(torch.int64)
     ids = torch.where((ids >= 0) & (ids < nb), ids, torch.zeros_like(ids))
