@@ -333,10 +333,20 @@ struct Latent16 {
   static constexpr bool HALF_PERIOD = (ROW / 4) % 64 == 32;
   static_assert(STAGE % 1024 == 0 && (HALF_PERIOD ? CPR % 8 == 0 : ((ROW / 4) % 64 == 0 && CPR % 16 == 0)),
                 "row length the swizzle is not made for");
-  // position of chunk c of row r inside the row
-  __device__ static constexpr int position(int r, int c) {
-    return HALF_PERIOD ? (c ^ ((r >> 1) & 7)) : (c ^ (r & 15));
+  // position of chunk c of row r inside the row: c ^ swizzle(r).  Two kinds of reads must find their
+  // lanes in different banks (64 banks of 4 bytes), and the LDS of this part serves them in these
+  // lane groups (measured with SQ_LDS_BANK_CONFLICT on pairs of active lanes): a 16-byte read in four
+  // groups of 16 lanes, {0-3, 12-15, 20-27}, {4-11, 16-19, 28-31} and the same plus 32; an 8-byte
+  // (transposing) read in two groups of 32 lanes.  The A operand of the score product reads row n,
+  // chunk 4 i + quad; the transposing read of the value columns reads rows 4 quad .. 4 quad + 3, an
+  // aligned pair of chunks each.  Rows of 1152 or 384 bytes start 32 banks apart, rows of 256 bytes in
+  // the same bank; the two swizzles below leave both reads without a conflict (the plain
+  // (r >> 1) & 7 and r & 15 gave every transposing read a two-way conflict: twice its LDS time).
+  __device__ static constexpr int swizzle(int r) {
+    const int m = (r >> 1) & 7;
+    return HALF_PERIOD ? ((((m & 3) << 1) | (m >> 2)) ^ ((m >> 2) << 2)) : ((((r & 7) ^ ((r >> 3) << 2)) << 1) | ((r >> 3) & 1));
   }
+  __device__ static constexpr int position(int r, int c) { return c ^ swizzle(r & 15); }
 };
 
 template <int DQK, int DV>
@@ -715,7 +725,7 @@ __global__ __launch_bounds__(512) void paged_decode_latent128_kernel(
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(piece + vfrag[vb % VBASES] + 16 * GC * (vb / VBASES)));
   };
   constexpr int KPRE = KSTEPS < 4 ? KSTEPS : 4;
-  constexpr int VPRE = VB < 6 ? VB : 6;
+  constexpr int VPRE = VB < 4 ? VB : 4;
 
   Cursor cur = locate_unit(a, s_pref, s_len, x);
   bf16x8 qf[KSTEPS];
@@ -755,35 +765,39 @@ __global__ __launch_bounds__(512) void paged_decode_latent128_kernel(
       __syncthreads();
     }
     if (wave_active) {
+      // Two pieces (32 keys) per step: one softmax for both, and the second product takes them as the
+      // 32-deep K dimension of one matrix instruction per block of 16 value columns (k index 8 quad + j
+      // stands for key 4 quad + j of the first piece for j < 4, of the second otherwise: the order in
+      // which the score tiles hold a lane's keys and the transposing reads their rows).
 #pragma unroll 1
-      for (int sub = 0; sub < NSUB; ++sub) {
-        if (SUB * sub >= nvalid) break;
-        const unsigned char *piece = smem + buf * STAGE + sub * L::STAGE;
+      for (int half = 0; half < NSUB / 2; ++half) {
+        if (2 * SUB * half >= nvalid) break;
+        const unsigned char *piece = smem + buf * STAGE + 2 * half * L::STAGE;
         // ---- S^T = K . Q^T -------------------------------------------------------------------
-        floatx4 st = {0.f, 0.f, 0.f, 0.f};
-        {
+        floatx4 st[2];
+#pragma unroll
+        for (int pc = 0; pc < 2; ++pc) {
+          st[pc] = floatx4{0.f, 0.f, 0.f, 0.f};
+          const unsigned char *pp = piece + pc * L::STAGE;
           bf16x8 ring[KPRE];
 #pragma unroll
-          for (int s = 0; s < KPRE; ++s) ring[s] = read_k(piece, s);
+          for (int s = 0; s < KPRE; ++s) ring[s] = read_k(pp, s);
 #pragma unroll
           for (int s = 0; s < KSTEPS; ++s) {
-            st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % KPRE], qf[s], st, 0, 0, 0);
-            if (s + KPRE < KSTEPS) ring[s % KPRE] = read_k(piece, s + KPRE);
-          }
-#pragma unroll
-          for (int s = 0; s < KSTEPS; ++s) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (s + KPRE < KSTEPS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            st[pc] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % KPRE], qf[s], st[pc], 0, 0, 0);
+            if (s + KPRE < KSTEPS) ring[s % KPRE] = read_k(pp, s + KPRE);
           }
         }
-        // ---- online softmax: lane (head, quad) holds keys 16 sub + 4 quad + r ---------------------
-        float sc[4], mloc = -INFINITY;
+        // ---- online softmax: lane (head, quad) holds keys 32 half + 16 pc + 4 quad + r ------------
+        float sc[8], mloc = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int key = SUB * sub + 4 * quad + r;
-          sc[r] = (key >= nvalid || key < nbelow) ? -INFINITY : st[r] * scale;
-          mloc = fmaxf(mloc, sc[r]);
-        }
+        for (int pc = 0; pc < 2; ++pc)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int key = 2 * SUB * half + SUB * pc + 4 * quad + r;
+            sc[4 * pc + r] = (key >= nvalid || key < nbelow) ? -INFINITY : st[pc][r] * scale;
+            mloc = fmaxf(mloc, sc[4 * pc + r]);
+          }
         mloc = max_over_quads(mloc);
         const bool move = !(mloc - m_run <= 8.0f);  // (lazy: also true from -inf)
         const float m_new = move ? mloc : m_run;
@@ -791,13 +805,13 @@ __global__ __launch_bounds__(512) void paged_decode_latent128_kernel(
         const float alpha = move ? __builtin_amdgcn_exp2f(m_run - m_safe) : 1.0f;
         m_run = m_new;
         float lsum = 0.f;
-        shortx4 pf;
+        bf16x8 pf;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
+        for (int r = 0; r < 8; ++r) {
           const float p = __builtin_amdgcn_exp2f(sc[r] - m_safe);
           const __bf16 pb = (__bf16)p;
           lsum += (float)pb;  // the normaliser sums the weights that multiply V
-          pf[r] = __builtin_bit_cast(short, pb);
+          pf[r] = pb;
         }
         l_run = l_run * alpha + lsum;
         if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
@@ -806,18 +820,17 @@ __global__ __launch_bounds__(512) void paged_decode_latent128_kernel(
         }
         // ---- O^T += V^T . P^T -------------------------------------------------------------------
         {
-          shortx4 vring[VPRE];
+          shortx4 lo[VPRE], hi[VPRE];
 #pragma unroll
-          for (int vb = 0; vb < VPRE; ++vb) vring[vb] = read_v(piece, vb);
-#pragma unroll
-          for (int vb = 0; vb < VB; ++vb) {
-            acc[vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vring[vb % VPRE], pf, acc[vb], 0, 0, 0);
-            if (vb + VPRE < VB) vring[vb % VPRE] = read_v(piece, vb + VPRE);
-          }
+          for (int vb = 0; vb < VPRE; ++vb) lo[vb] = read_v(piece, vb), hi[vb] = read_v(piece + L::STAGE, vb);
 #pragma unroll
           for (int vb = 0; vb < VB; ++vb) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (vb + VPRE < VB) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            const bf16x4 l4 = __builtin_bit_cast(bf16x4, lo[vb % VPRE]), h4 = __builtin_bit_cast(bf16x4, hi[vb % VPRE]);
+            bf16x8 vf;
+            vf[0] = l4[0], vf[1] = l4[1], vf[2] = l4[2], vf[3] = l4[3];
+            vf[4] = h4[0], vf[5] = h4[1], vf[6] = h4[2], vf[7] = h4[3];
+            acc[vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[vb], 0, 0, 0);
+            if (vb + VPRE < VB) lo[vb % VPRE] = read_v(piece, vb + VPRE), hi[vb % VPRE] = read_v(piece + L::STAGE, vb + VPRE);
           }
         }
       }
@@ -891,12 +904,11 @@ struct LatentPrefillArgs {
   float scale_log2e;
 };
 
-template <int DQK, int DV, int RB>
-__global__ __launch_bounds__(512 / RB) void latent_prefill_kernel(LatentPrefillArgs a) {
+template <int DQK, int DV>
+__global__ __launch_bounds__(512) void latent_prefill_kernel(LatentPrefillArgs a) {
   using L = Latent16<DQK, DV>;
   typedef float floatx4 __attribute__((ext_vector_type(4)));
-  // RB blocks of 16 rows per wavefront: a K or V^T fragment read from LDS feeds RB matrix instructions
-  constexpr int SUB = L::TILE, NSUB = 4, KEYS = SUB * NSUB, NWAVES = 8 / RB, WROWS = 16 * RB, ROWS = WROWS * NWAVES;
+  constexpr int SUB = L::TILE, NSUB = 4, KEYS = SUB * NSUB, NWAVES = 8, ROWS = 16 * NWAVES;
   constexpr int KSTEPS = DQK / 32, VB = DV / 16;
   constexpr int PER_WAVE = NSUB * L::NDMA / NWAVES;
   static_assert(NSUB * L::NDMA % NWAVES == 0, "a tile's requests must divide among the wavefronts");
@@ -915,18 +927,13 @@ __global__ __launch_bounds__(512 / RB) void latent_prefill_kernel(LatentPrefillA
   const int grp = (int)blockIdx.x % groups;
   const int b = grp / a.nkv, kvh = grp - b * a.nkv;
 
-  const int r0 = blk * ROWS + wave * WROWS;
+  const int r0 = blk * ROWS + wave * 16;
   const bool wave_active = r0 < rows_total;
-  int t[RB], head[RB], limit[RB];
-  bool row_valid[RB];
-#pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-    const int r = min(r0 + 16 * rb + n, rows_total - 1);
-    t[rb] = r / G, head[rb] = kvh * G + (r - t[rb] * G);
-    row_valid[rb] = r0 + 16 * rb + n < rows_total;
-    limit[rb] = a.causal ? t[rb] : a.s - 1;
-  }
-  const int wave_limit = a.causal ? min(r0 + WROWS - 1, rows_total - 1) / G : a.s - 1;
+  const int r = min(r0 + n, rows_total - 1);
+  const int t = r / G, head = kvh * G + (r - t * G);
+  const bool row_valid = r0 + n < rows_total;
+  const int limit = a.causal ? t : a.s - 1;
+  const int wave_limit = a.causal ? min(r0 + 15, rows_total - 1) / G : a.s - 1;
   const int wg_limit = a.causal ? min(blk * ROWS + ROWS - 1, rows_total - 1) / G : a.s - 1;
   const int ntiles = wg_limit / KEYS + 1;
 
@@ -979,28 +986,22 @@ __global__ __launch_bounds__(512 / RB) void latent_prefill_kernel(LatentPrefillA
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(piece + vfrag[vb % VBASES] + 16 * GC * (vb / VBASES)));
   };
   constexpr int KPRE = KSTEPS < 4 ? KSTEPS : 4;
-  constexpr int VPRE = VB < 6 ? VB : 6;
+  constexpr int VPRE = VB < 4 ? VB : 4;
 
   request_tile(0, 0);
   // B operand of the score product: lane (row, quad) holds features 32 s + 8 quad .. + 7 of its row
-  bf16x8 qf[RB][KSTEPS];
-  const uint16_t *mrow[RB];
+  bf16x8 qf[KSTEPS];
+  {
+    const uint16_t *qp = a.q + b * a.q_bs + head * a.q_hs + (int64_t)t * a.q_ts + 8 * quad;
 #pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-    const uint16_t *qp = a.q + b * a.q_bs + head[rb] * a.q_hs + (int64_t)t[rb] * a.q_ts + 8 * quad;
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) qf[rb][s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 32 * s));
-    mrow[rb] = a.mask ? a.mask + b * a.mask_bs + head[rb] * a.mask_hs + (int64_t)t[rb] * a.mask_rs : nullptr;
+    for (int s = 0; s < KSTEPS; ++s) qf[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 32 * s));
   }
+  const uint16_t *mrow = a.mask ? a.mask + b * a.mask_bs + head * a.mask_hs + (int64_t)t * a.mask_rs : nullptr;
 
-  floatx4 acc[RB][VB];
-  float m_run[RB], l_run[RB];
+  floatx4 acc[VB];
 #pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-#pragma unroll
-    for (int i = 0; i < VB; ++i) acc[rb][i] = floatx4{0.f, 0.f, 0.f, 0.f};
-    m_run[rb] = -INFINITY, l_run[rb] = 0.f;
-  }
+  for (int i = 0; i < VB; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
   const float scale = a.scale_log2e;
 
   for (int tile = 0; tile < ntiles; ++tile) {
@@ -1009,126 +1010,109 @@ __global__ __launch_bounds__(512 / RB) void latent_prefill_kernel(LatentPrefillA
     __syncthreads();                      // ... everybody's has, and the other stage is free
     if (tile + 1 < ntiles) request_tile(tile + 1, buf ^ 1);
     if (!wave_active) continue;
+    // Two pieces (32 keys) per step: one softmax for both, and the second product takes them as the
+    // 32-deep K dimension of one matrix instruction per block of 16 value columns.  k index 8 quad + j
+    // of that instruction stands for key 4 quad + j of the first piece (j < 4) or of the second: the
+    // order in which the score tiles hold the keys of a lane, and the transposing reads their rows.
 #pragma unroll 1
-    for (int sub = 0; sub < NSUB; ++sub) {
-      const int key0 = tile * KEYS + sub * SUB;
+    for (int half = 0; half < NSUB / 2; ++half) {
+      const int key0 = tile * KEYS + 2 * half * SUB;
       if (key0 > wave_limit) break;
-      const unsigned char *piece = smem + buf * STAGE + sub * L::STAGE;
+      const unsigned char *piece = smem + buf * STAGE + 2 * half * L::STAGE;
       // ---- S^T = K . Q^T ---------------------------------------------------------------------
-      floatx4 st[RB];
+      floatx4 st[2];
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) st[rb] = floatx4{0.f, 0.f, 0.f, 0.f};
-      {
+      for (int pc = 0; pc < 2; ++pc) {
+        st[pc] = floatx4{0.f, 0.f, 0.f, 0.f};
+        const unsigned char *pp = piece + pc * L::STAGE;
         bf16x8 ring[KPRE];
 #pragma unroll
-        for (int s = 0; s < KPRE; ++s) ring[s] = read_k(piece, s);
+        for (int s = 0; s < KPRE; ++s) ring[s] = read_k(pp, s);
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
-#pragma unroll
-          for (int rb = 0; rb < RB; ++rb)
-            st[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % KPRE], qf[rb][s], st[rb], 0, 0, 0);
-          if (s + KPRE < KSTEPS) ring[s % KPRE] = read_k(piece, s + KPRE);
-        }
-#pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) {
-          __builtin_amdgcn_sched_group_barrier(0x008, RB, 0);
-          if (s + KPRE < KSTEPS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          st[pc] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % KPRE], qf[s], st[pc], 0, 0, 0);
+          if (s + KPRE < KSTEPS) ring[s % KPRE] = read_k(pp, s + KPRE);
         }
       }
-      // ---- online softmax: lane (row, quad) holds keys key0 + 4 quad + r of its row ------------
-      shortx4 pf[RB];
+      // ---- online softmax: lane (row, quad) holds keys key0 + 16 pc + 4 quad + i of its row ------
+      float sc[8], mloc = -INFINITY;
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        float sc[4], mloc = -INFINITY;
+      for (int pc = 0; pc < 2; ++pc) {
         float madd[4] = {0.f, 0.f, 0.f, 0.f};
-        if (mrow[rb]) {  // wavefront-uniform
-          const int kq = min(key0 + 4 * quad, a.s - 4);
-          const uint2 mw = *reinterpret_cast<const uint2 *>(mrow[rb] + kq);
+        if (mrow) {  // wavefront-uniform
+          const int kq = min(key0 + 16 * pc + 4 * quad, a.s - 4);
+          const uint2 mw = *reinterpret_cast<const uint2 *>(mrow + kq);
           madd[0] = bf16_lo(mw.x) * 1.4426950408889634f, madd[1] = bf16_hi(mw.x) * 1.4426950408889634f;
           madd[2] = bf16_lo(mw.y) * 1.4426950408889634f, madd[3] = bf16_hi(mw.y) * 1.4426950408889634f;
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int key = key0 + 4 * quad + i;
-          sc[i] = key > limit[rb] ? -INFINITY : st[rb][i] * scale + madd[i];
-          mloc = fmaxf(mloc, sc[i]);
+          const int key = key0 + 16 * pc + 4 * quad + i;
+          sc[4 * pc + i] = key > limit ? -INFINITY : st[pc][i] * scale + madd[i];
+          mloc = fmaxf(mloc, sc[4 * pc + i]);
         }
-        mloc = max_over_quads(mloc);
-        const bool move = !(mloc - m_run[rb] <= 8.0f);  // (lazy: also true from -inf)
-        const float m_new = move ? mloc : m_run[rb];
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = move ? __builtin_amdgcn_exp2f(m_run[rb] - m_safe) : 1.0f;
-        m_run[rb] = m_new;
-        float lsum = 0.f;
+      }
+      mloc = max_over_quads(mloc);
+      const bool move = !(mloc - m_run <= 8.0f);  // (lazy: also true from -inf)
+      const float m_new = move ? mloc : m_run;
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = move ? __builtin_amdgcn_exp2f(m_run - m_safe) : 1.0f;
+      m_run = m_new;
+      float lsum = 0.f;
+      bf16x8 pf;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float pr = __builtin_amdgcn_exp2f(sc[i] - m_safe);
-          const __bf16 pb = (__bf16)pr;
-          lsum += (float)pb;
-          pf[rb][i] = __builtin_bit_cast(short, pb);
-        }
-        l_run[rb] = l_run[rb] * alpha + lsum;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+      for (int i = 0; i < 8; ++i) {
+        const float pr = __builtin_amdgcn_exp2f(sc[i] - m_safe);
+        const __bf16 pb = (__bf16)pr;
+        lsum += (float)pb;
+        pf[i] = pb;
+      }
+      l_run = l_run * alpha + lsum;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-          for (int i = 0; i < VB; ++i) acc[rb][i] *= alpha;
-        }
+        for (int i = 0; i < VB; ++i) acc[i] *= alpha;
       }
       // ---- O^T += V^T . P^T ---------------------------------------------------------------------
       {
-        shortx4 vring[VPRE];
+        shortx4 lo[VPRE], hi[VPRE];
 #pragma unroll
-        for (int vb = 0; vb < VPRE; ++vb) vring[vb] = read_v(piece, vb);
-#pragma unroll
-        for (int vb = 0; vb < VB; ++vb) {
-#pragma unroll
-          for (int rb = 0; rb < RB; ++rb)
-            acc[rb][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vring[vb % VPRE], pf[rb], acc[rb][vb], 0, 0, 0);
-          if (vb + VPRE < VB) vring[vb % VPRE] = read_v(piece, vb + VPRE);
-        }
+        for (int vb = 0; vb < VPRE; ++vb) lo[vb] = read_v(piece, vb), hi[vb] = read_v(piece + L::STAGE, vb);
 #pragma unroll
         for (int vb = 0; vb < VB; ++vb) {
-          __builtin_amdgcn_sched_group_barrier(0x008, RB, 0);
-          if (vb + VPRE < VB) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          const bf16x4 l4 = __builtin_bit_cast(bf16x4, lo[vb % VPRE]), h4 = __builtin_bit_cast(bf16x4, hi[vb % VPRE]);
+          bf16x8 vf;
+          vf[0] = l4[0], vf[1] = l4[1], vf[2] = l4[2], vf[3] = l4[3];
+          vf[4] = h4[0], vf[5] = h4[1], vf[6] = h4[2], vf[7] = h4[3];
+          acc[vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[vb], 0, 0, 0);
+          if (vb + VPRE < VB) lo[vb % VPRE] = read_v(piece, vb + VPRE), hi[vb % VPRE] = read_v(piece + L::STAGE, vb + VPRE);
         }
       }
     }
   }
   if (!wave_active) return;
   // ---- normalise and store: lane (row, quad) holds values 16 vb + 4 quad .. + 3 of its row --------
+  const float l_tot = sum_over_quads(l_run);
+  const float inv = 1.0f / l_tot;
+  if (row_valid) {
+    uint16_t *op = a.out + b * a.out_bs + head * a.out_hs + (int64_t)t * a.out_ts + 4 * quad;
 #pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-    const float l_tot = sum_over_quads(l_run[rb]);
-    const float inv = 1.0f / l_tot;
-    if (row_valid[rb]) {
-      uint16_t *op = a.out + b * a.out_bs + head[rb] * a.out_hs + (int64_t)t[rb] * a.out_ts + 4 * quad;
-#pragma unroll
-      for (int vb = 0; vb < VB; ++vb)
-        *reinterpret_cast<uint2 *>(op + 16 * vb) = make_uint2(pack_bf16x2(acc[rb][vb][0] * inv, acc[rb][vb][1] * inv),
-                                                              pack_bf16x2(acc[rb][vb][2] * inv, acc[rb][vb][3] * inv));
-    }
+    for (int vb = 0; vb < VB; ++vb)
+      *reinterpret_cast<uint2 *>(op + 16 * vb) =
+          make_uint2(pack_bf16x2(acc[vb][0] * inv, acc[vb][1] * inv), pack_bf16x2(acc[vb][2] * inv, acc[vb][3] * inv));
   }
-}
-
-template <int DQK, int DV, int RB>
-int launch_latent_prefill_rb(const LatentPrefillArgs &a, hipStream_t st) {
-  using L = Latent16<DQK, DV>;
-  const size_t lds = 2 * 4 * (size_t)L::STAGE;
-  static std::atomic<uint64_t> lds_ready{0};
-  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&latent_prefill_kernel<DQK, DV, RB>), lds, lds_ready))
-    return fail(TTPA_ERR_LAUNCH, "latent prefill: cannot reserve %zu bytes of LDS", lds);
-  const int64_t rows = (int64_t)(a.heads / a.nkv) * a.s;
-  const int64_t grid = (rows + 127) / 128 * a.batch * a.nkv;
-  launch_dominant(&latent_prefill_kernel<DQK, DV, RB>, dim3((unsigned)grid), dim3(512 / RB), lds, st, a);
-  return check_launch("latent_prefill");
 }
 
 template <int DQK, int DV>
 int launch_latent_prefill(const LatentPrefillArgs &a, hipStream_t st) {
-  // One block of 16 rows per wavefront.  With two (a fragment read from LDS feeding two matrix
-  // instructions, four wavefronts of 512 registers) the 256 accumulators and 144 Q registers of the
-  // (576, 512) shape leave the compiler too little: it keeps Q in scratch memory and the kernel runs
-  // eight times slower (4.3 ms against 0.54 on 4 x 2048 tokens, 16 heads).
-  return launch_latent_prefill_rb<DQK, DV, 1>(a, st);
+  using L = Latent16<DQK, DV>;
+  const size_t lds = 2 * 4 * (size_t)L::STAGE;
+  static std::atomic<uint64_t> lds_ready{0};
+  if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&latent_prefill_kernel<DQK, DV>), lds, lds_ready))
+    return fail(TTPA_ERR_LAUNCH, "latent prefill: cannot reserve %zu bytes of LDS", lds);
+  const int64_t rows = (int64_t)(a.heads / a.nkv) * a.s;
+  const int64_t grid = (rows + 127) / 128 * a.batch * a.nkv;
+  launch_dominant(&latent_prefill_kernel<DQK, DV>, dim3((unsigned)grid), dim3(512), lds, st, a);
+  return check_launch("latent_prefill");
 }
 
 template <int DQK, int DVW, bool SHARED_V>
