@@ -178,6 +178,19 @@ __device__ __forceinline__ void dma16_streaming_quad(const void *const (&bases)[
         "s"(bases[1]), "s"(bases[2]), "s"(bases[3]), "s"(lds_addr)
       : "memory", "m0");
 }
+// The same without the non-temporal hint (tiles that other workgroups read again).
+__device__ __forceinline__ void dma16_quad(const void *const (&bases)[4], const uint32_t (&lane_bytes)[4], uint32_t lds_addr) {
+  asm volatile(
+      "s_mov_b32 m0, %8\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, %4\n\t"
+      "global_load_lds_dwordx4 %1, %5 offset:1024\n\t"
+      "global_load_lds_dwordx4 %2, %6 offset:2048\n\t"
+      "global_load_lds_dwordx4 %3, %7 offset:3072"
+      :
+      : "v"(lane_bytes[0]), "v"(lane_bytes[1]), "v"(lane_bytes[2]), "v"(lane_bytes[3]), "s"(bases[0]),
+        "s"(bases[1]), "s"(bases[2]), "s"(bases[3]), "s"(lds_addr)
+      : "memory", "m0");
+}
 // The same for callers whose base / LDS address the compiler cannot prove uniform: both are
 // read from the first active lane, the address word by word (address_from_words).
 __device__ __forceinline__ void dma16_uniform(const void *uniform_base, uint32_t lane_bytes, uint32_t lds_addr) {

@@ -451,33 +451,40 @@ __global__ inline __launch_bounds__(256) void decode_combine_bf16_kernel(DecodeA
     *out = 0x7fc07fc0u;
     return;
   }
-  constexpr int kBatch = 8;
   const float *base = a.ws_slots + (int64_t)first * a.slot_floats;
   float mall = -INFINITY, num0 = 0.f, num1 = 0.f, den = 0.f;
-  for (int w = 0; w < nw; w += kBatch) {
-    float mv[kBatch], lv[kBatch];
-    uint32_t av[kBatch];
+  // partials are read in batches so that their loads overlap; a segment that few ranges share (the
+  // 128-head latent form: two or three) takes batches of its size instead of eight mostly repeated loads
+  auto merge = [&](auto batch_tag) {
+    constexpr int kBatch = decltype(batch_tag)::value;
+    for (int w = 0; w < nw; w += kBatch) {
+      float mv[kBatch], lv[kBatch];
+      uint32_t av[kBatch];
 #pragma unroll
-    for (int j = 0; j < kBatch; ++j) {
-      const float *sl = base + (int64_t)min(w + j, nw - 1) * a.slot_floats;
-      mv[j] = (w + j < nw) ? sl[pairs + g] : -INFINITY;
-      lv[j] = sl[pairs + G + g];
-      av[j] = reinterpret_cast<const uint32_t *>(sl)[p];
+      for (int j = 0; j < kBatch; ++j) {
+        const float *sl = base + (int64_t)min(w + j, nw - 1) * a.slot_floats;
+        mv[j] = (w + j < nw) ? sl[pairs + g] : -INFINITY;
+        lv[j] = sl[pairs + G + g];
+        av[j] = reinterpret_cast<const uint32_t *>(sl)[p];
+      }
+      float mnew = mall;
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) mnew = fmaxf(mnew, mv[j]);
+      const float resc = __builtin_amdgcn_exp2f(mall - mnew);
+      num0 *= resc, num1 *= resc, den *= resc;
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const float wgt = __builtin_amdgcn_exp2f(mv[j] - mnew);  // 0 for the padding entries
+        num0 = fmaf(wgt, bf16_lo(av[j]), num0);
+        num1 = fmaf(wgt, bf16_hi(av[j]), num1);
+        den = fmaf(wgt, lv[j], den);
+      }
+      mall = mnew;
     }
-    float mnew = mall;
-#pragma unroll
-    for (int j = 0; j < kBatch; ++j) mnew = fmaxf(mnew, mv[j]);
-    const float resc = __builtin_amdgcn_exp2f(mall - mnew);
-    num0 *= resc, num1 *= resc, den *= resc;
-#pragma unroll
-    for (int j = 0; j < kBatch; ++j) {
-      const float wgt = __builtin_amdgcn_exp2f(mv[j] - mnew);  // 0 for the padding entries
-      num0 = fmaf(wgt, bf16_lo(av[j]), num0);
-      num1 = fmaf(wgt, bf16_hi(av[j]), num1);
-      den = fmaf(wgt, lv[j], den);
-    }
-    mall = mnew;
-  }
+  };
+  if (nw <= 2) merge(std::integral_constant<int, 2>{});
+  else if (nw <= 4) merge(std::integral_constant<int, 4>{});
+  else merge(std::integral_constant<int, 8>{});
   if (a.sink) {
     const float sk = a.sink[h * G + g] * 1.4426950408889634f;
     const float mnew = fmaxf(mall, sk);

@@ -683,8 +683,14 @@ __global__ __launch_bounds__(512) void paged_decode_latent128_kernel(
         __builtin_amdgcn_readfirstlane((int)(uint32_t)addr), __builtin_amdgcn_readfirstlane((int)(uint32_t)(addr >> 32))));
     const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(
         (int)(lds0 + (uint32_t)(buf * STAGE + sub_w * L::STAGE + 1024 * (wave & 1) * PER_WAVE)));
+    const void *bases[4] = {src, src - 1024, src - 2048, src - 3072};
 #pragma unroll
-    for (int j = 0; j < PER_WAVE; ++j) dma16_streaming(src, src_off[j], dst + 1024u * j);
+    for (int j = 0; j + 4 <= PER_WAVE; j += 4) {
+      const uint32_t off[4] = {src_off[j], src_off[j + 1], src_off[j + 2], src_off[j + 3]};
+      dma16_streaming_quad(bases, off, dst + 1024u * j);
+    }
+#pragma unroll
+    for (int j = PER_WAVE / 4 * 4; j < PER_WAVE; ++j) dma16_streaming(src, src_off[j], dst + 1024u * j);
   };
   // Rows past the attended length may be cache rows nobody ever wrote: their scores are masked,
   // but as V rows they would turn 0 * Inf into NaN, so they are cleared in LDS.
@@ -953,8 +959,16 @@ __global__ __launch_bounds__(512) void latent_prefill_kernel(LatentPrefillArgs a
     const uint32_t dst0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)(buf * STAGE + 1024 * wave * PER_WAVE)));
     if ((tile + 1) * KEYS <= a.s) {
       const uint16_t *tile_base = kbase_g + (int64_t)tile * KEYS * a.k_ts;
+      // (four requests behind one write of M0: the instruction offset moves the LDS address too)
+      const char *tb = reinterpret_cast<const char *>(tile_base);
+      const void *bases[4] = {tb, tb - 1024, tb - 2048, tb - 3072};
 #pragma unroll
-      for (int j = 0; j < PER_WAVE; ++j) dma16(tile_base, req_off[j], dst0 + 1024u * j);
+      for (int j = 0; j + 4 <= PER_WAVE; j += 4) {
+        const uint32_t off[4] = {req_off[j], req_off[j + 1], req_off[j + 2], req_off[j + 3]};
+        dma16_quad(bases, off, dst0 + 1024u * j);
+      }
+#pragma unroll
+      for (int j = PER_WAVE / 4 * 4; j < PER_WAVE; ++j) dma16(tile_base, req_off[j], dst0 + 1024u * j);
     } else {
 #pragma unroll 1
       for (int j = 0; j < PER_WAVE; ++j) {
