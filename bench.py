@@ -52,13 +52,13 @@ MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
     # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
     # the rotating workload copies; the summaries under profiles/ hold the runs)
-    "config2": ("paged_decode_mfma16_kernel", "be3a15e04ef564b8", 310439571),
-    "config5": ("paged_decode_mfma16_kernel", "be3a15e04ef564b8", 168447693),
-    "config4": ("paged_decode_mfma16_kernel", "be3a15e04ef564b8", 3415584888),
-    "config3": ("prefill_kernel", "82cebe7e857b87ff", 244479198),
-    "latent": ("paged_decode_latent16_kernel", "0168059ef989a648", 654196617),
-    "latent128": ("paged_decode_latent128_kernel", "0168059ef989a648", 749333547),
-    "latent-prefill": ("latent_prefill_kernel", "0168059ef989a648", 333087947),
+    "config2": ("paged_decode_mfma16_kernel", "57ce30f89c503559", 310427869),
+    "config5": ("paged_decode_mfma16_kernel", "57ce30f89c503559", 168440746),
+    "config4": ("paged_decode_mfma16_kernel", "57ce30f89c503559", 3415570646),
+    "config3": ("prefill_kernel", "9e5dc9fce6518e7f", 244533644),
+    "latent": ("paged_decode_latent16_kernel", "a11e3796954bf311", 654198535),
+    "latent128": ("paged_decode_latent128_kernel", "a11e3796954bf311", 749341479),
+    "latent-prefill": ("latent_prefill_kernel", "a11e3796954bf311", 332749770),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}
