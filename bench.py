@@ -44,8 +44,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 KERNEL_SOURCES = {
     "paged_decode_mfma16_kernel": ["decode_mfma16_kernel.h", "decode_common.h", "common.h", "decode.hip"],  # the grid rule is in decode.hip
     "paged_decode_latent16_kernel": ["decode_wide.hip", "decode_common.h", "common.h"],
-    "paged_decode_latent128_kernel": ["decode_wide.hip", "decode_common.h", "common.h"],
-    "latent_prefill_kernel": ["decode_wide.hip", "decode_common.h", "common.h"],
+    "paged_decode_latent128_kernel": ["decode_wide.hip", "gen_latent_frag.py", "decode_common.h", "common.h"],
+    "latent_prefill_kernel": ["decode_wide.hip", "gen_latent_frag.py", "decode_common.h", "common.h"],
     "prefill_kernel": ["prefill.hip", "gen_prefill_stream.py", "common.h"],
 }
 MEASURED_TRAFFIC = {

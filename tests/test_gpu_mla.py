@@ -96,8 +96,8 @@ def test_mla_decode_16_heads_either_partial_format(monkeypatch, partials, dv):
 
 @pytest.mark.parametrize("kernel,partials", [("", "bf16"), ("", "f32"), ("wide", "f32")])
 def test_mla_decode_128_heads_every_form(monkeypatch, kernel, partials):
-    """All 128 heads of a latent layer on one GPU: the form in which eight wavefronts of a workgroup take
-    16 heads each on shared K tiles, with bfloat16 and with float partials, and the older form it
+    """All 128 heads of a latent layer on one GPU: the form in which four wavefronts of a workgroup take
+    32 heads each on shared K, with bfloat16 and with float partials, and the older form it
     replaced (TTPA_LATENT_KERNEL=wide: blocks of 32 heads, every score computed four times), which still
     serves masks and a separate V.  Contexts from one token to several tiles per workgroup range."""
     monkeypatch.setenv("TTPA_LATENT_PARTIALS", partials)
@@ -123,6 +123,22 @@ def test_mla_decode_128_heads_every_form(monkeypatch, kernel, partials):
                                               pos.cuda(), None, None).cpu()
     want = O.paged_flash_mla_decode(q, key, dv, table, None, pos, None)
     _check(f"mla decode 128 heads kernel={kernel or 'default'} partials={partials}", got, want)
+
+
+def test_mla_decode_128_heads_negative_scale():
+    """scale < 0: the softmax between the matrix instructions assumes a positive scale, so every step
+    must take the other one."""
+    users, hq, dh, dv, bs, width = 2, 128, 576, 512, 64, 8
+    g = torch.Generator().manual_seed(99)
+    nb = users * width
+    q = (_bf(g, 1, users, hq, dh).float() * 0.2).to(torch.bfloat16)
+    key = _bf(g, nb, 1, bs, dh)
+    table = torch.randperm(nb, generator=g).view(users, width).to(torch.int32)
+    pos = torch.tensor([500, 77], dtype=torch.int32)
+    got = torch.ops.tt.paged_flash_mla_decode(q.cuda(), key.cuda(), dv, table.cuda(), None, True, None,
+                                              pos.cuda(), None, -0.5).cpu()
+    want = O.paged_flash_mla_decode(q, key, dv, table, None, pos, -0.5)
+    _check("mla decode 128 heads, negative scale", got, want)
 
 
 def test_mla_decode_padded_row_sink_and_errors():
@@ -176,6 +192,35 @@ def test_flash_mla_prefill(b, hq, s, dh, nkv, dv, has_value):
     assert got.shape == (b, hq, s, dv)
     want = O.flash_mla_prefill(q.float(), k.float(), dv, None if v is None else v.float(), None, True, 1.0)
     _check(f"mla prefill b{b} h{hq} s{s} dh{dh} dv{dv}", got, want)
+
+
+@pytest.mark.parametrize("b,hq,s,dh,nkv,dv,scale", [
+    (1, 16, 224, 576, 1, 512, 1.0),     # every key for every row: all steps but a wavefront's first take the softmax
+    (2, 16, 96, 192, 1, 128, 1.0),      # that sits between the matrix instructions
+    (1, 32, 96, 128, 1, 128, 1.0),
+])
+def test_flash_mla_prefill_without_causal_limit(b, hq, s, dh, nkv, dv, scale):
+    """The operator accepts is_causal=False only together with a mask (reference custom_ops.py:723-726);
+    the library entry point below it also takes neither, which is the case where the masked softmax of
+    the kernel is left to a wavefront's first step: called directly."""
+    from tt_xla_amd import _native as N
+
+    print(f"case: mla prefill, every key, b{b} h{hq} s{s} dh{dh} dv{dv} scale{scale}", flush=True)
+    g = torch.Generator().manual_seed(7 * s + dh)
+    q = (_bf(g, b, hq, s, dh).float() * 0.15).to(torch.bfloat16)
+    k = _bf(g, b, nkv, s, dh)
+    qd, kd = q.cuda(), k.cuda()
+    out = torch.empty(b, hq, s, dv, dtype=torch.bfloat16, device="cuda")
+    N.call(
+        "ttpa_latent_prefill",
+        out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
+        qd.data_ptr(), qd.stride(0), qd.stride(1), qd.stride(2),
+        kd.data_ptr(), kd.stride(0), kd.stride(1), kd.stride(2),
+        0, 0, 0, 0, b, hq, nkv, s, dh, dv, 0, float(scale) * 1.0, torch.cuda.current_stream().cuda_stream,
+    )
+    torch.cuda.synchronize()
+    want = O.flash_mla_prefill(q.float(), k.float(), dv, None, None, False, scale)
+    _check(f"mla prefill, every key, s{s} dh{dh} dv{dv} scale{scale}", out.cpu(), want)
 
 
 MASKED_PREFILL = [

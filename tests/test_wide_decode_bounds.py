@@ -253,34 +253,43 @@ def test_every_address_of_the_16_head_form_stays_in_bounds(dqk, dv, sep_v, hq, n
     assert (waves * cus - 1) + (segs - 1) < waves * cus + segs     # slot index = wavefront + segment
 
 
-# ---- the 128-head form and the prefill kernel: eight wavefronts on shared tiles of four 16-row pieces ----
-def _shared_tile_checks(dqk, dv):
-    """What both kernels share: the stage of four pieces laid out like the 16-head form's, every chunk
-    of a tile requested exactly once by the wavefronts' shares, destinations inside the stage."""
-    row_bytes, sub, nsub, waves = 2 * dqk, 16, 4, 8
+# ---- the 128-head form and the prefill kernel: four wavefronts on shared steps of two 16-row pieces ----
+STEP_KEYS, STAGES, WAVES_SHARED, WAVE_ROWS = 32, 4, 4, 32
+
+
+def _shared_step_checks(dqk, dv):
+    """What both kernels share: a ring of four stages, each the two pieces of a step laid out like the
+    16-head form's stage, every chunk of a step requested exactly once by the wavefronts' shares
+    (wavefronts 2 i and 2 i + 1 fetch piece i), destinations inside the stage."""
+    row_bytes, sub, npieces, waves = 2 * dqk, 16, STEP_KEYS // 16, WAVES_SHARED
     cpr = row_bytes // 16
     piece = sub * row_bytes
     ndma = piece // 1024
-    stage = nsub * piece
-    assert piece % 1024 == 0 and (nsub * ndma) % waves == 0
-    per_wave = nsub * ndma // waves
-    assert STATIC_LDS + 2 * stage <= LDS_PER_CU
+    stage = npieces * piece
+    assert piece % 1024 == 0 and (npieces * ndma) % waves == 0
+    per_wave = npieces * ndma // waves
+    assert 2 * per_wave == ndma and per_wave < 16       # (the wait for a step counts the next step's requests: 4 bits)
+    assert STATIC_LDS + STAGES * stage <= LDS_PER_CU
     seen = set()
     for wave in range(waves):
         for j in range(per_wave):
             k = wave * per_wave + j
             piece_i, kk = k // ndma, k % ndma
+            assert piece_i == wave >> 1 and kk == (wave & 1) * per_wave + j
             for lane in range(64):
                 pos = 64 * kk + lane
                 rr, p = pos // cpr, pos % cpr
                 assert rr < sub
-                off = (sub * piece_i + rr, _position(row_bytes, rr, p))      # (row of the tile, chunk of the row)
+                off = (sub * piece_i + rr, _position(row_bytes, rr, p))      # (row of the step, chunk of the row)
                 assert off[1] < cpr
                 seen.add(off)
-            for buf in (0, 1):
-                dst = STATIC_LDS + buf * stage + 1024 * k
-                assert dst % 16 == 0 and dst + 1024 <= STATIC_LDS + (buf + 1) * stage <= LDS_PER_CU
-    assert len(seen) == nsub * sub * cpr, "every chunk of the tile is fetched exactly once"
+            for i in range(STAGES):
+                dst = STATIC_LDS + i * stage + 1024 * k
+                assert dst % 16 == 0 and dst + 1024 <= STATIC_LDS + (i + 1) * stage <= LDS_PER_CU
+    assert len(seen) == npieces * sub * cpr, "every chunk of the step is fetched exactly once"
+    # fragment reads of a lane: immediate offsets of the assembly blocks stay below 64 KiB
+    gc = 8 if (row_bytes // 4) % 64 == 32 else 16
+    assert piece + 16 * gc * (dqk // 32 // (gc // 4)) < 65536 and piece + 16 * gc * (dv // 16 // (gc // 2)) < 65536
     return row_bytes, piece, stage, per_wave, ndma
 
 
@@ -291,16 +300,15 @@ def test_the_128_head_form_is_exercised():
 
 @pytest.mark.parametrize("dqk,dv,sep_v,hq,nkv,bs,width,nb,users", SHAPES_128)
 def test_every_address_of_the_128_head_form_stays_in_bounds(dqk, dv, sep_v, hq, nkv, bs, width, nb, users):
-    row_bytes, piece, stage, per_wave, ndma = _shared_tile_checks(dqk, dv)
-    assert 2 * per_wave == ndma, "wavefronts 2 i and 2 i + 1 fetch piece i"
+    row_bytes, piece, stage, per_wave, ndma = _shared_step_checks(dqk, dv)
     g = hq // nkv
     nhb, gseg = (1, g) if g <= 128 else (g // 128, 128)
     assert nhb * gseg == g
     cache_bytes = nb * nkv * bs * row_bytes
     cap = width * bs
-    for t in {0, (cap - 1) // K_TILE}:
-        for wave in range(8):
-            tok0 = t * K_TILE + 16 * (wave >> 1)
+    for t, half in itertools.product({0, (cap - 1) // K_TILE}, (0, 1)):
+        for wave in range(WAVES_SHARED):
+            tok0 = t * K_TILE + STEP_KEYS * half + 16 * (wave >> 1)
             col = tok0 // bs
             assert tok0 - col * bs + 16 <= bs, "a piece lies inside one block"
             for phys, kvh in itertools.product({0, nb - 1}, {0, nkv - 1}):
@@ -310,8 +318,8 @@ def test_every_address_of_the_128_head_form_stays_in_bounds(dqk, dv, sep_v, hq, 
     vb = dv // 16
     slot_floats = (gseg * dv + 2 * gseg + 3) // 4 * 4
     slot_floats_bf16 = (gseg * dv // 2 + 2 * gseg + 3) // 4 * 4
-    for wave, n, quad in itertools.product(range(8), (0, 15), (0, 3)):
-        hg = 16 * wave + n
+    for wave, rb, n, quad in itertools.product(range(WAVES_SHARED), (0, 1), (0, 15), (0, 3)):
+        hg = WAVE_ROWS * wave + 16 * rb + n
         if hg < gseg:
             assert hg * dv + 4 * quad + 16 * (vb - 1) + 4 <= gseg * dv
             assert gseg * dv + gseg + hg < slot_floats
@@ -328,20 +336,20 @@ PREFILL_SHAPES = [(dh, dv, hq, nkv, s, b) for b, hq, s, dh, nkv, dv, has_v in G.
 
 @pytest.mark.parametrize("dqk,dv,hq,nkv,s,batch", sorted(set(PREFILL_SHAPES)))
 def test_every_address_of_the_prefill_kernel_stays_in_bounds(dqk, dv, hq, nkv, s, batch):
-    row_bytes, piece, stage, per_wave, ndma = _shared_tile_checks(dqk, dv)
+    row_bytes, piece, stage, per_wave, ndma = _shared_step_checks(dqk, dv)
     g = hq // nkv
     rows_total = g * s
     nblk = (rows_total + 127) // 128
     k_bytes = s * row_bytes                      # one (batch entry, KV head) of a contiguous K
     for blk in {0, nblk - 1}:
         last_row = min(blk * 128 + 127, rows_total - 1)
-        ntiles = (last_row // g) // K_TILE + 1
-        for tile in {0, ntiles - 1}:
-            for r in (0, 63):
-                key = min(tile * K_TILE + r, s - 1)
+        nsteps = (last_row // g) // STEP_KEYS + 1
+        for step in {0, nsteps - 1}:
+            for r in (0, STEP_KEYS - 1):
+                key = min(step * STEP_KEYS + r, s - 1)
                 assert key * row_bytes + row_bytes <= k_bytes
-        for wave, n in itertools.product(range(8), range(16)):
-            r = min(blk * 128 + 16 * wave + n, rows_total - 1)
+        for wave, rb, n in itertools.product(range(WAVES_SHARED), (0, 1), range(16)):
+            r = min(blk * 128 + WAVE_ROWS * wave + 16 * rb + n, rows_total - 1)
             t, head = r // g, r % g
             assert 0 <= t < s and head < g
             assert 32 * (dqk // 32 - 1) + 8 * 3 + 8 <= dqk and 16 * (dv // 16 - 1) + 4 * 3 + 4 <= dv

@@ -18,6 +18,7 @@
 #include "decode_common.h"
 
 #include <cstdlib>
+#include <utility>
 
 namespace ttpa {
 namespace decode {
@@ -620,23 +621,162 @@ bool launch_latent16(const DecodeArgs &a, const WideArgs &w, hipStream_t st) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// The arithmetic of one wavefront of the two kernels below on one step of 32 keys (two 16-row pieces
+// of K in LDS): the Q fragments of its two blocks of 16 rows, the running maxima and sums, and the
+// two products as the assembly blocks of build/latent_frag_asm.h (written by gen_latent_frag.py,
+// which says why assembly and where everything lives).  The output accumulators are registers that
+// no variable stands for: clear, scale, read16 and the second products are all that touches them.
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+#include "build/latent_frag_asm.h"
+
+template <int... Is, class F>
+__device__ __forceinline__ void static_for(std::integer_sequence<int, Is...>, F &&f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+
+template <int DQK, int DV>
+struct LatentMath {
+  using L = Latent16<DQK, DV>;
+  using B = LatentBlocks<DQK, DV>;
+  static constexpr int RB = 2;  // blocks of 16 rows
+  static constexpr int KSTEPS = DQK / 32, VB = DV / 16;
+  static constexpr int GC = L::HALF_PERIOD ? 8 : 16;  // chunks per swizzle group
+  static constexpr int KB = GC / 4, VBASES = GC / 2;
+  static constexpr int NQ16 = KSTEPS / 4, NA = VB / 4;
+  static constexpr int REQUESTS = B::REQUESTS;  // LDS-DMA requests of a wavefront per step
+  static_assert(VB % 4 == 0 && NQ16 >= 1 && (KSTEPS % 4 == 0 || KSTEPS % 4 == 2), "register blocks of 16");
+  u32x16 q16[RB][NQ16];
+  u32x8 q8[RB];
+  floatx4 ml;                         // running maxima (0, 1) and sums (2, 3) of the two row blocks
+  uint32_t kfrag[KB], vfrag[VBASES];  // the lane's fragment offsets inside a piece
+
+  // lane (n, quad): A operand of the score product = row n, chunk 4 s + quad; transposing read of
+  // the value columns = row 4 quad + n / 4, values 16 vb + 4 (n % 4) ..
+  __device__ __forceinline__ void init(int n, int quad) {
+#pragma unroll
+    for (int i = 0; i < KB; ++i) kfrag[i] = (uint32_t)(n * L::ROW + 16 * L::position(n, 4 * i + quad));
+    const int rv = 4 * quad + (n >> 2), q4 = n & 3;
+#pragma unroll
+    for (int i = 0; i < VBASES; ++i)
+      vfrag[i] = (uint32_t)(rv * L::ROW + 16 * L::position(rv, 2 * i + (q4 >> 1)) + 8 * (q4 & 1));
+#pragma unroll
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+      for (int r = 0; r < 8; ++r) q8[b][r] = 0;
+    restart();
+  }
+  __device__ __forceinline__ void restart() {
+    B::clear();
+    ml = floatx4{-INFINITY, -INFINITY, 0.f, 0.f};
+  }
+  // B operand of the score product: features 32 s + 8 quad .. + 7 of the lane's row in block b
+  __device__ __forceinline__ void set_q(int b, int s, const uint4 &t) {
+    if (s < 4 * NQ16) {
+      q16[b][s / 4][4 * (s % 4)] = t.x, q16[b][s / 4][4 * (s % 4) + 1] = t.y;
+      q16[b][s / 4][4 * (s % 4) + 2] = t.z, q16[b][s / 4][4 * (s % 4) + 3] = t.w;
+    } else {
+      const int j = 4 * (s - 4 * NQ16);
+      q8[b][j] = t.x, q8[b][j + 1] = t.y, q8[b][j + 2] = t.z, q8[b][j + 3] = t.w;
+    }
+  }
+  __device__ __forceinline__ float maximum(int b) const { return ml[b]; }
+  __device__ __forceinline__ float sum(int b) const { return ml[RB + b]; }
+  // f[4 j + r] = value 16 (4 I + j) + 4 quad + r of the lane's row in block BLK (unnormalised)
+  template <int BLK, int I>
+  __device__ __forceinline__ void read16(float (&f)[16]) const {
+    B::template read16<BLK, I>(f);
+  }
+
+  // `step`: LDS byte address of the first of the step's two pieces.  Lane (row, quad) receives in
+  // st[b][pc] the scores of keys 16 pc + 4 quad + r of its row in block b.
+  __device__ __forceinline__ void scores(uint32_t step, floatx4 (&st)[RB][2]) const { B::scores(step, st, kfrag, q16, q8); }
+  // The same with the wavefront's requests for a later step between the matrix instructions:
+  // 16 bytes per lane from `from` + off[j] to LDS address dst + 1024 j.  STREAMING: with the
+  // non-temporal hint (rows that nobody reads again).
+  template <bool STREAMING>
+  __device__ __forceinline__ void scores_requesting(uint32_t step, floatx4 (&st)[RB][2], const uint32_t (&off)[REQUESTS],
+                                                    const void *from, uint32_t dst) const {
+    B::template scores_requesting<STREAMING>(step, st, kfrag, q16, q8, off, static_cast<const char *>(from), dst);
+  }
+  // Online softmax of a step's scores, in C++, for steps with masked keys: bias(b, pc, e) is added to
+  // the scaled score of key 16 pc + 4 quad + e (-inf leaves the key out).  pf[b]: the lane's 8
+  // probabilities as bfloat16 pairs; afterwards the accumulators owe the factor of scale_accumulators.
+  template <class Bias>
+  __device__ __forceinline__ void softmax(floatx4 (&st)[RB][2], u32x4 (&pf)[RB], float (&alpha)[RB], float scale, Bias &&bias) {
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+      float sc[8], mloc = -INFINITY;
+#pragma unroll
+      for (int pc = 0; pc < 2; ++pc)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          sc[4 * pc + e] = st[b][pc][e] * scale + bias(b, pc, e);
+          mloc = fmaxf(mloc, sc[4 * pc + e]);
+        }
+      mloc = max_over_quads(mloc);
+      const float m_old = ml[b];
+      const bool move = !(mloc - m_old <= 8.0f);  // (lazy: also true from -inf)
+      const float m_new = move ? mloc : m_old;
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      alpha[b] = move ? __builtin_amdgcn_exp2f(m_old - m_safe) : 1.0f;
+      ml[b] = m_new;
+      float lsum = 0.f;
+      bf16x8 pb8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = __builtin_amdgcn_exp2f(sc[e] - m_safe);
+        const __bf16 pb = (__bf16)p;
+        lsum += (float)pb;  // the normaliser sums the weights that multiply V
+        pb8[e] = pb;
+      }
+      pf[b] = __builtin_bit_cast(u32x4, pb8);
+      ml[RB + b] = ml[RB + b] * alpha[b] + lsum;
+    }
+  }
+  // accumulators *= alpha where a maximum has moved (rare: the maximum moves lazily)
+  __device__ __forceinline__ void scale_accumulators(const float (&alpha)[RB]) {
+    if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.0f || alpha[1] != 1.0f) != 0) B::scale(alpha[0], alpha[1]);
+  }
+  // O^T += V^T . P^T of the step at `step` with probabilities pf
+  __device__ __forceinline__ void values(uint32_t step, const u32x4 (&pf)[RB]) { B::values(step, pf, vfrag); }
+  // The same and, between its matrix instructions, the softmax (no masks, scale > 0) of the score tiles
+  // st of the step after it; pf is replaced by the new probabilities.
+  __device__ __forceinline__ void values_softmax(uint32_t step, u32x4 (&pf)[RB], floatx4 (&st)[RB][2], float (&alpha)[RB], float scale) {
+    u32x4 pn[RB];
+    B::values_softmax(step, pn, alpha, st, ml, pf, vfrag, scale);
+    pf[0] = pn[0], pf[1] = pn[1];
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
 // More than 16 query heads per KV head with V taken from K (the latent layer with all of its 128
 // heads on one GPU): a segment is a block of up to 128 heads, a range of the flat list of 64-token
-// tiles belongs to a workgroup of eight wavefronts, and wavefront i computes heads 16 i .. 16 i + 15
-// exactly as the 16-head form does, on K tiles that the eight share in LDS (four 16-row pieces laid
-// out like that form's stages, one eighth of the requests per wavefront, two stages, one barrier per
-// tile).  Nothing is computed twice and a latent row is read from memory once per 128 heads; the
-// workgroup-shared form above re-reads it per block of 32 heads and computes every score four times.
+// tiles belongs to a workgroup of four wavefronts, one per SIMD, and wavefront i computes heads
+// 32 i .. 32 i + 31 as two blocks of 16 rows (LatentMath<.., 2>) on K that the four share in LDS:
+// a tile is two steps of 32 tokens, a step two 16-row pieces laid out like the 16-head form's stages
+// and requested by LDS-DMA, a quarter per wavefront.  Nothing is computed twice and a latent row is
+// read from memory once per 128 heads; the workgroup-shared form above re-reads it per block of 32
+// heads and computes every score four times.
+// The vector unit has no second wavefront to serve while the matrix unit works, so the softmax of a
+// step's scores sits between the matrix instructions of the second product of the step before
+// (values_softmax), and the requests for a later step between those of the score product
+// (scores_requesting); steps with masked keys (a sequence's last tile, the first of a sliding
+// window) and a segment's first step take the softmax below.  A step's second product thereby runs
+// one step late, so K lives in a ring of four stages with one barrier per step: past the barrier of
+// step i every wavefront has finished the second product of step i - 2, whose stage the requests for
+// step i + 2 overwrite.
 template <int DQK, int DV>
-__global__ __launch_bounds__(512) void paged_decode_latent128_kernel(
+__global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
     DecodeArgs a, WideArgs w, const int32_t *__restrict__ page_table, const void *__restrict__ cur_pos) {
   using L = Latent16<DQK, DV>;
-  typedef float floatx4 __attribute__((ext_vector_type(4)));
-  constexpr int SUB = L::TILE, NSUB = kTile / SUB, NWAVES = 8;
-  constexpr int KSTEPS = DQK / 32, VB = DV / 16;
-  constexpr int PER_WAVE = NSUB * L::NDMA / NWAVES;
-  static_assert(NSUB == 4 && 2 * PER_WAVE == L::NDMA, "two wavefronts request each 16-row piece");
-  constexpr int STAGE = NSUB * L::STAGE;
+  using M = LatentMath<DQK, DV>;
+  constexpr int RB = M::RB, SUB = L::TILE, KEYS = 2 * SUB, NWAVES = 4, NSTAGES = 4;
+  constexpr int KSTEPS = M::KSTEPS;
+  constexpr int PER_WAVE = M::REQUESTS;
+  static_assert(kTile == 2 * KEYS && 2 * PER_WAVE == L::NDMA && PER_WAVE < 16, "two wavefronts request each 16-row piece");
+  constexpr int STAGE = 2 * L::STAGE, WAVE_HEADS = 16 * RB;
 
   __shared__ int s_pref[kMaxUsersWide + 1];
   __shared__ int s_len[kMaxUsersWide];
@@ -659,9 +799,8 @@ __global__ __launch_bounds__(512) void paged_decode_latent128_kernel(
   int64_t x = (int64_t)wg * total / n_eff;
   const int64_t x_hi = (int64_t)(wg + 1) * total / n_eff;
   const int G = w.gseg;
-  const int hg = 16 * wave + n;  // this lane's head inside the segment
 
-  // ---- tile requests: wavefronts 2 i and 2 i + 1 fetch piece i (16 consecutive cache rows) -----
+  // ---- step requests: wavefronts 2 i and 2 i + 1 fetch piece i of a step (16 consecutive cache rows)
   const int sub_w = wave >> 1;
   uint32_t src_off[PER_WAVE];
 #pragma unroll
@@ -671,18 +810,25 @@ __global__ __launch_bounds__(512) void paged_decode_latent128_kernel(
     src_off[j] = (uint32_t)(rr * L::ROW + 16 * L::position(rr, p));
   }
   const uint32_t lds0 = lds_address(smem);
-  auto issue_tile = [&](const Cursor &cu, int buf) {
+  // the wavefront's piece of half `half` of tile cu: where its rows lie in the cache, where step i keeps them
+  auto piece_source = [&](const Cursor &cu, int half) {
     const int kvh = cu.h / w.nhb;
-    const int tok0 = cu.t * kTile + SUB * sub_w;
+    const int tok0 = cu.t * kTile + KEYS * half + SUB * sub_w;
     const int col = tok0 / a.bs;
     int phys = (col < a.w) ? page_table[(int64_t)cu.u * a.pt_rs + col] : 0;
     if ((unsigned)phys >= (unsigned)a.nb) phys = 0;
     const int64_t row0 = ((int64_t)phys * w.nkv + kvh) * a.bs + (tok0 - col * a.bs);
     const uint64_t addr = reinterpret_cast<uint64_t>(a.k) + (uint64_t)row0 * L::ROW;
-    const char *src = reinterpret_cast<const char *>(address_from_words(
-        __builtin_amdgcn_readfirstlane((int)(uint32_t)addr), __builtin_amdgcn_readfirstlane((int)(uint32_t)(addr >> 32))));
-    const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(
-        (int)(lds0 + (uint32_t)(buf * STAGE + sub_w * L::STAGE + 1024 * (wave & 1) * PER_WAVE)));
+    return reinterpret_cast<const char *>(address_from_words(__builtin_amdgcn_readfirstlane((int)(uint32_t)addr),
+                                                             __builtin_amdgcn_readfirstlane((int)(uint32_t)(addr >> 32))));
+  };
+  auto piece_stage = [&](int i) {
+    return (uint32_t)__builtin_amdgcn_readfirstlane(
+        (int)(lds0 + (uint32_t)((i % NSTAGES) * STAGE + sub_w * L::STAGE + 1024 * (wave & 1) * PER_WAVE)));
+  };
+  auto request_step = [&](const Cursor &cu, int half, int i) {
+    const char *src = piece_source(cu, half);
+    const uint32_t dst = piece_stage(i);
     const void *bases[4] = {src, src - 1024, src - 2048, src - 3072};
 #pragma unroll
     for (int j = 0; j + 4 <= PER_WAVE; j += 4) {
@@ -694,68 +840,48 @@ __global__ __launch_bounds__(512) void paged_decode_latent128_kernel(
   };
   // Rows past the attended length may be cache rows nobody ever wrote: their scores are masked,
   // but as V rows they would turn 0 * Inf into NaN, so they are cleared in LDS.
-  auto clear_unattended_rows = [&](int buf, int nvalid) {
-    for (int r = nvalid + wave; r < kTile; r += NWAVES) {
-      uint4 *row = reinterpret_cast<uint4 *>(smem + buf * STAGE + (r / SUB) * L::STAGE + (r % SUB) * L::ROW);
+  auto clear_unattended_rows = [&](int i, int nvalid) {
+    for (int r = nvalid + wave; r < KEYS; r += NWAVES) {
+      uint4 *row = reinterpret_cast<uint4 *>(smem + (i % NSTAGES) * STAGE + (r / SUB) * L::STAGE + (r % SUB) * L::ROW);
       for (int c = lane; c < L::ROW / 16; c += 64) row[c] = make_uint4(0, 0, 0, 0);
     }
   };
-  auto load_q = [&](const Cursor &cu, bf16x8 (&qf)[KSTEPS]) {
-    const uint16_t *qp = a.q + cu.u * a.q_us + (int64_t)(cu.h * G + min(hg, G - 1)) * a.q_hs + 8 * quad;
-    const uint32_t qmask = hg < G ? 0xffffffffu : 0u;
+  M m;
+  m.init(n, quad);
+  auto load_q = [&](const Cursor &cu) {
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-      uint4 t = *reinterpret_cast<const uint4 *>(qp + 32 * s);
-      t.x &= qmask, t.y &= qmask, t.z &= qmask, t.w &= qmask;
-      qf[s] = __builtin_bit_cast(bf16x8, t);
+    for (int rb = 0; rb < RB; ++rb) {
+      const int hg = WAVE_HEADS * wave + 16 * rb + n;  // this lane's head inside the segment
+      const uint16_t *qp = a.q + cu.u * a.q_us + (int64_t)(cu.h * G + min(hg, G - 1)) * a.q_hs + 8 * quad;
+      const uint32_t qmask = hg < G ? 0xffffffffu : 0u;
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {
+        uint4 t = *reinterpret_cast<const uint4 *>(qp + 32 * s);
+        t.x &= qmask, t.y &= qmask, t.z &= qmask, t.w &= qmask;
+        m.set_q(rb, s, t);
+      }
     }
   };
 
-  // ---- fragment addresses inside a 16-row piece (as in the 16-head form) -----------------------
-  constexpr int GC = L::HALF_PERIOD ? 8 : 16;
-  constexpr int KB = GC / 4, VBASES = GC / 2;
-  uint32_t kfrag[KB], vfrag[VBASES];
-#pragma unroll
-  for (int i = 0; i < KB; ++i) kfrag[i] = (uint32_t)(n * L::ROW + 16 * L::position(n, 4 * i + quad));
-  {
-    const int rv = 4 * quad + (n >> 2), q4 = n & 3;
-#pragma unroll
-    for (int i = 0; i < VBASES; ++i)
-      vfrag[i] = (uint32_t)(rv * L::ROW + 16 * L::position(rv, 2 * i + (q4 >> 1)) + 8 * (q4 & 1));
-  }
-  auto read_k = [&](const unsigned char *piece, int s) {
-    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(piece + kfrag[s % KB] + 16 * GC * (s / KB)));
-  };
-  auto read_v = [&](const unsigned char *piece, int vb) {
-    typedef __attribute__((address_space(3))) shortx4 *lds_v4;
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(piece + vfrag[vb % VBASES] + 16 * GC * (vb / VBASES)));
-  };
-  constexpr int KPRE = KSTEPS < 4 ? KSTEPS : 4;
-  constexpr int VPRE = VB < 4 ? VB : 4;
-
   Cursor cur = locate_unit(a, s_pref, s_len, x);
-  bf16x8 qf[KSTEPS];
-  issue_tile(cur, 0);
-  load_q(cur, qf);
+  request_step(cur, 0, 0);
+  request_step(cur, 1, 1);
+  load_q(cur);
   publish_segment_row(a, s_pref, total, n_eff);
 
-  floatx4 acc[VB];
-#pragma unroll
-  for (int i = 0; i < VB; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY, l_run = 0.f;
   const float scale = a.scale_log2e;
-  const bool wave_active = 16 * wave < G;
+  const bool wave_active = WAVE_HEADS * wave < G;
+  u32x4 pf[RB];
+  uint32_t prev = 0;
+  bool have_prev = false;  // a second product is owed: step `prev`, probabilities pf
+  bool drain = true;       // loads other than step requests are under way (Q)
+  int i = 0;               // step
 
-  for (int it = 0; x < x_hi; ++x, ++it) {
-    const int buf = it & 1;
+  for (; x < x_hi; ++x) {
     const int nvalid = cur.len - cur.t * kTile;
-    const bool partial = nvalid < kTile;
     const int nbelow = cur.lo - cur.t * kTile;  // sliding window: > 0 only in a segment's first tile
     const bool has_next = x + 1 < x_hi;
     const bool same_seg = has_next && cur.tiles_left > 1;
-
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's share of the tile has landed
-    __syncthreads();                     // the tile is complete; everybody has left the other stage
     Cursor nxt = cur;
     if (has_next) {
       if (same_seg) {
@@ -764,114 +890,98 @@ __global__ __launch_bounds__(512) void paged_decode_latent128_kernel(
       } else {
         nxt = locate_unit(a, s_pref, s_len, x + 1);
       }
-      issue_tile(nxt, buf ^ 1);
     }
-    if (partial) {
-      clear_unattended_rows(buf, max(nvalid, 0));
-      __syncthreads();
-    }
-    if (wave_active) {
+#pragma unroll 1
+    for (int half = 0; half < 2; ++half, ++i) {
+      // this wavefront's share of step i has landed (the requests of step i + 1 may still be under way)
+      if (!drain && (half == 0 || has_next)) __builtin_amdgcn_s_waitcnt(0x0F70 | PER_WAVE);
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
+      drain = false;
+      __syncthreads();  // ... everybody's has, and nobody reads the stage of step i - 2 any more
+      const int nv = nvalid - KEYS * half, nb = nbelow - KEYS * half;  // this step attends its keys nb .. nv - 1
+      const bool computing = wave_active && nv > 0;
+      // (a wavefront that computes sends the requests from inside the score product)
+      const bool inside = computing && has_next;
+      if (has_next && !inside) request_step(nxt, half, i + 2);
+      if (nv > 0 && nv < KEYS) {
+        clear_unattended_rows(i, nv);
+        __syncthreads();
+      }
+      if (!computing) {
+        if (have_prev) m.values(prev, pf), have_prev = false;
+        continue;
+      }
       // Two pieces (32 keys) per step: one softmax for both, and the second product takes them as the
       // 32-deep K dimension of one matrix instruction per block of 16 value columns (k index 8 quad + j
       // stands for key 4 quad + j of the first piece for j < 4, of the second otherwise: the order in
       // which the score tiles hold a lane's keys and the transposing reads their rows).
-#pragma unroll 1
-      for (int half = 0; half < NSUB / 2; ++half) {
-        if (2 * SUB * half >= nvalid) break;
-        const unsigned char *piece = smem + buf * STAGE + 2 * half * L::STAGE;
-        // ---- S^T = K . Q^T -------------------------------------------------------------------
-        floatx4 st[2];
-#pragma unroll
-        for (int pc = 0; pc < 2; ++pc) {
-          st[pc] = floatx4{0.f, 0.f, 0.f, 0.f};
-          const unsigned char *pp = piece + pc * L::STAGE;
-          bf16x8 ring[KPRE];
-#pragma unroll
-          for (int s = 0; s < KPRE; ++s) ring[s] = read_k(pp, s);
-#pragma unroll
-          for (int s = 0; s < KSTEPS; ++s) {
-            st[pc] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % KPRE], qf[s], st[pc], 0, 0, 0);
-            if (s + KPRE < KSTEPS) ring[s % KPRE] = read_k(pp, s + KPRE);
-          }
-        }
-        // ---- online softmax: lane (head, quad) holds keys 32 half + 16 pc + 4 quad + r ------------
-        float sc[8], mloc = -INFINITY;
-#pragma unroll
-        for (int pc = 0; pc < 2; ++pc)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int key = 2 * SUB * half + SUB * pc + 4 * quad + r;
-            sc[4 * pc + r] = (key >= nvalid || key < nbelow) ? -INFINITY : st[pc][r] * scale;
-            mloc = fmaxf(mloc, sc[4 * pc + r]);
-          }
-        mloc = max_over_quads(mloc);
-        const bool move = !(mloc - m_run <= 8.0f);  // (lazy: also true from -inf)
-        const float m_new = move ? mloc : m_run;
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = move ? __builtin_amdgcn_exp2f(m_run - m_safe) : 1.0f;
-        m_run = m_new;
-        float lsum = 0.f;
-        bf16x8 pf;
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          const float p = __builtin_amdgcn_exp2f(sc[r] - m_safe);
-          const __bf16 pb = (__bf16)p;
-          lsum += (float)pb;  // the normaliser sums the weights that multiply V
-          pf[r] = pb;
-        }
-        l_run = l_run * alpha + lsum;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-          for (int i = 0; i < VB; ++i) acc[i] *= alpha;
-        }
-        // ---- O^T += V^T . P^T -------------------------------------------------------------------
-        {
-          shortx4 lo[VPRE], hi[VPRE];
-#pragma unroll
-          for (int vb = 0; vb < VPRE; ++vb) lo[vb] = read_v(piece, vb), hi[vb] = read_v(piece + L::STAGE, vb);
-#pragma unroll
-          for (int vb = 0; vb < VB; ++vb) {
-            const bf16x4 l4 = __builtin_bit_cast(bf16x4, lo[vb % VPRE]), h4 = __builtin_bit_cast(bf16x4, hi[vb % VPRE]);
-            bf16x8 vf;
-            vf[0] = l4[0], vf[1] = l4[1], vf[2] = l4[2], vf[3] = l4[3];
-            vf[4] = h4[0], vf[5] = h4[1], vf[6] = h4[2], vf[7] = h4[3];
-            acc[vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[vb], 0, 0, 0);
-            if (vb + VPRE < VB) lo[vb % VPRE] = read_v(piece, vb + VPRE), hi[vb % VPRE] = read_v(piece + L::STAGE, vb + VPRE);
-          }
-        }
+      const uint32_t step = lds0 + (uint32_t)((i % NSTAGES) * STAGE);
+      floatx4 st[RB][2];
+      if (inside) m.template scores_requesting<true>(step, st, src_off, piece_source(nxt, half), piece_stage(i + 2));
+      else m.scores(step, st);
+      float alpha[RB];
+      if (have_prev && nv >= KEYS && nb <= 0 && scale > 0.f) {
+        m.values_softmax(prev, pf, st, alpha, scale);
+      } else {
+        if (have_prev) m.values(prev, pf);
+        // lane (head, quad) holds keys 16 pc + 4 quad + e of the step
+        m.softmax(st, pf, alpha, scale, [&](int, int pc, int e) {
+          const int key = SUB * pc + 4 * quad + e;
+          return (key >= nv || key < nb) ? -INFINITY : 0.f;
+        });
       }
+      m.scale_accumulators(alpha);
+      prev = step, have_prev = true;
     }
     // ---- close the segment: every wavefront writes its heads' part of the partial -----------------
     if (!same_seg) {
+      if (have_prev) m.values(prev, pf), have_prev = false;
       float *slot = a.ws_slots + ((int64_t)wg + (int64_t)cur.u * a.hkv + cur.h) * a.slot_floats;
-      const float l_tot = sum_over_quads(l_run);
-      if (hg < G) {
-        if (a.partial_bf16) {  // wavefront-uniform
-          uint32_t *dst = reinterpret_cast<uint32_t *>(slot) + (hg * DV + 4 * quad) / 2;
+      // (the lane's place in the slot is worked out here, behind an opaque copy of the lane number:
+      // kept across the loop it would not fit the register file)
+      int l = lane;
+      asm volatile("" : "+v"(l));
+      const int quad = l >> 4;
+      static_for(std::make_integer_sequence<int, RB>{}, [&](auto rbc) {
+        constexpr int rb = decltype(rbc)::value;
+        const int hg = WAVE_HEADS * wave + 16 * rb + (l & 15);
+        const float l_tot = sum_over_quads(m.sum(rb));
+        if (hg < G) {
+          if (a.partial_bf16) {  // wavefront-uniform
+            uint32_t *dst = reinterpret_cast<uint32_t *>(slot) + (hg * DV + 4 * quad) / 2;
+            static_for(std::make_integer_sequence<int, M::NA>{}, [&](auto ic) {
+              constexpr int bi = decltype(ic)::value;
+              float f[16];
+              m.template read16<rb, bi>(f);
 #pragma unroll
-          for (int vb = 0; vb < VB; ++vb)
-            *reinterpret_cast<uint2 *>(dst + 8 * vb) =
-                make_uint2(pack_bf16x2(acc[vb][0], acc[vb][1]), pack_bf16x2(acc[vb][2], acc[vb][3]));
-          if (quad == 0) {
-            slot[G * DV / 2 + hg] = m_run;
-            slot[G * DV / 2 + G + hg] = l_tot;
-          }
-        } else {
-          float *dst = slot + hg * DV + 4 * quad;
+              for (int j = 0; j < 4; ++j)
+                *reinterpret_cast<uint2 *>(dst + 8 * (4 * bi + j)) =
+                    make_uint2(pack_bf16x2(f[4 * j], f[4 * j + 1]), pack_bf16x2(f[4 * j + 2], f[4 * j + 3]));
+            });
+            if (quad == 0) {
+              slot[G * DV / 2 + hg] = m.maximum(rb);
+              slot[G * DV / 2 + G + hg] = l_tot;
+            }
+          } else {
+            float *dst = slot + hg * DV + 4 * quad;
+            static_for(std::make_integer_sequence<int, M::NA>{}, [&](auto ic) {
+              constexpr int bi = decltype(ic)::value;
+              float f[16];
+              m.template read16<rb, bi>(f);
 #pragma unroll
-          for (int vb = 0; vb < VB; ++vb)
-            *reinterpret_cast<float4 *>(dst + 16 * vb) = make_float4(acc[vb][0], acc[vb][1], acc[vb][2], acc[vb][3]);
-          if (quad == 0) {
-            slot[G * DV + hg] = m_run;
-            slot[G * DV + G + hg] = l_tot;
+              for (int j = 0; j < 4; ++j)
+                *reinterpret_cast<float4 *>(dst + 16 * (4 * bi + j)) = make_float4(f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]);
+            });
+            if (quad == 0) {
+              slot[G * DV + hg] = m.maximum(rb);
+              slot[G * DV + G + hg] = l_tot;
+            }
           }
         }
-      }
-#pragma unroll
-      for (int i = 0; i < VB; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
-      m_run = -INFINITY;
-      l_run = 0.f;
-      if (has_next) load_q(nxt, qf);
+      });
+      m.restart();
+      if (has_next) load_q(nxt);
+      drain = true;
     }
     cur = nxt;
   }
@@ -884,7 +994,7 @@ bool launch_latent128(const DecodeArgs &a, const WideArgs &w, hipStream_t st) {
   static std::atomic<uint64_t> lds_ready{0};
   if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&paged_decode_latent128_kernel<DQK, DV>), lds, lds_ready))
     return false;
-  launch_dominant(&paged_decode_latent128_kernel<DQK, DV>, dim3(a.n_waves), dim3(512), lds, st, a, w, a.pt, a.cur);
+  launch_dominant(&paged_decode_latent128_kernel<DQK, DV>, dim3(a.n_waves), dim3(256), lds, st, a, w, a.pt, a.cur);
   return true;
 }
 
@@ -911,14 +1021,14 @@ struct LatentPrefillArgs {
 };
 
 template <int DQK, int DV>
-__global__ __launch_bounds__(512) void latent_prefill_kernel(LatentPrefillArgs a) {
+__global__ __launch_bounds__(256) void latent_prefill_kernel(LatentPrefillArgs a) {
   using L = Latent16<DQK, DV>;
-  typedef float floatx4 __attribute__((ext_vector_type(4)));
-  constexpr int SUB = L::TILE, NSUB = 4, KEYS = SUB * NSUB, NWAVES = 8, ROWS = 16 * NWAVES;
-  constexpr int KSTEPS = DQK / 32, VB = DV / 16;
-  constexpr int PER_WAVE = NSUB * L::NDMA / NWAVES;
-  static_assert(NSUB * L::NDMA % NWAVES == 0, "a tile's requests must divide among the wavefronts");
-  constexpr int STAGE = NSUB * L::STAGE;
+  using M = LatentMath<DQK, DV>;
+  constexpr int RB = M::RB, SUB = L::TILE, KEYS = 2 * SUB, NWAVES = 4, WROWS = 16 * RB, ROWS = WROWS * NWAVES, NSTAGES = 4;
+  constexpr int KSTEPS = M::KSTEPS;
+  constexpr int PER_WAVE = M::REQUESTS;
+  static_assert(NWAVES * PER_WAVE == 2 * L::NDMA && PER_WAVE < 16, "a step's requests divide among the wavefronts");
+  constexpr int STAGE = 2 * L::STAGE;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   const int lane = threadIdx.x & 63;
@@ -933,20 +1043,28 @@ __global__ __launch_bounds__(512) void latent_prefill_kernel(LatentPrefillArgs a
   const int grp = (int)blockIdx.x % groups;
   const int b = grp / a.nkv, kvh = grp - b * a.nkv;
 
-  const int r0 = blk * ROWS + wave * 16;
+  const int r0 = blk * ROWS + wave * WROWS;
   const bool wave_active = r0 < rows_total;
-  const int r = min(r0 + n, rows_total - 1);
-  const int t = r / G, head = kvh * G + (r - t * G);
-  const bool row_valid = r0 + n < rows_total;
-  const int limit = a.causal ? t : a.s - 1;
-  const int wave_limit = a.causal ? min(r0 + 15, rows_total - 1) / G : a.s - 1;
+  // Token and head of the lane's row in block rb (rows past the end repeat the last one and are not
+  // stored).  Worked out where it is needed, behind an opaque copy of the lane number: kept across
+  // the loop, the rows' tokens, heads and mask addresses would not fit the register file.
+  auto row_of = [&](int rb, int &t, int &head) {
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    const int r = min(r0 + 16 * rb + (l & 15), rows_total - 1);
+    t = r / G, head = kvh * G + (r - t * G);
+  };
+  const int first_limit = a.causal ? min(r0, rows_total - 1) / G : a.s - 1;  // the smallest limit among the rows
+  const int wave_limit = a.causal ? min(r0 + WROWS - 1, rows_total - 1) / G : a.s - 1;
   const int wg_limit = a.causal ? min(blk * ROWS + ROWS - 1, rows_total - 1) / G : a.s - 1;
-  const int ntiles = wg_limit / KEYS + 1;
+  const int nsteps = wg_limit / KEYS + 1;
+  const float scale = a.scale_log2e;
+  const bool plain = a.mask == nullptr;  // (the scale is positive: the entry point checks)
 
-  // ---- tile requests: instruction k = wave * PER_WAVE + j of the tile's NSUB * NDMA -----------
+  // ---- step requests: instruction k = wave * PER_WAVE + j of the step's 2 * NDMA ---------------
   const uint16_t *kbase_g = a.k + b * a.k_bs + kvh * a.k_hs;
   const uint32_t row_bytes = 2u * (uint32_t)a.k_ts;
-  // (offsets inside a tile whose 64 keys all exist; the last tile of a sequence clamps row by row)
+  // (offsets inside a step whose 32 keys all exist; the last step of a sequence clamps row by row)
   uint32_t req_off[PER_WAVE];
 #pragma unroll
   for (int j = 0; j < PER_WAVE; ++j) {
@@ -955,12 +1073,13 @@ __global__ __launch_bounds__(512) void latent_prefill_kernel(LatentPrefillArgs a
     req_off[j] = (uint32_t)(SUB * sub + rr) * row_bytes + 16u * (uint32_t)L::position(rr, p);
   }
   const uint32_t lds0 = lds_address(smem);
-  auto request_tile = [&](int tile, int buf) {
-    const uint32_t dst0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)(buf * STAGE + 1024 * wave * PER_WAVE)));
-    if ((tile + 1) * KEYS <= a.s) {
-      const uint16_t *tile_base = kbase_g + (int64_t)tile * KEYS * a.k_ts;
+  auto request_step = [&](int i) {
+    const uint32_t dst0 =
+        (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)((i % NSTAGES) * STAGE + 1024 * wave * PER_WAVE)));
+    if ((i + 1) * KEYS <= a.s) {
+      const uint16_t *step_base = kbase_g + (int64_t)i * KEYS * a.k_ts;
       // (four requests behind one write of M0: the instruction offset moves the LDS address too)
-      const char *tb = reinterpret_cast<const char *>(tile_base);
+      const char *tb = reinterpret_cast<const char *>(step_base);
       const void *bases[4] = {tb, tb - 1024, tb - 2048, tb - 3072};
 #pragma unroll
       for (int j = 0; j + 4 <= PER_WAVE; j += 4) {
@@ -968,164 +1087,122 @@ __global__ __launch_bounds__(512) void latent_prefill_kernel(LatentPrefillArgs a
         dma16_quad(bases, off, dst0 + 1024u * j);
       }
 #pragma unroll
-      for (int j = PER_WAVE / 4 * 4; j < PER_WAVE; ++j) dma16(tile_base, req_off[j], dst0 + 1024u * j);
+      for (int j = PER_WAVE / 4 * 4; j < PER_WAVE; ++j) dma16(step_base, req_off[j], dst0 + 1024u * j);
     } else {
 #pragma unroll 1
       for (int j = 0; j < PER_WAVE; ++j) {
         const int k = wave * PER_WAVE + j, sub = k / L::NDMA, kk = k % L::NDMA;
         const int P = 64 * kk + lane, rr = P / L::CPR, p = P % L::CPR;
-        const int key = min(tile * KEYS + SUB * sub + rr, a.s - 1);  // rows past the end repeat the last one
+        const int key = min(i * KEYS + SUB * sub + rr, a.s - 1);  // rows past the end repeat the last one
         dma16(kbase_g, (uint32_t)key * row_bytes + 16u * (uint32_t)L::position(rr, p), dst0 + 1024u * (uint32_t)j);
       }
     }
   };
 
-  // ---- fragment addresses inside a 16-row piece (as in the 16-head decode form) ----------------
-  constexpr int GC = L::HALF_PERIOD ? 8 : 16;
-  constexpr int KB = GC / 4, VBASES = GC / 2;
-  uint32_t kfrag[KB], vfrag[VBASES];
+  M m;
+  m.init(n, quad);
 #pragma unroll
-  for (int i = 0; i < KB; ++i) kfrag[i] = (uint32_t)(n * L::ROW + 16 * L::position(n, 4 * i + quad));
-  {
-    const int rv = 4 * quad + (n >> 2), q4 = n & 3;
-#pragma unroll
-    for (int i = 0; i < VBASES; ++i)
-      vfrag[i] = (uint32_t)(rv * L::ROW + 16 * L::position(rv, 2 * i + (q4 >> 1)) + 8 * (q4 & 1));
-  }
-  auto read_k = [&](const unsigned char *piece, int s) {
-    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(piece + kfrag[s % KB] + 16 * GC * (s / KB)));
-  };
-  auto read_v = [&](const unsigned char *piece, int vb) {
-    typedef __attribute__((address_space(3))) shortx4 *lds_v4;
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)(piece + vfrag[vb % VBASES] + 16 * GC * (vb / VBASES)));
-  };
-  constexpr int KPRE = KSTEPS < 4 ? KSTEPS : 4;
-  constexpr int VPRE = VB < 4 ? VB : 4;
-
-  request_tile(0, 0);
-  // B operand of the score product: lane (row, quad) holds features 32 s + 8 quad .. + 7 of its row
-  bf16x8 qf[KSTEPS];
-  {
+  for (int rb = 0; rb < RB; ++rb) {
+    int t, head;
+    row_of(rb, t, head);
     const uint16_t *qp = a.q + b * a.q_bs + head * a.q_hs + (int64_t)t * a.q_ts + 8 * quad;
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) qf[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 32 * s));
+    for (int s = 0; s < KSTEPS; ++s) m.set_q(rb, s, *reinterpret_cast<const uint4 *>(qp + 32 * s));
   }
-  const uint16_t *mrow = a.mask ? a.mask + b * a.mask_bs + head * a.mask_hs + (int64_t)t * a.mask_rs : nullptr;
+  // (behind the Q loads: the waits below count this wavefront's requests only from here on)
+  request_step(0);
+  if (nsteps > 1) request_step(1);
 
-  floatx4 acc[VB];
-#pragma unroll
-  for (int i = 0; i < VB; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY, l_run = 0.f;
-  const float scale = a.scale_log2e;
+  u32x4 pf[RB];
+  uint32_t prev = 0;
+  bool have_prev = false;  // a second product is owed: step `prev`, probabilities pf
 
-  for (int tile = 0; tile < ntiles; ++tile) {
-    const int buf = tile & 1;
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's share of the tile has landed
-    __syncthreads();                      // ... everybody's has, and the other stage is free
-    if (tile + 1 < ntiles) request_tile(tile + 1, buf ^ 1);
-    if (!wave_active) continue;
+  for (int i = 0; i < nsteps; ++i) {
+    // this wavefront's share of step i has landed (the requests of step i + 1 may still be under way)
+    if (i + 1 < nsteps) __builtin_amdgcn_s_waitcnt(0x0F70 | PER_WAVE);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();  // ... everybody's has, and nobody reads the stage of step i - 2 any more
+    const int key0 = i * KEYS;
+    const bool computing = wave_active && key0 <= wave_limit;
+    // (a wavefront that computes sends whole steps' requests from inside the score product)
+    const bool inside = computing && i + 2 < nsteps && (i + 3) * KEYS <= a.s;
+    if (i + 2 < nsteps && !inside) request_step(i + 2);
+    if (!computing) {
+      if (have_prev) m.values(prev, pf), have_prev = false;
+      continue;
+    }
     // Two pieces (32 keys) per step: one softmax for both, and the second product takes them as the
     // 32-deep K dimension of one matrix instruction per block of 16 value columns.  k index 8 quad + j
     // of that instruction stands for key 4 quad + j of the first piece (j < 4) or of the second: the
     // order in which the score tiles hold the keys of a lane, and the transposing reads their rows.
-#pragma unroll 1
-    for (int half = 0; half < NSUB / 2; ++half) {
-      const int key0 = tile * KEYS + 2 * half * SUB;
-      if (key0 > wave_limit) break;
-      const unsigned char *piece = smem + buf * STAGE + 2 * half * L::STAGE;
-      // ---- S^T = K . Q^T ---------------------------------------------------------------------
-      floatx4 st[2];
-#pragma unroll
-      for (int pc = 0; pc < 2; ++pc) {
-        st[pc] = floatx4{0.f, 0.f, 0.f, 0.f};
-        const unsigned char *pp = piece + pc * L::STAGE;
-        bf16x8 ring[KPRE];
-#pragma unroll
-        for (int s = 0; s < KPRE; ++s) ring[s] = read_k(pp, s);
-#pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) {
-          st[pc] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % KPRE], qf[s], st[pc], 0, 0, 0);
-          if (s + KPRE < KSTEPS) ring[s % KPRE] = read_k(pp, s + KPRE);
-        }
-      }
-      // ---- online softmax: lane (row, quad) holds keys key0 + 16 pc + 4 quad + i of its row ------
-      float sc[8], mloc = -INFINITY;
-#pragma unroll
-      for (int pc = 0; pc < 2; ++pc) {
-        float madd[4] = {0.f, 0.f, 0.f, 0.f};
-        if (mrow) {  // wavefront-uniform
-          const int kq = min(key0 + 16 * pc + 4 * quad, a.s - 4);
-          const uint2 mw = *reinterpret_cast<const uint2 *>(mrow + kq);
-          madd[0] = bf16_lo(mw.x) * 1.4426950408889634f, madd[1] = bf16_hi(mw.x) * 1.4426950408889634f;
-          madd[2] = bf16_lo(mw.y) * 1.4426950408889634f, madd[3] = bf16_hi(mw.y) * 1.4426950408889634f;
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = key0 + 16 * pc + 4 * quad + i;
-          sc[4 * pc + i] = key > limit ? -INFINITY : st[pc][i] * scale + madd[i];
-          mloc = fmaxf(mloc, sc[4 * pc + i]);
-        }
-      }
-      mloc = max_over_quads(mloc);
-      const bool move = !(mloc - m_run <= 8.0f);  // (lazy: also true from -inf)
-      const float m_new = move ? mloc : m_run;
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = move ? __builtin_amdgcn_exp2f(m_run - m_safe) : 1.0f;
-      m_run = m_new;
-      float lsum = 0.f;
-      bf16x8 pf;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float pr = __builtin_amdgcn_exp2f(sc[i] - m_safe);
-        const __bf16 pb = (__bf16)pr;
-        lsum += (float)pb;
-        pf[i] = pb;
-      }
-      l_run = l_run * alpha + lsum;
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-        for (int i = 0; i < VB; ++i) acc[i] *= alpha;
-      }
-      // ---- O^T += V^T . P^T ---------------------------------------------------------------------
-      {
-        shortx4 lo[VPRE], hi[VPRE];
-#pragma unroll
-        for (int vb = 0; vb < VPRE; ++vb) lo[vb] = read_v(piece, vb), hi[vb] = read_v(piece + L::STAGE, vb);
-#pragma unroll
-        for (int vb = 0; vb < VB; ++vb) {
-          const bf16x4 l4 = __builtin_bit_cast(bf16x4, lo[vb % VPRE]), h4 = __builtin_bit_cast(bf16x4, hi[vb % VPRE]);
-          bf16x8 vf;
-          vf[0] = l4[0], vf[1] = l4[1], vf[2] = l4[2], vf[3] = l4[3];
-          vf[4] = h4[0], vf[5] = h4[1], vf[6] = h4[2], vf[7] = h4[3];
-          acc[vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[vb], 0, 0, 0);
-          if (vb + VPRE < VB) lo[vb % VPRE] = read_v(piece, vb + VPRE), hi[vb % VPRE] = read_v(piece + L::STAGE, vb + VPRE);
-        }
-      }
+    const uint32_t step = lds0 + (uint32_t)((i % NSTAGES) * STAGE);
+    floatx4 st[RB][2];
+    if (inside) {
+      const uint32_t dst0 = (uint32_t)__builtin_amdgcn_readfirstlane(
+          (int)(lds0 + (uint32_t)(((i + 2) % NSTAGES) * STAGE + 1024 * wave * PER_WAVE)));
+      m.template scores_requesting<false>(step, st, req_off, kbase_g + (int64_t)(i + 2) * KEYS * a.k_ts, dst0);
+    } else {
+      m.scores(step, st);
     }
+    float alpha[RB];
+    if (have_prev && plain && key0 + KEYS - 1 <= first_limit) {
+      m.values_softmax(prev, pf, st, alpha, scale);
+    } else {
+      if (have_prev) m.values(prev, pf);
+      // lane (row, quad) holds keys key0 + 16 pc + 4 quad + e of its rows
+      int limit[RB], t[RB], head[RB];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        row_of(rb, t[rb], head[rb]);
+        limit[rb] = a.causal ? t[rb] : a.s - 1;
+      }
+      m.softmax(st, pf, alpha, scale, [&](int rb, int pc, int e) {
+        const int key = key0 + 16 * pc + 4 * quad + e;
+        float add = 0.f;
+        if (a.mask) {
+          const int kq = min(key0 + 16 * pc + 4 * quad, a.s - 4);
+          const uint2 mw = *reinterpret_cast<const uint2 *>(a.mask + b * a.mask_bs + head[rb] * a.mask_hs + (int64_t)t[rb] * a.mask_rs + kq);
+          add = (e == 0 ? bf16_lo(mw.x) : e == 1 ? bf16_hi(mw.x) : e == 2 ? bf16_lo(mw.y) : bf16_hi(mw.y)) * 1.4426950408889634f;
+        }
+        return key > limit[rb] ? -INFINITY : add;
+      });
+    }
+    m.scale_accumulators(alpha);
+    prev = step, have_prev = true;
   }
   if (!wave_active) return;
-  // ---- normalise and store: lane (row, quad) holds values 16 vb + 4 quad .. + 3 of its row --------
-  const float l_tot = sum_over_quads(l_run);
-  const float inv = 1.0f / l_tot;
-  if (row_valid) {
-    uint16_t *op = a.out + b * a.out_bs + head * a.out_hs + (int64_t)t * a.out_ts + 4 * quad;
+  if (have_prev) m.values(prev, pf);
+  // ---- normalise and store: lane (row, quad) holds values 16 vb + 4 quad .. + 3 of its rows --------
+  static_for(std::make_integer_sequence<int, RB>{}, [&](auto rbc) {
+    constexpr int rb = decltype(rbc)::value;
+    const float inv = 1.0f / sum_over_quads(m.sum(rb));
+    if (r0 + 16 * rb + n < rows_total) {
+      int t, head;
+      row_of(rb, t, head);
+      uint16_t *op = a.out + b * a.out_bs + head * a.out_hs + (int64_t)t * a.out_ts + 4 * quad;
+      static_for(std::make_integer_sequence<int, M::NA>{}, [&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        float f[16];
+        m.template read16<rb, i>(f);
 #pragma unroll
-    for (int vb = 0; vb < VB; ++vb)
-      *reinterpret_cast<uint2 *>(op + 16 * vb) =
-          make_uint2(pack_bf16x2(acc[vb][0] * inv, acc[vb][1] * inv), pack_bf16x2(acc[vb][2] * inv, acc[vb][3] * inv));
-  }
+        for (int j = 0; j < 4; ++j)
+          *reinterpret_cast<uint2 *>(op + 16 * (4 * i + j)) =
+              make_uint2(pack_bf16x2(f[4 * j] * inv, f[4 * j + 1] * inv), pack_bf16x2(f[4 * j + 2] * inv, f[4 * j + 3] * inv));
+      });
+    }
+  });
 }
 
 template <int DQK, int DV>
 int launch_latent_prefill(const LatentPrefillArgs &a, hipStream_t st) {
   using L = Latent16<DQK, DV>;
-  const size_t lds = 2 * 4 * (size_t)L::STAGE;
+  const size_t lds = 4 * 2 * (size_t)L::STAGE;
   static std::atomic<uint64_t> lds_ready{0};
   if (!ensure_dynamic_lds(reinterpret_cast<const void *>(&latent_prefill_kernel<DQK, DV>), lds, lds_ready))
     return fail(TTPA_ERR_LAUNCH, "latent prefill: cannot reserve %zu bytes of LDS", lds);
   const int64_t rows = (int64_t)(a.heads / a.nkv) * a.s;
   const int64_t grid = (rows + 127) / 128 * a.batch * a.nkv;
-  launch_dominant(&latent_prefill_kernel<DQK, DV>, dim3((unsigned)grid), dim3(512), lds, st, a);
+  launch_dominant(&latent_prefill_kernel<DQK, DV>, dim3((unsigned)grid), dim3(256), lds, st, a);
   return check_launch("latent_prefill");
 }
 
