@@ -237,7 +237,7 @@ def softmax_groups(R, scale, alpha):
     the accumulators still owe in operand alpha + b (1.0 unless the maximum moved by more than 8), and
     the probabilities as bfloat16 pairs in R.pn + 4 b ...  The maximum only moves when it has to (as
     the C++ form does), sums are taken before rounding to bfloat16, `scale` is positive.
-    Returns groups of instructions that stay together; the two row blocks alternate phase by phase."""
+    Returns groups of instructions that stay together."""
     phases = []
     for b in range(RB):
         S = [f"v{R.st + 8 * b + k}" for k in range(8)]
@@ -264,10 +264,15 @@ def softmax_groups(R, scale, alpha):
                    [f"v_add_f32 {T[0]}, {T[0]}, {T[2]}"], [f"v_fma_f32 {L}, {L}, {AL}, {T[0]}"]])
         ph.append([[f"v_cvt_pk_bf16_f32 {P[k]}, {S[2 * k]}, {S[2 * k + 1]}"] for k in range(4)])
         phases.append(ph)
+    # the two row blocks alternate group by group, so that neighbours do not depend on each other
+    # (a wavefront issues in order: a vector instruction that waits holds up the matrix instruction behind it)
     out = []
     for i in range(len(phases[0])):
-        for b in range(RB):
-            out += phases[b][i]
+        if len(phases[0][i]) == 1:  # (the group that keeps vcc)
+            out += [phases[b][i][0] for b in range(RB)]
+        else:
+            for groups in zip(*(phases[b][i] for b in range(RB))):
+                out += list(groups)
     return out
 
 
