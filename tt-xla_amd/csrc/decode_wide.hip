@@ -935,6 +935,8 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
     }
     // ---- close the segment: every wavefront writes its heads' part of the partial -----------------
     if (!same_seg) {
+      // (the next segment's Q first: its loads run while the partial is written)
+      if (has_next) load_q(nxt);
       if (have_prev) m.values(prev, pf), have_prev = false;
       float *slot = a.ws_slots + ((int64_t)wg + (int64_t)cur.u * a.hkv + cur.h) * a.slot_floats;
       // (the lane's place in the slot is worked out here, behind an opaque copy of the lane number:
@@ -980,7 +982,6 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
         }
       });
       m.restart();
-      if (has_next) load_q(nxt);
       drain = true;
     }
     cur = nxt;
