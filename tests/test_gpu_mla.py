@@ -41,11 +41,11 @@ DECODE = [
     (8, 16, 4, 192, 128, False, 32, 16, 1.0),
     (8, 8, 8, 128, 128, True, 32, 16, 1.0),
     (4, 16, 1, 576, 512, False, 32, 24, None),    # latent serving shape, 16 heads per rank
-    (3, 128, 1, 576, 512, False, 64, 12, None),   # all 128 heads: four head blocks per user
+    (3, 128, 1, 576, 512, False, 64, 12, None),   # all 128 heads of the layer
     (2, 64, 2, 192, 128, False, 16, 40, 0.11),
     (3, 16, 1, 576, 384, False, 32, 12, None),    # a value width that is not a power of two (merge kernel)
-    (2, 48, 1, 192, 128, False, 32, 6, 0.2),      # three of the eight wavefronts of the 128-head form have heads
-    (2, 40, 2, 128, 128, False, 16, 20, 0.2),     # 20 heads per KV head: a wavefront with four heads
+    (2, 48, 1, 192, 128, False, 32, 6, 0.2),      # two of the four wavefronts of the 128-head form have heads, one of them 16
+    (2, 40, 2, 128, 128, False, 16, 20, 0.2),     # 20 heads per KV head: a row block with four heads
     (2, 256, 1, 576, 512, False, 64, 6, None),    # two segments of 128 heads per user
     (6, 128, 1, 576, 384, False, 128, 5, None),   # blocks of two tiles
 ]
