@@ -650,6 +650,7 @@ struct LatentMath {
   u32x16 q16[RB][NQ16];
   u32x8 q8[RB];
   floatx4 ml;                         // running maxima (0, 1) and sums (2, 3) of the two row blocks
+  float th[RB];                       // (maximum + 8) / scale: the raw score above which a maximum moves
   uint32_t kfrag[KB], vfrag[VBASES];  // the lane's fragment offsets inside a piece
 
   // lane (n, quad): A operand of the score product = row n, chunk 4 s + quad; transposing read of
@@ -670,6 +671,7 @@ struct LatentMath {
   __device__ __forceinline__ void restart() {
     B::clear();
     ml = floatx4{-INFINITY, -INFINITY, 0.f, 0.f};
+    th[0] = th[1] = -INFINITY;
   }
   // B operand of the score product: features 32 s + 8 quad .. + 7 of the lane's row in block b
   __device__ __forceinline__ void set_q(int b, int s, const uint4 &t) {
@@ -722,6 +724,7 @@ struct LatentMath {
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
       alpha[b] = move ? __builtin_amdgcn_exp2f(m_old - m_safe) : 1.0f;
       ml[b] = m_new;
+      th[b] = (m_new + 8.0f) * __builtin_amdgcn_rcpf(scale);
       float lsum = 0.f;
       bf16x8 pb8;
 #pragma unroll
@@ -742,11 +745,22 @@ struct LatentMath {
   // O^T += V^T . P^T of the step at `step` with probabilities pf
   __device__ __forceinline__ void values(uint32_t step, const u32x4 (&pf)[RB]) { B::values(step, pf, vfrag); }
   // The same and, between its matrix instructions, the softmax (no masks, scale > 0) of the score tiles
-  // st of the step after it; pf is replaced by the new probabilities.
+  // st of the step after it; pf is replaced by the new probabilities.  The block keeps the running
+  // maxima as they are; where a score would move one (rarely: a maximum moves by 8 at least), the
+  // softmax above redoes the step.
   __device__ __forceinline__ void values_softmax(uint32_t step, u32x4 (&pf)[RB], floatx4 (&st)[RB][2], float (&alpha)[RB], float scale) {
     u32x4 pn[RB];
-    B::values_softmax(step, pn, alpha, st, ml, pf, vfrag, scale);
-    pf[0] = pn[0], pf[1] = pn[1];
+    float sum[RB];
+    uint64_t moved;
+    const float m[RB] = {ml[0], ml[1]};
+    B::values_softmax(step, pn, sum, moved, st, m, th, pf, vfrag, scale);
+    if (moved == 0) {
+      pf[0] = pn[0], pf[1] = pn[1];
+      ml[RB] += sum[0], ml[RB + 1] += sum[1];
+      alpha[0] = alpha[1] = 1.0f;
+    } else {
+      softmax(st, pf, alpha, scale, [](int, int, int) { return 0.f; });
+    }
   }
 };
 

@@ -21,7 +21,7 @@ a later step are placed between the matrix instructions here.  Registers are fix
   v[0:2 DQK/8)        Q fragments, DQK / 8 per row block, 4 per step of 32 features
   then                a ring of 5 fragments (4 registers: a K fragment or a pair of V^T fragments),
                       the four score tiles (16), softmax temporaries (8), the next step's probabilities
-                      (8), the running maxima and sums of the two row blocks (4)
+                      (8)
 
 Two row blocks of (576, 512) fill all 256 accumulation registers, more than the compiler binds to
 the operands of one assembly statement, so no variable stands for the accumulators: the blocks below
@@ -82,18 +82,23 @@ class Regs:
         return [f'"v{r}"' for r in range(self.ring, self.ring + 4 * DEPTH)]
 
 
-def pipeline(n, reads_per_step, read, mma):
+def pipeline(n, reads_per_step, read, mma, every=1):
     """n steps; read(j, slot) returns the read instructions of step j into ring slot `slot`, mma(j, slot)
     the matrix instructions that use them.  The slot of step j - 1 is refilled behind the first matrix
-    instruction of step j."""
+    instruction of step j.  A wait in front of every `every`-th step covers that many steps (a
+    wavefront alone on its SIMD issues one instruction per four cycles, whatever the kind: a wait is not
+    free)."""
     depth = min(DEPTH, n)
     lines, issued = [], []
     for j in range(depth):
         lines += read(j, j % depth)
         issued.append(j)
     for j in range(n):
-        behind = reads_per_step * len([x for x in issued if x > j])
-        lines.append(f"s_waitcnt lgkmcnt({behind})")
+        if j % every == 0:
+            last = min(j + every - 1, n - 1)
+            assert all(x in issued for x in range(j, last + 1)), "a wait covers reads that are under way"
+            behind = reads_per_step * len([x for x in issued if x > last])
+            lines.append(f"s_waitcnt lgkmcnt({behind})")
         ops = mma(j, j % depth)
         lines.append(ops[0])
         nxt = j - 1 + depth
@@ -206,7 +211,7 @@ def scores(dqk, dv, gc, requests=0, nt=False):
     return statement(comment, name, args, lines, outs, ins, clob)
 
 
-def values_pipeline(R, dv, gc, piece, pf_in, vb_in):
+def values_pipeline(R, dv, gc, piece, pf_in, vb_in, every=1):
     vbases = gc // 2
 
     def read(j, slot):
@@ -217,7 +222,7 @@ def values_pipeline(R, dv, gc, piece, pf_in, vb_in):
     def mma(j, slot):
         return [f"v_mfma_f32_16x16x32_bf16 {R.accum(b, j)}, {R.slot(slot)}, %{pf_in + b}, {R.accum(b, j)}" for b in range(RB)]
 
-    return pipeline(dv // 16, 2, read, mma)
+    return pipeline(dv // 16, 2, read, mma, every)
 
 
 def values(dqk, dv, gc):
@@ -231,48 +236,38 @@ def values(dqk, dv, gc):
                      f"latent_values_{dqk}_{dv}", args, lines, [], ins, R.ring_clobbers() + ACC_CLOBBERS)
 
 
-def softmax_groups(R, scale, alpha):
-    """Online softmax of the score tiles of one step, without masks: per row block b the 8 scores of a
-    lane (R.st + 8 b ..), the running maximum R.ml + b and sum R.ml + 2 + b (updated), the factor that
-    the accumulators still owe in operand alpha + b (1.0 unless the maximum moved by more than 8), and
-    the probabilities as bfloat16 pairs in R.pn + 4 b ...  The maximum only moves when it has to (as
-    the C++ form does), sums are taken before rounding to bfloat16, `scale` is positive.
-    Returns groups of instructions that stay together."""
+def softmax_groups(R, scale, m, th, total, moved):
+    """Softmax of the score tiles of one step against the running maxima as they are, without masks:
+    per row block b the 8 scores of a lane (R.st + 8 b .., left as they are), the running maximum in
+    operand m + b, the probabilities exp2(score * scale - maximum) as bfloat16 pairs in R.pn + 4 b ..
+    and their sum (taken before rounding) in operand total + b.  A maximum moves only when a score
+    exceeds it by more than 8 (as in the C++ form): operand th + b holds (maximum + 8) / scale, and
+    the scalar pair `moved` collects the lanes with a raw score above it; the caller redoes the
+    softmax of a step where any lane has one.  `scale` is positive.
+    Returns groups of instructions that stay together; the two row blocks alternate group by group, so
+    that neighbours do not depend on each other (a wavefront issues in order: a vector instruction
+    that waits holds up the matrix instruction behind it)."""
     phases = []
     for b in range(RB):
         S = [f"v{R.st + 8 * b + k}" for k in range(8)]
         T = [f"v{R.tmp + 4 * b + k}" for k in range(4)]
         P = [f"v{R.pn + 4 * b + k}" for k in range(4)]
-        M, L, AL = f"v{R.ml + b}", f"v{R.ml + RB + b}", f"%{alpha + b}"
-        ph = []
-        ph.append([[f"v_max3_f32 {T[0]}, {S[0]}, {S[1]}, {S[2]}"], [f"v_max3_f32 {T[0]}, {T[0]}, {S[3]}, {S[4]}"],
-                   [f"v_max3_f32 {T[0]}, {T[0]}, {S[5]}, {S[6]}"], [f"v_max_f32 {T[0]}, {T[0]}, {S[7]}"],
-                   [f"v_mul_f32 {T[0]}, {scale}, {T[0]}"]])
-        # maximum over the four 16-lane groups that hold a row
-        ph.append([[f"v_mov_b32 {T[1]}, {T[0]}"], ["s_nop 1", f"v_permlane16_swap_b32 {T[0]}, {T[1]}"], [f"v_max_f32 {T[0]}, {T[0]}, {T[1]}"],
-                   [f"v_mov_b32 {T[1]}, {T[0]}"], ["s_nop 1", f"v_permlane32_swap_b32 {T[0]}, {T[1]}"], [f"v_max_f32 {T[0]}, {T[0]}, {T[1]}"]])
-        # (vcc lives from the comparison to the second selection: one group)
-        ph.append([[f"v_sub_f32 {T[1]}, {T[0]}, {M}",
-                    f"v_cmp_nge_f32 vcc, 0x41000000, {T[1]}",      # not (8.0 >= new - old): also true from -inf
-                    f"v_cndmask_b32 {T[2]}, {M}, {T[0]}, vcc",     # the maximum to use
-                    f"v_sub_f32 {T[3]}, {M}, {T[2]}", f"v_exp_f32 {T[3]}, {T[3]}", f"v_mov_b32 {M}, {T[2]}", "s_nop 0",
-                    f"v_cndmask_b32 {AL}, 1.0, {T[3]}, vcc"]])
-        ph.append([[f"v_fma_f32 {x}, {x}, {scale}, -{T[2]}"] for x in S])
-        ph.append([[f"v_exp_f32 {x}, {x}"] for x in S])
-        ph.append([[f"v_add_f32 {T[0]}, {S[0]}, {S[1]}"], [f"v_add_f32 {T[1]}, {S[2]}, {S[3]}"], [f"v_add_f32 {T[2]}, {S[4]}, {S[5]}"],
-                   [f"v_add_f32 {T[3]}, {S[6]}, {S[7]}"], [f"v_add_f32 {T[0]}, {T[0]}, {T[1]}"], [f"v_add_f32 {T[2]}, {T[2]}, {T[3]}"],
-                   [f"v_add_f32 {T[0]}, {T[0]}, {T[2]}"], [f"v_fma_f32 {L}, {L}, {AL}, {T[0]}"]])
-        ph.append([[f"v_cvt_pk_bf16_f32 {P[k]}, {S[2 * k]}, {S[2 * k + 1]}"] for k in range(4)])
-        phases.append(ph)
-    # the two row blocks alternate group by group, so that neighbours do not depend on each other
-    # (a wavefront issues in order: a vector instruction that waits holds up the matrix instruction behind it)
+        M, TH, SUM = f"%{m + b}", f"%{th + b}", f"%{total + b}"
+        g = [[f"v_max3_f32 {T[0]}, {S[0]}, {S[1]}, {S[2]}"], [f"v_max3_f32 {T[0]}, {T[0]}, {S[3]}, {S[4]}"],
+             [f"v_max3_f32 {T[0]}, {T[0]}, {S[5]}, {S[6]}"], [f"v_max_f32 {T[0]}, {T[0]}, {S[7]}"],
+             [f"v_cmp_gt_f32 vcc, {T[0]}, {TH}", f"s_or_b64 {moved}, {moved}, vcc"]]
+        for k in range(4):
+            x, y = (T[1], T[2]) if k % 2 == 0 else (T[3], T[0])  # (two pairs of temporaries in turn; the maximum is done with)
+            g += [[f"v_fma_f32 {x}, {S[2 * k]}, {scale}, -{M}"], [f"v_fma_f32 {y}, {S[2 * k + 1]}, {scale}, -{M}"],
+                  [f"v_exp_f32 {x}, {x}"], [f"v_exp_f32 {y}, {y}"],
+                  [f"v_add_f32 {SUM}, {x}, {y}"] if k == 0 else [f"v_add_f32 {SUM}, {SUM}, {x}"]]
+            if k:
+                g += [[f"v_add_f32 {SUM}, {SUM}, {y}"]]
+            g += [[f"v_cvt_pk_bf16_f32 {P[k]}, {x}, {y}"]]
+        phases.append(g)
     out = []
-    for i in range(len(phases[0])):
-        if len(phases[0][i]) == 1:  # (the group that keeps vcc)
-            out += [phases[b][i][0] for b in range(RB)]
-        else:
-            for groups in zip(*(phases[b][i] for b in range(RB))):
-                out += list(groups)
+    for groups in zip(*phases):
+        out += list(groups)
     return out
 
 
@@ -281,26 +276,34 @@ def values_softmax(dqk, dv, gc):
     instructions."""
     R = Regs(dqk, dv)
     vbases = gc // 2
-    # operands: outputs 0..1 next probabilities, 2..3 alpha; in/out 4..7 score tiles, 8 maxima and sums;
-    # inputs 9.. : probabilities of the step whose second product this is, V^T bases, scale
-    n_out = 4 * RB + 1
-    pf_in, vb_in, scale = n_out, n_out + RB, f"%{n_out + RB + vbases}"
-    product = values_pipeline(R, dv, gc, 32 * dqk, pf_in, vb_in)
-    lines = ([MARK_BEGIN, "s_nop 1", "s_waitcnt lgkmcnt(0)"] + spread(product, softmax_groups(R, scale, RB)) +
-             ["s_nop 7", "s_nop 7", MARK_END])
-    args = ([f"u32x4 &pn{b}" for b in range(RB)] + [f"float &alpha{b}" for b in range(RB)] +
-            [f"floatx4 &st{2 * b + pc}" for b in range(RB) for pc in range(2)] + ["floatx4 &ml"] +
-            [f"const u32x4 &pf{b}" for b in range(RB)] + [f"uint32_t vb{i}" for i in range(vbases)] + ["float scale"])
-    outs = ([f'"=&{{v[{R.pn + 4 * b}:{R.pn + 4 * b + 3}]}}"(pn{b})' for b in range(RB)] + [f'"=&v"(alpha{b})' for b in range(RB)] +
-            [f'"+{{{R.score(b, pc)}}}"(st{2 * b + pc})' for b in range(RB) for pc in range(2)] +
-            [f'"+{{v[{R.ml}:{R.ml + 2 * RB - 1}]}}"(ml)'])
-    ins = [f'"v"(pf{b})' for b in range(RB)] + [f'"v"(vb{i})' for i in range(vbases)] + ['"s"(scale)']
-    assert len(outs) == n_out and len(outs) + 2 * RB + 1 + len(ins) <= 30  # ("+" operands count twice)
-    clob = R.ring_clobbers() + [f'"v{r}"' for r in range(R.tmp, R.tmp + 4 * RB)] + ['"vcc"'] + ACC_CLOBBERS
-    comment = (f"// O^T += V^T . P^T of one step ({dv // 16} blocks of 16 value columns) and, between its matrix instructions, the\n"
-               "// softmax of the score tiles st.. of the next step (no masks, scale > 0): ml = the running maxima and sums of the\n"
-               "// two row blocks, alpha what the accumulators owe afterwards, pn the next probabilities")
-    return statement(comment, f"latent_values_softmax_{dqk}_{dv}", args, lines, outs, ins, clob)
+    # operands: outputs 0..1 next probabilities, 2..3 their sums, 4 the lanes whose maximum has to move;
+    # inputs: 5..8 score tiles, 9..10 maxima, 11..12 thresholds, 13..14 probabilities of the step whose
+    # second product this is, V^T bases, scale
+    n_out = 2 * RB + 1
+    moved = f"%{2 * RB}"
+    st_in = n_out
+    m_in, th_in = st_in + 2 * RB, st_in + 3 * RB
+    pf_in = th_in + RB
+    vb_in = pf_in + RB
+    scale = f"%{vb_in + vbases}"
+    product = values_pipeline(R, dv, gc, 32 * dqk, pf_in, vb_in, every=2)
+    lines = ([MARK_BEGIN, f"s_mov_b64 {moved}, 0", "s_nop 0", "s_waitcnt lgkmcnt(0)"] +
+             spread(product, softmax_groups(R, scale, m_in, th_in, RB, moved), first=2) + ["s_nop 7", "s_nop 7", MARK_END])
+    args = ([f"u32x4 &pn{b}" for b in range(RB)] + [f"float &sum{b}" for b in range(RB)] + ["uint64_t &moved"] +
+            [f"const floatx4 &st{2 * b + pc}" for b in range(RB) for pc in range(2)] + [f"float m{b}" for b in range(RB)] +
+            [f"float th{b}" for b in range(RB)] + [f"const u32x4 &pf{b}" for b in range(RB)] +
+            [f"uint32_t vb{i}" for i in range(vbases)] + ["float scale"])
+    outs = ([f'"=&{{v[{R.pn + 4 * b}:{R.pn + 4 * b + 3}]}}"(pn{b})' for b in range(RB)] + [f'"=&v"(sum{b})' for b in range(RB)] +
+            ['"=&s"(moved)'])
+    ins = ([f'"{{{R.score(b, pc)}}}"(st{2 * b + pc})' for b in range(RB) for pc in range(2)] + [f'"v"(m{b})' for b in range(RB)] +
+           [f'"v"(th{b})' for b in range(RB)] + [f'"v"(pf{b})' for b in range(RB)] + [f'"v"(vb{i})' for i in range(vbases)] +
+           ['"s"(scale)'])
+    assert len(outs) == n_out and len(outs) + len(ins) <= 30
+    clob = R.ring_clobbers() + [f'"v{r}"' for r in range(R.tmp, R.tmp + 4 * RB)] + ['"vcc"', '"scc"'] + ACC_CLOBBERS
+    comment = (f"// O^T += V^T . P^T of one step ({dv // 16} blocks of 16 value columns) and, between its matrix instructions, the\\n"
+               "// softmax of the score tiles st.. of the next step against the running maxima m.. as they are (no masks,\\n"
+               "// scale > 0): pn the probabilities, sum their sums, moved != 0 where a score exceeds th = (m + 8) / scale")
+    return statement(comment.replace("\\n", "\n"), f"latent_values_softmax_{dqk}_{dv}", args, lines, outs, ins, clob)
 
 
 def accumulator_access(dv):
@@ -364,9 +367,10 @@ struct LatentBlocks<{dqk}, {dv}> {{
   static __device__ __forceinline__ void values(uint32_t step, const u32x4 (&pf)[2], const uint32_t (&vf)[{vbases}]) {{
     latent_values_{dqk}_{dv}(pf[0], pf[1], {vf});
   }}
-  static __device__ __forceinline__ void values_softmax(uint32_t step, u32x4 (&pn)[2], float (&alpha)[2], floatx4 (&st)[2][2], floatx4 &ml,
+  static __device__ __forceinline__ void values_softmax(uint32_t step, u32x4 (&pn)[2], float (&sum)[2], uint64_t &moved,
+                                                        const floatx4 (&st)[2][2], const float (&m)[2], const float (&th)[2],
                                                         const u32x4 (&pf)[2], const uint32_t (&vf)[{vbases}], float scale) {{
-    latent_values_softmax_{dqk}_{dv}(pn[0], pn[1], alpha[0], alpha[1], {st}, ml, pf[0], pf[1], {vf}, scale);
+    latent_values_softmax_{dqk}_{dv}(pn[0], pn[1], sum[0], sum[1], moved, {st}, m[0], m[1], th[0], th[1], pf[0], pf[1], {vf}, scale);
   }}
   static __device__ __forceinline__ void clear() {{ latent_acc_clear_{dv}(); }}
   static __device__ __forceinline__ void scale(float alpha0, float alpha1) {{ latent_acc_scale_{dqk}_{dv}(alpha0, alpha1); }}
