@@ -52,13 +52,13 @@ MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
     # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
     # the rotating workload copies; the summaries under profiles/ hold the runs)
-    "config2": ("paged_decode_mfma16_kernel", "57ce30f89c503559", 310428385),
-    "config5": ("paged_decode_mfma16_kernel", "57ce30f89c503559", 168441012),
-    "config4": ("paged_decode_mfma16_kernel", "57ce30f89c503559", 3415575463),
-    "config3": ("prefill_kernel", "9e5dc9fce6518e7f", 244494236),
-    "latent": ("paged_decode_latent16_kernel", "a3580e2bacac3b3c", 654190586),
-    "latent128": ("paged_decode_latent128_kernel", "57869affdd297548", 743907672),
-    "latent-prefill": ("latent_prefill_kernel", "57869affdd297548", 332232193),
+    "config2": ("paged_decode_mfma16_kernel", "57ce30f89c503559", 310428587),
+    "config5": ("paged_decode_mfma16_kernel", "57ce30f89c503559", 168440615),
+    "config4": ("paged_decode_mfma16_kernel", "57ce30f89c503559", 3415576119),
+    "config3": ("prefill_kernel", "9e5dc9fce6518e7f", 244464543),
+    "latent": ("paged_decode_latent16_kernel", "87f771815d47e9f8", 654195478),
+    "latent128": ("paged_decode_latent128_kernel", "c394a61fcc308551", 743929974),
+    "latent-prefill": ("latent_prefill_kernel", "c394a61fcc308551", 332296701),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}
