@@ -194,19 +194,23 @@ def test_flash_mla_prefill(b, hq, s, dh, nkv, dv, has_value):
     _check(f"mla prefill b{b} h{hq} s{s} dh{dh} dv{dv}", got, want)
 
 
-@pytest.mark.parametrize("b,hq,s,dh,nkv,dv,scale", [
-    (1, 16, 224, 576, 1, 512, 1.0),     # every key for every row: all steps but a wavefront's first take the softmax
-    (2, 16, 96, 192, 1, 128, 1.0),      # that sits between the matrix instructions
-    (1, 32, 96, 128, 1, 128, 1.0),
+@pytest.mark.parametrize("b,hq,s,dh,nkv,dv,causal", [
+    (1, 16, 224, 576, 1, 512, False),   # every key for every row: all steps but a wavefront's first take the softmax
+    (2, 16, 96, 192, 1, 128, False),    # that sits between the matrix instructions
+    (1, 32, 96, 128, 1, 128, False),
+    (1, 16, 100, 576, 1, 512, False),   # a sequence that ends inside a step of 32 keys (the operator asks for multiples
+    (1, 16, 100, 576, 1, 512, True),    # of 32, the library does not): rows past the end are requested as the last one
+    (2, 8, 44, 192, 1, 128, True),
 ])
-def test_flash_mla_prefill_without_causal_limit(b, hq, s, dh, nkv, dv, scale):
-    """The operator accepts is_causal=False only together with a mask (reference custom_ops.py:723-726);
-    the library entry point below it also takes neither, which is the case where the masked softmax of
-    the kernel is left to a wavefront's first step: called directly."""
+def test_flash_mla_prefill_through_the_library(b, hq, s, dh, nkv, dv, causal):
+    """The operator accepts is_causal=False only together with a mask and sequence lengths that are multiples of 32
+    (reference custom_ops.py:723-726, :238); the library entry point below it takes neither restriction: called
+    directly.  Without a mask and without a causal limit, the masked softmax of the kernel is left to a
+    wavefront's first step."""
     from tt_xla_amd import _native as N
 
-    print(f"case: mla prefill, every key, b{b} h{hq} s{s} dh{dh} dv{dv} scale{scale}", flush=True)
-    g = torch.Generator().manual_seed(7 * s + dh)
+    print(f"case: mla prefill through the library b{b} h{hq} s{s} dh{dh} dv{dv} causal={causal}", flush=True)
+    g = torch.Generator().manual_seed(7 * s + dh + int(causal))
     q = (_bf(g, b, hq, s, dh).float() * 0.15).to(torch.bfloat16)
     k = _bf(g, b, nkv, s, dh)
     qd, kd = q.cuda(), k.cuda()
@@ -216,11 +220,11 @@ def test_flash_mla_prefill_without_causal_limit(b, hq, s, dh, nkv, dv, scale):
         out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
         qd.data_ptr(), qd.stride(0), qd.stride(1), qd.stride(2),
         kd.data_ptr(), kd.stride(0), kd.stride(1), kd.stride(2),
-        0, 0, 0, 0, b, hq, nkv, s, dh, dv, 0, float(scale) * 1.0, torch.cuda.current_stream().cuda_stream,
+        0, 0, 0, 0, b, hq, nkv, s, dh, dv, int(causal), 1.0, torch.cuda.current_stream().cuda_stream,
     )
     torch.cuda.synchronize()
-    want = O.flash_mla_prefill(q.float(), k.float(), dv, None, None, False, scale)
-    _check(f"mla prefill, every key, s{s} dh{dh} dv{dv} scale{scale}", out.cpu(), want)
+    want = O.flash_mla_prefill(q.float(), k.float(), dv, None, None, causal, 1.0)
+    _check(f"mla prefill through the library s{s} dh{dh} dv{dv} causal={causal}", out.cpu(), want)
 
 
 MASKED_PREFILL = [
