@@ -797,21 +797,27 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
   __shared__ int s_wsum[NWAVES];
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
-  build_prefix(a, cur_pos, s_pref, s_len, s_wsum);
+  const int seg_units = a.seg_units;
+  build_prefix(a, cur_pos, s_pref, s_len, s_wsum, seg_units);
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 15, quad = lane >> 4;
   const int wg = blockIdx.x;
-  const int total_tiles = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
-  const int64_t total = (int64_t)total_tiles * a.hkv;
-  const int n_eff = (int)(total < a.n_waves ? total : a.n_waves);  // workgroups that get work
+  // The flat list in units: per segment `seg_units` units that stand for the cost of closing it (the
+  // partial, the next segment's Q), then its tiles.  A range of more than seg_units units holds at
+  // least one tile.
+  const int total_units = __builtin_amdgcn_readfirstlane(s_pref[a.users]);
+  const int64_t total = (int64_t)total_units * a.hkv;
+  const int64_t max_ranges = total / (seg_units + 1);
+  const int n_eff = (int)(max_ranges < a.n_waves ? max_ranges : a.n_waves);  // workgroups that get work
   if (total == 0 || wg >= n_eff) {
-    publish_segment_row(a, s_pref, total, n_eff);
+    publish_segment_row(a, s_pref, total, n_eff, seg_units);
     return;
   }
-  int64_t x = (int64_t)wg * total / n_eff;
+  const int64_t x_lo = (int64_t)wg * total / n_eff;
   const int64_t x_hi = (int64_t)(wg + 1) * total / n_eff;
+  int64_t x = x_lo;  // set below to the unit of the first tile at or behind x_lo
   const int G = w.gseg;
 
   // ---- step requests: wavefronts 2 i and 2 i + 1 fetch piece i of a step (16 consecutive cache rows)
@@ -877,11 +883,11 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
     }
   };
 
-  Cursor cur = locate_unit(a, s_pref, s_len, x);
+  Cursor cur = locate_unit(a, s_pref, s_len, x_lo, seg_units, &x);
   request_step(cur, 0, 0);
   request_step(cur, 1, 1);
   load_q(cur);
-  publish_segment_row(a, s_pref, total, n_eff);
+  publish_segment_row(a, s_pref, total, n_eff, seg_units);
 
   const float scale = a.scale_log2e;
   const bool wave_active = WAVE_HEADS * wave < G;
@@ -891,10 +897,12 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
   bool drain = true;       // loads other than step requests are under way (Q)
   int i = 0;               // step
 
-  for (; x < x_hi; ++x) {
+  while (x < x_hi) {
     const int nvalid = cur.len - cur.t * kTile;
     const int nbelow = cur.lo - cur.t * kTile;  // sliding window: > 0 only in a segment's first tile
-    const bool has_next = x + 1 < x_hi;
+    // the unit of the tile behind this one: the next, or behind the next segment's leading units
+    const int64_t x_next = x + (cur.tiles_left > 1 ? 1 : 1 + seg_units);
+    const bool has_next = x_next < x_hi;
     const bool same_seg = has_next && cur.tiles_left > 1;
     Cursor nxt = cur;
     if (has_next) {
@@ -902,7 +910,7 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
         nxt.t = cur.t + 1;
         nxt.tiles_left = cur.tiles_left - 1;
       } else {
-        nxt = locate_unit(a, s_pref, s_len, x + 1);
+        nxt = locate_unit(a, s_pref, s_len, x + 1, seg_units);
       }
     }
 #pragma unroll 1
@@ -998,7 +1006,7 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
       m.restart();
       drain = true;
     }
-    cur = nxt;
+    cur = nxt, x = x_next;
   }
 }
 
@@ -1376,6 +1384,8 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
     a.partial_bf16 = !(pf && pf[0] == 'f') && out_user_stride % 2 == 0 && out_head_stride % 2 == 0 &&
                      reinterpret_cast<uintptr_t>(out) % 4 == 0;
     if (a.partial_bf16) a.slot_floats = slot_floats_bf16_for(gseg, head_dim_v);
+    // units in front of every segment of the flat list: what closing a segment costs, in tiles
+    a.seg_units = segment_units(2);
     if (head_size == 576 && head_dim_v == 512) ok = launch_latent128<576, 512>(a, w, st);
     else if (head_size == 576 && head_dim_v == 384) ok = launch_latent128<576, 384>(a, w, st);
     else if (head_size == 192 && head_dim_v == 128) ok = launch_latent128<192, 128>(a, w, st);
