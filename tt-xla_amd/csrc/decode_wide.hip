@@ -895,6 +895,7 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
   uint32_t prev = 0;
   bool have_prev = false;  // a second product is owed: step `prev`, probabilities pf
   bool drain = true;       // loads other than step requests are under way (Q)
+  bool landed = false;     // the next step's K and Q have been waited for already
   int i = 0;               // step
 
   while (x < x_hi) {
@@ -916,9 +917,14 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
 #pragma unroll 1
     for (int half = 0; half < 2; ++half, ++i) {
       // this wavefront's share of step i has landed (the requests of step i + 1 may still be under way)
-      if (!drain && (half == 0 || has_next)) __builtin_amdgcn_s_waitcnt(0x0F70 | PER_WAVE);
-      else __builtin_amdgcn_s_waitcnt(0x0F70);
-      drain = false;
+      if (landed) {
+        // (waited for while the segment was closed; the partial's stores need not be waited for)
+      } else if (!drain && (half == 0 || has_next)) {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | PER_WAVE);
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+      }
+      drain = landed = false;
       __syncthreads();  // ... everybody's has, and nobody reads the stage of step i - 2 any more
       const int nv = nvalid - KEYS * half, nb = nbelow - KEYS * half;  // this step attends its keys nb .. nv - 1
       const bool computing = wave_active && nv > 0;
@@ -960,6 +966,10 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
       // (the next segment's Q first: its loads run while the partial is written)
       if (has_next) load_q(nxt);
       if (have_prev) m.values(prev, pf), have_prev = false;
+      // Everything requested so far (Q, the next two steps) has to land before the next step anyway:
+      // waited for here, behind the second product above and in front of the partial's stores, which
+      // the next step then does not have to wait for.
+      __builtin_amdgcn_s_waitcnt(0x0F70);
       float *slot = a.ws_slots + ((int64_t)wg + (int64_t)cur.u * a.hkv + cur.h) * a.slot_floats;
       // (the lane's place in the slot is worked out here, behind an opaque copy of the lane number:
       // kept across the loop it would not fit the register file)
@@ -1004,7 +1014,7 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
         }
       });
       m.restart();
-      drain = true;
+      landed = true;
     }
     cur = nxt, x = x_next;
   }
@@ -1384,8 +1394,10 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
     a.partial_bf16 = !(pf && pf[0] == 'f') && out_user_stride % 2 == 0 && out_head_stride % 2 == 0 &&
                      reinterpret_cast<uintptr_t>(out) % 4 == 0;
     if (a.partial_bf16) a.slot_floats = slot_floats_bf16_for(gseg, head_dim_v);
-    // units in front of every segment of the flat list: what closing a segment costs, in tiles
-    a.seg_units = segment_units(2);
+    // units in front of every segment of the flat list: what a change of segment costs a range, in tiles
+    // (the partial, the next segment's Q and first step; 128 users of 512 ... 8192 tokens: 180 us with none,
+    // 167 with two, 163 with three to five)
+    a.seg_units = segment_units(4);
     if (head_size == 576 && head_dim_v == 512) ok = launch_latent128<576, 512>(a, w, st);
     else if (head_size == 576 && head_dim_v == 384) ok = launch_latent128<576, 384>(a, w, st);
     else if (head_size == 192 && head_dim_v == 128) ok = launch_latent128<192, 128>(a, w, st);
