@@ -317,13 +317,27 @@ def test_every_address_of_the_128_head_form_stays_in_bounds(dqk, dv, sep_v, hq, 
                 assert base % 16 == 0 and base + piece <= cache_bytes
     vb = dv // 16
     slot_floats = (gseg * dv + 2 * gseg + 3) // 4 * 4
-    slot_floats_bf16 = (gseg * dv // 2 + 2 * gseg + 3) // 4 * 4
-    for wave, rb, n, quad in itertools.product(range(WAVES_SHARED), (0, 1), (0, 15), (0, 3)):
+    # bfloat16 partials lie in blocks of 16 heads x 16 columns, the last block of heads padded
+    vals_bf16 = (gseg + 15) // 16 * 16 * dv // 2
+    slot_floats_bf16 = (vals_bf16 + 2 * gseg + 3) // 4 * 4
+    assert slot_floats_bf16 <= slot_floats, "the workspace is sized for float partials"
+    words = set()
+    for wave, rb, n, quad in itertools.product(range(WAVES_SHARED), (0, 1), range(16), range(4)):
         hg = WAVE_ROWS * wave + 16 * rb + n
         if hg < gseg:
             assert hg * dv + 4 * quad + 16 * (vb - 1) + 4 <= gseg * dv
             assert gseg * dv + gseg + hg < slot_floats
-            assert gseg * dv // 2 + gseg + hg < slot_floats_bf16
+            assert vals_bf16 + gseg + hg < slot_floats_bf16
+            for blk in range(vb):
+                w0 = (((2 * wave + rb) * vb + blk) * 16 + n) * 8 + 2 * quad
+                assert w0 + 2 <= vals_bf16
+                for w in (w0, w0 + 1):
+                    assert w not in words
+                    words.add(w)
+                    # what the merge kernel makes of the word: the head and the first of its two columns
+                    b, inb = w >> 7, w & 127
+                    assert (16 * (b // vb) + (inb >> 3), 16 * (b % vb) + 2 * (inb & 7)) == (hg, 16 * blk + 4 * quad + 2 * (w - w0))
+    assert len(words) == gseg * dv // 2
     for seg_h in (0, nkv * nhb - 1):
         assert seg_h * gseg + gseg - 1 < hq and seg_h // nhb < nkv
     segs, cus = users * nkv * nhb, 256

@@ -982,19 +982,24 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
         const float l_tot = sum_over_quads(m.sum(rb));
         if (hg < G) {
           if (a.partial_bf16) {  // wavefront-uniform
-            uint32_t *dst = reinterpret_cast<uint32_t *>(slot) + (hg * DV + 4 * quad) / 2;
+            // in blocks of 16 heads x 16 columns (decode_combine_bf16_kernel<true>): the 64 lanes of a
+            // store write 512 consecutive bytes (head by head they wrote 16 pieces of 32 bytes, and the
+            // partial took 7 us of the 10 us that a change of segment cost)
+            constexpr int HEADS16 = WAVE_HEADS / 16;
+            uint32_t *dst = reinterpret_cast<uint32_t *>(slot) + ((HEADS16 * wave + rb) * (DV / 16) * 16 + (l & 15)) * 8 + 2 * quad;
             static_for(std::make_integer_sequence<int, M::NA>{}, [&](auto ic) {
               constexpr int bi = decltype(ic)::value;
               float f[16];
               m.template read16<rb, bi>(f);
 #pragma unroll
               for (int j = 0; j < 4; ++j)
-                *reinterpret_cast<uint2 *>(dst + 8 * (4 * bi + j)) =
+                *reinterpret_cast<uint2 *>(dst + 128 * (4 * bi + j)) =
                     make_uint2(pack_bf16x2(f[4 * j], f[4 * j + 1]), pack_bf16x2(f[4 * j + 2], f[4 * j + 3]));
             });
+            const int vals = (G + 15) / 16 * 16 * DV / 2;
             if (quad == 0) {
-              slot[G * DV / 2 + hg] = m.maximum(rb);
-              slot[G * DV / 2 + G + hg] = l_tot;
+              slot[vals + hg] = m.maximum(rb);
+              slot[vals + G + hg] = l_tot;
             }
           } else {
             float *dst = slot + hg * DV + 4 * quad;
@@ -1393,7 +1398,7 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
     const char *pf = getenv("TTPA_LATENT_PARTIALS");
     a.partial_bf16 = !(pf && pf[0] == 'f') && out_user_stride % 2 == 0 && out_head_stride % 2 == 0 &&
                      reinterpret_cast<uintptr_t>(out) % 4 == 0;
-    if (a.partial_bf16) a.slot_floats = slot_floats_bf16_for(gseg, head_dim_v);
+    if (a.partial_bf16) a.slot_floats = slot_floats_bf16_blocks_for(gseg, head_dim_v);
     // units in front of every segment of the flat list: what a change of segment costs a range, in tiles
     // (the partial, the next segment's Q and first step; 128 users of 512 ... 8192 tokens: 180 us with none,
     // 167 with two, 163 with three to five)
@@ -1405,7 +1410,7 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
     if (!ok) return fail(TTPA_ERR_LAUNCH, "latent decode: cannot configure the kernel");
     if (int rc = check_launch("paged_mla_decode")) return rc;
     if (a.partial_bf16)
-      decode_combine_bf16_kernel<<<dim3(users * kv_heads * nhb, combine_pieces(gseg, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+      decode_combine_bf16_kernel<true><<<dim3(users * kv_heads * nhb, combine_pieces((gseg + 15) / 16 * 16, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
     else
       decode_combine_kernel<<<dim3(users * kv_heads * nhb, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
     return check_launch("paged_mla_decode");
@@ -1443,7 +1448,7 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
       if (!ok) return fail(TTPA_ERR_LAUNCH, "latent decode: cannot configure the kernel");
       if (int rc = check_launch("paged_mla_decode")) return rc;
       if (a.partial_bf16)
-        decode_combine_bf16_kernel<<<dim3(users * kv_heads, combine_pieces(gseg, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+        decode_combine_bf16_kernel<false><<<dim3(users * kv_heads, combine_pieces(gseg, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
       else
         decode_combine_kernel<<<dim3(users * kv_heads, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
       return check_launch("paged_mla_decode");
