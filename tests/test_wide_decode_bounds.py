@@ -246,9 +246,12 @@ def test_every_address_of_the_16_head_form_stays_in_bounds(dqk, dv, sep_v, hq, n
             assert off // row_bytes == rv and off + 8 <= stage
         assert 8 * quad + 32 * (ksteps - 1) + 8 <= dqk
         slot_floats = (g * dv + 2 * g + 3) // 4 * 4
+        # bfloat16 partials: one block of 16 heads x 16 columns per block of columns
+        slot_floats_bf16 = (16 * dv // 2 + 2 * g + 3) // 4 * 4
         if n < g:
             assert n * dv + 4 * quad + 16 * (vb - 1) + 4 <= g * dv
             assert g * dv + g + n < slot_floats
+            assert (128 * (vb - 1) + 8 * n + 2 * quad) + 2 <= 16 * dv // 2 and 16 * dv // 2 + g + n < slot_floats_bf16
     segs, cus = users * nkv, 256
     assert (waves * cus - 1) + (segs - 1) < waves * cus + segs     # slot index = wavefront + segment
 

@@ -578,14 +578,16 @@ __global__ __launch_bounds__(256, 1) void paged_decode_latent16_kernel(
       const float l_tot = sum_over_quads(l_run);
       if (n < G) {
         if (a.partial_bf16) {  // wavefront-uniform
-          uint32_t *dst = reinterpret_cast<uint32_t *>(slot) + (n * DV + 4 * quad) / 2;
+          // in blocks of 16 heads x 16 columns (decode_combine_bf16_kernel<true>; here one block of
+          // heads): the 64 lanes of a store write 512 consecutive bytes
+          uint32_t *dst = reinterpret_cast<uint32_t *>(slot) + 8 * n + 2 * quad;
 #pragma unroll
           for (int vb = 0; vb < VB; ++vb)
-            *reinterpret_cast<uint2 *>(dst + 8 * vb) =
+            *reinterpret_cast<uint2 *>(dst + 128 * vb) =
                 make_uint2(pack_bf16x2(acc[vb][0], acc[vb][1]), pack_bf16x2(acc[vb][2], acc[vb][3]));
           if (quad == 0) {
-            slot[G * DV / 2 + n] = m_run;
-            slot[G * DV / 2 + G + n] = l_tot;
+            slot[16 * DV / 2 + n] = m_run;
+            slot[16 * DV / 2 + G + n] = l_tot;
           }
         } else {
           float *dst = slot + n * DV + 4 * quad;
@@ -1300,7 +1302,8 @@ extern "C" size_t ttpa_paged_mla_decode_workspace_bytes(int32_t users, int32_t q
   // (error text of a geometry the workgroup-shared form refuses is not this function's business)
   if (wide_geometry(q_heads, kv_heads, nhb, gseg) == TTPA_OK) {
     const size_t segs = (size_t)users * kv_heads * nhb;
-    const size_t slot = (size_t)slot_floats_for(gseg, head_dim_v) * sizeof(float);
+    // (float partials, or bfloat16 ones in blocks of 16 heads: more when a group has fewer than 8)
+    const size_t slot = (size_t)std::max(slot_floats_for(gseg, head_dim_v), slot_floats_bf16_blocks_for(gseg, head_dim_v)) * sizeof(float);
     // one slot per range of the largest grid (at most four wavefront ranges per CU in the 16-head form)
     need = header_bytes(users, kv_heads * nhb) + ((size_t)cus * kWavesPerBlockHost + segs) * slot;
   }
@@ -1436,7 +1439,7 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
     // (the merge then stores output pairs as words: rows on 4-byte boundaries)
     a.partial_bf16 = !(pf && pf[0] == 'f') && out_user_stride % 2 == 0 && out_head_stride % 2 == 0 &&
                      reinterpret_cast<uintptr_t>(out) % 4 == 0;
-    if (a.partial_bf16) a.slot_floats = slot_floats_bf16_for(gseg, head_dim_v);
+    if (a.partial_bf16) a.slot_floats = slot_floats_bf16_blocks_for(gseg, head_dim_v);
     bool have = true;
     if (head_size == 576 && head_dim_v == 512) ok = launch_latent16<576, 512>(a, w, st);
     else if (head_size == 576 && head_dim_v == 384) ok = launch_latent16<576, 384>(a, w, st);
@@ -1448,7 +1451,7 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
       if (!ok) return fail(TTPA_ERR_LAUNCH, "latent decode: cannot configure the kernel");
       if (int rc = check_launch("paged_mla_decode")) return rc;
       if (a.partial_bf16)
-        decode_combine_bf16_kernel<false><<<dim3(users * kv_heads, combine_pieces(gseg, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+        decode_combine_bf16_kernel<true><<<dim3(users * kv_heads, combine_pieces(16, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
       else
         decode_combine_kernel<<<dim3(users * kv_heads, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
       return check_launch("paged_mla_decode");
