@@ -434,29 +434,22 @@ __global__ inline __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a
   }
 }
 
-// The same merge over partials whose values are bfloat16 (DecodeArgs::partial_bf16): a thread owns
-// two neighbouring output elements, one 32-bit word of every partial, and stores them as one word
-// (the caller checks that output rows start on 4-byte boundaries).  Grid: x = segment, y = piece
-// of kCombinePiece element pairs.
-// HEAD_BLOCKS: the values of a partial lie in blocks of 16 heads x 16 elements (element e of head g
-// at ((g / 16 * (D / 16) + e / 16) * 16 + g % 16) * 16 + e % 16, the last block of heads padded), the
-// order in which the 128-head latent kernel holds them: its 64 lanes then store 512 consecutive bytes.
-// A thread owns a word of the partials, in their order, whichever it is.
-template <bool HEAD_BLOCKS = false>
+// The same merge over partials whose values are bfloat16 (DecodeArgs::partial_bf16).  They lie in
+// blocks of 16 heads x 16 elements (element e of head g at
+// ((g / 16 * (D / 16) + e / 16) * 16 + g % 16) * 16 + e % 16, the last block of heads padded), the order
+// in which the latent kernels hold them: the 64 lanes of a store then write 512 consecutive bytes.  A
+// thread owns one 32-bit word of every partial, in that order, and stores its two neighbouring
+// output elements as one word (the caller checks that output rows start on 4-byte boundaries).
+// Grid: x = segment, y = piece of kCombinePiece words.
 __global__ inline __launch_bounds__(256) void decode_combine_bf16_kernel(DecodeArgs a, int G, int D) {
   const int seg = blockIdx.x;
-  const int pairs = (HEAD_BLOCKS ? (G + 15) / 16 * 16 : G) * D / 2;  // words of values in a partial
+  const int pairs = (G + 15) / 16 * 16 * D / 2;  // words of values in a partial
   const int p = blockIdx.y * kCombinePiece + threadIdx.x;
   if (p >= pairs) return;
   const int u = seg / a.hkv, h = seg % a.hkv;
-  int g, e;
-  if constexpr (HEAD_BLOCKS) {
-    const int blk = p >> 7, in_blk = p & 127;  // 16 heads x 8 words
-    g = 16 * (blk / (D / 16)) + (in_blk >> 3), e = 16 * (blk % (D / 16)) + 2 * (in_blk & 7);
-    if (g >= G) return;
-  } else {
-    g = 2 * p / D, e = 2 * p - g * D;
-  }
+  const int blk = p >> 7, in_blk = p & 127;  // a block: 16 heads x 8 words
+  const int g = 16 * (blk / (D / 16)) + (in_blk >> 3), e = 16 * (blk % (D / 16)) + 2 * (in_blk & 7);
+  if (g >= G) return;
   const int first = a.ws_seg[2 * seg], nw = a.ws_seg[2 * seg + 1];
   uint32_t *out = reinterpret_cast<uint32_t *>(a.out + u * a.out_us + (int64_t)(h * G + g) * a.out_hs + e);
   if (nw == 0) {  // padded row: no attended position -> NaN like softmax over nothing
@@ -508,10 +501,8 @@ __global__ inline __launch_bounds__(256) void decode_combine_bf16_kernel(DecodeA
 }
 
 inline int slot_floats_for(int g, int d) { return ((g * d + 2 * g + 3) / 4) * 4; }
-// the same with the values as bfloat16 (g * d even)
-inline int slot_floats_bf16_for(int g, int d) { return ((g * d / 2 + 2 * g + 3) / 4) * 4; }
-// the same in blocks of 16 heads (decode_combine_bf16_kernel<true>)
-inline int slot_floats_bf16_blocks_for(int g, int d) { return (((g + 15) / 16 * 16 * d / 2 + 2 * g + 3) / 4) * 4; }
+// the same with the values as bfloat16, in blocks of 16 heads (decode_combine_bf16_kernel)
+inline int slot_floats_bf16_for(int g, int d) { return (((g + 15) / 16 * 16 * d / 2 + 2 * g + 3) / 4) * 4; }
 inline size_t header_bytes(int users, int hkv) { return (((size_t)users * hkv * 8 + 255) / 256) * 256; }
 
 

@@ -578,7 +578,7 @@ __global__ __launch_bounds__(256, 1) void paged_decode_latent16_kernel(
       const float l_tot = sum_over_quads(l_run);
       if (n < G) {
         if (a.partial_bf16) {  // wavefront-uniform
-          // in blocks of 16 heads x 16 columns (decode_combine_bf16_kernel<true>; here one block of
+          // in blocks of 16 heads x 16 columns (decode_combine_bf16_kernel; here one block of
           // heads): the 64 lanes of a store write 512 consecutive bytes
           uint32_t *dst = reinterpret_cast<uint32_t *>(slot) + 8 * n + 2 * quad;
 #pragma unroll
@@ -984,7 +984,7 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
         const float l_tot = sum_over_quads(m.sum(rb));
         if (hg < G) {
           if (a.partial_bf16) {  // wavefront-uniform
-            // in blocks of 16 heads x 16 columns (decode_combine_bf16_kernel<true>): the 64 lanes of a
+            // in blocks of 16 heads x 16 columns (decode_combine_bf16_kernel): the 64 lanes of a
             // store write 512 consecutive bytes (head by head they wrote 16 pieces of 32 bytes, and the
             // partial took 7 us of the 10 us that a change of segment cost)
             constexpr int HEADS16 = WAVE_HEADS / 16;
@@ -1303,7 +1303,7 @@ extern "C" size_t ttpa_paged_mla_decode_workspace_bytes(int32_t users, int32_t q
   if (wide_geometry(q_heads, kv_heads, nhb, gseg) == TTPA_OK) {
     const size_t segs = (size_t)users * kv_heads * nhb;
     // (float partials, or bfloat16 ones in blocks of 16 heads: more when a group has fewer than 8)
-    const size_t slot = (size_t)std::max(slot_floats_for(gseg, head_dim_v), slot_floats_bf16_blocks_for(gseg, head_dim_v)) * sizeof(float);
+    const size_t slot = (size_t)std::max(slot_floats_for(gseg, head_dim_v), slot_floats_bf16_for(gseg, head_dim_v)) * sizeof(float);
     // one slot per range of the largest grid (at most four wavefront ranges per CU in the 16-head form)
     need = header_bytes(users, kv_heads * nhb) + ((size_t)cus * kWavesPerBlockHost + segs) * slot;
   }
@@ -1401,7 +1401,7 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
     const char *pf = getenv("TTPA_LATENT_PARTIALS");
     a.partial_bf16 = !(pf && pf[0] == 'f') && out_user_stride % 2 == 0 && out_head_stride % 2 == 0 &&
                      reinterpret_cast<uintptr_t>(out) % 4 == 0;
-    if (a.partial_bf16) a.slot_floats = slot_floats_bf16_blocks_for(gseg, head_dim_v);
+    if (a.partial_bf16) a.slot_floats = slot_floats_bf16_for(gseg, head_dim_v);
     // units in front of every segment of the flat list: what a change of segment costs a range, in tiles
     // (the partial, the next segment's Q and first step; 128 users of 512 ... 8192 tokens: 180 us with none,
     // 167 with two, 163 with three to five)
@@ -1413,7 +1413,7 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
     if (!ok) return fail(TTPA_ERR_LAUNCH, "latent decode: cannot configure the kernel");
     if (int rc = check_launch("paged_mla_decode")) return rc;
     if (a.partial_bf16)
-      decode_combine_bf16_kernel<true><<<dim3(users * kv_heads * nhb, combine_pieces((gseg + 15) / 16 * 16, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+      decode_combine_bf16_kernel<<<dim3(users * kv_heads * nhb, combine_pieces((gseg + 15) / 16 * 16, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
     else
       decode_combine_kernel<<<dim3(users * kv_heads * nhb, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
     return check_launch("paged_mla_decode");
@@ -1439,7 +1439,7 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
     // (the merge then stores output pairs as words: rows on 4-byte boundaries)
     a.partial_bf16 = !(pf && pf[0] == 'f') && out_user_stride % 2 == 0 && out_head_stride % 2 == 0 &&
                      reinterpret_cast<uintptr_t>(out) % 4 == 0;
-    if (a.partial_bf16) a.slot_floats = slot_floats_bf16_blocks_for(gseg, head_dim_v);
+    if (a.partial_bf16) a.slot_floats = slot_floats_bf16_for(gseg, head_dim_v);
     bool have = true;
     if (head_size == 576 && head_dim_v == 512) ok = launch_latent16<576, 512>(a, w, st);
     else if (head_size == 576 && head_dim_v == 384) ok = launch_latent16<576, 384>(a, w, st);
@@ -1451,7 +1451,7 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
       if (!ok) return fail(TTPA_ERR_LAUNCH, "latent decode: cannot configure the kernel");
       if (int rc = check_launch("paged_mla_decode")) return rc;
       if (a.partial_bf16)
-        decode_combine_bf16_kernel<true><<<dim3(users * kv_heads, combine_pieces(16, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+        decode_combine_bf16_kernel<<<dim3(users * kv_heads, combine_pieces(16, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
       else
         decode_combine_kernel<<<dim3(users * kv_heads, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
       return check_launch("paged_mla_decode");
