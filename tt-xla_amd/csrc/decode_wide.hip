@@ -1210,25 +1210,39 @@ __global__ __launch_bounds__(256) void latent_prefill_kernel(LatentPrefillArgs a
     m.scale_accumulators(alpha);
     prev = step, have_prev = true;
   }
+  if (wave_active && have_prev) m.values(prev, pf);
+  // ---- normalise and store --------------------------------------------------------------------
+  // Lane (row, quad) holds values 16 vb + 4 quad .. + 3 of its rows: stored from there, a store would
+  // write 16 pieces of 32 bytes (7.7 us per workgroup, a tenth of its time).  Instead the rows of a row
+  // block go through LDS (nobody reads K any more), a wavefront's own 16 rows of 2 DV + 16 bytes (the
+  // pitch puts the 16 rows of a 8-byte write into different banks), and come back 16 bytes per lane
+  // along the rows: a store writes whole rows.
+  __syncthreads();
   if (!wave_active) return;
-  if (have_prev) m.values(prev, pf);
-  // ---- normalise and store: lane (row, quad) holds values 16 vb + 4 quad .. + 3 of its rows --------
+  constexpr int PITCH = 2 * DV + 16, LPR = DV / 8, RPI = 64 / LPR;  // bytes per staged row, lanes per row, rows per store
+  static_assert((PITCH / 4) % 64 == 4 && 64 % LPR == 0 && 16 % RPI == 0 && NWAVES * 16 * PITCH <= NSTAGES * STAGE, "staging area of the output");
+  unsigned char *staged = smem + (lds0 - lds_address(smem)) + wave * (16 * PITCH);
   static_for(std::make_integer_sequence<int, RB>{}, [&](auto rbc) {
     constexpr int rb = decltype(rbc)::value;
     const float inv = 1.0f / sum_over_quads(m.sum(rb));
-    if (r0 + 16 * rb + n < rows_total) {
-      int t, head;
-      row_of(rb, t, head);
-      uint16_t *op = a.out + b * a.out_bs + head * a.out_hs + (int64_t)t * a.out_ts + 4 * quad;
-      static_for(std::make_integer_sequence<int, M::NA>{}, [&](auto ic) {
-        constexpr int i = decltype(ic)::value;
-        float f[16];
-        m.template read16<rb, i>(f);
+    static_for(std::make_integer_sequence<int, M::NA>{}, [&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      float f[16];
+      m.template read16<rb, i>(f);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          *reinterpret_cast<uint2 *>(op + 16 * (4 * i + j)) =
-              make_uint2(pack_bf16x2(f[4 * j] * inv, f[4 * j + 1] * inv), pack_bf16x2(f[4 * j + 2] * inv, f[4 * j + 3] * inv));
-      });
+      for (int j = 0; j < 4; ++j)
+        *reinterpret_cast<uint2 *>(staged + n * PITCH + 32 * (4 * i + j) + 8 * quad) =
+            make_uint2(pack_bf16x2(f[4 * j] * inv, f[4 * j + 1] * inv), pack_bf16x2(f[4 * j + 2] * inv, f[4 * j + 3] * inv));
+    });
+#pragma unroll 4
+    for (int r = 0; r < 16; r += RPI) {
+      const int rs = r + lane / LPR;  // the lane's row among the 16, 16 bytes of it at chunk lane % LPR
+      const int row = r0 + 16 * rb + rs;
+      if (row < rows_total) {
+        const int t = row / G, head = kvh * G + (row - t * G);
+        const uint4 v = *reinterpret_cast<const uint4 *>(staged + rs * PITCH + 16 * (lane % LPR));
+        *reinterpret_cast<uint4 *>(a.out + b * a.out_bs + head * a.out_hs + (int64_t)t * a.out_ts + 8 * (lane % LPR)) = v;
+      }
     }
   });
 }
@@ -1533,13 +1547,12 @@ extern "C" int ttpa_latent_prefill(void *out, int64_t out_batch_stride, int64_t 
                head_size);
   TTPA_REQUIRE(!(mask && causal), "an additive mask excludes causal masking");
   TTPA_REQUIRE(scale > 0.f, "latent prefill: scale %g must be positive", (double)scale);
-  TTPA_REQUIRE(aligned16(q) && aligned16(k) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0,
-               "latent prefill: q / k must be 16-byte aligned, out 8-byte aligned");
+  TTPA_REQUIRE(aligned16(q) && aligned16(k) && aligned16(out), "latent prefill: q / k / out must be 16-byte aligned");
   TTPA_REQUIRE(q_batch_stride % 8 == 0 && q_head_stride % 8 == 0 && q_token_stride % 8 == 0 && k_batch_stride % 8 == 0 &&
                    k_head_stride % 8 == 0 && k_token_stride % 8 == 0,
                "latent prefill: q / k strides must be multiples of 8 elements");
-  TTPA_REQUIRE(out_batch_stride % 4 == 0 && out_head_stride % 4 == 0 && out_token_stride % 4 == 0,
-               "latent prefill: out strides must be multiples of 4 elements");
+  TTPA_REQUIRE(out_batch_stride % 8 == 0 && out_head_stride % 8 == 0 && out_token_stride % 8 == 0,
+               "latent prefill: out strides must be multiples of 8 elements");
   TTPA_REQUIRE((int64_t)seq_len * k_token_stride * 2 < (1ll << 32), "latent prefill: a K head must stay below 4 GiB");
   if (mask) {
     TTPA_REQUIRE(seq_len % 4 == 0 && (reinterpret_cast<uintptr_t>(mask) & 7u) == 0 && mask_batch_stride % 4 == 0 &&
