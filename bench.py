@@ -52,13 +52,13 @@ MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
     # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
     # the rotating workload copies; the summaries under profiles/ hold the runs)
-    "config2": ("paged_decode_mfma16_kernel", "57ce30f89c503559", 310428587),
-    "config5": ("paged_decode_mfma16_kernel", "57ce30f89c503559", 168440615),
-    "config4": ("paged_decode_mfma16_kernel", "57ce30f89c503559", 3415576119),
-    "config3": ("prefill_kernel", "9e5dc9fce6518e7f", 244464543),
-    "latent": ("paged_decode_latent16_kernel", "87f771815d47e9f8", 654195478),
-    "latent128": ("paged_decode_latent128_kernel", "c394a61fcc308551", 743929974),
-    "latent-prefill": ("latent_prefill_kernel", "c394a61fcc308551", 332296701),
+    "config2": ("paged_decode_mfma16_kernel", "df5353961e3de31b", 310422502),
+    "config5": ("paged_decode_mfma16_kernel", "df5353961e3de31b", 168457019),
+    "config4": ("paged_decode_mfma16_kernel", "df5353961e3de31b", 3415575004),
+    "config3": ("prefill_kernel", "9e5dc9fce6518e7f", 244434883),
+    "latent": ("paged_decode_latent16_kernel", "96465725840a6f73", 654193569),
+    "latent128": ("paged_decode_latent128_kernel", "2f1fa3176d0b8668", 739290014),
+    "latent-prefill": ("latent_prefill_kernel", "2f1fa3176d0b8668", 332038139),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}
