@@ -341,6 +341,12 @@ def test_every_address_of_the_128_head_form_stays_in_bounds(dqk, dv, sep_v, hq, 
                     b, inb = w >> 7, w & 127
                     assert (16 * (b // vb) + (inb >> 3), 16 * (b % vb) + 2 * (inb & 7)) == (hg, 16 * blk + 4 * quad + 2 * (w - w0))
     assert len(words) == gseg * dv // 2
+    # the merge's threads of four words: aligned, inside one head's eight, 16-byte output pieces
+    assert slot_floats_bf16 % 4 == 0 and vals_bf16 % 4 == 0
+    for w0 in range(0, vals_bf16, 4):
+        heads = {16 * ((w >> 7) // vb) + ((w & 127) >> 3) for w in range(w0, w0 + 4)}
+        cols = [16 * ((w >> 7) % vb) + 2 * (w & 7) for w in range(w0, w0 + 4)]
+        assert len(heads) == 1 and cols[0] % 8 == 0 and cols == list(range(cols[0], cols[0] + 8, 2))
     for seg_h in (0, nkv * nhb - 1):
         assert seg_h * gseg + gseg - 1 < hq and seg_h // nhb < nkv
     segs, cus = users * nkv * nhb, 256

@@ -438,50 +438,64 @@ __global__ inline __launch_bounds__(256) void decode_combine_kernel(DecodeArgs a
 // blocks of 16 heads x 16 elements (element e of head g at
 // ((g / 16 * (D / 16) + e / 16) * 16 + g % 16) * 16 + e % 16, the last block of heads padded), the order
 // in which the latent kernels hold them: the 64 lanes of a store then write 512 consecutive bytes.  A
-// thread owns one 32-bit word of every partial, in that order, and stores its two neighbouring
-// output elements as one word (the caller checks that output rows start on 4-byte boundaries).
-// Grid: x = segment, y = piece of kCombinePiece words.
+// thread owns W consecutive 32-bit words of every partial, in that order, and stores its 2 W
+// neighbouring output elements at once: W = 4 (16 bytes per load and store) where output rows start
+// on 16-byte boundaries, W = 1 where only on 4-byte ones (the caller checks).
+// Grid: x = segment, y = piece of kCombinePiece threads.
+template <int W>
 __global__ inline __launch_bounds__(256) void decode_combine_bf16_kernel(DecodeArgs a, int G, int D) {
+  static_assert(W == 1 || W == 4, "a thread's words stay inside one head's eight");
+  typedef uint32_t words_t __attribute__((ext_vector_type(W)));
   const int seg = blockIdx.x;
   const int pairs = (G + 15) / 16 * 16 * D / 2;  // words of values in a partial
-  const int p = blockIdx.y * kCombinePiece + threadIdx.x;
+  const int p = W * (blockIdx.y * kCombinePiece + threadIdx.x);
   if (p >= pairs) return;
   const int u = seg / a.hkv, h = seg % a.hkv;
   const int blk = p >> 7, in_blk = p & 127;  // a block: 16 heads x 8 words
   const int g = 16 * (blk / (D / 16)) + (in_blk >> 3), e = 16 * (blk % (D / 16)) + 2 * (in_blk & 7);
   if (g >= G) return;
   const int first = a.ws_seg[2 * seg], nw = a.ws_seg[2 * seg + 1];
-  uint32_t *out = reinterpret_cast<uint32_t *>(a.out + u * a.out_us + (int64_t)(h * G + g) * a.out_hs + e);
+  words_t *out = reinterpret_cast<words_t *>(a.out + u * a.out_us + (int64_t)(h * G + g) * a.out_hs + e);
   if (nw == 0) {  // padded row: no attended position -> NaN like softmax over nothing
-    *out = 0x7fc07fc0u;
+    words_t nan;
+#pragma unroll
+    for (int k = 0; k < W; ++k) nan[k] = 0x7fc07fc0u;
+    *out = nan;
     return;
   }
   const float *base = a.ws_slots + (int64_t)first * a.slot_floats;
-  float mall = -INFINITY, num0 = 0.f, num1 = 0.f, den = 0.f;
+  float mall = -INFINITY, den = 0.f, num[2 * W];
+#pragma unroll
+  for (int k = 0; k < 2 * W; ++k) num[k] = 0.f;
   // partials are read in batches so that their loads overlap; a segment that few ranges share (the
   // 128-head latent form: two or three) takes batches of its size instead of eight mostly repeated loads
   auto merge = [&](auto batch_tag) {
     constexpr int kBatch = decltype(batch_tag)::value;
     for (int w = 0; w < nw; w += kBatch) {
       float mv[kBatch], lv[kBatch];
-      uint32_t av[kBatch];
+      words_t av[kBatch];
 #pragma unroll
       for (int j = 0; j < kBatch; ++j) {
         const float *sl = base + (int64_t)min(w + j, nw - 1) * a.slot_floats;
         mv[j] = (w + j < nw) ? sl[pairs + g] : -INFINITY;
         lv[j] = sl[pairs + G + g];
-        av[j] = reinterpret_cast<const uint32_t *>(sl)[p];
+        av[j] = *reinterpret_cast<const words_t *>(reinterpret_cast<const uint32_t *>(sl) + p);
       }
       float mnew = mall;
 #pragma unroll
       for (int j = 0; j < kBatch; ++j) mnew = fmaxf(mnew, mv[j]);
       const float resc = __builtin_amdgcn_exp2f(mall - mnew);
-      num0 *= resc, num1 *= resc, den *= resc;
+      den *= resc;
+#pragma unroll
+      for (int k = 0; k < 2 * W; ++k) num[k] *= resc;
 #pragma unroll
       for (int j = 0; j < kBatch; ++j) {
         const float wgt = __builtin_amdgcn_exp2f(mv[j] - mnew);  // 0 for the padding entries
-        num0 = fmaf(wgt, bf16_lo(av[j]), num0);
-        num1 = fmaf(wgt, bf16_hi(av[j]), num1);
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+          num[2 * k] = fmaf(wgt, bf16_lo(av[j][k]), num[2 * k]);
+          num[2 * k + 1] = fmaf(wgt, bf16_hi(av[j][k]), num[2 * k + 1]);
+        }
         den = fmaf(wgt, lv[j], den);
       }
       mall = mnew;
@@ -494,10 +508,15 @@ __global__ inline __launch_bounds__(256) void decode_combine_bf16_kernel(DecodeA
     const float sk = a.sink[h * G + g] * 1.4426950408889634f;
     const float mnew = fmaxf(mall, sk);
     const float resc = __builtin_amdgcn_exp2f(mall - mnew);
-    num0 *= resc, num1 *= resc;
+#pragma unroll
+    for (int k = 0; k < 2 * W; ++k) num[k] *= resc;
     den = den * resc + __builtin_amdgcn_exp2f(sk - mnew);
   }
-  *out = f32_to_bf16_bits(num0 / den) | (f32_to_bf16_bits(num1 / den) << 16);
+  const float inv = 1.0f / den;
+  words_t res;
+#pragma unroll
+  for (int k = 0; k < W; ++k) res[k] = f32_to_bf16_bits(num[2 * k] * inv) | (f32_to_bf16_bits(num[2 * k + 1] * inv) << 16);
+  *out = res;
 }
 
 inline int slot_floats_for(int g, int d) { return ((g * d + 2 * g + 3) / 4) * 4; }

@@ -1280,6 +1280,16 @@ using namespace ttpa;
 using namespace ttpa::decode;
 
 // Workspace: the segment table followed by (workgroups + segments) partial slots.
+// The merge of bfloat16 partials: 16 bytes per thread where the output rows allow it.
+static void launch_combine_bf16(const DecodeArgs &a, int segments, int gseg, int head_dim_v, const void *out, int64_t out_user_stride,
+                                int64_t out_head_stride, hipStream_t st) {
+  const int words = (gseg + 15) / 16 * 16 * head_dim_v / 2;
+  if (out_user_stride % 8 == 0 && out_head_stride % 8 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0)
+    decode_combine_bf16_kernel<4><<<dim3(segments, combine_pieces(words / 4, 1)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+  else
+    decode_combine_bf16_kernel<1><<<dim3(segments, combine_pieces(words, 1)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+}
+
 static int wide_geometry(int32_t q_heads, int32_t kv_heads, int32_t &nhb, int32_t &gseg) {
   const int g = q_heads / kv_heads;
   if (g <= 32) {
@@ -1427,7 +1437,7 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
     if (!ok) return fail(TTPA_ERR_LAUNCH, "latent decode: cannot configure the kernel");
     if (int rc = check_launch("paged_mla_decode")) return rc;
     if (a.partial_bf16)
-      decode_combine_bf16_kernel<<<dim3(users * kv_heads * nhb, combine_pieces((gseg + 15) / 16 * 16, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+      launch_combine_bf16(a, users * kv_heads * nhb, gseg, head_dim_v, out, out_user_stride, out_head_stride, st);
     else
       decode_combine_kernel<<<dim3(users * kv_heads * nhb, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
     return check_launch("paged_mla_decode");
@@ -1465,7 +1475,7 @@ static int mla_decode_impl(void *out, int64_t out_user_stride, int64_t out_head_
       if (!ok) return fail(TTPA_ERR_LAUNCH, "latent decode: cannot configure the kernel");
       if (int rc = check_launch("paged_mla_decode")) return rc;
       if (a.partial_bf16)
-        decode_combine_bf16_kernel<<<dim3(users * kv_heads, combine_pieces(16, head_dim_v / 2)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
+        launch_combine_bf16(a, users * kv_heads, gseg, head_dim_v, out, out_user_stride, out_head_stride, st);
       else
         decode_combine_kernel<<<dim3(users * kv_heads, combine_pieces(gseg, head_dim_v)), dim3(256), 0, st>>>(a, gseg, head_dim_v);
       return check_launch("paged_mla_decode");
