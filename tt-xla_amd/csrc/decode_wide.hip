@@ -746,16 +746,36 @@ struct LatentMath {
   }
   // O^T += V^T . P^T of the step at `step` with probabilities pf
   __device__ __forceinline__ void values(uint32_t step, const u32x4 (&pf)[RB]) { B::values(step, pf, vfrag); }
-  // The same and, between its matrix instructions, the softmax (no masks, scale > 0) of the score tiles
-  // st of the step after it; pf is replaced by the new probabilities.  The block keeps the running
-  // maxima as they are; where a score would move one (rarely: a maximum moves by 8 at least), the
-  // softmax above redoes the step.
-  __device__ __forceinline__ void values_softmax(uint32_t step, u32x4 (&pf)[RB], floatx4 (&st)[RB][2], float (&alpha)[RB], float scale) {
+  // A whole step as one block: the scores of the step at `step`, the second product of the step at
+  // `before` (probabilities pf) and, between the matrix instructions of the latter, the softmax (no
+  // masks, scale > 0) of the new scores; pf is replaced by the new probabilities.  The block keeps the
+  // running maxima as they are; where a score would move one (rarely: a maximum moves by 8 at least),
+  // the softmax above redoes the step.
+  __device__ __forceinline__ void whole_step(uint32_t step, uint32_t before, u32x4 (&pf)[RB], floatx4 (&st)[RB][2], float (&alpha)[RB], float scale) {
     u32x4 pn[RB];
     float sum[RB];
     uint64_t moved;
     const float m[RB] = {ml[0], ml[1]};
-    B::values_softmax(step, pn, sum, moved, st, m, th, pf, vfrag, scale);
+    B::whole_step(step, before, st, pn, sum, moved, kfrag, vfrag, q16, q8, m, th, pf, scale);
+    take(moved, pn, sum, pf, st, alpha, scale);
+  }
+  // The same with the wavefront's requests between the matrix instructions of the score product
+  // (scores_requesting)
+  template <bool STREAMING>
+  __device__ __forceinline__ void whole_step_requesting(uint32_t step, uint32_t before, u32x4 (&pf)[RB], floatx4 (&st)[RB][2], float (&alpha)[RB],
+                                                        float scale, const uint32_t (&off)[REQUESTS], const void *from, uint32_t dst) {
+    u32x4 pn[RB];
+    float sum[RB];
+    uint64_t moved;
+    const float m[RB] = {ml[0], ml[1]};
+    B::template whole_step_requesting<STREAMING>(step, before, st, pn, sum, moved, kfrag, vfrag, q16, q8, m, th, pf, scale, off,
+                                                 static_cast<const char *>(from), dst);
+    take(moved, pn, sum, pf, st, alpha, scale);
+  }
+
+ private:
+  __device__ __forceinline__ void take(uint64_t moved, const u32x4 (&pn)[RB], const float (&sum)[RB], u32x4 (&pf)[RB], floatx4 (&st)[RB][2],
+                                       float (&alpha)[RB], float scale) {
     if (moved == 0) {
       pf[0] = pn[0], pf[1] = pn[1];
       ml[RB] += sum[0], ml[RB + 1] += sum[1];
@@ -777,7 +797,7 @@ struct LatentMath {
 // heads and computes every score four times.
 // The vector unit has no second wavefront to serve while the matrix unit works, so the softmax of a
 // step's scores sits between the matrix instructions of the second product of the step before
-// (values_softmax), and the requests for a later step between those of the score product
+// (whole_step), and the requests for a later step between those of the score product
 // (scores_requesting); steps with masked keys (a sequence's last tile, the first of a sliding
 // window) and a segment's first step take the softmax below.  A step's second product thereby runs
 // one step late, so K lives in a ring of four stages with one barrier per step: past the barrier of
@@ -947,12 +967,13 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
       // which the score tiles hold a lane's keys and the transposing reads their rows).
       const uint32_t step = lds0 + (uint32_t)((i % NSTAGES) * STAGE);
       floatx4 st[RB][2];
-      if (inside) m.template scores_requesting<true>(step, st, src_off, piece_source(nxt, half), piece_stage(i + 2));
-      else m.scores(step, st);
       float alpha[RB];
       if (have_prev && nv >= KEYS && nb <= 0 && scale > 0.f) {
-        m.values_softmax(prev, pf, st, alpha, scale);
+        if (inside) m.template whole_step_requesting<true>(step, prev, pf, st, alpha, scale, src_off, piece_source(nxt, half), piece_stage(i + 2));
+        else m.whole_step(step, prev, pf, st, alpha, scale);
       } else {
+        if (inside) m.template scores_requesting<true>(step, st, src_off, piece_source(nxt, half), piece_stage(i + 2));
+        else m.scores(step, st);
         if (have_prev) m.values(prev, pf);
         // lane (head, quad) holds keys 16 pc + 4 quad + e of the step
         m.softmax(st, pf, alpha, scale, [&](int, int pc, int e) {
@@ -1177,17 +1198,16 @@ __global__ __launch_bounds__(256) void latent_prefill_kernel(LatentPrefillArgs a
     // order in which the score tiles hold the keys of a lane, and the transposing reads their rows.
     const uint32_t step = lds0 + (uint32_t)((i % NSTAGES) * STAGE);
     floatx4 st[RB][2];
-    if (inside) {
-      const uint32_t dst0 = (uint32_t)__builtin_amdgcn_readfirstlane(
-          (int)(lds0 + (uint32_t)(((i + 2) % NSTAGES) * STAGE + 1024 * wave * PER_WAVE)));
-      m.template scores_requesting<false>(step, st, req_off, kbase_g + (int64_t)(i + 2) * KEYS * a.k_ts, dst0);
-    } else {
-      m.scores(step, st);
-    }
     float alpha[RB];
+    const uint32_t dst0 = (uint32_t)__builtin_amdgcn_readfirstlane(
+        (int)(lds0 + (uint32_t)(((i + 2) % NSTAGES) * STAGE + 1024 * wave * PER_WAVE)));
+    const uint16_t *from = kbase_g + (int64_t)(i + 2) * KEYS * a.k_ts;
     if (have_prev && plain && key0 + KEYS - 1 <= first_limit) {
-      m.values_softmax(prev, pf, st, alpha, scale);
+      if (inside) m.template whole_step_requesting<false>(step, prev, pf, st, alpha, scale, req_off, from, dst0);
+      else m.whole_step(step, prev, pf, st, alpha, scale);
     } else {
+      if (inside) m.template scores_requesting<false>(step, st, req_off, from, dst0);
+      else m.scores(step, st);
       if (have_prev) m.values(prev, pf);
       // lane (row, quad) holds keys key0 + 16 pc + 4 quad + e of its rows
       int limit[RB], t[RB], head[RB];

@@ -30,6 +30,10 @@ kernels for that), every one of them lists all 256 as clobbered, and volatile st
 order.  Everything else (LDS addresses of the lane's fragments, probabilities) comes in registers
 that the compiler chooses.
 
+A step without masks is one statement (whole_step): its two products share one pipeline of fragment
+reads, so the second one starts on fragments that were requested while the first one ran.  The
+products also exist on their own (scores, values) for steps whose softmax is C++ (masks).
+
 A ring slot is refilled one matrix instruction after the last one that read it.  Waits are counted: a
 block starts with lgkmcnt(0), so the counter holds its own reads only.  Matrix results are read by
 vector instructions no earlier than 16 wait states after the last matrix instruction (s_nop at the
@@ -82,32 +86,46 @@ class Regs:
         return [f'"v{r}"' for r in range(self.ring, self.ring + 4 * DEPTH)]
 
 
-def pipeline(n, reads_per_step, read, mma, every=1):
-    """n steps; read(j, slot) returns the read instructions of step j into ring slot `slot`, mma(j, slot)
-    the matrix instructions that use them.  The slot of step j - 1 is refilled behind the first matrix
-    instruction of step j.  A wait in front of every `every`-th step covers that many steps (a
-    wavefront alone on its SIMD issues one instruction per four cycles, whatever the kind: a wait is not
-    free)."""
+def pipeline(n, read, mma, covers):
+    """n steps; read(j, slot) returns the read instructions of step j into ring slot `slot` = j % depth,
+    mma(j, slot) the matrix instructions that use them.  The slot of step j - 1 is refilled behind the
+    first matrix instruction of step j.  covers(j): the last step whose reads the wait in front of step
+    j covers, or None for no wait there (a wavefront alone on its SIMD issues one instruction per four
+    cycles, whatever the kind: a wait is not free)."""
     depth = min(DEPTH, n)
-    lines, issued = [], []
+    lines, queue = [], []  # queue: (step, read instructions) in the order of issue
+
+    def issue(j):
+        r = read(j, j % depth)
+        queue.append((j, len(r)))
+        return r
+
     for j in range(depth):
-        lines += read(j, j % depth)
-        issued.append(j)
+        lines += issue(j)
+    waited = -1
     for j in range(n):
-        if j % every == 0:
-            last = min(j + every - 1, n - 1)
-            assert all(x in issued for x in range(j, last + 1)), "a wait covers reads that are under way"
-            behind = reads_per_step * len([x for x in issued if x > last])
+        last = covers(j)
+        if last is not None:
+            at = [k for k, (step, _) in enumerate(queue) if step == last]
+            assert len(at) == 1 and last >= j, "a wait covers reads that are under way"
+            behind = sum(c for _, c in queue[at[0] + 1:])
+            assert behind <= 15
             lines.append(f"s_waitcnt lgkmcnt({behind})")
+            waited = last
+        assert waited >= j
         ops = mma(j, j % depth)
         lines.append(ops[0])
         nxt = j - 1 + depth
         if j >= 1 and nxt < n:
-            lines += read(nxt, nxt % depth)
-            issued.append(nxt)
+            lines += issue(nxt)
         lines += ops[1:]
-    assert sorted(issued) == list(range(n))
+    assert [step for step, _ in queue] == list(range(n))
     return lines
+
+
+def every(k, n):
+    """covers() of pipeline: a wait in front of every k-th of n steps."""
+    return lambda j: min(j + k - 1, n - 1) if j % k == 0 else None
 
 
 def spread(lines, extra, first=1, last_fraction=1.0):
@@ -161,12 +179,8 @@ def q_operands(R, dqk):
 
 def scores(dqk, dv, gc, requests=0, nt=False):
     """Both pieces of a step, their steps of 32 features alternating (four independent accumulation
-    chains).  requests > 0: the wavefront's LDS-DMA requests for a later step go out between the
-    matrix instructions (a 1 KiB request occupies the address path for 16 cycles, and a wavefront
-    that waits for it issues nothing else): request j reads 16 bytes per lane at base (j % 4) +
-    offset j and lands at LDS address dst + 1024 j (base i = the step's address - 1024 i: the
-    instruction offset 1024 i moves the LDS address and the global address alike, so four requests
-    share a value of M0)."""
+    chains).  requests > 0: with the wavefront's LDS-DMA requests for a later step between the matrix
+    instructions (request_groups)."""
     R = Regs(dqk, dv)
     ksteps, piece, kb = dqk // 32, 32 * dqk, gc // 4
     n_out = 2 * RB
@@ -183,7 +197,7 @@ def scores(dqk, dv, gc, requests=0, nt=False):
         return [f"v_mfma_f32_16x16x32_bf16 {R.score(b, pc)}, {R.slot(slot)}, {R.q(b, s)}, {'0' if s == 0 else R.score(b, pc)}"
                 for b in range(RB)]
 
-    lines = ["s_waitcnt lgkmcnt(0)"] + pipeline(2 * ksteps, 1, read, mma) + ["s_nop 7", "s_nop 7"]
+    lines = ["s_waitcnt lgkmcnt(0)"] + pipeline(2 * ksteps, read, mma, every(1, 2 * ksteps)) + ["s_nop 7", "s_nop 7"]
     args = [f"floatx4 &st{2 * b + pc}" for b in range(RB) for pc in range(2)] + [f"uint32_t kb{i}" for i in range(kb)]
     outs = [f'"=&{{{R.score(b, pc)}}}"(st{2 * b + pc})' for b in range(RB) for pc in range(2)]
     ins = [f'"v"(kb{i})' for i in range(kb)]
@@ -196,14 +210,7 @@ def scores(dqk, dv, gc, requests=0, nt=False):
         args += [f"uint32_t off{j}" for j in range(requests)] + [f"const void *base{i}" for i in range(4)] + ["uint32_t dst"]
         ins += [f'"v"(off{j})' for j in range(requests)] + [f'"s"(base{i})' for i in range(4)] + ['"s"(dst)']
         assert len(outs) + len(ins) <= 30
-        req = []
-        for j in range(requests):
-            r = []
-            if j % 4 == 0:
-                r += [f"s_mov_b32 m0, %{dst}" if j == 0 else f"s_add_u32 m0, %{dst}, {1024 * j}", "s_nop 0"]
-            r.append(f"global_load_lds_dwordx4 %{off + j}, %{base + j % 4}" + (f" offset:{1024 * (j % 4)}" if j % 4 else "") +
-                     (" nt" if nt else ""))
-            req.append(r)
+        req = request_groups(requests, off, base, dst, nt)
         lines = spread(lines, req, first=4, last_fraction=0.75)
         clob, name = clob + ['"m0"', '"scc"'], name + "_req" + ("_nt" if nt else "")
     comment = (f"// S^T = K . Q^T of the two pieces of a step: {ksteps} steps of 32 features, swizzle groups of {gc} chunks" +
@@ -211,7 +218,7 @@ def scores(dqk, dv, gc, requests=0, nt=False):
     return statement(comment, name, args, lines, outs, ins, clob)
 
 
-def values_pipeline(R, dv, gc, piece, pf_in, vb_in, every=1):
+def values_pipeline(R, dv, gc, piece, pf_in, vb_in):
     vbases = gc // 2
 
     def read(j, slot):
@@ -222,7 +229,7 @@ def values_pipeline(R, dv, gc, piece, pf_in, vb_in, every=1):
     def mma(j, slot):
         return [f"v_mfma_f32_16x16x32_bf16 {R.accum(b, j)}, {R.slot(slot)}, %{pf_in + b}, {R.accum(b, j)}" for b in range(RB)]
 
-    return pipeline(dv // 16, 2, read, mma, every)
+    return pipeline(dv // 16, read, mma, every(1, dv // 16))
 
 
 def values(dqk, dv, gc):
@@ -271,39 +278,102 @@ def softmax_groups(R, scale, m, th, total, moved):
     return out
 
 
-def values_softmax(dqk, dv, gc):
-    """The second product of one step with the softmax of the next step's scores between its matrix
-    instructions."""
+def request_groups(requests, off, base, dst, nt):
+    """The wavefront's LDS-DMA requests for a later step (a 1 KiB request occupies the address path for
+    16 cycles, and a wavefront that waits for it issues nothing else): request j reads 16 bytes per
+    lane at base (j % 4) + offset j and lands at LDS address dst + 1024 j (base i = the step's address
+    - 1024 i: the instruction offset 1024 i moves the LDS address and the global address alike, so
+    four requests share a value of M0).  off, base, dst: the first operand numbers."""
+    req = []
+    for j in range(requests):
+        r = []
+        if j % 4 == 0:
+            r += [f"s_mov_b32 m0, %{dst}" if j == 0 else f"s_add_u32 m0, %{dst}, {1024 * j}", "s_nop 0"]
+        r.append(f"global_load_lds_dwordx4 %{off + j}, %{base + j % 4}" + (f" offset:{1024 * (j % 4)}" if j % 4 else "") +
+                 (" nt" if nt else ""))
+        req.append(r)
+    return req
+
+
+def whole_step(dqk, dv, gc, requests=0, nt=False):
+    """A step as one statement and one pipeline: the score product of the step at kb.., then the second
+    product of the step before (at vb.., probabilities pf) with the softmax of the new scores between
+    its matrix instructions.  The ring slots that the last score steps leave take the first V^T
+    fragments, so the matrix unit goes from one product to the other without a gap (as two statements
+    the second one starts with reads of its own and their latency: a twentieth of a step)."""
     R = Regs(dqk, dv)
-    vbases = gc // 2
-    # operands: outputs 0..1 next probabilities, 2..3 their sums, 4 the lanes whose maximum has to move;
-    # inputs: 5..8 score tiles, 9..10 maxima, 11..12 thresholds, 13..14 probabilities of the step whose
-    # second product this is, V^T bases, scale
-    n_out = 2 * RB + 1
-    moved = f"%{2 * RB}"
-    st_in = n_out
-    m_in, th_in = st_in + 2 * RB, st_in + 3 * RB
-    pf_in = th_in + RB
-    vb_in = pf_in + RB
-    scale = f"%{vb_in + vbases}"
-    product = values_pipeline(R, dv, gc, 32 * dqk, pf_in, vb_in, every=2)
-    lines = ([MARK_BEGIN, f"s_mov_b64 {moved}, 0", "s_nop 0", "s_waitcnt lgkmcnt(0)"] +
-             spread(product, softmax_groups(R, scale, m_in, th_in, RB, moved), first=2) + ["s_nop 7", "s_nop 7", MARK_END])
-    args = ([f"u32x4 &pn{b}" for b in range(RB)] + [f"float &sum{b}" for b in range(RB)] + ["uint64_t &moved"] +
-            [f"const floatx4 &st{2 * b + pc}" for b in range(RB) for pc in range(2)] + [f"float m{b}" for b in range(RB)] +
-            [f"float th{b}" for b in range(RB)] + [f"const u32x4 &pf{b}" for b in range(RB)] +
-            [f"uint32_t vb{i}" for i in range(vbases)] + ["float scale"])
-    outs = ([f'"=&{{v[{R.pn + 4 * b}:{R.pn + 4 * b + 3}]}}"(pn{b})' for b in range(RB)] + [f'"=&v"(sum{b})' for b in range(RB)] +
-            ['"=&s"(moved)'])
-    ins = ([f'"{{{R.score(b, pc)}}}"(st{2 * b + pc})' for b in range(RB) for pc in range(2)] + [f'"v"(m{b})' for b in range(RB)] +
-           [f'"v"(th{b})' for b in range(RB)] + [f'"v"(pf{b})' for b in range(RB)] + [f'"v"(vb{i})' for i in range(vbases)] +
-           ['"s"(scale)'])
-    assert len(outs) == n_out and len(outs) + len(ins) <= 30
-    clob = R.ring_clobbers() + [f'"v{r}"' for r in range(R.tmp, R.tmp + 4 * RB)] + ['"vcc"', '"scc"'] + ACC_CLOBBERS
-    comment = (f"// O^T += V^T . P^T of one step ({dv // 16} blocks of 16 value columns) and, between its matrix instructions, the\\n"
-               "// softmax of the score tiles st.. of the next step against the running maxima m.. as they are (no masks,\\n"
-               "// scale > 0): pn the probabilities, sum their sums, moved != 0 where a score exceeds th = (m + 8) / scale")
-    return statement(comment.replace("\\n", "\n"), f"latent_values_softmax_{dqk}_{dv}", args, lines, outs, ins, clob)
+    ksteps, piece, kb, vbases = dqk // 32, 32 * dqk, gc // 4, gc // 2
+    ns, nv = 2 * ksteps, dv // 16
+    # operands: outputs 0..3 score tiles, 4..5 next probabilities, 6..7 their sums, 8 the lanes whose
+    # maximum has to move; inputs: K bases, V^T bases, Q, maxima, thresholds, probabilities, scale, (requests)
+    n_out = 4 * RB + 1
+    st_out, pn_out, sum_out, moved = 0, 2 * RB, 3 * RB, f"%{4 * RB}"
+    kb_in = n_out
+    vb_in = kb_in + kb
+    qa, qi = q_operands(R, dqk)
+    m_in = vb_in + vbases + len(qi)
+    th_in, pf_in = m_in + RB, m_in + 2 * RB
+    scale = f"%{pf_in + RB}"
+
+    def read(j, slot):
+        if j < ns:
+            pc, f = j % 2, j // 2  # piece, step of 32 features
+            return [f"ds_read_b128 {R.slot(slot)}, %{kb_in + f % kb} offset:{pc * piece + 16 * gc * (f // kb)}"]
+        t = j - ns
+        base, off = f"%{vb_in + t % vbases}", 16 * gc * (t // vbases)
+        return [f"ds_read_b64_tr_b16 {R.slot(slot, 0, 2)}, {base} offset:{off}",
+                f"ds_read_b64_tr_b16 {R.slot(slot, 2, 2)}, {base} offset:{off + piece}"]
+
+    def mma(j, slot):
+        if j < ns:
+            pc, f = j % 2, j // 2
+            return [f"v_mfma_f32_16x16x32_bf16 {R.score(b, pc)}, {R.slot(slot)}, {R.q(b, f)}, {'0' if f == 0 else R.score(b, pc)}"
+                    for b in range(RB)]
+        t = j - ns
+        return [f"v_mfma_f32_16x16x32_bf16 {R.accum(b, t)}, {R.slot(slot)}, %{pf_in + b}, {R.accum(b, t)}" for b in range(RB)]
+
+    def covers(j):  # every score step, every second step of the second product
+        if j < ns:
+            return j
+        return min(j + 1, ns + nv - 1) if (j - ns) % 2 == 0 else None
+
+    lines = pipeline(ns + nv, read, mma, covers)
+    split = min(k for k, ln in enumerate(lines) if ln.startswith("v_mfma") and " a[" in ln)
+    first, second = lines[:split], lines[split:]
+    # the vector unit reads the score tiles no earlier than 16 wait states behind their last matrix instruction
+    count = seen = 0
+    for ln in second:
+        count += 1
+        seen += ln.startswith("v_mfma")
+        if count >= 16:
+            break
+    assert count >= 16 and seen + 1 < 2 * nv
+    second = spread(second, softmax_groups(R, scale, m_in, th_in, sum_out, moved), first=seen + 1)
+    args = ([f"floatx4 &st{2 * b + pc}" for b in range(RB) for pc in range(2)] + [f"u32x4 &pn{b}" for b in range(RB)] +
+            [f"float &sum{b}" for b in range(RB)] + ["uint64_t &moved"] + [f"uint32_t kb{i}" for i in range(kb)] +
+            [f"uint32_t vb{i}" for i in range(vbases)] + qa + [f"float m{b}" for b in range(RB)] + [f"float th{b}" for b in range(RB)] +
+            [f"const u32x4 &pf{b}" for b in range(RB)] + ["float scale"])
+    outs = ([f'"=&{{{R.score(b, pc)}}}"(st{2 * b + pc})' for b in range(RB) for pc in range(2)] +
+            [f'"=&{{v[{R.pn + 4 * b}:{R.pn + 4 * b + 3}]}}"(pn{b})' for b in range(RB)] + [f'"=&v"(sum{b})' for b in range(RB)] + ['"=&s"(moved)'])
+    ins = ([f'"v"(kb{i})' for i in range(kb)] + [f'"v"(vb{i})' for i in range(vbases)] + qi + [f'"v"(m{b})' for b in range(RB)] +
+           [f'"v"(th{b})' for b in range(RB)] + [f'"v"(pf{b})' for b in range(RB)] + ['"s"(scale)'])
+    assert len(outs) == n_out and R.score(0, 0) == f"v[{R.st}:{R.st + 3}]"
+    clob = R.ring_clobbers() + [f'"v{r}"' for r in range(R.tmp, R.tmp + 4 * RB)] + ['"vcc"', '"scc"']
+    name = f"latent_step_{dqk}_{dv}"
+    if requests:
+        at = len(outs) + len(ins)
+        args += [f"uint32_t off{j}" for j in range(requests)] + [f"const void *base{i}" for i in range(4)] + ["uint32_t dst"]
+        ins += [f'"v"(off{j})' for j in range(requests)] + [f'"s"(base{i})' for i in range(4)] + ['"s"(dst)']
+        first = spread(first, request_groups(requests, at, at + requests, at + requests + 4, nt), first=4, last_fraction=0.75)
+        clob, name = clob + ['"m0"'], name + "_req" + ("_nt" if nt else "")
+    lines = ([MARK_BEGIN, f"s_mov_b64 {moved}, 0", "s_nop 0", "s_waitcnt lgkmcnt(0)"] + first + second + ["s_nop 7", "s_nop 7", MARK_END])
+    comment = (f"// One step: S^T = K . Q^T of the two pieces at kb.. ({ksteps} steps of 32 features), then O^T += V^T . P^T of the step\n"
+               f"// at vb.. ({nv} blocks of 16 value columns, probabilities pf) and, between its matrix instructions, the softmax of\n"
+               "// the new score tiles st.. against the running maxima m.. as they are (no masks, scale > 0): pn the\n"
+               "// probabilities, sum their sums, moved != 0 where a score exceeds th = (m + 8) / scale" +
+               (f"\n// (with {requests} LDS-DMA requests{', non-temporal,' if nt else ''} between the matrix instructions of the first product)"
+                if requests else ""))
+    return statement(comment.replace("\\n", "\n"), name, args, lines, outs, ins, clob + ACC_CLOBBERS)
 
 
 def accumulator_access(dv):
@@ -345,6 +415,7 @@ def wrappers(dqk, dv, gc, requests):
     st = ", ".join(f"st[{b}][{pc}]" for b in range(RB) for pc in range(2))
     kf = ", ".join(f"step + kf[{i}]" for i in range(kb))
     vf = ", ".join(f"step + vf[{i}]" for i in range(vbases))
+    vp = ", ".join(f"before + vf[{i}]" for i in range(vbases))
     offs = ", ".join(f"off[{j}]" for j in range(requests))
     reads = "\n".join(f"    {'if' if k == 0 else 'else if'} constexpr (B == {k // per} && I == {k % per}) latent_acc_read_{dv}_{k // per}_{k % per}(f);"
                       for k in range(RB * per))
@@ -367,10 +438,26 @@ struct LatentBlocks<{dqk}, {dv}> {{
   static __device__ __forceinline__ void values(uint32_t step, const u32x4 (&pf)[2], const uint32_t (&vf)[{vbases}]) {{
     latent_values_{dqk}_{dv}(pf[0], pf[1], {vf});
   }}
-  static __device__ __forceinline__ void values_softmax(uint32_t step, u32x4 (&pn)[2], float (&sum)[2], uint64_t &moved,
-                                                        const floatx4 (&st)[2][2], const float (&m)[2], const float (&th)[2],
-                                                        const u32x4 (&pf)[2], const uint32_t (&vf)[{vbases}], float scale) {{
-    latent_values_softmax_{dqk}_{dv}(pn[0], pn[1], sum[0], sum[1], moved, {st}, m[0], m[1], th[0], th[1], pf[0], pf[1], {vf}, scale);
+  // (`before`: the step whose second product this is)
+  static __device__ __forceinline__ void whole_step(uint32_t step, uint32_t before, floatx4 (&st)[2][2], u32x4 (&pn)[2], float (&sum)[2],
+                                                    uint64_t &moved, const uint32_t (&kf)[{kb}], const uint32_t (&vf)[{vbases}],
+                                                    const u32x16 (&q16)[2][{nq16}], const u32x8 (&q8)[2], const float (&m)[2],
+                                                    const float (&th)[2], const u32x4 (&pf)[2], float scale) {{
+    latent_step_{dqk}_{dv}({st}, pn[0], pn[1], sum[0], sum[1], moved, {kf}, {vp}, {qs}, m[0], m[1], th[0], th[1], pf[0], pf[1], scale);
+  }}
+  template <bool STREAMING>
+  static __device__ __forceinline__ void whole_step_requesting(uint32_t step, uint32_t before, floatx4 (&st)[2][2], u32x4 (&pn)[2],
+                                                               float (&sum)[2], uint64_t &moved, const uint32_t (&kf)[{kb}],
+                                                               const uint32_t (&vf)[{vbases}], const u32x16 (&q16)[2][{nq16}],
+                                                               const u32x8 (&q8)[2], const float (&m)[2], const float (&th)[2],
+                                                               const u32x4 (&pf)[2], float scale, const uint32_t (&off)[{requests}],
+                                                               const char *from, uint32_t dst) {{
+    if constexpr (STREAMING)
+      latent_step_{dqk}_{dv}_req_nt({st}, pn[0], pn[1], sum[0], sum[1], moved, {kf}, {vp}, {qs}, m[0], m[1], th[0], th[1], pf[0], pf[1], scale,
+                                    {offs}, from, from - 1024, from - 2048, from - 3072, dst);
+    else
+      latent_step_{dqk}_{dv}_req({st}, pn[0], pn[1], sum[0], sum[1], moved, {kf}, {vp}, {qs}, m[0], m[1], th[0], th[1], pf[0], pf[1], scale,
+                                 {offs}, from, from - 1024, from - 2048, from - 3072, dst);
   }}
   static __device__ __forceinline__ void clear() {{ latent_acc_clear_{dv}(); }}
   static __device__ __forceinline__ void scale(float alpha0, float alpha1) {{ latent_acc_scale_{dqk}_{dv}(alpha0, alpha1); }}
@@ -400,7 +487,9 @@ def main():
             once(("req", dqk), scores(dqk, dv, gc, requests=requests))
             once(("req_nt", dqk), scores(dqk, dv, gc, requests=requests, nt=True))
             f.write(values(dqk, dv, gc) + "\n")
-            f.write(values_softmax(dqk, dv, gc) + "\n")
+            f.write(whole_step(dqk, dv, gc) + "\n")
+            f.write(whole_step(dqk, dv, gc, requests=requests) + "\n")
+            f.write(whole_step(dqk, dv, gc, requests=requests, nt=True) + "\n")
             once(("acc", dv), accumulator_access(dv))
             f.write(accumulator_scale(dqk, dv) + "\n")
             f.write(wrappers(dqk, dv, gc, requests) + "\n")
