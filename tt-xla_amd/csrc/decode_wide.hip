@@ -746,7 +746,8 @@ struct LatentMath {
   }
   // O^T += V^T . P^T of the step at `step` with probabilities pf
   __device__ __forceinline__ void values(uint32_t step, const u32x4 (&pf)[RB]) { B::values(step, pf, vfrag); }
-  // A whole step as one block: the scores of the step at `step`, the second product of the step at
+  // A whole step as one block that starts with the workgroup's barrier of the step (the caller has
+  // waited for its own requests and does not call __syncthreads): the scores of the step at `step`, the second product of the step at
   // `before` (probabilities pf) and, between the matrix instructions of the latter, the softmax (no
   // masks, scale > 0) of the new scores; pf is replaced by the new probabilities.  The block keeps the
   // running maxima as they are; where a score would move one (rarely: a maximum moves by 8 at least),
@@ -947,11 +948,27 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
         __builtin_amdgcn_s_waitcnt(0x0F70);
       }
       drain = landed = false;
-      __syncthreads();  // ... everybody's has, and nobody reads the stage of step i - 2 any more
+      // ... and behind the workgroup's barrier everybody's has, and nobody reads the stage of step i - 2
+      // any more.  A wavefront whose step needs no masks runs it as one block that starts with the barrier.
       const int nv = nvalid - KEYS * half, nb = nbelow - KEYS * half;  // this step attends its keys nb .. nv - 1
       const bool computing = wave_active && nv > 0;
       // (a wavefront that computes sends the requests from inside the score product)
       const bool inside = computing && has_next;
+      // Two pieces (32 keys) per step: one softmax for both, and the second product takes them as the
+      // 32-deep K dimension of one matrix instruction per block of 16 value columns (k index 8 quad + j
+      // stands for key 4 quad + j of the first piece for j < 4, of the second otherwise: the order in
+      // which the score tiles hold a lane's keys and the transposing reads their rows).
+      const uint32_t step = lds0 + (uint32_t)((i % NSTAGES) * STAGE);
+      floatx4 st[RB][2];
+      float alpha[RB];
+      if (computing && have_prev && nv >= KEYS && nb <= 0 && scale > 0.f) {
+        if (inside) m.template whole_step_requesting<true>(step, prev, pf, st, alpha, scale, src_off, piece_source(nxt, half), piece_stage(i + 2));
+        else m.whole_step(step, prev, pf, st, alpha, scale);
+        m.scale_accumulators(alpha);
+        prev = step;
+        continue;
+      }
+      __syncthreads();
       if (has_next && !inside) request_step(nxt, half, i + 2);
       if (nv > 0 && nv < KEYS) {
         clear_unattended_rows(i, nv);
@@ -961,17 +978,7 @@ __global__ __launch_bounds__(256) void paged_decode_latent128_kernel(
         if (have_prev) m.values(prev, pf), have_prev = false;
         continue;
       }
-      // Two pieces (32 keys) per step: one softmax for both, and the second product takes them as the
-      // 32-deep K dimension of one matrix instruction per block of 16 value columns (k index 8 quad + j
-      // stands for key 4 quad + j of the first piece for j < 4, of the second otherwise: the order in
-      // which the score tiles hold a lane's keys and the transposing reads their rows).
-      const uint32_t step = lds0 + (uint32_t)((i % NSTAGES) * STAGE);
-      floatx4 st[RB][2];
-      float alpha[RB];
-      if (have_prev && nv >= KEYS && nb <= 0 && scale > 0.f) {
-        if (inside) m.template whole_step_requesting<true>(step, prev, pf, st, alpha, scale, src_off, piece_source(nxt, half), piece_stage(i + 2));
-        else m.whole_step(step, prev, pf, st, alpha, scale);
-      } else {
+      {
         if (inside) m.template scores_requesting<true>(step, st, src_off, piece_source(nxt, half), piece_stage(i + 2));
         else m.scores(step, st);
         if (have_prev) m.values(prev, pf);
@@ -1182,11 +1189,26 @@ __global__ __launch_bounds__(256) void latent_prefill_kernel(LatentPrefillArgs a
     // this wavefront's share of step i has landed (the requests of step i + 1 may still be under way)
     if (i + 1 < nsteps) __builtin_amdgcn_s_waitcnt(0x0F70 | PER_WAVE);
     else __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();  // ... everybody's has, and nobody reads the stage of step i - 2 any more
+    // ... and behind the workgroup's barrier everybody's has, and nobody reads the stage of step i - 2 any
+    // more.  A wavefront whose step needs no masks runs the step as one block that starts with the barrier.
     const int key0 = i * KEYS;
     const bool computing = wave_active && key0 <= wave_limit;
     // (a wavefront that computes sends whole steps' requests from inside the score product)
     const bool inside = computing && i + 2 < nsteps && (i + 3) * KEYS <= a.s;
+    const uint32_t step = lds0 + (uint32_t)((i % NSTAGES) * STAGE);
+    floatx4 st[RB][2];
+    float alpha[RB];
+    const uint32_t dst0 = (uint32_t)__builtin_amdgcn_readfirstlane(
+        (int)(lds0 + (uint32_t)(((i + 2) % NSTAGES) * STAGE + 1024 * wave * PER_WAVE)));
+    const uint16_t *from = kbase_g + (int64_t)(i + 2) * KEYS * a.k_ts;
+    if (computing && have_prev && plain && key0 + KEYS - 1 <= first_limit && (inside || i + 2 >= nsteps)) {
+      if (inside) m.template whole_step_requesting<false>(step, prev, pf, st, alpha, scale, req_off, from, dst0);
+      else m.whole_step(step, prev, pf, st, alpha, scale);
+      m.scale_accumulators(alpha);
+      prev = step;
+      continue;
+    }
+    __syncthreads();
     if (i + 2 < nsteps && !inside) request_step(i + 2);
     if (!computing) {
       if (have_prev) m.values(prev, pf), have_prev = false;
@@ -1196,16 +1218,7 @@ __global__ __launch_bounds__(256) void latent_prefill_kernel(LatentPrefillArgs a
     // 32-deep K dimension of one matrix instruction per block of 16 value columns.  k index 8 quad + j
     // of that instruction stands for key 4 quad + j of the first piece (j < 4) or of the second: the
     // order in which the score tiles hold the keys of a lane, and the transposing reads their rows.
-    const uint32_t step = lds0 + (uint32_t)((i % NSTAGES) * STAGE);
-    floatx4 st[RB][2];
-    float alpha[RB];
-    const uint32_t dst0 = (uint32_t)__builtin_amdgcn_readfirstlane(
-        (int)(lds0 + (uint32_t)(((i + 2) % NSTAGES) * STAGE + 1024 * wave * PER_WAVE)));
-    const uint16_t *from = kbase_g + (int64_t)(i + 2) * KEYS * a.k_ts;
-    if (have_prev && plain && key0 + KEYS - 1 <= first_limit) {
-      if (inside) m.template whole_step_requesting<false>(step, prev, pf, st, alpha, scale, req_off, from, dst0);
-      else m.whole_step(step, prev, pf, st, alpha, scale);
-    } else {
+    {
       if (inside) m.template scores_requesting<false>(step, st, req_off, from, dst0);
       else m.scores(step, st);
       if (have_prev) m.values(prev, pf);

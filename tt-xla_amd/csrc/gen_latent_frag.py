@@ -86,12 +86,13 @@ class Regs:
         return [f'"v{r}"' for r in range(self.ring, self.ring + 4 * DEPTH)]
 
 
-def pipeline(n, read, mma, covers):
+def pipeline(n, read, mma, covers, after_fill=()):
     """n steps; read(j, slot) returns the read instructions of step j into ring slot `slot` = j % depth,
     mma(j, slot) the matrix instructions that use them.  The slot of step j - 1 is refilled behind the
     first matrix instruction of step j.  covers(j): the last step whose reads the wait in front of step
     j covers, or None for no wait there (a wavefront alone on its SIMD issues one instruction per four
-    cycles, whatever the kind: a wait is not free)."""
+    cycles, whatever the kind: a wait is not free).  after_fill: lines behind the reads that fill the
+    ring at the start."""
     depth = min(DEPTH, n)
     lines, queue = [], []  # queue: (step, read instructions) in the order of issue
 
@@ -102,6 +103,7 @@ def pipeline(n, read, mma, covers):
 
     for j in range(depth):
         lines += issue(j)
+    lines += list(after_fill)
     waited = -1
     for j in range(n):
         last = covers(j)
@@ -296,7 +298,8 @@ def request_groups(requests, off, base, dst, nt):
 
 
 def whole_step(dqk, dv, gc, requests=0, nt=False):
-    """A step as one statement and one pipeline: the score product of the step at kb.., then the second
+    """A step as one statement and one pipeline, the workgroup's barrier included (the caller has
+    waited for its own requests): the score product of the step at kb.., then the second
     product of the step before (at vb.., probabilities pf) with the softmax of the new scores between
     its matrix instructions.  The ring slots that the last score steps leave take the first V^T
     fragments, so the matrix unit goes from one product to the other without a gap (as two statements
@@ -315,30 +318,42 @@ def whole_step(dqk, dv, gc, requests=0, nt=False):
     th_in, pf_in = m_in + RB, m_in + 2 * RB
     scale = f"%{pf_in + RB}"
 
+    # The statement starts with the workgroup's barrier of the step (behind it the step's K is in LDS).
+    # The step before has been there since the barrier before, so where the second product is long enough
+    # its first `early` blocks go first: their reads go out in front of the barrier and their matrix
+    # instructions run while the first K fragments are on their way.
+    early = DEPTH if nv >= 4 * DEPTH else 0
+    order = [("v", t) for t in range(early)] + [("s", k) for k in range(ns)] + [("v", t) for t in range(early, nv)]
+
     def read(j, slot):
-        if j < ns:
-            pc, f = j % 2, j // 2  # piece, step of 32 features
+        kind, t = order[j]
+        if kind == "s":
+            pc, f = t % 2, t // 2  # piece, step of 32 features
             return [f"ds_read_b128 {R.slot(slot)}, %{kb_in + f % kb} offset:{pc * piece + 16 * gc * (f // kb)}"]
-        t = j - ns
         base, off = f"%{vb_in + t % vbases}", 16 * gc * (t // vbases)
         return [f"ds_read_b64_tr_b16 {R.slot(slot, 0, 2)}, {base} offset:{off}",
                 f"ds_read_b64_tr_b16 {R.slot(slot, 2, 2)}, {base} offset:{off + piece}"]
 
     def mma(j, slot):
-        if j < ns:
-            pc, f = j % 2, j // 2
+        kind, t = order[j]
+        if kind == "s":
+            pc, f = t % 2, t // 2
             return [f"v_mfma_f32_16x16x32_bf16 {R.score(b, pc)}, {R.slot(slot)}, {R.q(b, f)}, {'0' if f == 0 else R.score(b, pc)}"
                     for b in range(RB)]
-        t = j - ns
         return [f"v_mfma_f32_16x16x32_bf16 {R.accum(b, t)}, {R.slot(slot)}, %{pf_in + b}, {R.accum(b, t)}" for b in range(RB)]
 
-    def covers(j):  # every score step, every second step of the second product
-        if j < ns:
+    def covers(j):  # every step up to the last score step, then every second one
+        late = j - early - ns
+        if late < 0:
             return j
-        return min(j + 1, ns + nv - 1) if (j - ns) % 2 == 0 else None
+        return min(j + 1, ns + nv - 1) if late % 2 == 0 else None
 
-    lines = pipeline(ns + nv, read, mma, covers)
-    split = min(k for k, ln in enumerate(lines) if ln.startswith("v_mfma") and " a[" in ln)
+    if early:
+        assert early == DEPTH  # (the reads that fill the ring are those of the step before)
+        lines = pipeline(ns + nv, read, mma, covers, after_fill=["s_barrier"])
+    else:
+        lines = ["s_barrier"] + pipeline(ns + nv, read, mma, covers)
+    split = 1 + max(k for k, ln in enumerate(lines) if ln.startswith("v_mfma") and " a[" not in ln)
     first, second = lines[:split], lines[split:]
     # the vector unit reads the score tiles no earlier than 16 wait states behind their last matrix instruction
     count = seen = 0
@@ -347,7 +362,7 @@ def whole_step(dqk, dv, gc, requests=0, nt=False):
         seen += ln.startswith("v_mfma")
         if count >= 16:
             break
-    assert count >= 16 and seen + 1 < 2 * nv
+    assert count >= 16 and seen + 1 < 2 * (nv - early)
     second = spread(second, softmax_groups(R, scale, m_in, th_in, sum_out, moved), first=seen + 1)
     args = ([f"floatx4 &st{2 * b + pc}" for b in range(RB) for pc in range(2)] + [f"u32x4 &pn{b}" for b in range(RB)] +
             [f"float &sum{b}" for b in range(RB)] + ["uint64_t &moved"] + [f"uint32_t kb{i}" for i in range(kb)] +
@@ -367,7 +382,7 @@ def whole_step(dqk, dv, gc, requests=0, nt=False):
         first = spread(first, request_groups(requests, at, at + requests, at + requests + 4, nt), first=4, last_fraction=0.75)
         clob, name = clob + ['"m0"'], name + "_req" + ("_nt" if nt else "")
     lines = ([MARK_BEGIN, f"s_mov_b64 {moved}, 0", "s_nop 0", "s_waitcnt lgkmcnt(0)"] + first + second + ["s_nop 7", "s_nop 7", MARK_END])
-    comment = (f"// One step: S^T = K . Q^T of the two pieces at kb.. ({ksteps} steps of 32 features), then O^T += V^T . P^T of the step\n"
+    comment = (f"// One step, from the workgroup's barrier on: S^T = K . Q^T of the two pieces at kb.. ({ksteps} steps of 32 features), then O^T += V^T . P^T of the step\n"
                f"// at vb.. ({nv} blocks of 16 value columns, probabilities pf) and, between its matrix instructions, the softmax of\n"
                "// the new score tiles st.. against the running maxima m.. as they are (no masks, scale > 0): pn the\n"
                "// probabilities, sum their sums, moved != 0 where a score exceeds th = (m + 8) / scale" +
