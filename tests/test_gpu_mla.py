@@ -125,6 +125,33 @@ def test_mla_decode_128_heads_every_form(monkeypatch, kernel, partials):
     _check(f"mla decode 128 heads kernel={kernel or 'default'} partials={partials}", got, want)
 
 
+@pytest.mark.parametrize("hq", [16, 128])
+@pytest.mark.parametrize("pad", [8, 2, 1])
+def test_mla_decode_output_rows_by_strides(monkeypatch, hq, pad):
+    """The output is addressed by strides (ttpa_paged_mla_decode): rows that start on 16-byte boundaries
+    take the merge with 16 bytes per thread (pad 8), rows on 4-byte boundaries the one with 4 (pad 2),
+    and rows on odd element offsets the float partials (pad 1).  A small grid cuts every user's context
+    into several partials."""
+    from tt_xla_amd import custom_ops as C
+
+    monkeypatch.setenv("TTPA_DECODE_WAVES_PER_CU", "0.25")
+    users, dh, dv, bs, width = 3, 576, 512, 64, 24
+    print(f"case: mla decode strided output h{hq} pad{pad}", flush=True)
+    g = torch.Generator().manual_seed(31 * hq + pad)
+    nb = users * width
+    q = _bf(g, 1, users, hq, dh)
+    key = _bf(g, nb, 1, bs, dh)
+    table = torch.randperm(nb, generator=g).view(users, width).to(torch.int32)
+    pos = torch.tensor([width * bs - 1, 130, 900], dtype=torch.int32)
+    buf = torch.full((users, hq, dv + pad), 7.0, dtype=torch.bfloat16, device="cuda")
+    out = buf[:, :, :dv]
+    C._mla_decode_launch(out, q[0].cuda(), key.cuda(), None, table.cuda(), pos.cuda(), dv, 1.0 / math.sqrt(dh), None)
+    torch.cuda.synchronize()
+    want = O.paged_flash_mla_decode(q, key, dv, table, None, pos, None)
+    _check(f"mla decode strided output h{hq} pad{pad}", out.cpu(), want[0])
+    assert (buf[:, :, dv:] == 7.0).all(), "the columns behind a row stay as they were"
+
+
 def test_mla_decode_128_heads_negative_scale():
     """scale < 0: the softmax between the matrix instructions assumes a positive scale, so every step
     must take the other one."""
