@@ -52,13 +52,13 @@ MEASURED_TRAFFIC = {
     # workload: (kernel, hash of its sources, HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of the
     # kernel, each scaled by what the same counter reads for a plain copy of known size, mean over
     # the rotating workload copies; the summaries under profiles/ hold the runs)
-    "config2": ("paged_decode_mfma16_kernel", "df5353961e3de31b", 310422502),
-    "config5": ("paged_decode_mfma16_kernel", "df5353961e3de31b", 168457019),
-    "config4": ("paged_decode_mfma16_kernel", "df5353961e3de31b", 3415575004),
-    "config3": ("prefill_kernel", "9e5dc9fce6518e7f", 244434883),
-    "latent": ("paged_decode_latent16_kernel", "96465725840a6f73", 654193569),
-    "latent128": ("paged_decode_latent128_kernel", "2f1fa3176d0b8668", 739290014),
-    "latent-prefill": ("latent_prefill_kernel", "2f1fa3176d0b8668", 332038139),
+    "config2": ("paged_decode_mfma16_kernel", "8ba1b647faebb44c", 310422335),
+    "config5": ("paged_decode_mfma16_kernel", "8ba1b647faebb44c", 168457090),
+    "config4": ("paged_decode_mfma16_kernel", "8ba1b647faebb44c", 3415575936),
+    "config3": ("prefill_kernel", "9e5dc9fce6518e7f", 244468287),
+    "latent": ("paged_decode_latent16_kernel", "cb2ca9fa245030d1", 654198293),
+    "latent128": ("paged_decode_latent128_kernel", "b26a62d6c1d0a108", 739381753),
+    "latent-prefill": ("latent_prefill_kernel", "b26a62d6c1d0a108", 332193335),
 }
 DECODE_KERNEL_NAME = {"config2": "paged_decode_mfma16_kernel", "config4": "paged_decode_mfma16_kernel",
                       "config5": "paged_decode_mfma16_kernel"}
