@@ -109,3 +109,60 @@ def test_config4_chunk_pass_full_size():
     out_h = torch.ops.tt.chunked_scaled_dot_product_attention(q, kc, (vc.float() * 0.5).to(torch.bfloat16),
                                                               w.page_table, w.chunk_start)
     torch.testing.assert_close(out_h.float() * 2, out.float(), atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("hq", [16, 128])
+def test_latent_decode_full_size(monkeypatch, hq):
+    """The latent decode workloads of the benchmark (128 users, contexts 512 .. 8192 on a shuffled
+    pool, one latent head of 576 features, 16 or 128 query heads): the oracle on the three shortest
+    users and the longest, invariance under a permutation of users, and at 128 heads agreement
+    with the workgroup-shared kernel, which computes the same thing another way."""
+    users, dh, dv, bs, lo, hi = 128, 576, 512, 64, 512, 8192
+    print(f"case: latent decode full size h{hq}", flush=True)
+    g = torch.Generator().manual_seed(11)
+    ctx = torch.randint(lo, hi + 1, (users,), generator=g)
+    w = (hi + bs) // bs
+    nb = users * w + 1
+    gd = torch.Generator(device="cuda").manual_seed(12)
+    key = torch.randn(nb, 1, bs, dh, generator=gd, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    table = (torch.randperm(nb - 1, generator=g)[: users * w] + 1).view(users, w).to(torch.int32)
+    q = torch.randn(1, users, hq, dh, generator=g).to(torch.bfloat16)
+    pos = ctx.to(torch.int32)
+    run = lambda qq, tt, pp: torch.ops.tt.paged_flash_mla_decode(qq, key, dv, tt, None, True, None, pp, None, None)  # noqa: E731
+    out = run(q.cuda(), table.cuda(), pos.cuda())
+    assert torch.isfinite(out.float()).all()
+    order = torch.argsort(pos)
+    for u in order[:3].tolist() + [int(order[-1])]:
+        nblk = int(pos[u]) // bs + 1
+        kk = key[table[u, :nblk].long().cuda()].cpu()  # this user's blocks, in order
+        t1 = torch.arange(nblk, dtype=torch.int32).view(1, nblk)
+        want = O.paged_flash_mla_decode(q[:, u : u + 1], kk, dv, t1, None, pos[u : u + 1], None)
+        err = (out[0, u].cpu().float() - want[0, 0].float()).abs().max().item()
+        print(f"latent decode h{hq} user {u} context {int(pos[u]) + 1}: max-abs error {err:.3e}", flush=True)
+        torch.testing.assert_close(out[0, u].cpu().float(), want[0, 0].float(), atol=2e-2, rtol=2e-2)
+    perm = torch.randperm(users, generator=torch.Generator().manual_seed(1))
+    out_p = run(q[:, perm].cuda(), table[perm].cuda(), pos[perm].cuda())
+    torch.testing.assert_close(out_p.float(), out[:, perm.cuda()].float(), atol=4e-3, rtol=4e-3)
+    if hq == 128:
+        monkeypatch.setenv("TTPA_LATENT_KERNEL", "wide")
+        out_w = run(q.cuda(), table.cuda(), pos.cuda())
+        torch.testing.assert_close(out_w.float(), out.float(), atol=8e-3, rtol=8e-3)
+
+
+def test_latent_prefill_full_size():
+    """4 x 2048 tokens, 16 heads over one latent head (576 / 512), causal: batch 0 against the oracle,
+    and a causal prefill of the first 1024 tokens must reproduce the first 1024 rows."""
+    b, hq, s, dh, dv = 4, 16, 2048, 576, 512
+    print("case: latent prefill full size", flush=True)
+    g = torch.Generator().manual_seed(21)
+    q = (torch.randn(b, hq, s, dh, generator=g) * 0.15).to(torch.bfloat16)
+    k = torch.randn(b, 1, s, dh, generator=g).to(torch.bfloat16)
+    scale = dh ** -0.5
+    out = torch.ops.tt.flash_mla_prefill(q.cuda(), k.cuda(), dv, None, None, True, scale)
+    assert out.shape == (b, hq, s, dv) and torch.isfinite(out.float()).all()
+    want = O.flash_mla_prefill(q[:1].float(), k[:1].float(), dv, None, None, True, scale)
+    err = (out[:1].cpu().float() - want).abs().max().item()
+    print(f"latent prefill 4 x 2048, batch 0: max-abs error {err:.3e}", flush=True)
+    torch.testing.assert_close(out[:1].cpu().float(), want, atol=2e-2, rtol=2e-2)
+    head = torch.ops.tt.flash_mla_prefill(q[:, :, :1024].contiguous().cuda(), k[:, :, :1024].contiguous().cuda(), dv, None, None, True, scale)
+    torch.testing.assert_close(head.float(), out[:, :, :1024].float(), atol=4e-3, rtol=4e-3)
