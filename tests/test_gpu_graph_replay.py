@@ -1,6 +1,6 @@
 """GPU tests of the operators under HIP-graph replay, the way bench.py (and a serving loop that
-captures its decode forward) runs them: the decode step operator and the one-operator prefill
-pass are captured once and replayed several times with fresh inputs copied into the captured
+captures its decode forward) runs them: the decode step operator, the one-operator prefill
+pass and the two latent operators are captured once and replayed several times with fresh inputs copied into the captured
 tensors and eager work between the replays; every replay must equal the eager result on the
 same inputs (caches bit for bit, outputs bit for bit: same kernels, same order)."""
 
@@ -91,3 +91,47 @@ def test_prefill_pass_replays():
         torch.cuda.synchronize()
         assert torch.equal(out_g, out_e), f"replay {it}: output differs"
         assert torch.equal(kc_g, kc_e) and torch.equal(vc_g, vc_e), f"replay {it}: caches differ"
+
+
+@pytest.mark.parametrize("hq", [16, 128])
+def test_latent_decode_replays(hq):
+    """tt::paged_flash_mla_decode (attention + merge of the partials) captured once: positions, queries
+    and cache contents change between the replays."""
+    users, dh, dv, bs, width = 5, 576, 512, 64, 20
+    g = torch.Generator(device="cuda").manual_seed(17 + hq)
+    nb = users * width + 1
+    rnd = lambda *shape: torch.randn(*shape, generator=g, device="cuda").to(torch.bfloat16)  # noqa: E731
+    q, key = rnd(1, users, hq, dh), rnd(nb, 1, bs, dh)
+    table = (torch.randperm(nb - 1, generator=g, device="cuda")[: users * width] + 1).view(users, width).to(torch.int32)
+    pos = torch.tensor([0, 63, 500, 1279, 64], dtype=torch.int32, device="cuda")
+
+    def run():
+        return torch.ops.tt.paged_flash_mla_decode(q, key, dv, table, None, True, None, pos, None, None)
+
+    graph, out_graph = _capture(run)
+    for it in range(3):
+        q.copy_(rnd(1, users, hq, dh))
+        key[1 + it :: 7].copy_(rnd(*key[1 + it :: 7].shape))
+        pos.copy_(torch.tensor([it, 63 + it, 500 - 100 * it, 1279 - it, 64 * (it + 1)], dtype=torch.int32, device="cuda"))
+        graph.replay()
+        want = run()  # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(out_graph, want), f"replay {it}: output differs"
+
+
+def test_latent_prefill_replays():
+    b, hq, s, dh, dv = 2, 16, 160, 576, 512
+    g = torch.Generator(device="cuda").manual_seed(23)
+    rnd = lambda *shape: torch.randn(*shape, generator=g, device="cuda").to(torch.bfloat16)  # noqa: E731
+    q, k = rnd(b, hq, s, dh), rnd(b, 1, s, dh)
+
+    def run():
+        return torch.ops.tt.flash_mla_prefill(q, k, dv, None, None, True, dh ** -0.5)
+
+    graph, out_graph = _capture(run)
+    for it in range(3):
+        q.copy_(rnd(b, hq, s, dh)), k.copy_(rnd(b, 1, s, dh))
+        graph.replay()
+        want = run()
+        torch.cuda.synchronize()
+        assert torch.equal(out_graph, want), f"replay {it}: output differs"
